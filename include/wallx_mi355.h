@@ -1,0 +1,170 @@
+/*
+ * wallx_mi355.h -- C ABI of libwallx_mi355.so: the wall-x per-layer MoE hot path on MI355X (gfx950).
+ *
+ * Every entry point takes raw device pointers, sizes, strides (in elements) and a HIP stream, enqueues
+ * its kernels on that stream and returns immediately: no allocation, no host synchronisation, no
+ * torch types.  Return value: WX_OK (0) or a negative wx_status; wx_last_error_string() describes the
+ * last failure on the calling thread.  Inputs are never modified.
+ *
+ * Each entry point names the reference interface it replaces (paths relative to the wall-x repository:
+ * csrc/ = native ops bound by csrc/ops.cu:11-21 into module `wallx_csrc`, ops.py =
+ * wall_x/fusions/ops.py, act.py / vl.py = wall_x/model/qwen2_5_based/modeling_qwen2_5_vl{_act,}.py).
+ */
+#ifndef WALLX_MI355_H
+#define WALLX_MI355_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* wx_stream_t; /* hipStream_t */
+
+typedef enum {
+  WX_OK = 0,
+  WX_ERR_INVALID_ARGUMENT = -1, /* null pointer, negative size, misaligned row, bad enum */
+  WX_ERR_UNSUPPORTED = -2,      /* dtype / size outside what the kernels implement */
+  WX_ERR_WORKSPACE = -3,        /* workspace too small */
+  WX_ERR_LAUNCH = -4            /* hipGetLastError() after a launch */
+} wx_status;
+
+typedef enum { WX_F32 = 0, WX_F16 = 1, WX_BF16 = 2 } wx_dtype;
+typedef enum { WX_I32 = 0, WX_I64 = 1, WX_U8 = 2 /* torch.bool */ } wx_itype;
+/* Which rotary channel takes which of the (t, h, w) position planes:
+ * WX_MROPE_HF   sections [s0,s1,s2,s0,s1,s2] cycling t,h,w,t,h,w     (vl.py:763-769, the PyTorch path)
+ * WX_MROPE_CSRC sections [2*s0, 2*s1, 2*s2] contiguous t,h,w           (csrc/rope.cu:104-117) */
+typedef enum { WX_MROPE_HF = 0, WX_MROPE_CSRC = 1 } wx_mrope_layout;
+
+const char* wx_last_error_string(void);
+int wx_abi_version(void);
+
+/* ------------------------------------------------------------------------------------------------
+ * Token partition.  Replaces cub::DeviceRadixSort::SortPairs + moe_permute_topK_row_map
+ * (csrc/permute.cu:39-67, 472-494) and the caller's per-expert bookkeeping (act.py:1274-1283).
+ *
+ * ids[num_tokens * num_topk] (row-major [T, K]) hold expert ids in [0, num_experts), num_experts <= 256.
+ * Stable counting partition:  row_id_map[k*T + t] = sorted position of (t, k), or -1 when that position
+ * is >= num_out_tokens (num_out_tokens <= 0 means T*K).  sorted_row_id[p] = t*K + k (may be NULL).
+ * expert_offsets[num_experts + 1] = exclusive prefix of per-expert counts (may be NULL).
+ * status (may be NULL): device word, set to 1 when an id lies outside [0, num_experts) (such ids are
+ * clamped into range so the outputs stay a permutation), otherwise left untouched.
+ * workspace: wx_partition_workspace_bytes(T*K) bytes of device memory, 256-byte aligned. */
+size_t wx_partition_workspace_bytes(int64_t num_expanded_tokens);
+int wx_partition_build(const void* ids, int id_type /* wx_itype */, int64_t num_tokens, int num_topk,
+                       int num_experts, int64_t num_out_tokens, int32_t* row_id_map,
+                       int32_t* sorted_row_id, int32_t* expert_offsets, int32_t* status,
+                       void* workspace, size_t workspace_bytes, wx_stream_t stream);
+
+/* Row scatter of the permute op: out[row_id_map[k*T + t], :] = x[t, :] for every k with a map entry
+ * != -1.  Replaces moe_permute_topK_kernel, forward branch (csrc/permute.cu:156-262, 294-305).
+ * num_cols * sizeof(dtype) must be a multiple of 16 and rows 16-byte aligned. */
+int wx_permute_rows(const void* x, void* out, const int32_t* row_id_map, int64_t num_tokens,
+                    int num_topk, int64_t num_cols, int dtype /* wx_dtype */, wx_stream_t stream);
+
+/* out[t, :] = sum_k prob[t, k] * y[row_id_map[k*T + t], :] (entries == -1 skipped; all skipped -> 0).
+ * probs == NULL or num_topk == 1: no scaling (csrc/permute.cu:405-415 drops probs at K == 1).
+ * Replaces moe_recover_topK_kernel (csrc/permute.cu:69-154, 398-441, 638-779). */
+int wx_unpermute_rows(const void* y, void* out, const int32_t* row_id_map, const float* probs,
+                      int64_t num_tokens, int num_topk, int64_t num_cols, int dtype,
+                      wx_stream_t stream);
+
+/* Backward of wx_unpermute_rows: act_grad[row_id_map[k*T+t], :] = grad_out[t, :] * prob[t, k]
+ * (no factor at K == 1), prob_grad[t, k] = <grad_out[t, :], y_fwd[row, :]> in fp32 (written only when
+ * K > 1; prob_grad may be NULL at K == 1).  Rows of act_grad that no token maps to are not written.
+ * Replaces moe_permute_topK_kernel, unpermute-backward branch (csrc/permute.cu:156-262, 781-942). */
+int wx_unpermute_rows_bwd(const void* grad_out, const void* y_fwd, void* act_grad, float* prob_grad,
+                          const int32_t* row_id_map, const float* probs, int64_t num_tokens,
+                          int num_topk, int64_t num_cols, int dtype, wx_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * Dual asymmetric grouped GEMM: out_e = op(in_e) @ op(w_e), e in {0, 1}, in ONE launch; bf16 in/out,
+ * fp32 accumulate.  Replaces AsymmetricDualExpertGemm (csrc/dual_asym_grouped_gemm.cu:308-366,
+ * ops.py:6-165).  trans_a: in_e stored [k_e, m_e]; trans_b: w_e stored [n_e, k_e] (nn.Linear layout).
+ * All matrices packed row-major; k_e and n_e multiples of 8 (16-byte rows).  m_e == 0 is allowed. */
+int wx_dual_gemm(const void* in0, const void* in1, const void* w0, const void* w1, void* out0,
+                 void* out1, int64_t m0, int64_t n0, int64_t k0, int64_t m1, int64_t n1, int64_t k1,
+                 int trans_a, int trans_b, wx_stream_t stream);
+
+/* Both experts' SwiGLU FFN over expert-sorted rows, two launches (gate/up + SwiGLU, then down), each
+ * covering both experts:  out[r, :] = down_e( silu(x[r] @ gate_e^T) * (x[r] @ up_e^T) ) for rows
+ * r in [expert_offsets[e], expert_offsets[e+1]).  Replaces the per-expert loop of
+ * SparseMoeBlock.forward over BlockSparseMLP (act.py:79-82, 142-154).
+ * x, out: [num_rows, hidden] bf16;  gate_e, up_e: [inter_e, hidden];  down_e: [hidden, inter_e].
+ * expert_offsets: DEVICE int32[3] (from wx_partition_build), read by the kernels -- no host sync.
+ * hmid: device scratch, num_rows * max(inter0, inter1) bf16.
+ * Intermediate rounding follows eager bf16 evaluation: gate, up, silu(gate) and the product are each
+ * rounded to bf16 (fp32 accumulation inside each contraction). */
+int wx_dual_swiglu_ffn(const void* x, void* out, const int32_t* expert_offsets, const void* gate0,
+                       const void* up0, const void* down0, const void* gate1, const void* up1,
+                       const void* down1, void* hmid, int64_t num_rows, int64_t hidden,
+                       int64_t inter0, int64_t inter1, wx_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * 3D multimodal RoPE:  out = x * cos_sel + rotate_half(x) * sin_sel for q and k, where channel d of
+ * cos_sel / sin_sel comes from plane axis(d) of cos / sin [3, B, S, D] (contiguous, dtype of q).
+ * Replaces launch_multimodal_rope_forward (csrc/rope.cu:48-178, 453-509; ops.py:402-497) and follows
+ * apply_multimodal_rotary_pos_emb (vl.py:731-773) when layout == WX_MROPE_HF.
+ * q is addressed as q[b, h, s, d] = q + b*q_sb + h*q_sh + s*q_ss + d (strides in elements, d
+ * contiguous), so the [B, S, H, D] projection output can be passed without a transposing copy; same for
+ * k and the two outputs.  Each product and the sum are rounded to the storage dtype, as eager
+ * evaluation does.  D must be a multiple of 16 and at most 256. */
+int wx_mrope_apply(const void* q, const void* k, const void* cos, const void* sin, void* q_out,
+                   void* k_out, int64_t batch, int64_t seq, int n_q_heads, int n_kv_heads,
+                   int head_dim, const int64_t q_strides[3] /* b, h, s */, const int64_t k_strides[3],
+                   const int64_t qo_strides[3], const int64_t ko_strides[3],
+                   const int mrope_section[3], int layout /* wx_mrope_layout */, int dtype,
+                   wx_stream_t stream);
+
+/* Adjoint w.r.t. q and k: g_in = g*cos_sel + rotate_half^T(g*sin_sel).  Replaces
+ * launch_multimodal_rope_backward (csrc/rope.cu:181-330, 511-571).  fp32 math, one rounding. */
+int wx_mrope_apply_bwd(const void* gq_out, const void* gk_out, const void* cos, const void* sin,
+                       void* gq, void* gk, int64_t batch, int64_t seq, int n_q_heads,
+                       int n_kv_heads, int head_dim, const int64_t gqo_strides[3],
+                       const int64_t gko_strides[3], const int64_t gq_strides[3],
+                       const int64_t gk_strides[3], const int mrope_section[3], int layout,
+                       int dtype, wx_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * 3D position ids.  Replaces get_rope_index (csrc/rope_index.cu:464-569) with the semantics of the
+ * PyTorch path (act.py:929-1149), exact integer arithmetic.
+ * input_ids [B, S] int64; attention_mask [B, S] int64 or NULL (all ones);
+ * image_grid_thw [n_image, 3] / video_grid_thw [n_video, 3] int64 (NULL when absent);
+ * second_per_grid_ts [n_video] fp32 or NULL (1.0).  Both grids NULL selects the text-only branch
+ * (act.py:1123-1149).  position_ids [3, B, S] int64, deltas [B] int64.
+ * status (may be NULL): device word set to 1 when a row is malformed in a way that makes the PyTorch
+ * path raise (a vision item without its tokens, more items than grids, a fully masked row).
+ * workspace: wx_rope_index_workspace_bytes(B) bytes. */
+size_t wx_rope_index_workspace_bytes(int64_t batch);
+int wx_rope_index(const int64_t* input_ids, const int64_t* attention_mask,
+                  const int64_t* image_grid_thw, int64_t n_image, const int64_t* video_grid_thw,
+                  int64_t n_video, const float* second_per_grid_ts, int64_t batch, int64_t seq,
+                  int spatial_merge_size, int64_t image_token_id, int64_t video_token_id,
+                  int64_t vision_start_token_id, float tokens_per_second, int64_t* position_ids,
+                  int64_t* deltas, int32_t* status, void* workspace, size_t workspace_bytes,
+                  wx_stream_t stream);
+
+/* Vision-tower rotary table.  Replaces fused_rot_pos_emb_cuda (csrc/rot_pos.cu:187-312) and follows
+ * rot_pos_emb (vl.py:473-500).  grid_thw [n_grid, 3] int32 or int64 on the device; total_patches =
+ * sum t*h*w (the caller sizes the outputs from its host copy of grid_thw).
+ * table (may be NULL): fp32 [total_patches, 2*n_freq] = [h_pos * inv_freq, w_pos * inv_freq].
+ * pos_ids (may be NULL): int64 [total_patches, 2] = (h_pos, w_pos). */
+int wx_rot_pos_emb(const float* inv_freq, int n_freq, const void* grid_thw, int grid_type,
+                   int64_t n_grid, int spatial_merge_size, int64_t total_patches, float* table,
+                   int64_t* pos_ids, wx_stream_t stream);
+
+/* Vision-tower window permutation.  Replaces get_window_index_cuda (csrc/window_index.cu:208-286)
+ * and follows get_window_index (vl.py:502-547) with one cumulative entry per non-empty window.
+ * grid_thw [n_grid, 3] int32 or int64 on the device.  window_index int32 [total_tokens], total_tokens =
+ * sum t*(h/m)*(w/m); cu_window_seqlens int32 [total_windows + 1], total_windows =
+ * sum t*ceil(h/m/ws)*ceil(w/m/ws) (the caller sizes both from its host copy of grid_thw). */
+int wx_window_index(const void* grid_thw, int grid_type, int64_t n_grid, int spatial_merge_size,
+                    int vit_merger_window_size, int spatial_merge_unit, int64_t total_tokens,
+                    int64_t total_windows, int32_t* window_index, int32_t* cu_window_seqlens,
+                    wx_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* WALLX_MI355_H */

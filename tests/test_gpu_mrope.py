@@ -1,0 +1,107 @@
+"""GPU parity: 3D M-RoPE apply against the oracle (eager bf16 evaluation of vl.py:731-773)."""
+
+import warnings
+
+import pytest
+import torch
+
+import oracle
+from wallx_mi355 import native, workloads as wl
+from wallx_mi355.fusions import ops
+
+pytestmark = pytest.mark.gpu
+
+ATOL, RTOL = 2e-2, 1e-2  # |x - ref| <= 2e-2 + 1e-2 |ref| for bf16 outputs
+
+
+def _close(got, ref, atol=ATOL, rtol=RTOL):
+    got, ref = got.float().cpu(), ref.float()
+    bad = (got - ref).abs() > atol + rtol * ref.abs()
+    assert not bad.any(), f"{int(bad.sum())} of {bad.numel()} outside tolerance, max abs {float((got - ref).abs().max())}"
+
+
+def _inputs(B, S, dtype, seed, hq=4, hk=2):
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn(B, S, hq, 128, generator=g).to(dtype)
+    k = torch.randn(B, S, hk, 128, generator=g).to(dtype)
+    pos = torch.randint(0, 2000, (3, B, S), generator=g)
+    cos, sin = oracle.rotary_cos_sin_ref(pos, wl.text_inv_freq(), dtype)
+    return q, k, cos, sin
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("layout", ["hf", "csrc"])
+def test_mrope_matches_eager_bit_for_bit(dev, dtype, layout):
+    q, k, cos, sin = _inputs(2, 37, dtype, 5)
+    qt, kt = q.transpose(1, 2), k.transpose(1, 2)  # [B, H, S, D] views of token-major memory
+    rq, rk = oracle.mrope_apply_ref(qt, kt, cos, sin, list(wl.MROPE_SECTION), layout, eager_rounding=True)
+    native.set_mrope_layout(layout)
+    try:
+        gq, gk = ops.multimodal_rope(qt.to(dev), kt.to(dev), cos.to(dev), sin.to(dev), list(wl.MROPE_SECTION))
+    finally:
+        native.set_mrope_layout("hf")
+    assert gq.shape == rq.shape and gq.is_contiguous() and gk.is_contiguous()
+    # the kernel rounds each product and the sum exactly like eager evaluation, so the match is exact
+    assert torch.equal(gq.cpu(), rq) and torch.equal(gk.cpu(), rk)
+    _close(gq, rq)
+
+
+def test_mrope_strided_views_need_no_copy(dev):
+    q, k, cos, sin = _inputs(3, 20, torch.bfloat16, 7)
+    qd, kd = q.to(dev), k.to(dev)
+    with warnings.catch_warnings():
+        warnings.simplefilter("error")  # no "discontiguous" warning: strided [B,H,S,D] views are read in place
+        gq, gk = ops.multimodal_rope(qd.transpose(1, 2), kd.transpose(1, 2), cos.to(dev), sin.to(dev), [16, 24, 24])
+    cq, ck = ops.multimodal_rope(qd.transpose(1, 2).contiguous(), kd.transpose(1, 2).contiguous(), cos.to(dev),
+                                 sin.to(dev), [16, 24, 24])
+    assert torch.equal(gq, cq) and torch.equal(gk, ck)
+
+
+def test_mrope_config2_full_size(dev):
+    """B = 16, S = 896, q [14336,16,128], k [14336,2,128] bf16 with the real position ids of the layout."""
+    ids, grid = wl.config2_tokens()
+    pos, _ = oracle.rope_index_ref(ids, 2, wl.IMAGE_TOKEN_ID, wl.VIDEO_TOKEN_ID, wl.VISION_START_TOKEN_ID, 2,
+                                   image_grid_thw=grid)
+    cos, sin = oracle.rotary_cos_sin_ref(pos, wl.text_inv_freq(), torch.bfloat16)
+    q, k = wl.qk_inputs(16, 896)
+    qt, kt = q.transpose(1, 2), k.transpose(1, 2)
+    rq, rk = oracle.mrope_apply_ref(qt, kt, cos, sin, list(wl.MROPE_SECTION), "hf")
+    gq, gk = ops.multimodal_rope(qt.to(dev), kt.to(dev), cos.to(dev), sin.to(dev), list(wl.MROPE_SECTION))
+    _close(gq, rq)
+    _close(gk, rk)
+    assert torch.equal(gq.cpu(), rq) and torch.equal(gk.cpu(), rk)
+    # fp32-math oracle (one rounding) is within the stated tolerance as well
+    fq, fk = oracle.mrope_apply_ref(qt, kt, cos, sin, list(wl.MROPE_SECTION), "hf", eager_rounding=False)
+    _close(gq, fq)
+    # rotation pairs (d, d + 64) keep their norm up to bf16 rounding
+    n_in = (qt[..., :64].float() ** 2 + qt[..., 64:].float() ** 2)
+    n_out = (gq[..., :64].float().cpu() ** 2 + gq[..., 64:].float().cpu() ** 2)
+    assert torch.all((n_in - n_out).abs() <= 0.05 * n_in + 0.05)
+
+
+def test_mrope_non_multiple_of_8_sections(dev):
+    q, k, cos, sin = _inputs(1, 9, torch.bfloat16, 9)
+    sec = [10, 27, 27]
+    rq, rk = oracle.mrope_apply_ref(q.transpose(1, 2), k.transpose(1, 2), cos, sin, sec, "hf")
+    gq, gk = ops.multimodal_rope(q.transpose(1, 2).to(dev), k.transpose(1, 2).to(dev), cos.to(dev), sin.to(dev), sec)
+    assert torch.equal(gq.cpu(), rq) and torch.equal(gk.cpu(), rk)
+    with pytest.raises(RuntimeError, match="covers"):
+        ops.multimodal_rope(q.transpose(1, 2).to(dev), k.transpose(1, 2).to(dev), cos.to(dev), sin.to(dev), [16, 24, 20])
+
+
+@pytest.mark.parametrize("layout", ["hf", "csrc"])
+def test_mrope_backward(dev, layout):
+    q, k, cos, sin = _inputs(2, 11, torch.float32, 13)
+    qd = q.transpose(1, 2).to(dev).requires_grad_(True)
+    kd = k.transpose(1, 2).to(dev).requires_grad_(True)
+    native.set_mrope_layout(layout)
+    try:
+        oq, ok = ops.multimodal_rope(qd, kd, cos.to(dev), sin.to(dev), list(wl.MROPE_SECTION))
+        g = torch.Generator().manual_seed(3)
+        gq, gk = torch.randn(oq.shape, generator=g), torch.randn(ok.shape, generator=g)
+        torch.autograd.backward([oq, ok], [gq.to(dev), gk.to(dev)])
+    finally:
+        native.set_mrope_layout("hf")
+    rq, rk = oracle.mrope_apply_bwd_ref(gq, gk, cos, sin, list(wl.MROPE_SECTION), layout)
+    assert torch.allclose(qd.grad.cpu(), rq, rtol=1e-5, atol=1e-5)
+    assert torch.allclose(kd.grad.cpu(), rk, rtol=1e-5, atol=1e-5)

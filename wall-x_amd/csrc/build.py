@@ -1,0 +1,82 @@
+"""Builds libwallx_mi355.so (the C-ABI library) for gfx950 with hipcc.
+
+    python wall-x_amd/csrc/build.py [--force]
+
+Sources are compiled one by one (objects under csrc/build/) and linked into
+wall-x_amd/wallx_mi355/libwallx_mi355.so, next to the Python package that loads it.
+"""
+
+import os
+import shutil
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+REPO = os.path.dirname(os.path.dirname(HERE))
+INCLUDE = os.path.join(REPO, "include")
+OUT_DIR = os.path.join(os.path.dirname(HERE), "wallx_mi355")
+LIB = os.path.join(OUT_DIR, "libwallx_mi355.so")
+OBJ_DIR = os.path.join(HERE, "build")
+
+SOURCES = ["common.hip", "partition.hip", "dual_gemm.hip", "mrope.hip", "rope_index.hip", "vision_index.hip"]
+HEADERS = ["common.h", "grid_prefix.h", os.path.join(INCLUDE, "wallx_mi355.h")]
+
+FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
+    # packed fp32 math is kept off for every kernel in this library
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+    f"-I{INCLUDE}", f"-I{HERE}",
+]
+
+
+def _hipcc() -> str:
+    exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(exe):
+        raise RuntimeError("hipcc not found; libwallx_mi355.so cannot be built")
+    return exe
+
+
+def _newer(target: str, deps) -> bool:
+    if not os.path.exists(target):
+        return False
+    t = os.path.getmtime(target)
+    return all(os.path.getmtime(d) <= t for d in deps)
+
+
+def _run(cmd):
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    noise = "is not a recognized feature for this target"
+    err = "\n".join(line for line in proc.stderr.splitlines() if noise not in line)
+    if proc.returncode != 0:
+        raise RuntimeError(f"command failed: {' '.join(cmd)}\n{proc.stdout}\n{err}")
+    if err.strip():
+        sys.stderr.write(err + "\n")
+
+
+def build(force: bool = False, verbose: bool = True) -> str:
+    hipcc = _hipcc()
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    headers = [h if os.path.isabs(h) else os.path.join(HERE, h) for h in HEADERS]
+    objs, jobs = [], []
+    for src in SOURCES:
+        path = os.path.join(HERE, src)
+        obj = os.path.join(OBJ_DIR, src.replace(".hip", ".o"))
+        objs.append(obj)
+        if force or not _newer(obj, [path] + headers):
+            jobs.append([hipcc] + FLAGS + ["-c", path, "-o", obj])
+    if jobs:
+        if verbose:
+            print(f"[wallx_mi355] compiling {len(jobs)} source(s) for gfx950", flush=True)
+        with ThreadPoolExecutor(max_workers=min(len(jobs), 6)) as pool:
+            list(pool.map(_run, jobs))
+    if jobs or force or not _newer(LIB, objs):
+        _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs)
+        if verbose:
+            print(f"[wallx_mi355] linked {LIB}", flush=True)
+    return LIB
+
+
+if __name__ == "__main__":
+    build(force="--force" in sys.argv)

@@ -1,0 +1,42 @@
+// Error reporting and device queries shared by every entry point of libwallx_mi355.
+#include "common.h"
+
+#include <cstdarg>
+#include <cstdio>
+
+namespace wx {
+
+static thread_local char g_error[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int check_launch(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e == hipSuccess) return WX_OK;
+  return fail(WX_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e));
+}
+
+int device_cu_count() {
+  static thread_local int cached_dev = -1;
+  static thread_local int cached_cus = 0;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return 256;
+  if (dev != cached_dev) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cached_dev = dev;
+    cached_cus = n;
+  }
+  return cached_cus;
+}
+
+}  // namespace wx
+
+extern "C" const char* wx_last_error_string(void) { return wx::g_error; }
+extern "C" int wx_abi_version(void) { return 1; }

@@ -1,0 +1,208 @@
+// 3D multimodal RoPE apply (forward and adjoint) for gfx950.
+//
+// HBM-bound elementwise kernel.  A thread owns one rotation group of a token: the 8 channels
+// [8j, 8j+8) of the low half together with their partners in the high half, so both operands of every
+// rotation are in registers and each access is a full 16-byte lane (32 bytes for fp32).  The thread
+// loads the selected cos/sin values for its channels once and then walks the heads of q and k that
+// its head group covers, which amortises the table over the heads.  q/k/outputs are addressed
+// through (batch, head, seq) strides so the projection's [B, S, H, D] memory is read in place.
+#include "common.h"
+
+namespace wx {
+namespace {
+
+constexpr int kMaxHeadDim = 256;
+
+struct AxisTable {
+  uint8_t axis[kMaxHeadDim];        // position plane (0 t, 1 h, 2 w) per channel
+  uint8_t uniform[kMaxHeadDim / 8]; // 1 when the 8 channels starting at 8*i share one plane
+};
+
+struct Strides {
+  int64_t b, h, s;
+};
+
+template <int DT>
+__device__ __forceinline__ void load8(const void* base, int64_t elem_off, float* f) {
+  if constexpr (DT == WX_F32) {
+    const u32x4* p = reinterpret_cast<const u32x4*>(static_cast<const float*>(base) + elem_off);
+    unpack16<DT>(p[0], f);
+    unpack16<DT>(p[1], f + 4);
+  } else {
+    unpack16<DT>(*reinterpret_cast<const u32x4*>(static_cast<const uint16_t*>(base) + elem_off), f);
+  }
+}
+template <int DT>
+__device__ __forceinline__ void store8(void* base, int64_t elem_off, const float* f) {
+  if constexpr (DT == WX_F32) {
+    u32x4* p = reinterpret_cast<u32x4*>(static_cast<float*>(base) + elem_off);
+    p[0] = pack16<DT>(f);
+    p[1] = pack16<DT>(f + 4);
+  } else {
+    *reinterpret_cast<u32x4*>(static_cast<uint16_t*>(base) + elem_off) = pack16<DT>(f);
+  }
+}
+template <int DT>
+__device__ __forceinline__ float load1(const void* base, int64_t elem_off) {
+  if constexpr (DT == WX_F32) return static_cast<const float*>(base)[elem_off];
+  else return Elem<DT>::load(static_cast<const uint16_t*>(base)[elem_off]);
+}
+
+// cos/sin for channels [d0, d0+8) of one token, each channel from its own position plane.
+template <int DT>
+__device__ __forceinline__ void load_selected(const void* table, const AxisTable& ax, int64_t plane_stride,
+                                              int64_t token_off, int d0, float* f) {
+  if (ax.uniform[d0 >> 3]) {
+    load8<DT>(table, ax.axis[d0] * plane_stride + token_off + d0, f);
+  } else {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) f[e] = load1<DT>(table, ax.axis[d0 + e] * plane_stride + token_off + d0 + e);
+  }
+}
+
+template <int DT, bool BWD>
+__global__ __launch_bounds__(256) void mrope_kernel(
+    const void* __restrict__ q, const void* __restrict__ k, const void* __restrict__ cos_t,
+    const void* __restrict__ sin_t, void* __restrict__ q_out, void* __restrict__ k_out, int64_t n_tokens,
+    int64_t seq, int n_q_heads, int n_kv_heads, int head_dim, Strides sq, Strides sk, Strides sqo, Strides sko,
+    AxisTable ax, int head_groups) {
+  const int groups = head_dim / 16;  // rotation groups per head
+  const int64_t gid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const int j = static_cast<int>(gid % groups);
+  const int hg = static_cast<int>((gid / groups) % head_groups);
+  const int64_t token = gid / (static_cast<int64_t>(groups) * head_groups);
+  if (token >= n_tokens) return;
+  const int64_t b = token / seq, s = token - b * seq;
+  const int half = head_dim / 2;
+  const int d_lo = 8 * j, d_hi = half + 8 * j;
+  const int64_t plane = n_tokens * head_dim, tok_off = token * head_dim;
+
+  float c_lo[8], c_hi[8], s_lo[8], s_hi[8];
+  load_selected<DT>(cos_t, ax, plane, tok_off, d_lo, c_lo);
+  load_selected<DT>(cos_t, ax, plane, tok_off, d_hi, c_hi);
+  load_selected<DT>(sin_t, ax, plane, tok_off, d_lo, s_lo);
+  load_selected<DT>(sin_t, ax, plane, tok_off, d_hi, s_hi);
+
+  const int n_heads = n_q_heads + n_kv_heads;
+  for (int h = hg; h < n_heads; h += head_groups) {
+    const bool is_q = h < n_q_heads;
+    const int hh = is_q ? h : h - n_q_heads;
+    const Strides& si = is_q ? sq : sk;
+    const Strides& so = is_q ? sqo : sko;
+    const void* in = is_q ? q : k;
+    void* out = is_q ? q_out : k_out;
+    const int64_t in_off = b * si.b + hh * si.h + s * si.s;
+    const int64_t out_off = b * so.b + hh * so.h + s * so.s;
+    float x_lo[8], x_hi[8], o_lo[8], o_hi[8];
+    load8<DT>(in, in_off + d_lo, x_lo);
+    load8<DT>(in, in_off + d_hi, x_hi);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      if constexpr (!BWD) {
+        // eager evaluation order of (x * cos) + (rotate_half(x) * sin): every product and the sum are
+        // rounded to the storage type; rotate_half(x) = (-x_hi, x_lo)
+        const float p1 = Elem<DT>::round(__fmul_rn(x_lo[e], c_lo[e]));
+        const float p2 = Elem<DT>::round(__fmul_rn(-x_hi[e], s_lo[e]));
+        o_lo[e] = __fadd_rn(p1, p2);
+        const float p3 = Elem<DT>::round(__fmul_rn(x_hi[e], c_hi[e]));
+        const float p4 = Elem<DT>::round(__fmul_rn(x_lo[e], s_hi[e]));
+        o_hi[e] = __fadd_rn(p3, p4);
+      } else {
+        // adjoint: g*cos + rotate_half^T(g*sin), rotate_half^T(y) = (y_hi, -y_lo)
+        o_lo[e] = x_lo[e] * c_lo[e] + x_hi[e] * s_hi[e];
+        o_hi[e] = x_hi[e] * c_hi[e] - x_lo[e] * s_lo[e];
+      }
+    }
+    store8<DT>(out, out_off + d_lo, o_lo);
+    store8<DT>(out, out_off + d_hi, o_hi);
+  }
+}
+
+int build_axis_table(const int sec[3], int head_dim, int layout, AxisTable& ax) {
+  int d = 0;
+  auto put = [&](int axis, int n) {
+    for (int i = 0; i < n && d < kMaxHeadDim; ++i) ax.axis[d++] = static_cast<uint8_t>(axis);
+  };
+  if (layout == WX_MROPE_HF) {
+    for (int rep = 0; rep < 2; ++rep)
+      for (int a = 0; a < 3; ++a) put(a, sec[a]);
+  } else if (layout == WX_MROPE_CSRC) {
+    put(0, 2 * sec[0]);
+    put(1, 2 * sec[1]);
+    while (d < head_dim) put(2, 1);  // csrc/rope.cu:104-117: everything past s0+s1 is the w plane
+  } else {
+    return fail(WX_ERR_INVALID_ARGUMENT, "mrope: bad layout %d", layout);
+  }
+  if (d != head_dim)
+    return fail(WX_ERR_INVALID_ARGUMENT, "mrope: mrope_section [%d,%d,%d] covers %d channels, head_dim is %d", sec[0],
+                sec[1], sec[2], d, head_dim);
+  for (int c = 0; c < head_dim / 8; ++c) {
+    bool same = true;
+    for (int e = 1; e < 8; ++e) same = same && ax.axis[8 * c + e] == ax.axis[8 * c];
+    ax.uniform[c] = same;
+  }
+  return WX_OK;
+}
+
+template <bool BWD>
+int launch(const void* q, const void* k, const void* cos_t, const void* sin_t, void* q_out, void* k_out,
+           int64_t batch, int64_t seq, int n_q, int n_kv, int head_dim, const int64_t* sq, const int64_t* sk,
+           const int64_t* sqo, const int64_t* sko, const int sec[3], int layout, int dtype, wx_stream_t stream) {
+  const char* who = BWD ? "wx_mrope_apply_bwd" : "wx_mrope_apply";
+  if (batch < 0 || seq < 0 || n_q < 0 || n_kv < 0) return fail(WX_ERR_INVALID_ARGUMENT, "%s: negative size", who);
+  if (head_dim <= 0 || head_dim % 16 != 0 || head_dim > kMaxHeadDim)
+    return fail(WX_ERR_UNSUPPORTED, "%s: head_dim %d must be a multiple of 16 and <= %d", who, head_dim, kMaxHeadDim);
+  if (!sq || !sk || !sqo || !sko || !sec) return fail(WX_ERR_INVALID_ARGUMENT, "%s: null stride/section", who);
+  const int64_t n_tokens = batch * seq;
+  if (n_tokens == 0 || n_q + n_kv == 0) return WX_OK;
+  if (!cos_t || !sin_t || (n_q && (!q || !q_out)) || (n_kv && (!k || !k_out)))
+    return fail(WX_ERR_INVALID_ARGUMENT, "%s: null pointer", who);
+  const int align = dtype == WX_F32 ? 4 : 8;  // elements per 16 bytes
+  const int64_t* all[4] = {sq, sk, sqo, sko};
+  for (auto* st : all)
+    for (int i = 0; i < 3; ++i)
+      if (st[i] % align != 0) return fail(WX_ERR_UNSUPPORTED, "%s: strides must keep rows 16-byte aligned", who);
+  AxisTable ax{};
+  if (int rc = build_axis_table(sec, head_dim, layout, ax)) return rc;
+  const Strides a{sq[0], sq[1], sq[2]}, b{sk[0], sk[1], sk[2]}, c{sqo[0], sqo[1], sqo[2]}, d{sko[0], sko[1], sko[2]};
+  // spread heads over a few threads per rotation group when there are few tokens to fill the chip
+  const int groups = head_dim / 16;
+  int head_groups = 1;
+  const int64_t target_threads = static_cast<int64_t>(device_cu_count()) * 2048;
+  while (head_groups * 2 <= n_q + n_kv && n_tokens * groups * head_groups < target_threads) head_groups *= 2;
+  const int64_t threads = n_tokens * groups * head_groups;
+  const dim3 grid(static_cast<unsigned>((threads + 255) / 256)), block(256);
+  hipStream_t s = as_stream(stream);
+#define WX_LAUNCH(DT)                                                                                             \
+  hipLaunchKernelGGL((mrope_kernel<DT, BWD>), grid, block, 0, s, q, k, cos_t, sin_t, q_out, k_out, n_tokens, seq, \
+                     n_q, n_kv, head_dim, a, b, c, d, ax, head_groups)
+  switch (dtype) {
+    case WX_F32: WX_LAUNCH(WX_F32); break;
+    case WX_F16: WX_LAUNCH(WX_F16); break;
+    case WX_BF16: WX_LAUNCH(WX_BF16); break;
+    default: return fail(WX_ERR_UNSUPPORTED, "%s: dtype %d", who, dtype);
+  }
+#undef WX_LAUNCH
+  return check_launch(who);
+}
+
+}  // namespace
+}  // namespace wx
+
+extern "C" int wx_mrope_apply(const void* q, const void* k, const void* cos, const void* sin, void* q_out,
+                              void* k_out, int64_t batch, int64_t seq, int n_q_heads, int n_kv_heads, int head_dim,
+                              const int64_t q_strides[3], const int64_t k_strides[3], const int64_t qo_strides[3],
+                              const int64_t ko_strides[3], const int mrope_section[3], int layout, int dtype,
+                              wx_stream_t stream) {
+  return wx::launch<false>(q, k, cos, sin, q_out, k_out, batch, seq, n_q_heads, n_kv_heads, head_dim, q_strides,
+                           k_strides, qo_strides, ko_strides, mrope_section, layout, dtype, stream);
+}
+
+extern "C" int wx_mrope_apply_bwd(const void* gq_out, const void* gk_out, const void* cos, const void* sin, void* gq,
+                                  void* gk, int64_t batch, int64_t seq, int n_q_heads, int n_kv_heads, int head_dim,
+                                  const int64_t gqo_strides[3], const int64_t gko_strides[3],
+                                  const int64_t gq_strides[3], const int64_t gk_strides[3],
+                                  const int mrope_section[3], int layout, int dtype, wx_stream_t stream) {
+  return wx::launch<true>(gq_out, gk_out, cos, sin, gq, gk, batch, seq, n_q_heads, n_kv_heads, head_dim, gqo_strides,
+                          gko_strides, gq_strides, gk_strides, mrope_section, layout, dtype, stream);
+}

@@ -1,0 +1,417 @@
+// Modality-routed token partition, row scatter (permute) and row gather (unpermute) for gfx950.
+//
+// The partition is a stable counting sort over at most 256 expert bins.  The key stream is cut into
+// segments, one per wavefront.  Inside a segment a wavefront walks 64 keys at a time and ranks equal
+// keys with ballots (rank = popcount of the equal-key mask below the lane), so order within a bin is
+// source order -- the contract of a stable sort -- without any sorting network or atomics.
+//   pass 1  partition_count    per-segment histogram  -> hist[segment][256]
+//   pass 2  partition_scatter  per-block prefix over hist (bins, then earlier segments), then ranks
+// The row movers are pure HBM streams: one wavefront per token row, 16-byte lanes, several rows in flight.
+#include "common.h"
+
+namespace wx {
+namespace {
+
+constexpr int kBins = 256;
+constexpr int kWavesPerBlock = 4;
+constexpr int kBlock = kWavesPerBlock * kWave;
+
+__host__ __device__ inline int64_t segment_len(int64_t n) {
+  // 512 keys per wavefront until that would need more than 1024 segments
+  int64_t seg = 512;
+  if (n > seg * 1024) seg = ((n + 1023) / 1024 + 63) / 64 * 64;
+  return seg;
+}
+
+__device__ __forceinline__ int load_key(const void* ids, int itype, int64_t i, int num_experts, bool& bad) {
+  int64_t v = load_index(ids, itype, i);
+  if (v < 0) { bad = true; v = 0; }
+  if (v >= num_experts) { bad = true; v = num_experts - 1; }
+  return static_cast<int>(v);
+}
+
+// Calls f(key, mask) once per distinct key among the active lanes; mask = lanes holding that key.
+template <typename F>
+__device__ __forceinline__ void for_each_key_group(int key, bool active, F f) {
+  uint64_t todo = __ballot(active);
+  while (todo) {
+    const int leader = __ffsll(static_cast<long long>(todo)) - 1;
+    const int k = __builtin_amdgcn_readlane(key, leader);
+    const uint64_t mask = __ballot(active && key == k);
+    f(k, mask);
+    todo &= ~mask;
+  }
+}
+
+__global__ __launch_bounds__(kBlock) void partition_count(const void* __restrict__ ids, int itype, int64_t n,
+                                                          int num_experts, int64_t seg_len,
+                                                          int32_t* __restrict__ hist, int32_t* status) {
+  __shared__ int32_t s_hist[kWavesPerBlock][kBins];
+  const int w = threadIdx.x / kWave, lane = lane_id();
+  for (int i = lane; i < kBins; i += kWave) s_hist[w][i] = 0;
+  const int64_t seg = static_cast<int64_t>(blockIdx.x) * kWavesPerBlock + w;
+  const int64_t begin = seg * seg_len;
+  const int64_t end = begin + seg_len < n ? begin + seg_len : n;
+  bool bad = false;
+  for (int64_t base = begin; base < end; base += kWave) {
+    const int64_t i = base + lane;
+    const bool active = i < end;
+    const int key = active ? load_key(ids, itype, i, num_experts, bad) : 0;
+    for_each_key_group(key, active, [&](int k, uint64_t mask) {
+      if (lane == 0) s_hist[w][k] += __popcll(mask);
+    });
+  }
+  if (begin < n) {
+    for (int i = lane; i < kBins; i += kWave) hist[seg * kBins + i] = s_hist[w][i];
+  }
+  if (status != nullptr && __ballot(bad) != 0 && lane == 0) *status = 1;
+}
+
+__global__ __launch_bounds__(kBlock) void partition_scatter(
+    const void* __restrict__ ids, int itype, int64_t num_tokens, int num_topk, int num_experts,
+    int64_t num_out, int64_t seg_len, int64_t num_seg, const int32_t* __restrict__ hist,
+    int32_t* __restrict__ row_id_map, int32_t* __restrict__ sorted_row_id,
+    int32_t* __restrict__ expert_offsets) {
+  __shared__ int32_t s_run[kWavesPerBlock][kBins];  // next free sorted position per (wave, bin)
+  __shared__ int32_t s_wave_total[kWavesPerBlock];
+  const int tid = threadIdx.x, w = tid / kWave, lane = lane_id();
+  const int64_t n = num_tokens * num_topk;
+  const int64_t first_seg = static_cast<int64_t>(blockIdx.x) * kWavesPerBlock;
+
+  // bin `tid`: rows of this bin in all segments (total) and in segments before this block (before)
+  int32_t total = 0, before = 0;
+  for (int64_t s = 0; s < num_seg; ++s) {
+    const int32_t v = hist[s * kBins + tid];
+    total += v;
+    if (s < first_seg) before += v;
+  }
+  // exclusive prefix of `total` over the 256 bins: wave scan, then wave totals through LDS
+  int32_t incl = total;
+#pragma unroll
+  for (int d = 1; d < kWave; d <<= 1) {
+    const int32_t up = __shfl_up(incl, d);
+    if (lane >= d) incl += up;
+  }
+  if (lane == kWave - 1) s_wave_total[w] = incl;
+  __syncthreads();
+  int32_t bin_base = incl - total;
+  for (int i = 0; i < w; ++i) bin_base += s_wave_total[i];
+  if (blockIdx.x == 0 && expert_offsets != nullptr) {
+    if (tid < num_experts) expert_offsets[tid] = bin_base;
+    if (tid == 0) expert_offsets[num_experts] = static_cast<int32_t>(n);
+  }
+  int32_t run = bin_base + before;
+#pragma unroll
+  for (int i = 0; i < kWavesPerBlock; ++i) {
+    s_run[i][tid] = run;
+    if (first_seg + i < num_seg) run += hist[(first_seg + i) * kBins + tid];
+  }
+  __syncthreads();
+
+  const int64_t seg = first_seg + w;
+  const int64_t begin = seg * seg_len;
+  const int64_t end = begin + seg_len < n ? begin + seg_len : n;
+  const uint64_t below = (1ull << lane) - 1ull;
+  bool bad = false;
+  for (int64_t base = begin; base < end; base += kWave) {
+    const int64_t i = base + lane;
+    const bool active = i < end;
+    const int key = active ? load_key(ids, itype, i, num_experts, bad) : 0;
+    int32_t pos = 0;
+    for_each_key_group(key, active, [&](int k, uint64_t mask) {
+      const int32_t start = s_run[w][k];  // same address for the whole wave: LDS broadcast
+      if (active && key == k) pos = start + __popcll(mask & below);
+      __builtin_amdgcn_wave_barrier();
+      if (lane == 0) s_run[w][k] = start + __popcll(mask);
+      __builtin_amdgcn_wave_barrier();
+    });
+    if (active) {
+      const int64_t t = i / num_topk, k = i - t * num_topk;
+      row_id_map[k * num_tokens + t] = pos < num_out ? pos : -1;
+      if (sorted_row_id != nullptr) sorted_row_id[pos] = static_cast<int32_t>(i);
+    }
+  }
+}
+
+// ---- row movers ---------------------------------------------------------------------------------
+constexpr int kMoverWaves = 4;
+
+__device__ __forceinline__ u32x4 ld16(const u32x4* p) { return __builtin_nontemporal_load(p); }
+__device__ __forceinline__ void st16(u32x4* p, const u32x4& v) { __builtin_nontemporal_store(v, p); }
+
+// out[row_id_map[k*T + t]] = x[t] for every k; one wavefront per source row.
+__global__ __launch_bounds__(kMoverWaves* kWave) void permute_rows_kernel(
+    const u32x4* __restrict__ x, u32x4* __restrict__ out, const int32_t* __restrict__ row_id_map,
+    int64_t num_tokens, int num_topk, int64_t vec_per_row) {
+  const int lane = lane_id();
+  const int64_t wave = static_cast<int64_t>(blockIdx.x) * kMoverWaves + threadIdx.x / kWave;
+  const int64_t n_waves = static_cast<int64_t>(gridDim.x) * kMoverWaves;
+  for (int64_t t = wave; t < num_tokens; t += n_waves) {
+    const u32x4* src = x + t * vec_per_row;
+    if (num_topk == 1) {
+      const int32_t dst_row = row_id_map[t];
+      if (dst_row < 0) continue;
+      u32x4* dst = out + static_cast<int64_t>(dst_row) * vec_per_row;
+      int64_t v = lane;
+      for (; v + 3 * kWave < vec_per_row; v += 4 * kWave) {
+        const u32x4 a = ld16(src + v), b = ld16(src + v + kWave), c = ld16(src + v + 2 * kWave),
+                    d = ld16(src + v + 3 * kWave);
+        st16(dst + v, a); st16(dst + v + kWave, b); st16(dst + v + 2 * kWave, c); st16(dst + v + 3 * kWave, d);
+      }
+      for (; v < vec_per_row; v += kWave) st16(dst + v, ld16(src + v));
+    } else {
+      for (int64_t v = lane; v < vec_per_row; v += kWave) {
+        const u32x4 a = ld16(src + v);
+        for (int k = 0; k < num_topk; ++k) {
+          const int32_t dst_row = row_id_map[k * num_tokens + t];
+          if (dst_row >= 0) st16(out + static_cast<int64_t>(dst_row) * vec_per_row + v, a);
+        }
+      }
+    }
+  }
+}
+
+// out[t] = y[row_id_map[t]] (zeros when the map entry is -1); one wavefront per destination row.
+__global__ __launch_bounds__(kMoverWaves* kWave) void gather_rows_kernel(
+    const u32x4* __restrict__ y, u32x4* __restrict__ out, const int32_t* __restrict__ row_id_map,
+    int64_t num_tokens, int64_t vec_per_row) {
+  const int lane = lane_id();
+  const int64_t wave = static_cast<int64_t>(blockIdx.x) * kMoverWaves + threadIdx.x / kWave;
+  const int64_t n_waves = static_cast<int64_t>(gridDim.x) * kMoverWaves;
+  for (int64_t t = wave; t < num_tokens; t += n_waves) {
+    const int32_t src_row = row_id_map[t];
+    u32x4* dst = out + t * vec_per_row;
+    if (src_row < 0) {
+      for (int64_t v = lane; v < vec_per_row; v += kWave) st16(dst + v, u32x4{0, 0, 0, 0});
+      continue;
+    }
+    const u32x4* src = y + static_cast<int64_t>(src_row) * vec_per_row;
+    int64_t v = lane;
+    for (; v + 3 * kWave < vec_per_row; v += 4 * kWave) {
+      const u32x4 a = ld16(src + v), b = ld16(src + v + kWave), c = ld16(src + v + 2 * kWave),
+                  d = ld16(src + v + 3 * kWave);
+      st16(dst + v, a); st16(dst + v + kWave, b); st16(dst + v + 2 * kWave, c); st16(dst + v + 3 * kWave, d);
+    }
+    for (; v < vec_per_row; v += kWave) st16(dst + v, ld16(src + v));
+  }
+}
+
+// out[t] = sum_k prob[t,k] * y[row_id_map[k*T+t]] for topK > 1.  The reference kernel multiplies and
+// accumulates in the storage type (csrc/permute.cu:69-154 with TCompute == T for 16-bit types), one
+// rounding per operation in k order; Elem<DT>::round reproduces that.
+template <int DT>
+__global__ __launch_bounds__(kMoverWaves* kWave) void combine_rows_kernel(
+    const u32x4* __restrict__ y, u32x4* __restrict__ out, const int32_t* __restrict__ row_id_map,
+    const float* __restrict__ probs, int64_t num_tokens, int num_topk, int64_t vec_per_row) {
+  constexpr int E = elems_per_16<DT>();
+  const int lane = lane_id();
+  const int64_t wave = static_cast<int64_t>(blockIdx.x) * kMoverWaves + threadIdx.x / kWave;
+  const int64_t n_waves = static_cast<int64_t>(gridDim.x) * kMoverWaves;
+  for (int64_t t = wave; t < num_tokens; t += n_waves) {
+    for (int64_t v = lane; v < vec_per_row; v += kWave) {
+      float acc[E];
+#pragma unroll
+      for (int e = 0; e < E; ++e) acc[e] = 0.f;
+      for (int k = 0; k < num_topk; ++k) {
+        const int32_t r = row_id_map[k * num_tokens + t];
+        if (r < 0) continue;  // a dropped copy adds nothing (for k == 0 the sum starts at zero)
+        float f[E];
+        unpack16<DT>(ld16(y + static_cast<int64_t>(r) * vec_per_row + v), f);
+        const float p = probs != nullptr ? Elem<DT>::round(probs[t * num_topk + k]) : 1.f;
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+          const float term = probs != nullptr ? Elem<DT>::round(f[e] * p) : f[e];
+          acc[e] = k == 0 ? term : Elem<DT>::round(acc[e] + term);
+        }
+      }
+      st16(out + t * vec_per_row + v, pack16<DT>(acc));
+    }
+  }
+}
+
+// Backward of the weighted combine; one wavefront per token.
+template <int DT>
+__global__ __launch_bounds__(kMoverWaves* kWave) void combine_rows_bwd_kernel(
+    const u32x4* __restrict__ grad_out, const u32x4* __restrict__ y_fwd, u32x4* __restrict__ act_grad,
+    float* __restrict__ prob_grad, const int32_t* __restrict__ row_id_map, const float* __restrict__ probs,
+    int64_t num_tokens, int num_topk, int64_t vec_per_row) {
+  constexpr int E = elems_per_16<DT>();
+  const int lane = lane_id();
+  const int64_t wave = static_cast<int64_t>(blockIdx.x) * kMoverWaves + threadIdx.x / kWave;
+  const int64_t n_waves = static_cast<int64_t>(gridDim.x) * kMoverWaves;
+  const bool weighted = num_topk > 1 && probs != nullptr;
+  for (int64_t t = wave; t < num_tokens; t += n_waves) {
+    for (int k = 0; k < num_topk; ++k) {
+      const int32_t r = row_id_map[k * num_tokens + t];
+      float dot = 0.f;
+      if (r >= 0) {
+        const float p = weighted ? Elem<DT>::round(probs[t * num_topk + k]) : 1.f;
+        for (int64_t v = lane; v < vec_per_row; v += kWave) {
+          const u32x4 g16 = ld16(grad_out + t * vec_per_row + v);
+          if (!weighted) {
+            st16(act_grad + static_cast<int64_t>(r) * vec_per_row + v, g16);
+            continue;
+          }
+          float g[E], yv[E], o[E];
+          unpack16<DT>(g16, g);
+          unpack16<DT>(ld16(y_fwd + static_cast<int64_t>(r) * vec_per_row + v), yv);
+#pragma unroll
+          for (int e = 0; e < E; ++e) {
+            o[e] = Elem<DT>::round(g[e] * p);
+            dot += Elem<DT>::round(g[e] * yv[e]);
+          }
+          st16(act_grad + static_cast<int64_t>(r) * vec_per_row + v, pack16<DT>(o));
+        }
+      }
+      if (weighted && prob_grad != nullptr) {
+#pragma unroll
+        for (int d = kWave / 2; d > 0; d >>= 1) dot += __shfl_xor(dot, d);
+        if (lane == 0) prob_grad[t * num_topk + k] = dot;
+      }
+    }
+  }
+}
+
+int elem_bytes(int dtype) {
+  switch (dtype) {
+    case WX_F32: return 4;
+    case WX_F16:
+    case WX_BF16: return 2;
+    default: return 0;
+  }
+}
+
+int mover_grid(int64_t rows) {
+  // enough resident wavefronts to cover HBM latency: 8 blocks of 4 waves per CU, capped by the row count
+  const int64_t want = static_cast<int64_t>(device_cu_count()) * 8;
+  const int64_t need = (rows + kMoverWaves - 1) / kMoverWaves;
+  return static_cast<int>(need < want ? (need < 1 ? 1 : need) : want);
+}
+
+int check_rows(const char* who, const void* a, const void* b, const void* map, int64_t num_tokens, int num_topk,
+               int64_t num_cols, int dtype) {
+  const int eb = elem_bytes(dtype);
+  if (eb == 0) return fail(WX_ERR_UNSUPPORTED, "%s: dtype %d is not fp32/fp16/bf16", who, dtype);
+  if (num_tokens < 0 || num_cols <= 0 || num_topk < 1) return fail(WX_ERR_INVALID_ARGUMENT, "%s: bad sizes", who);
+  if (num_topk > 128) return fail(WX_ERR_UNSUPPORTED, "%s: num_topK cannot exceed 128.", who);
+  if ((num_cols * eb) % 16 != 0)
+    return fail(WX_ERR_UNSUPPORTED, "%s: row size %lld bytes is not a multiple of 16", who,
+                static_cast<long long>(num_cols * eb));
+  if (num_tokens > 0 && (a == nullptr || b == nullptr || map == nullptr))
+    return fail(WX_ERR_INVALID_ARGUMENT, "%s: null pointer", who);
+  if ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) & 15)
+    return fail(WX_ERR_INVALID_ARGUMENT, "%s: buffers must be 16-byte aligned", who);
+  if (num_tokens * num_topk > INT32_MAX) return fail(WX_ERR_UNSUPPORTED, "%s: more than 2^31-1 rows", who);
+  return WX_OK;
+}
+
+}  // namespace
+}  // namespace wx
+
+using namespace wx;
+
+extern "C" size_t wx_partition_workspace_bytes(int64_t n) {
+  if (n <= 0) return 256;
+  const int64_t seg = segment_len(n);
+  const int64_t num_seg = (n + seg - 1) / seg;
+  const int64_t padded = (num_seg + kWavesPerBlock - 1) / kWavesPerBlock * kWavesPerBlock;
+  return static_cast<size_t>(padded) * kBins * sizeof(int32_t);
+}
+
+extern "C" int wx_partition_build(const void* ids, int id_type, int64_t num_tokens, int num_topk, int num_experts,
+                                  int64_t num_out_tokens, int32_t* row_id_map, int32_t* sorted_row_id,
+                                  int32_t* expert_offsets, int32_t* status, void* workspace,
+                                  size_t workspace_bytes, wx_stream_t stream) {
+  if (num_tokens < 0 || num_topk < 1) return fail(WX_ERR_INVALID_ARGUMENT, "wx_partition_build: bad sizes");
+  if (num_topk > 128) return fail(WX_ERR_UNSUPPORTED, "wx_partition_build: num_topK cannot exceed 128.");
+  if (num_experts < 1 || num_experts > kBins)
+    return fail(WX_ERR_UNSUPPORTED, "wx_partition_build: num_experts %d outside [1, %d]", num_experts, kBins);
+  if (id_type != WX_I32 && id_type != WX_I64 && id_type != WX_U8)
+    return fail(WX_ERR_INVALID_ARGUMENT, "wx_partition_build: bad id_type %d", id_type);
+  const int64_t n = num_tokens * num_topk;
+  if (n > INT32_MAX) return fail(WX_ERR_UNSUPPORTED, "wx_partition_build: more than 2^31-1 expanded tokens");
+  if (n > 0 && (ids == nullptr || row_id_map == nullptr || workspace == nullptr))
+    return fail(WX_ERR_INVALID_ARGUMENT, "wx_partition_build: null pointer");
+  if (workspace_bytes < wx_partition_workspace_bytes(n))
+    return fail(WX_ERR_WORKSPACE, "wx_partition_build: workspace %zu < %zu bytes", workspace_bytes,
+                wx_partition_workspace_bytes(n));
+  hipStream_t s = as_stream(stream);
+  const int64_t seg = segment_len(n > 0 ? n : 1);
+  const int64_t num_seg = n > 0 ? (n + seg - 1) / seg : 0;
+  // at least one block even for n == 0 so expert_offsets are written
+  const int blocks = static_cast<int>(num_seg > 0 ? (num_seg + kWavesPerBlock - 1) / kWavesPerBlock : 1);
+  const int64_t num_out = num_out_tokens > 0 ? num_out_tokens : n;
+  int32_t* hist = static_cast<int32_t*>(workspace);
+  if (n > 0) {
+    hipLaunchKernelGGL(partition_count, dim3(blocks), dim3(kBlock), 0, s, ids, id_type, n, num_experts, seg, hist,
+                       status);
+    if (int rc = check_launch("partition_count")) return rc;
+  }
+  hipLaunchKernelGGL(partition_scatter, dim3(blocks), dim3(kBlock), 0, s, ids, id_type, num_tokens, num_topk,
+                     num_experts, num_out, seg, num_seg, hist, row_id_map, sorted_row_id, expert_offsets);
+  return check_launch("partition_scatter");
+}
+
+extern "C" int wx_permute_rows(const void* x, void* out, const int32_t* row_id_map, int64_t num_tokens,
+                               int num_topk, int64_t num_cols, int dtype, wx_stream_t stream) {
+  if (int rc = check_rows("wx_permute_rows", x, out, row_id_map, num_tokens, num_topk, num_cols, dtype)) return rc;
+  if (num_tokens == 0) return WX_OK;
+  const int64_t vec = num_cols * elem_bytes(dtype) / 16;
+  hipLaunchKernelGGL(permute_rows_kernel, dim3(mover_grid(num_tokens)), dim3(kMoverWaves * kWave), 0,
+                     as_stream(stream), static_cast<const u32x4*>(x), static_cast<u32x4*>(out), row_id_map,
+                     num_tokens, num_topk, vec);
+  return check_launch("permute_rows_kernel");
+}
+
+extern "C" int wx_unpermute_rows(const void* y, void* out, const int32_t* row_id_map, const float* probs,
+                                 int64_t num_tokens, int num_topk, int64_t num_cols, int dtype,
+                                 wx_stream_t stream) {
+  if (int rc = check_rows("wx_unpermute_rows", y, out, row_id_map, num_tokens, num_topk, num_cols, dtype)) return rc;
+  if (num_tokens == 0) return WX_OK;
+  const int64_t vec = num_cols * elem_bytes(dtype) / 16;
+  const dim3 grid(mover_grid(num_tokens)), block(kMoverWaves * kWave);
+  hipStream_t s = as_stream(stream);
+  const u32x4* yy = static_cast<const u32x4*>(y);
+  u32x4* oo = static_cast<u32x4*>(out);
+  if (num_topk == 1) {
+    hipLaunchKernelGGL(gather_rows_kernel, grid, block, 0, s, yy, oo, row_id_map, num_tokens, vec);
+  } else if (dtype == WX_F32) {
+    hipLaunchKernelGGL(combine_rows_kernel<WX_F32>, grid, block, 0, s, yy, oo, row_id_map, probs, num_tokens,
+                       num_topk, vec);
+  } else if (dtype == WX_F16) {
+    hipLaunchKernelGGL(combine_rows_kernel<WX_F16>, grid, block, 0, s, yy, oo, row_id_map, probs, num_tokens,
+                       num_topk, vec);
+  } else {
+    hipLaunchKernelGGL(combine_rows_kernel<WX_BF16>, grid, block, 0, s, yy, oo, row_id_map, probs, num_tokens,
+                       num_topk, vec);
+  }
+  return check_launch("wx_unpermute_rows");
+}
+
+extern "C" int wx_unpermute_rows_bwd(const void* grad_out, const void* y_fwd, void* act_grad, float* prob_grad,
+                                     const int32_t* row_id_map, const float* probs, int64_t num_tokens,
+                                     int num_topk, int64_t num_cols, int dtype, wx_stream_t stream) {
+  if (int rc = check_rows("wx_unpermute_rows_bwd", grad_out, act_grad, row_id_map, num_tokens, num_topk, num_cols,
+                          dtype))
+    return rc;
+  if (num_topk > 1 && (probs == nullptr || y_fwd == nullptr || prob_grad == nullptr))
+    return fail(WX_ERR_INVALID_ARGUMENT, "wx_unpermute_rows_bwd: probs, y_fwd and prob_grad are required for topK > 1");
+  if (num_tokens == 0) return WX_OK;
+  const int64_t vec = num_cols * elem_bytes(dtype) / 16;
+  const dim3 grid(mover_grid(num_tokens)), block(kMoverWaves * kWave);
+  hipStream_t s = as_stream(stream);
+  const u32x4* g = static_cast<const u32x4*>(grad_out);
+  const u32x4* yf = static_cast<const u32x4*>(y_fwd);
+  u32x4* ag = static_cast<u32x4*>(act_grad);
+  if (dtype == WX_F32) {
+    hipLaunchKernelGGL(combine_rows_bwd_kernel<WX_F32>, grid, block, 0, s, g, yf, ag, prob_grad, row_id_map, probs,
+                       num_tokens, num_topk, vec);
+  } else if (dtype == WX_F16) {
+    hipLaunchKernelGGL(combine_rows_bwd_kernel<WX_F16>, grid, block, 0, s, g, yf, ag, prob_grad, row_id_map, probs,
+                       num_tokens, num_topk, vec);
+  } else {
+    hipLaunchKernelGGL(combine_rows_bwd_kernel<WX_BF16>, grid, block, 0, s, g, yf, ag, prob_grad, row_id_map, probs,
+                       num_tokens, num_topk, vec);
+  }
+  return check_launch("wx_unpermute_rows_bwd");
+}

@@ -1,0 +1,86 @@
+"""ctypes binding of libwallx_mi355.so (the C ABI declared in include/wallx_mi355.h).
+
+The library is built in-tree by ``wall-x_amd/csrc/build.py``; there is no fallback path: if it is
+missing, loading raises.
+"""
+
+import ctypes
+import os
+import threading
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libwallx_mi355.so")
+
+WX_F32, WX_F16, WX_BF16 = 0, 1, 2
+WX_I32, WX_I64, WX_U8 = 0, 1, 2
+WX_MROPE_HF, WX_MROPE_CSRC = 0, 1
+
+_c = ctypes
+_vp, _i64, _i32, _sz, _f32 = _c.c_void_p, _c.c_int64, _c.c_int, _c.c_size_t, _c.c_float
+
+# name -> (restype, argtypes); mirrors include/wallx_mi355.h one to one
+PROTOTYPES = {
+    "wx_last_error_string": (_c.c_char_p, []),
+    "wx_abi_version": (_i32, []),
+    "wx_partition_workspace_bytes": (_sz, [_i64]),
+    "wx_partition_build": (_i32, [_vp, _i32, _i64, _i32, _i32, _i64, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "wx_permute_rows": (_i32, [_vp, _vp, _vp, _i64, _i32, _i64, _i32, _vp]),
+    "wx_unpermute_rows": (_i32, [_vp, _vp, _vp, _vp, _i64, _i32, _i64, _i32, _vp]),
+    "wx_unpermute_rows_bwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i32, _i64, _i32, _vp]),
+    "wx_dual_gemm": (_i32, [_vp] * 6 + [_i64] * 6 + [_i32, _i32, _vp]),
+    "wx_dual_swiglu_ffn": (_i32, [_vp] * 10 + [_i64] * 4 + [_vp]),
+    "wx_mrope_apply": (_i32, [_vp] * 6 + [_i64, _i64, _i32, _i32, _i32] + [_c.POINTER(_i64)] * 4
+                       + [_c.POINTER(_i32), _i32, _i32, _vp]),
+    "wx_mrope_apply_bwd": (_i32, [_vp] * 6 + [_i64, _i64, _i32, _i32, _i32] + [_c.POINTER(_i64)] * 4
+                           + [_c.POINTER(_i32), _i32, _i32, _vp]),
+    "wx_rope_index_workspace_bytes": (_sz, [_i64]),
+    "wx_rope_index": (_i32, [_vp, _vp, _vp, _i64, _vp, _i64, _vp, _i64, _i64, _i32, _i64, _i64, _i64, _f32,
+                             _vp, _vp, _vp, _vp, _sz, _vp]),
+    "wx_rot_pos_emb": (_i32, [_vp, _i32, _vp, _i32, _i64, _i32, _i64, _vp, _vp, _vp]),
+    "wx_window_index": (_i32, [_vp, _i32, _i64, _i32, _i32, _i32, _i64, _i64, _vp, _vp, _vp]),
+}
+
+_lock = threading.Lock()
+_lib = None
+
+
+class WallxLibraryError(RuntimeError):
+    pass
+
+
+def load():
+    """Returns the loaded library; raises WallxLibraryError when it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    with _lock:
+        if _lib is None:
+            if not os.path.exists(LIB_PATH):
+                raise WallxLibraryError(
+                    f"{LIB_PATH} is missing: build it with `python wall-x_amd/csrc/build.py` "
+                    "(hipcc, gfx950). There is no fallback implementation.")
+            lib = ctypes.CDLL(LIB_PATH)
+            for name, (res, args) in PROTOTYPES.items():
+                fn = getattr(lib, name)  # AttributeError here means header and library disagree
+                fn.restype = res
+                fn.argtypes = args
+            _lib = lib
+    return _lib
+
+
+def check(rc: int, exc=RuntimeError):
+    if rc != 0:
+        msg = load().wx_last_error_string().decode("utf-8", "replace")
+        raise exc(f"wallx_mi355: {msg} (status {rc})")
+
+
+def call(name: str, *args, exc=RuntimeError):
+    check(getattr(load(), name)(*args), exc)
+
+
+def i64x3(vals):
+    return (_i64 * 3)(*[int(v) for v in vals])
+
+
+def i32x3(vals):
+    return (_i32 * 3)(*[int(v) for v in vals])

@@ -1,0 +1,118 @@
+"""Drop-in for the reference's modality-routed MoE block (act.py:67-162) on the fused kernels.
+
+The reference's SparseMoeBlock permutes the tokens, loops over the experts in Python (six cuBLAS GEMMs,
+four elementwise kernels and two slice copies per layer, bounds read from CPU tensors) and unpermutes.
+Here one layer is: partition (2 small launches, reusable across layers) -> row scatter -> gate/up + SwiGLU
+for both experts (1 launch) -> down for both experts (1 launch) -> row gather.  The per-expert row ranges
+stay on the device (expert_offsets from the partition), so nothing synchronises with the host.
+
+Parameter names match the reference (``experts.{e}.{gate,up,down}_proj.weight``), so its checkpoints load.
+"""
+
+from dataclasses import dataclass
+from typing import List, Optional
+
+import torch
+from torch import nn
+
+from . import native
+
+
+class ExpertMLP(nn.Module):
+    """Weights of one SwiGLU expert, laid out like BlockSparseMLP (act.py:67-82)."""
+
+    def __init__(self, config: dict):
+        super().__init__()
+        self.hidden_size = config["hidden_size"]
+        self.intermediate_size = config["intermediate_size"]
+        self.hidden_act = config.get("hidden_act", "silu")
+        if self.hidden_act != "silu":
+            raise ValueError(f"the fused expert kernel implements silu gating only, got {self.hidden_act!r}")
+        self.gate_proj = nn.Linear(self.hidden_size, self.intermediate_size, bias=False)
+        self.up_proj = nn.Linear(self.hidden_size, self.intermediate_size, bias=False)
+        self.down_proj = nn.Linear(self.intermediate_size, self.hidden_size, bias=False)
+
+    def weights(self):
+        return (self.gate_proj.weight, self.up_proj.weight, self.down_proj.weight)
+
+
+@dataclass
+class Routing:
+    """Result of the token partition; valid for every layer of a forward pass (token types do not change)."""
+
+    row_id_map: torch.Tensor      # int32 [T]: sorted position of each token
+    expert_offsets: torch.Tensor  # int32 [E + 1] on the device
+    num_tokens: int
+
+
+class _DualExpertFFN(torch.autograd.Function):
+    """Inference-only for now: the fused path has no backward (training falls outside this build's scope)."""
+
+    @staticmethod
+    def forward(ctx, x_sorted, expert_offsets, hmid, *weights):
+        w = ((weights[0], weights[1], weights[2]), (weights[3], weights[4], weights[5]))
+        return native.dual_swiglu_ffn(x_sorted, expert_offsets, w, hmid=hmid)
+
+    @staticmethod
+    def backward(ctx, grad):
+        raise NotImplementedError("wallx_mi355.moe: the fused dual-expert FFN implements the forward pass only")
+
+
+class SparseMoeBlock(nn.Module):
+    """Same constructor and forward signature as the reference block (act.py:85-162)."""
+
+    def __init__(self, config, num_experts: int):
+        super().__init__()
+        if num_experts != 2:
+            raise ValueError("the dual-expert kernel runs exactly two experts (VL and action)")
+        self.num_experts = num_experts
+        self.experts = nn.ModuleList([ExpertMLP(config.experts[i]) for i in range(num_experts)])
+        self._partition_ws: Optional[List[torch.Tensor]] = None
+        self._hmid: Optional[torch.Tensor] = None
+
+    def route(self, experts_indices: torch.Tensor) -> Routing:
+        """Stable partition of the flattened token types; reuse the result for all layers of a forward."""
+        ids = experts_indices.reshape(-1)
+        row_id_map, offsets, _, self._partition_ws = native.partition(ids, self.num_experts, 0, self._partition_ws)
+        return Routing(row_id_map, offsets, ids.numel())
+
+    def forward(self, hidden_states: torch.Tensor, experts_indices: torch.Tensor,
+                start_indices: Optional[torch.Tensor] = None, end_indices: Optional[torch.Tensor] = None,
+                routing: Optional[Routing] = None) -> torch.Tensor:
+        """hidden_states [B, S, H] bf16; experts_indices [B, S] (bool or integer expert id).
+
+        start_indices / end_indices are accepted for signature parity and not read: the row ranges come from
+        the partition on the device.
+        """
+        del start_indices, end_indices
+        batch, seq, hidden = hidden_states.shape
+        x = hidden_states.reshape(-1, hidden)
+        if x.dtype != torch.bfloat16:
+            raise RuntimeError("All tensors must be BFloat16 for this kernel")
+        if routing is None:
+            routing = self.route(experts_indices)
+        if routing.num_tokens != x.size(0):
+            raise RuntimeError(f"routing was built for {routing.num_tokens} tokens, got {x.size(0)}")
+        x_sorted = native.permute_rows(x.contiguous(), routing.row_id_map, 1, x.size(0))
+        need = x.size(0) * max(e.intermediate_size for e in self.experts)
+        if self._hmid is None or self._hmid.numel() < need or self._hmid.device != x.device:
+            self._hmid = torch.empty(need, dtype=torch.bfloat16, device=x.device)
+        flat = [w for e in self.experts for w in e.weights()]
+        y_sorted = _DualExpertFFN.apply(x_sorted, routing.expert_offsets, self._hmid, *flat)
+        y = native.unpermute(y_sorted, routing.row_id_map, torch.tensor([]), x.size(0), 1)
+        return y.view(batch, seq, hidden)
+
+
+def moe_layer_forward(x: torch.Tensor, token_types: torch.Tensor, weights, routing: Optional[Routing] = None,
+                      hmid: Optional[torch.Tensor] = None, workspace=None):
+    """Functional form of one layer: permute -> dual-expert SwiGLU FFN -> unpermute.
+
+    x [T, H] bf16, token_types [T] (bool / int), weights ((g0,u0,d0),(g1,u1,d1)).  Returns (y [T, H], routing).
+    """
+    if routing is None:
+        row_id_map, offsets, _, _ = native.partition(token_types.reshape(-1), 2, 0, workspace)
+        routing = Routing(row_id_map, offsets, x.size(0))
+    x_sorted = native.permute_rows(x, routing.row_id_map, 1, x.size(0))
+    y_sorted = native.dual_swiglu_ffn(x_sorted, routing.expert_offsets, weights, hmid=hmid)
+    y = native.unpermute(y_sorted, routing.row_id_map, torch.tensor([]), x.size(0), 1)
+    return y, routing

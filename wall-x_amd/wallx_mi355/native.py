@@ -1,0 +1,383 @@
+"""The nine native ops of the reference's ``wallx_csrc`` extension module (csrc/ops.cu:11-21), with the
+same names, argument order and ownership rules, implemented on libwallx_mi355.so.
+
+torch is used for allocation and stream lookup only; every computation is a HIP kernel behind the C ABI.
+Nothing here falls back to PyTorch math: without the library, or with CPU tensors, calls raise.
+"""
+
+from typing import List, Optional, Tuple
+
+import torch
+
+from . import _lib
+from ._lib import WX_BF16, WX_F16, WX_F32, WX_I32, WX_I64, WX_U8, WX_MROPE_CSRC, WX_MROPE_HF
+
+_DTYPES = {torch.float32: WX_F32, torch.float16: WX_F16, torch.bfloat16: WX_BF16}
+_ITYPES = {torch.int32: WX_I32, torch.int64: WX_I64, torch.bool: WX_U8, torch.uint8: WX_U8}
+
+# Channel layout used by rope()/rope_bwd().  "hf" follows the reference's PyTorch path
+# (vl.py:763-769); "csrc" follows its CUDA kernel (csrc/rope.cu:104-117).  They differ on 80 of 128
+# channels for mrope_section [16, 24, 24] and coincide only when the three position planes are equal.
+_mrope_layout = WX_MROPE_HF
+
+
+def set_mrope_layout(name: str) -> None:
+    global _mrope_layout
+    _mrope_layout = {"hf": WX_MROPE_HF, "csrc": WX_MROPE_CSRC}[name]
+
+
+def get_mrope_layout() -> str:
+    return "hf" if _mrope_layout == WX_MROPE_HF else "csrc"
+
+
+def _stream(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    if t is None or t.numel() == 0:
+        return None
+    return t.data_ptr()
+
+
+def _need_cuda(name: str, t: torch.Tensor) -> None:
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must be a CUDA tensor")
+
+
+def _dtype_code(t: torch.Tensor) -> int:
+    try:
+        return _DTYPES[t.dtype]
+    except KeyError:
+        raise RuntimeError("Wrong activation tensor type.")  # csrc/permute.cu:626
+
+
+class _DeviceGuard:
+    """Makes the tensor's device current for the launch when it is not already."""
+
+    def __init__(self, t: torch.Tensor):
+        self.idx = t.device.index
+        self.prev = None
+
+    def __enter__(self):
+        cur = torch.cuda.current_device()
+        if self.idx is not None and self.idx != cur:
+            self.prev = cur
+            torch.cuda.set_device(self.idx)
+
+    def __exit__(self, *exc):
+        if self.prev is not None:
+            torch.cuda.set_device(self.prev)
+
+
+# ----------------------------------------------------------------------------- dual grouped GEMM
+def asym_dual_gmm(input_expert0, input_expert1, weight_expert0, weight_expert1, output_expert0,
+                  output_expert1, trans_a: bool, trans_b: bool) -> None:
+    """csrc/dual_asym_grouped_gemm.cu:308-366.  Writes into the caller's outputs."""
+    ts = (input_expert0, input_expert1, weight_expert0, weight_expert1, output_expert0, output_expert1)
+    for t in ts:
+        _need_cuda("All tensors", t)
+        if t.device != ts[0].device:
+            raise RuntimeError("All tensors must be on the same device")
+        if t.dtype != torch.bfloat16:
+            raise RuntimeError("All tensors must be BFloat16 for this kernel")
+    if not (output_expert0.is_contiguous() and output_expert1.is_contiguous()):
+        # the reference silently writes a temporary here (csrc/dual_asym_grouped_gemm.cu:335-336); refuse instead
+        raise RuntimeError("output tensors must be contiguous")
+    a0, a1 = input_expert0.contiguous(), input_expert1.contiguous()
+    w0, w1 = weight_expert0.contiguous(), weight_expert1.contiguous()
+
+    def dims(a, w):
+        m, k = (a.size(1), a.size(0)) if trans_a else (a.size(0), a.size(1))
+        n, kw = (w.size(0), w.size(1)) if trans_b else (w.size(1), w.size(0))
+        if k != kw:
+            raise RuntimeError(f"inner dimensions disagree: {k} vs {kw}")
+        return m, n, k
+
+    m0, n0, k0 = dims(a0, w0)
+    m1, n1, k1 = dims(a1, w1)
+    if tuple(output_expert0.shape) != (m0, n0) or tuple(output_expert1.shape) != (m1, n1):
+        raise RuntimeError("output shape mismatch")
+    with _DeviceGuard(a0):
+        _lib.call("wx_dual_gemm", _ptr(a0), _ptr(a1), _ptr(w0), _ptr(w1), _ptr(output_expert0),
+                  _ptr(output_expert1), m0, n0, k0, m1, n1, k1, int(bool(trans_a)), int(bool(trans_b)),
+                  _stream(a0))
+
+
+# ----------------------------------------------------------------------------- permute / unpermute
+def partition(indices: torch.Tensor, num_experts: int, num_out_tokens: int = 0,
+              workspace: Optional[List[torch.Tensor]] = None, want_sorted: bool = False):
+    """Stable partition of expert ids [T] or [T, K] (int32 / int64 / bool, no cast kernel needed).
+
+    Returns (row_id_map int32 [T*K], expert_offsets int32 [E+1], sorted_row_id or None, workspace).
+    workspace = [hist scratch, status word]; pass the returned list back in to avoid reallocation.
+    """
+    _need_cuda("indices", indices)
+    ids = indices if indices.is_contiguous() else indices.contiguous()
+    if ids.dtype not in _ITYPES:
+        ids = ids.to(torch.int32)
+    T = ids.size(0)
+    K = ids.size(1) if ids.dim() == 2 else 1
+    n = T * K
+    dev = ids.device
+    need = _lib.load().wx_partition_workspace_bytes(n)
+    if not workspace or workspace[0].numel() < need or workspace[0].device != dev:
+        workspace = [torch.empty(need, dtype=torch.uint8, device=dev),
+                     torch.zeros(1, dtype=torch.int32, device=dev)]
+    row_id_map = torch.empty(n, dtype=torch.int32, device=dev)
+    offsets = torch.empty(num_experts + 1, dtype=torch.int32, device=dev)
+    sorted_row_id = torch.empty(n, dtype=torch.int32, device=dev) if want_sorted else None
+    with _DeviceGuard(ids):
+        _lib.call("wx_partition_build", _ptr(ids), _ITYPES[ids.dtype], T, K, int(num_experts),
+                  int(num_out_tokens), _ptr(row_id_map), _ptr(sorted_row_id), offsets.data_ptr(),
+                  workspace[1].data_ptr(), workspace[0].data_ptr(), workspace[0].numel(), _stream(ids))
+    return row_id_map, offsets, sorted_row_id, workspace
+
+
+def permute_rows(input: torch.Tensor, row_id_map: torch.Tensor, num_topk: int, num_out: int) -> torch.Tensor:
+    out = torch.empty((num_out, input.size(1)), dtype=input.dtype, device=input.device)
+    with _DeviceGuard(input):
+        _lib.call("wx_permute_rows", _ptr(input), _ptr(out), _ptr(row_id_map), input.size(0), int(num_topk),
+                  input.size(1), _dtype_code(input), _stream(input))
+    return out
+
+
+# Expert ids the partition distinguishes.  The reference sorts arbitrary int32 keys with a radix sort;
+# MoE expert ids are small, and 256 bins cover every configuration of the model (it has 2 experts).
+MAX_EXPERTS = 256
+
+
+def permute(input: torch.Tensor, indices: torch.Tensor, num_out_tokens: int, workspace: List[torch.Tensor],
+            max_expanded_token_num: int) -> Tuple[torch.Tensor, torch.Tensor, List[torch.Tensor]]:
+    """csrc/permute.cu:450-630: (permuted [num_out, H], row_id_map int32 [T*K], workspace)."""
+    _need_cuda("input", input)
+    _need_cuda("indices", indices)
+    if input.dim() != 2 or indices.dim() != 2:
+        raise RuntimeError("permute expects input [T, H] and indices [T, K]")
+    dt = _dtype_code(input)  # raises "Wrong activation tensor type." for unsupported dtypes
+    del dt
+    if not input.is_contiguous():
+        input = input.contiguous()
+    T, K = indices.shape
+    if K > 128:
+        raise RuntimeError("num_topK cannot exceed 128.")  # csrc/permute.cu:394
+    row_id_map, _, _, workspace = partition(indices, MAX_EXPERTS, num_out_tokens, workspace)
+    num_out = num_out_tokens if num_out_tokens and num_out_tokens > 0 else T * K
+    permuted = permute_rows(input, row_id_map, K, num_out)
+    return permuted, row_id_map, workspace
+
+
+def unpermute(input: torch.Tensor, row_id_map: torch.Tensor, prob: torch.Tensor, num_tokens: int,
+              num_topK: int) -> torch.Tensor:
+    """csrc/permute.cu:638-779.  prob may be an empty tensor (no scaling); ignored when num_topK == 1."""
+    _need_cuda("input", input)
+    if not input.is_contiguous():
+        input = input.contiguous()
+    if num_topK > 128:
+        raise RuntimeError("num_topK cannot exceed 128.")
+    row_id_map = row_id_map.to(device=input.device, dtype=torch.int32).contiguous()
+    if row_id_map.numel() < num_tokens * num_topK:
+        raise RuntimeError("row_id_map is shorter than num_tokens * num_topK")
+    probs = None
+    if prob is not None and prob.numel() and num_topK > 1:
+        probs = prob.to(device=input.device, dtype=torch.float32).contiguous()
+    out = torch.empty((num_tokens, input.size(1)), dtype=input.dtype, device=input.device)
+    with _DeviceGuard(input):
+        _lib.call("wx_unpermute_rows", _ptr(input), _ptr(out), _ptr(row_id_map), _ptr(probs), int(num_tokens),
+                  int(num_topK), input.size(1), _dtype_code(input), _stream(input))
+    return out
+
+
+def unpermute_bwd(input_bwd: torch.Tensor, input_fwd: torch.Tensor, row_id_map: torch.Tensor,
+                  prob: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """csrc/permute.cu:781-942: (act_grad [rows of input_fwd, H], prob_grad fp32 [T, K]).
+
+    Rows of act_grad that no token maps to are returned as zeros (the reference leaves them
+    uninitialised); prob_grad is zeros when K == 1 (the reference leaves it uninitialised).
+    """
+    _need_cuda("input_bwd", input_bwd)
+    T, K = prob.shape
+    input_bwd = input_bwd.contiguous()
+    input_fwd = input_fwd.contiguous()
+    row_id_map = row_id_map.to(device=input_bwd.device, dtype=torch.int32).contiguous()
+    prob = prob.to(device=input_bwd.device, dtype=torch.float32).contiguous()
+    act_grad = torch.zeros((input_fwd.size(0), input_bwd.size(1)), dtype=input_bwd.dtype, device=input_bwd.device)
+    prob_grad = torch.zeros((T, K), dtype=torch.float32, device=input_bwd.device)
+    with _DeviceGuard(input_bwd):
+        _lib.call("wx_unpermute_rows_bwd", _ptr(input_bwd), _ptr(input_fwd), _ptr(act_grad), _ptr(prob_grad),
+                  _ptr(row_id_map), _ptr(prob), T, K, input_bwd.size(1), _dtype_code(input_bwd),
+                  _stream(input_bwd))
+    return act_grad, prob_grad
+
+
+# ----------------------------------------------------------------------------- M-RoPE
+def _bhsd_strides(t: torch.Tensor):
+    if t.dim() != 4 or t.stride(3) != 1:
+        raise RuntimeError("expected a [B, H, S, D] tensor with a contiguous last dimension")
+    return _lib.i64x3((t.stride(0), t.stride(1), t.stride(2)))
+
+
+def _rope_common(fn_name, q_in, k_in, cos, sin, q_out, k_out, mrope_section_doubled):
+    for name, t in (("q", q_in), ("k", k_in), ("cos", cos), ("sin", sin), ("q_out", q_out), ("k_out", k_out)):
+        _need_cuda(name, t)
+    if len(mrope_section_doubled) != 3:
+        raise RuntimeError("mrope_section_doubled must have 3 entries")
+    B, Hq, S, D = q_in.shape
+    Hk = k_in.size(1)
+    if tuple(k_in.shape) != (B, Hk, S, D) or tuple(q_out.shape) != tuple(q_in.shape) or \
+            tuple(k_out.shape) != tuple(k_in.shape):
+        raise RuntimeError("q/k/q_out/k_out shapes are inconsistent")
+    if tuple(cos.shape) != (3, B, S, D) or tuple(sin.shape) != (3, B, S, D):
+        raise RuntimeError(f"cos/sin must have shape [3, {B}, {S}, {D}]")
+    if not (q_in.dtype == k_in.dtype == cos.dtype == sin.dtype == q_out.dtype == k_out.dtype):
+        raise RuntimeError("q, k, cos, sin and the outputs must share one dtype")
+    cos = cos.contiguous()
+    sin = sin.contiguous()
+    section = _lib.i32x3([int(v) // 2 for v in mrope_section_doubled])
+    with _DeviceGuard(q_in):
+        _lib.call(fn_name, _ptr(q_in), _ptr(k_in), _ptr(cos), _ptr(sin), _ptr(q_out), _ptr(k_out), B, S, Hq, Hk,
+                  D, _bhsd_strides(q_in), _bhsd_strides(k_in), _bhsd_strides(q_out), _bhsd_strides(k_out),
+                  section, _mrope_layout, _dtype_code(q_in), _stream(q_in))
+
+
+def rope(q, k, cos, sin, q_out, k_out, mrope_section_doubled) -> None:
+    """csrc/rope.cu:453-509.  q [B,Hq,S,D], k [B,Hkv,S,D] (any batch/head/seq strides), cos/sin [3,B,S,D]."""
+    _rope_common("wx_mrope_apply", q, k, cos, sin, q_out, k_out, mrope_section_doubled)
+
+
+def rope_bwd(grad_q_out, grad_k_out, q, k, cos, sin, grad_q, grad_k, mrope_section_doubled) -> None:
+    """csrc/rope.cu:511-571.  q and k are accepted for signature parity; the adjoint does not need them."""
+    _rope_common("wx_mrope_apply_bwd", grad_q_out, grad_k_out, cos, sin, grad_q, grad_k, mrope_section_doubled)
+
+
+# ----------------------------------------------------------------------------- index builders
+def rope_index(input_ids, image_grid_thw, video_grid_thw, second_per_grid_ts, attention_mask,
+               spatial_merge_size: int, image_token_id: int, video_token_id: int, vision_start_token_id: int,
+               tokens_per_second: float, return_status: bool = False):
+    """csrc/rope_index.cu:464-569 with the PyTorch path's semantics (act.py:929-1149).
+
+    Returns (position_ids int64 [3, B, S], mrope_deltas int64 [B, 1]).
+    """
+    if input_ids is None:
+        raise RuntimeError("input_ids is required")
+    _need_cuda("input_ids", input_ids)
+    dev = input_ids.device
+
+    def as_i64(t):
+        return None if t is None else t.to(device=dev, dtype=torch.int64).contiguous()
+
+    ids = as_i64(input_ids)
+    B, S = ids.shape
+    mask = as_i64(attention_mask)
+    ig, vg = as_i64(image_grid_thw), as_i64(video_grid_thw)
+    spg = None if second_per_grid_ts is None else second_per_grid_ts.to(device=dev, dtype=torch.float32).contiguous()
+    pos = torch.empty((3, B, S), dtype=torch.int64, device=dev)
+    deltas = torch.empty((B, 1), dtype=torch.int64, device=dev)
+    status = torch.zeros(1, dtype=torch.int32, device=dev)
+    ws_bytes = _lib.load().wx_rope_index_workspace_bytes(B)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    with _DeviceGuard(ids):
+        _lib.call("wx_rope_index", _ptr(ids), _ptr(mask), None if ig is None else ig.data_ptr(),
+                  0 if ig is None else ig.size(0), None if vg is None else vg.data_ptr(),
+                  0 if vg is None else vg.size(0), _ptr(spg), B, S, int(spatial_merge_size), int(image_token_id),
+                  int(video_token_id), int(vision_start_token_id), float(tokens_per_second), _ptr(pos),
+                  _ptr(deltas), status.data_ptr(), ws.data_ptr(), ws_bytes, _stream(ids))
+    if return_status:
+        return pos, deltas, status
+    return pos, deltas
+
+
+def _host_grid(grid_thw: torch.Tensor, grid_thw_host):
+    """grid_thw as a host list of (t, h, w); copies device -> host (one sync) unless a host copy is given."""
+    if grid_thw_host is not None:
+        src = grid_thw_host
+    else:
+        src = grid_thw
+    return [tuple(int(v) for v in row) for row in src.cpu().tolist()]
+
+
+def rot_pos_emb(inv_freq: torch.Tensor, grid_thw: torch.Tensor, spatial_merge_size: int,
+                grid_thw_host: Optional[torch.Tensor] = None, return_ids: bool = False):
+    """csrc/rot_pos.cu:187-312: fp32 [sum t*h*w, 2*len(inv_freq)].
+
+    The output size depends on grid_thw's values; pass grid_thw_host (the CPU copy the processor produced)
+    to avoid the device -> host read the reference also performs.
+    """
+    _need_cuda("inv_freq", inv_freq)
+    _need_cuda("grid_thw", grid_thw)
+    if inv_freq.dtype != torch.float32:
+        raise RuntimeError("inv_freq must be float32")
+    if grid_thw.dtype not in (torch.int32, torch.int64):
+        raise RuntimeError("grid_thw must be int32 or int64")
+    grid = grid_thw.contiguous()
+    inv = inv_freq.contiguous()
+    rows = _host_grid(grid, grid_thw_host)
+    total = sum(t * h * w for t, h, w in rows)
+    F = inv.numel()
+    table = torch.empty((total, 2 * F), dtype=torch.float32, device=inv.device)
+    ids = torch.empty((total, 2), dtype=torch.int64, device=inv.device) if return_ids else None
+    with _DeviceGuard(inv):
+        _lib.call("wx_rot_pos_emb", _ptr(inv), F, _ptr(grid), _ITYPES[grid.dtype], grid.size(0),
+                  int(spatial_merge_size), total, _ptr(table), _ptr(ids), _stream(inv))
+    return (table, ids) if return_ids else table
+
+
+def get_window_index(grid_thw: torch.Tensor, spatial_merge_size: int, vit_merger_window_size: int,
+                     patch_size: int, spatial_merge_unit: int, grid_thw_host: Optional[torch.Tensor] = None):
+    """csrc/window_index.cu:208-286: (window_index int32 [N], cu_window_seqlens int32 [W + 1])."""
+    _need_cuda("grid_thw", grid_thw)
+    if grid_thw.dim() != 2 or grid_thw.size(1) != 3:
+        raise RuntimeError("grid_thw must have shape [num_grids, 3]")
+    if grid_thw.dtype != torch.int32:
+        raise RuntimeError("grid_thw must be int32")  # csrc/window_index.cu:217
+    del patch_size  # part of the reference signature; the window size arrives already divided by it
+    grid = grid_thw.contiguous()
+    dev = grid.device
+    if grid.size(0) == 0:  # csrc/window_index.cu:220-225
+        return torch.empty(0, dtype=torch.int32, device=dev), torch.zeros(1, dtype=torch.int32, device=dev)
+    rows = _host_grid(grid, grid_thw_host)
+    m, ws = int(spatial_merge_size), int(vit_merger_window_size)
+    n_tok = sum(t * (h // m) * (w // m) for t, h, w in rows)
+    n_win = sum(t * (-(-(h // m) // ws)) * (-(-(w // m) // ws)) for t, h, w in rows)
+    if n_tok == 0 or n_win == 0:  # csrc/window_index.cu:253-258
+        return torch.empty(0, dtype=torch.int32, device=dev), torch.zeros(1, dtype=torch.int32, device=dev)
+    window_index = torch.empty(n_tok, dtype=torch.int32, device=dev)
+    cu = torch.empty(n_win + 1, dtype=torch.int32, device=dev)
+    with _DeviceGuard(grid):
+        _lib.call("wx_window_index", _ptr(grid), WX_I32, grid.size(0), m, ws, int(spatial_merge_unit), n_tok,
+                  n_win, _ptr(window_index), _ptr(cu), _stream(grid))
+    return window_index, cu
+
+
+# ----------------------------------------------------------------------------- fused dual-expert FFN
+def dual_swiglu_ffn(x: torch.Tensor, expert_offsets: torch.Tensor, weights, hmid: Optional[torch.Tensor] = None,
+                    out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Both experts' SwiGLU FFN over expert-sorted rows in two launches (act.py:79-82, 142-154).
+
+    x [T, H] bf16 sorted by expert; expert_offsets int32 [3] ON THE DEVICE (from partition());
+    weights = ((gate0, up0, down0), (gate1, up1, down1)) in nn.Linear layout.
+    """
+    _need_cuda("x", x)
+    if x.dtype != torch.bfloat16:
+        raise RuntimeError("All tensors must be BFloat16 for this kernel")
+    (g0, u0, d0), (g1, u1, d1) = weights
+    for w in (g0, u0, d0, g1, u1, d1):
+        if w.dtype != torch.bfloat16 or not w.is_cuda or not w.is_contiguous():
+            raise RuntimeError("expert weights must be contiguous BFloat16 CUDA tensors")
+    T, H = x.shape
+    I0, I1 = g0.size(0), g1.size(0)
+    if tuple(g0.shape) != (I0, H) or tuple(u0.shape) != (I0, H) or tuple(d0.shape) != (H, I0) or \
+            tuple(g1.shape) != (I1, H) or tuple(u1.shape) != (I1, H) or tuple(d1.shape) != (H, I1):
+        raise RuntimeError("expert weight shapes are inconsistent with hidden size")
+    if expert_offsets.dtype != torch.int32 or expert_offsets.numel() < 3 or not expert_offsets.is_cuda:
+        raise RuntimeError("expert_offsets must be an int32 CUDA tensor with 3 entries")
+    x = x.contiguous()
+    need = T * max(I0, I1)
+    if hmid is None or hmid.numel() < need or hmid.dtype != torch.bfloat16:
+        hmid = torch.empty(need, dtype=torch.bfloat16, device=x.device)
+    if out is None:
+        out = torch.empty_like(x)
+    with _DeviceGuard(x):
+        _lib.call("wx_dual_swiglu_ffn", _ptr(x), _ptr(out), expert_offsets.data_ptr(), _ptr(g0), _ptr(u0), _ptr(d0),
+                  _ptr(g1), _ptr(u1), _ptr(d1), hmid.data_ptr(), T, H, I0, I1, _stream(x))
+    return out
