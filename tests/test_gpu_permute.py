@@ -63,8 +63,10 @@ def test_permute_num_out_tokens(dev):
     p, rmap = ops.permute(x.to(dev), ids.to(dev), num_out_tokens=200)
     assert p.shape == (200, 16)
     assert torch.equal(rmap.cpu(), ref_map) and torch.equal(p.cpu(), ref_p)
-    y = ops.unpermute(p, rmap)
+    # without probs the op infers the token count from its input (ops.py:350), so pass them like the model does
+    y = ops.unpermute(p, rmap, torch.ones(300, 1, device=dev))
     assert torch.equal(y.cpu(), oracle.unpermute_ref(ref_p, ref_map))  # dropped rows come back as zeros
+    assert ops.unpermute(p, rmap).shape == (200, 16)
 
 
 def test_out_of_range_ids_raise_the_status_word(dev):

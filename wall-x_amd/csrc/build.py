@@ -26,6 +26,8 @@ FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
     # packed fp32 math is kept off for every kernel in this library
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # no implicit fused multiply-add: the elementwise kernels reproduce eager mul-then-add rounding exactly
+    "-ffp-contract=off",
     "-Wno-unused-command-line-argument",
     f"-I{INCLUDE}", f"-I{HERE}",
 ]
