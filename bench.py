@@ -1,0 +1,275 @@
+#!/usr/bin/env python3
+"""Throughput of the per-layer MoE hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--ops-only]
+
+One step = one pass of the hot path over the serving batch of BASELINE config 3: 32 sequences x 912 tokens
+(880 VL + 32 action per sequence, seeded per-token mask), hidden 2048, VL expert 11008, action expert 1024,
+bf16: token partition -> row permute -> gate/up GEMM + SwiGLU (both experts, one launch) -> down GEMM (both
+experts, one launch) -> row unpermute.  Inputs are resident in HBM before the timed region.
+
+Prints ONE JSON line.  `value` = algorithmic FFN FLOPs (6*H*(m0*I0 + m1*I1)) / whole-step time, i.e. the
+permute and unpermute passes are inside the timed step.  `roofline` is the dominant kernel (gate/up + SwiGLU)
+timed by itself with HIP events on its stream.  `cpu_baseline` is the CPU oracle (a restatement of the
+reference's PyTorch path) on a bounded sample of the same batch, on this box's host cores.
+"""
+
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "wall-x_amd"))
+sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
+PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--ops-only", action="store_true", help="skip the side measurements (M-RoPE, index builders)")
+    ap.add_argument("--cpu-seqs", type=int, default=4, help="sequences of the batch the CPU baseline runs")
+    return ap.parse_args()
+
+
+def event_ms(fn, iters, warm=3):
+    """Median duration of fn() in ms from HIP events on the current stream."""
+    import torch
+
+    for _ in range(warm):
+        fn()
+    times = []
+    for _ in range(iters):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        fn()
+        b.record()
+        b.synchronize()
+        times.append(a.elapsed_time(b))
+    return statistics.median(times), sum(times) / len(times)
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this hot path has no cross-GPU step and every box here has a single "
+              "MI355X; run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (torch.cuda.is_available() is False)", file=sys.stderr)
+        sys.exit(1)
+    from wallx_mi355 import _lib, native, workloads as wl
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    H, I0, I1 = wl.HIDDEN, wl.INTER_VL, wl.INTER_ACT
+    B, S, NA = 32, 912, 32
+    T = B * S
+
+    # ---- synthetic inputs, resident in HBM ----------------------------------------------------------
+    x_cpu, types_cpu, w_cpu = wl.config3()
+    x = x_cpu.view(T, H).to(dev)
+    types = types_cpu.view(T).to(dev)
+    weights = [w.to(dev).as_tuple() for w in w_cpu]
+    (g0, u0, d0), (g1, u1, d1) = weights
+    m1 = int(types_cpu.sum())
+    m0 = T - m1
+    ffn_flops = 6.0 * H * (m0 * I0 + m1 * I1)
+    gate_up_flops = 4.0 * H * (m0 * I0 + m1 * I1)
+    down_flops = 2.0 * H * (m0 * I0 + m1 * I1)
+    row_bytes = 2.0 * T * H * 2 + 8.0 * T  # read + write of [T, H] bf16 plus the index traffic
+
+    hmid = torch.empty(T * max(I0, I1), dtype=torch.bfloat16, device=dev)
+    x_sorted = torch.empty_like(x)
+    y_sorted = torch.empty_like(x)
+    y = torch.empty_like(x)
+    ws = None
+    stream = torch.cuda.current_stream().cuda_stream
+
+    row_id_map, offsets, _, ws = native.partition(types, 2, 0, ws)
+
+    def partition():
+        nonlocal row_id_map, offsets, ws
+        row_id_map, offsets, _, ws = native.partition(types, 2, 0, ws)
+
+    def permute():
+        _lib.call("wx_permute_rows", x.data_ptr(), x_sorted.data_ptr(), row_id_map.data_ptr(), T, 1, H,
+                  _lib.WX_BF16, stream)
+
+    def gate_up():
+        _lib.call("wx_dual_swiglu_gate_up", x_sorted.data_ptr(), hmid.data_ptr(), offsets.data_ptr(), g0.data_ptr(),
+                  u0.data_ptr(), g1.data_ptr(), u1.data_ptr(), T, H, I0, I1, stream)
+
+    def down():
+        _lib.call("wx_dual_down_proj", hmid.data_ptr(), y_sorted.data_ptr(), offsets.data_ptr(), d0.data_ptr(),
+                  d1.data_ptr(), T, H, I0, I1, stream)
+
+    def unpermute():
+        _lib.call("wx_unpermute_rows", y_sorted.data_ptr(), y.data_ptr(), row_id_map.data_ptr(), None, T, 1, H,
+                  _lib.WX_BF16, stream)
+
+    def step():
+        partition()
+        permute()
+        gate_up()
+        down()
+        unpermute()
+
+    # ---- the timed region ----------------------------------------------------------------------------
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed * 1e3 / args.steps
+    tflops = ffn_flops / (elapsed / args.steps) / 1e12
+
+    # ---- per-kernel timings (HIP events on the launch stream) ------------------------------------------
+    iters = max(10, args.steps)
+    t_gate_up, t_gate_up_avg = event_ms(gate_up, iters)
+    t_down, _ = event_ms(down, iters)
+    t_perm, _ = event_ms(permute, iters)
+    t_unperm, _ = event_ms(unpermute, iters)
+    t_part, _ = event_ms(partition, iters)
+    gate_up_tflops = gate_up_flops / (t_gate_up_avg * 1e-3) / 1e12
+
+    extra = {
+        "gate_up_swiglu_ms": round(t_gate_up, 4), "gate_up_tflops": round(gate_up_flops / t_gate_up / 1e9, 1),
+        "down_ms": round(t_down, 4), "down_tflops": round(down_flops / t_down / 1e9, 1),
+        "ffn_kernels_tflops": round(ffn_flops / (t_gate_up + t_down) / 1e9, 1),
+        "permute_ms": round(t_perm, 4), "permute_GBps": round(row_bytes / t_perm / 1e6, 1),
+        "unpermute_ms": round(t_unperm, 4), "unpermute_GBps": round(row_bytes / t_unperm / 1e6, 1),
+        "permute_frac_hbm_peak": round(row_bytes / t_perm / 1e6 / PEAK_HBM_GBS, 4),
+        "partition_us": round(t_part * 1e3, 2),
+    }
+
+    if not args.ops_only:
+        extra.update(side_measurements(dev, iters))
+
+    result = {
+        "metric": "dual_expert_ffn_tflops",
+        "value": round(tflops, 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": "config 3 (BASELINE.json configs[2]): dual-expert FFN layer, 32 seq x 912 tokens, hidden 2048, "
+                        "VL expert 11008 on 28160 tokens, action expert 1024 on 1024 tokens; "
+                        "partition + permute + gate/up+SwiGLU + down + unpermute",
+            "tokens": T, "vl_tokens": m0, "action_tokens": m1, "hidden": H, "inter_vl": I0, "inter_action": I1,
+            "flops_per_step": ffn_flops,
+        },
+        "frac_mfma_peak": round(tflops / PEAK_BF16_TFLOPS, 4),
+        "roofline": {
+            "kernel": "dual_gemm_kernel<swiglu> (gate/up GEMM + SwiGLU, both experts)",
+            "bound": "mfma",
+            "achieved": round(gate_up_tflops, 2),
+            "peak": PEAK_BF16_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": round(gate_up_tflops / PEAK_BF16_TFLOPS, 4),
+            "flops_per_launch": gate_up_flops,
+            "avg_launch_ms": round(t_gate_up_avg, 4),
+            "traffic": None,
+        },
+        "extra": extra,
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(x_cpu, types_cpu, w_cpu, args.cpu_seqs, H, I0, I1)
+    print(json.dumps(result), flush=True)
+
+
+def side_measurements(dev, iters):
+    """M-RoPE bandwidth and index-builder latencies at BASELINE config 2 shapes (reported, not part of `value`)."""
+    import torch
+    from wallx_mi355 import native, workloads as wl
+    from wallx_mi355.fusions import ops
+
+    out = {}
+    ids_cpu, grid_cpu = wl.config2_tokens()
+    ids, grid = ids_cpu.to(dev), grid_cpu.to(dev)
+    grid32 = grid.to(torch.int32)
+    args = (2, wl.IMAGE_TOKEN_ID, wl.VIDEO_TOKEN_ID, wl.VISION_START_TOKEN_ID, 2)
+    pos, _ = ops.get_rope_index(ids, *args, image_grid_thw=grid)
+    t, _ = event_ms(lambda: ops.get_rope_index(ids, *args, image_grid_thw=grid), iters)
+    out["rope_index_us"] = round(t * 1e3, 2)
+    inv_v = wl.vision_inv_freq().to(dev)
+    t, _ = event_ms(lambda: native.rot_pos_emb(inv_v, grid, 2, grid_thw_host=grid_cpu), iters)
+    out["rot_pos_emb_us"] = round(t * 1e3, 2)
+    t, _ = event_ms(lambda: native.get_window_index(grid32, 2, 4, 14, 4, grid_thw_host=grid_cpu), iters)
+    out["window_index_us"] = round(t * 1e3, 2)
+
+    # M-RoPE at B = 16, S = 896: q [14336, 16, 128], k [14336, 2, 128] bf16, cos/sin from the positions above
+    B, S, D = ids.shape[0], ids.shape[1], wl.HEAD_DIM
+    inv = wl.text_inv_freq().to(dev)
+    freqs = pos.float()[..., None] * inv
+    emb = torch.cat((freqs, freqs), -1)
+    cos, sin = emb.cos().to(torch.bfloat16), emb.sin().to(torch.bfloat16)
+    q = torch.randn(B, S, wl.N_Q_HEADS, D, device=dev).to(torch.bfloat16).transpose(1, 2)
+    k = torch.randn(B, S, wl.N_KV_HEADS, D, device=dev).to(torch.bfloat16).transpose(1, 2)
+    qo = torch.empty(B, wl.N_Q_HEADS, S, D, dtype=torch.bfloat16, device=dev)
+    ko = torch.empty(B, wl.N_KV_HEADS, S, D, dtype=torch.bfloat16, device=dev)
+    sec2 = [2 * v for v in wl.MROPE_SECTION]
+    t, _ = event_ms(lambda: native.rope(q, k, cos, sin, qo, ko, sec2), iters)
+    tokens = B * S
+    rope_bytes = 2.0 * 2 * tokens * D * (wl.N_Q_HEADS + wl.N_KV_HEADS) + 2.0 * 2 * tokens * D
+    out["mrope_us"] = round(t * 1e3, 2)
+    out["mrope_GBps"] = round(rope_bytes / t / 1e6, 1)
+    out["mrope_frac_hbm_peak"] = round(rope_bytes / t / 1e6 / PEAK_HBM_GBS, 4)
+    return out
+
+
+def cpu_baseline(x_cpu, types_cpu, w_cpu, n_seq, H, I0, I1):
+    """The CPU oracle on the first n_seq sequences of the same batch (bf16 inputs upcast to fp32 inside)."""
+    import torch
+    import oracle
+
+    xs, ts = x_cpu[:n_seq], types_cpu[:n_seq]
+    weights = [w.as_tuple() for w in w_cpu]
+    m1 = int(ts.sum())
+    m0 = ts.numel() - m1
+    flops = 6.0 * H * (m0 * I0 + m1 * I1)
+    w32 = [tuple(t.float() for t in w) for w in weights]  # upcast once, outside the timed region
+    x32 = xs.float()
+
+    def run():
+        return oracle.sparse_moe_block_ref(x32, ts, w32, eager_rounding=False)
+
+    run()
+    times = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        run()
+        times.append(time.perf_counter() - t0)
+    best = statistics.median(times)
+    return {
+        "value": round(flops / best / 1e12, 4),
+        "unit": "TFLOP/s",
+        "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": f"first {n_seq} of 32 sequences of the same batch ({ts.numel()} tokens, {flops / 1e12:.3f} TFLOP), "
+                  f"fp32 math on bf16-valued inputs, median of 3 runs after 1 warm-up, {best * 1e3:.0f} ms per run",
+    }
+
+
+if __name__ == "__main__":
+    main()

@@ -101,6 +101,16 @@ int wx_dual_swiglu_ffn(const void* x, void* out, const int32_t* expert_offsets, 
                        const void* down1, void* hmid, int64_t num_rows, int64_t hidden,
                        int64_t inter0, int64_t inter1, wx_stream_t stream);
 
+/* The two launches of wx_dual_swiglu_ffn on their own, for callers that put work between them (and for
+ * timing each kernel): hmid = silu(x @ gate^T) * (x @ up^T), then out = hmid @ down^T, per expert.
+ * Same arguments and layouts as above; they replace the same reference lines (act.py:79-82, 142-154). */
+int wx_dual_swiglu_gate_up(const void* x, void* hmid, const int32_t* expert_offsets, const void* gate0,
+                           const void* up0, const void* gate1, const void* up1, int64_t num_rows,
+                           int64_t hidden, int64_t inter0, int64_t inter1, wx_stream_t stream);
+int wx_dual_down_proj(const void* hmid, void* out, const int32_t* expert_offsets, const void* down0,
+                      const void* down1, int64_t num_rows, int64_t hidden, int64_t inter0,
+                      int64_t inter1, wx_stream_t stream);
+
 /* ------------------------------------------------------------------------------------------------
  * 3D multimodal RoPE:  out = x * cos_sel + rotate_half(x) * sin_sel for q and k, where channel d of
  * cos_sel / sin_sel comes from plane axis(d) of cos / sin [3, B, S, D] (contiguous, dtype of q).

@@ -342,45 +342,93 @@ extern "C" int wx_dual_gemm(const void* in0, const void* in1, const void* w0, co
   return check_launch("dual_gemm_reference_layout_kernel");
 }
 
+namespace {
+
+struct FfnArgs {
+  const void *x, *gate[2], *up[2], *down[2];
+  void *out, *hmid;
+  const int32_t* offsets;
+  int64_t rows, hidden, inter[2];
+};
+
+int check_ffn(const char* who, const FfnArgs& a, bool need_gate_up, bool need_down) {
+  if (int rc = check_dims(who, a.rows, a.inter[0], a.hidden)) return rc;
+  if (int rc = check_dims(who, a.rows, a.hidden, a.inter[1])) return rc;
+  if (a.rows == 0) return WX_OK;
+  if (!a.offsets || !a.hmid || (need_gate_up && !a.x) || (need_down && !a.out))
+    return fail(WX_ERR_INVALID_ARGUMENT, "%s: null pointer", who);
+  for (int e = 0; e < 2; ++e) {
+    if (a.inter[e] == 0) continue;
+    if ((need_gate_up && (!a.gate[e] || !a.up[e])) || (need_down && !a.down[e]))
+      return fail(WX_ERR_INVALID_ARGUMENT, "%s: null weight pointer for expert %d", who, e);
+  }
+  const int64_t max_inter = a.inter[0] > a.inter[1] ? a.inter[0] : a.inter[1];
+  if (a.rows * max_inter * 2 >= (1ll << 40)) return fail(WX_ERR_UNSUPPORTED, "%s: intermediate too large", who);
+  return WX_OK;
+}
+
+// hmid_e = silu(x_e @ gate_e^T) * (x_e @ up_e^T); expert e's rows are packed with row length inter_e
+int launch_gate_up(const FfnArgs& a, hipStream_t s) {
+  Params p{};
+  for (int e = 0; e < 2; ++e) {
+    Group& g = p.g[e];
+    g.a = static_cast<const __bf16*>(a.x);
+    g.b0 = static_cast<const __bf16*>(a.gate[e]);
+    g.b1 = static_cast<const __bf16*>(a.up[e]);
+    g.c = static_cast<__bf16*>(a.hmid);
+    g.m = 0; g.n = static_cast<int>(a.inter[e]); g.k = static_cast<int>(a.hidden);
+    g.lda = static_cast<int>(a.hidden); g.ldb = static_cast<int>(a.hidden); g.ldc = static_cast<int>(a.inter[e]);
+  }
+  p.offsets = a.offsets;
+  return launch_mfma<true>(p, s, "dual_gemm_kernel<swiglu>");
+}
+
+// out_e = hmid_e @ down_e^T
+int launch_down(const FfnArgs& a, hipStream_t s) {
+  Params p{};
+  for (int e = 0; e < 2; ++e) {
+    Group& g = p.g[e];
+    g.a = static_cast<const __bf16*>(a.hmid);
+    g.b0 = static_cast<const __bf16*>(a.down[e]);
+    g.b1 = nullptr;
+    g.c = static_cast<__bf16*>(a.out);
+    g.m = 0; g.n = static_cast<int>(a.hidden); g.k = static_cast<int>(a.inter[e]);
+    g.lda = static_cast<int>(a.inter[e]); g.ldb = static_cast<int>(a.inter[e]); g.ldc = static_cast<int>(a.hidden);
+  }
+  p.offsets = a.offsets;
+  return launch_mfma<false>(p, s, "dual_gemm_kernel<down>");
+}
+
+}  // namespace
+
+extern "C" int wx_dual_swiglu_gate_up(const void* x, void* hmid, const int32_t* expert_offsets, const void* gate0,
+                                      const void* up0, const void* gate1, const void* up1, int64_t num_rows,
+                                      int64_t hidden, int64_t inter0, int64_t inter1, wx_stream_t stream) {
+  const FfnArgs a{x, {gate0, gate1}, {up0, up1}, {nullptr, nullptr}, nullptr, hmid, expert_offsets,
+                  num_rows, hidden, {inter0, inter1}};
+  if (int rc = check_ffn("wx_dual_swiglu_gate_up", a, true, false)) return rc;
+  if (num_rows == 0) return WX_OK;
+  return launch_gate_up(a, as_stream(stream));
+}
+
+extern "C" int wx_dual_down_proj(const void* hmid, void* out, const int32_t* expert_offsets, const void* down0,
+                                 const void* down1, int64_t num_rows, int64_t hidden, int64_t inter0,
+                                 int64_t inter1, wx_stream_t stream) {
+  const FfnArgs a{nullptr, {nullptr, nullptr}, {nullptr, nullptr}, {down0, down1}, out, const_cast<void*>(hmid),
+                  expert_offsets, num_rows, hidden, {inter0, inter1}};
+  if (int rc = check_ffn("wx_dual_down_proj", a, false, true)) return rc;
+  if (num_rows == 0) return WX_OK;
+  return launch_down(a, as_stream(stream));
+}
+
 extern "C" int wx_dual_swiglu_ffn(const void* x, void* out, const int32_t* expert_offsets, const void* gate0,
                                   const void* up0, const void* down0, const void* gate1, const void* up1,
                                   const void* down1, void* hmid, int64_t num_rows, int64_t hidden, int64_t inter0,
                                   int64_t inter1, wx_stream_t stream) {
-  if (int rc = check_dims("wx_dual_swiglu_ffn", num_rows, inter0, hidden)) return rc;
-  if (int rc = check_dims("wx_dual_swiglu_ffn", num_rows, hidden, inter1)) return rc;
+  const FfnArgs a{x, {gate0, gate1}, {up0, up1}, {down0, down1}, out, hmid, expert_offsets,
+                  num_rows, hidden, {inter0, inter1}};
+  if (int rc = check_ffn("wx_dual_swiglu_ffn", a, true, true)) return rc;
   if (num_rows == 0) return WX_OK;
-  if (!x || !out || !expert_offsets || !hmid) return fail(WX_ERR_INVALID_ARGUMENT, "wx_dual_swiglu_ffn: null pointer");
-  if ((inter0 > 0 && (!gate0 || !up0 || !down0)) || (inter1 > 0 && (!gate1 || !up1 || !down1)))
-    return fail(WX_ERR_INVALID_ARGUMENT, "wx_dual_swiglu_ffn: null weight pointer");
-  const int64_t max_inter = inter0 > inter1 ? inter0 : inter1;
-  if (num_rows * max_inter * 2 >= (1ll << 40)) return fail(WX_ERR_UNSUPPORTED, "wx_dual_swiglu_ffn: intermediate too large");
-  hipStream_t s = as_stream(stream);
-  const void* gates[2] = {gate0, gate1};
-  const void* ups[2] = {up0, up1};
-  const void* downs[2] = {down0, down1};
-  const int64_t inters[2] = {inter0, inter1};
-  // launch 1: hmid_e = silu(x_e @ gate_e^T) * (x_e @ up_e^T); expert e's rows are packed with row length inter_e
-  Params p1{};
-  Params p2{};
-  for (int e = 0; e < 2; ++e) {
-    Group& g = p1.g[e];
-    g.a = static_cast<const __bf16*>(x);
-    g.b0 = static_cast<const __bf16*>(gates[e]);
-    g.b1 = static_cast<const __bf16*>(ups[e]);
-    g.c = static_cast<__bf16*>(hmid);
-    g.m = 0; g.n = static_cast<int>(inters[e]); g.k = static_cast<int>(hidden);
-    g.lda = static_cast<int>(hidden); g.ldb = static_cast<int>(hidden); g.ldc = static_cast<int>(inters[e]);
-    // launch 2: out_e = hmid_e @ down_e^T
-    Group& d = p2.g[e];
-    d.a = static_cast<const __bf16*>(hmid);
-    d.b0 = static_cast<const __bf16*>(downs[e]);
-    d.b1 = nullptr;
-    d.c = static_cast<__bf16*>(out);
-    d.m = 0; d.n = static_cast<int>(hidden); d.k = static_cast<int>(inters[e]);
-    d.lda = static_cast<int>(inters[e]); d.ldb = static_cast<int>(inters[e]); d.ldc = static_cast<int>(hidden);
-  }
-  p1.offsets = expert_offsets;
-  p2.offsets = expert_offsets;
-  if (int rc = launch_mfma<true>(p1, s, "dual_gemm_kernel<swiglu>")) return rc;
-  return launch_mfma<false>(p2, s, "dual_gemm_kernel<down>");
+  if (int rc = launch_gate_up(a, as_stream(stream))) return rc;
+  return launch_down(a, as_stream(stream));
 }
