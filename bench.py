@@ -37,6 +37,10 @@ def parse():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--ops-only", action="store_true", help="skip the side measurements (M-RoPE, index builders)")
     ap.add_argument("--cpu-seqs", type=int, default=4, help="sequences of the batch the CPU baseline runs")
+    ap.add_argument("--kernel-loop", default=None,
+                    choices=["gate_up", "down", "permute", "unpermute", "partition", "copy"],
+                    help="profiling aid: run only this kernel --steps times (no JSON line); 'copy' is a plain "
+                         "device-to-device copy of the [T, H] activations, the known-size yardstick for HBM counters")
     return ap.parse_args()
 
 
@@ -124,6 +128,15 @@ def main():
         gate_up()
         down()
         unpermute()
+
+    if args.kernel_loop:
+        permute(); gate_up(); down()
+        fn = {"gate_up": gate_up, "down": down, "permute": permute, "unpermute": unpermute, "partition": partition,
+              "copy": lambda: x_sorted.copy_(x)}[args.kernel_loop]
+        for _ in range(args.steps):
+            fn()
+        torch.cuda.synchronize()
+        return
 
     # ---- the timed region ----------------------------------------------------------------------------
     for _ in range(args.warmup):

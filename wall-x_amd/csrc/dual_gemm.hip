@@ -48,8 +48,14 @@ struct Params {
 
 #define LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
 
+// Buffer descriptor for `bytes` readable bytes at `base`.  Both are wave-uniform by construction; passing them
+// through readfirstlane pins the descriptor to scalar registers.
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes) {
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, static_cast<int>(bytes), 0x00020000);
+  const uint64_t v = reinterpret_cast<uint64_t>(base);
+  const uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v));
+  const uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v >> 32));
+  void* p = reinterpret_cast<void*>((static_cast<uint64_t>(hi) << 32) | lo);
+  return __builtin_amdgcn_make_buffer_rsrc(p, 0, static_cast<int>(__builtin_amdgcn_readfirstlane(bytes)), 0x00020000);
 }
 
 struct TileCoord {
@@ -84,7 +90,8 @@ __global__ __launch_bounds__(kThreads, 1) void dual_gemm_kernel(Params p) {
   __shared__ __attribute__((aligned(1024))) unsigned char s_a1[kTileBytes];
   __shared__ __attribute__((aligned(1024))) unsigned char s_b1[kTileBytes];
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keeps descriptors and LDS bases scalar
   const int wm = wave >> 2, wn = wave & 3;
   const int l32 = lane & 31, lhi = lane >> 5;
 
@@ -129,48 +136,157 @@ __global__ __launch_bounds__(kThreads, 1) void dual_gemm_kernel(Params p) {
   const int b_row_off0 = (SWIGLU ? wn * 32 + l32 : wn * 64 + l32) * kRowBytes;
   const int b_row_off1 = (SWIGLU ? 128 + wn * 32 + l32 : wn * 64 + 32 + l32) * kRowBytes;
 
-  for (int64_t t = blockIdx.x; t < padded; t += gridDim.x) {
-    TileCoord tc;
-    if (!map_tile(t, total, tiles_m, tiles_n, tc)) continue;
+  // ---- per-tile state ------------------------------------------------------------------------------
+  struct Loader {   // where this thread's eight 16-byte loads per K step come from
+    const __bf16 *a_base, *b_base;
+    uint32_t a_bytes, b_bytes;
+    uint32_t voff_a[4], voff_b[4];
+    int K, nk;
+  };
+  struct Store {    // where the finished tile goes
+    __bf16* c_base;
+    int rows, cols_left, ldc;  // valid rows / columns from the tile origin
+  };
+
+  auto setup = [&](const TileCoord& tc, Loader& L, Store& S) {
     const Group G = tc.group ? g1 : g0;
     const int row0 = tc.tm * BM, col0 = tc.tn * kTileN;
-    const int K = G.k;
-    const int nk = (K + BK - 1) / BK;
-
-    // ---- loader addressing ------------------------------------------------------------------------
     const int rows_a = G.m - row0 < BM ? G.m - row0 : BM;
     const int rows_b = G.n - col0 < kTileN ? G.n - col0 : kTileN;
-    const __bf16* a_base = G.a + static_cast<int64_t>(row0) * G.lda;
+    L.K = G.k;
+    L.nk = (G.k + BK - 1) / BK;
+    L.a_base = G.a + static_cast<int64_t>(row0) * G.lda;
     const bool up_half = SWIGLU && wave >= 4;
-    const __bf16* b_src = up_half ? G.b1 : G.b0;
-    const __bf16* b_base = b_src + static_cast<int64_t>(col0) * G.ldb;
-    const uint32_t a_bytes = static_cast<uint32_t>(rows_a) * G.lda * 2u;
-    const uint32_t b_bytes = static_cast<uint32_t>(rows_b) * G.ldb * 2u;
+    L.b_base = (up_half ? G.b1 : G.b0) + static_cast<int64_t>(col0) * G.ldb;
+    L.a_bytes = static_cast<uint32_t>(rows_a) * G.lda * 2u;
+    L.b_bytes = static_cast<uint32_t>(rows_b) * G.ldb * 2u;
     const int b_ld_row0 = SWIGLU ? (wave & 3) * 32 + (lane >> 3) : ld_row0;  // row inside the gate / up half
-    uint32_t voff_a[4], voff_b[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      voff_a[i] = static_cast<uint32_t>(ld_row0 + 8 * i) * G.lda * 2u + ld_chunk[i] * 16u;
-      voff_b[i] = static_cast<uint32_t>(b_ld_row0 + 8 * i) * G.ldb * 2u + ld_chunk[i] * 16u;
+      L.voff_a[i] = static_cast<uint32_t>(ld_row0 + 8 * i) * G.lda * 2u + ld_chunk[i] * 16u;
+      L.voff_b[i] = static_cast<uint32_t>(b_ld_row0 + 8 * i) * G.ldb * 2u + ld_chunk[i] * 16u;
     }
+    S.c_base = G.c + static_cast<int64_t>(row0) * G.ldc + col0;
+    S.rows = rows_a;
+    S.cols_left = G.n - col0;
+    S.ldc = G.ldc;
+  };
 
-    auto issue = [&](int ks, unsigned char* sa, unsigned char* sb) {
-      const int k0 = ks * BK;
-      // advancing the base keeps the absolute end of the readable range: rows past the matrix and, through the
-      // per-lane select below, K chunks past the row end read as zero
-      const __amdgpu_buffer_rsrc_t ra = make_rsrc(a_base + k0, a_bytes - 2u * k0);
-      const __amdgpu_buffer_rsrc_t rb = make_rsrc(b_base + k0, b_bytes - 2u * k0);
-      const bool k_tail = k0 + BK > K;
+  // One K step of global -> LDS for this wave: rows [wave*32, +32) of the A tile and of the B tile.
+  auto issue = [&](const Loader& L, int ks, unsigned char* sa, unsigned char* sb) {
+    const int k0 = ks * BK;
+    // advancing the base keeps the absolute end of the readable range: rows past the matrix and, through the
+    // per-lane select below, K chunks past the row end read as zero
+    const __amdgpu_buffer_rsrc_t ra = make_rsrc(L.a_base + k0, L.a_bytes - 2u * k0);
+    const __amdgpu_buffer_rsrc_t rb = make_rsrc(L.b_base + k0, L.b_bytes - 2u * k0);
+    const bool k_tail = k0 + BK > L.K;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        uint32_t va = voff_a[i], vb = voff_b[i];
-        if (k_tail && k0 + ld_chunk[i] * 8 >= K) va = vb = 0x80000000u;
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, LDS_PTR(sa + (wave * 32 + 8 * i) * kRowBytes), 16, va, 0, 0, 0);
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, LDS_PTR(sb + (wave * 32 + 8 * i) * kRowBytes), 16, vb, 0, 0, 0);
-      }
-    };
+    for (int i = 0; i < 4; ++i) {
+      uint32_t va = L.voff_a[i], vb = L.voff_b[i];
+      if (k_tail && k0 + ld_chunk[i] * 8 >= L.K) va = vb = 0x80000000u;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, LDS_PTR(sa + (wave * 32 + 8 * i) * kRowBytes), 16, va, 0, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, LDS_PTR(sb + (wave * 32 + 8 * i) * kRowBytes), 16, vb, 0, 0, 0);
+    }
+  };
 
-    f32x16 acc[4][2];
+  f32x16 acc[4][2];
+  bf16x8 fa[2][4], fb[2][2];  // two fragment sets: one feeds the MFMAs while the other is being read from LDS
+
+  auto read_frags = [&](const unsigned char* sa, const unsigned char* sb, int kk, int set) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      fa[set][i] = *reinterpret_cast<const bf16x8*>(sa + a_row_off + i * 32 * kRowBytes + frag_off[kk]);
+    fb[set][0] = *reinterpret_cast<const bf16x8*>(sb + b_row_off0 + frag_off[kk]);
+    fb[set][1] = *reinterpret_cast<const bf16x8*>(sb + b_row_off1 + frag_off[kk]);
+  };
+  auto mma = [&](int set) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[set][i], fb[set][j], acc[i][j], 0, 0, 0);
+  };
+  // scheduling hints: interleave the six LDS reads of the next fragment set with the eight MFMAs of this one
+  auto interleave_reads = [&]() {
+#pragma unroll
+    for (int q = 0; q < 6; ++q) {
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one LDS read
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+  };
+
+  // One K step.  On entry fragment set 0 holds kk = 0 of the current stage.  The barrier sits before the last
+  // quarter: by then every wave has its kk = 3 fragments in registers, so the current stage can be refilled
+  // (K step ks + 2) right after it, and the next stage -- issued a whole K step earlier -- is complete.
+  auto k_step = [&](const Loader& L, int ks, unsigned char* sa_cur, unsigned char* sb_cur, unsigned char* sa_nxt,
+                    unsigned char* sb_nxt) {
+    read_frags(sa_cur, sb_cur, 1, 1);
+    mma(0);
+    interleave_reads();
+    read_frags(sa_cur, sb_cur, 2, 0);
+    mma(1);
+    interleave_reads();
+    read_frags(sa_cur, sb_cur, 3, 1);
+    mma(0);
+    interleave_reads();
+    if (ks + 1 < L.nk) {
+      __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0): my loads for ks+1 landed, my LDS reads returned
+      __syncthreads();
+      if (ks + 2 < L.nk) issue(L, ks + 2, sa_cur, sb_cur);
+      read_frags(sa_nxt, sb_nxt, 0, 0);
+    }
+    mma(1);
+  };
+
+  auto epilogue = [&](const Store& S) {
+    // accumulator register r of lane l holds row 8*(r/4) + 4*(l/32) + r%4, column l%32 of its 32x32 block
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int row = wm * 128 + i * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
+        if (row >= S.rows) continue;
+        __bf16* c_row = S.c_base + static_cast<int64_t>(row) * S.ldc;
+        if constexpr (SWIGLU) {
+          const int col = wn * 32 + l32;
+          if (col < S.cols_left) {
+            // eager bf16 evaluation of act_fn(gate) * up (act.py:80-82): gate, up, silu(gate) and the product are
+            // each rounded to bf16
+            const float g = round_bf16(acc[i][0][r]);
+            const float u = round_bf16(acc[i][1][r]);
+            const float sg = round_bf16(g / (1.0f + expf(-g)));
+            c_row[col] = static_cast<__bf16>(sg * u);
+          }
+        } else {
+#pragma unroll
+          for (int j = 0; j < 2; ++j) {
+            const int col = wn * 64 + j * 32 + l32;
+            if (col < S.cols_left) c_row[col] = static_cast<__bf16>(acc[i][j][r]);
+          }
+        }
+      }
+    }
+  };
+
+  // first two K steps of a tile go out together; later ones are issued from inside k_step
+  auto prologue = [&](const Loader& L) {
+    issue(L, 0, s_a0, s_b0);
+    if (L.nk > 1) issue(L, 1, s_a1, s_b1);
+  };
+
+  // ---- persistent tile loop -----------------------------------------------------------------------
+  int64_t t = blockIdx.x;
+  TileCoord tc;
+  bool have = false;
+  for (; t < padded && !have; t += have ? 0 : gridDim.x) have = map_tile(t, total, tiles_m, tiles_n, tc);
+  if (!have) return;
+  Loader L;
+  Store S;
+  setup(tc, L, S);
+  prologue(L);
+
+  while (true) {
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
@@ -178,69 +294,27 @@ __global__ __launch_bounds__(kThreads, 1) void dual_gemm_kernel(Params p) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-    auto compute = [&](const unsigned char* sa, const unsigned char* sb) {
-#pragma unroll
-      for (int kk = 0; kk < 4; ++kk) {
-        bf16x8 fa[4], fb[2];
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-          fa[i] = *reinterpret_cast<const bf16x8*>(sa + a_row_off + i * 32 * kRowBytes + frag_off[kk]);
-        fb[0] = *reinterpret_cast<const bf16x8*>(sb + b_row_off0 + frag_off[kk]);
-        fb[1] = *reinterpret_cast<const bf16x8*>(sb + b_row_off1 + frag_off[kk]);
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-#pragma unroll
-          for (int j = 0; j < 2; ++j)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
-      }
-    };
-
-    // ---- main loop: stage s holds K step ks with (ks & 1) == s ------------------------------------
-    __syncthreads();  // the previous tile's last reads of stage 0 are done
-    issue(0, s_a0, s_b0);
-    for (int ks = 0; ks < nk; ks += 2) {
-      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's loads for step ks have landed
-      __syncthreads();                     // ... and everyone else's; stage 1 is no longer being read
-      if (ks + 1 < nk) issue(ks + 1, s_a1, s_b1);
-      compute(s_a0, s_b0);
-      if (ks + 1 < nk) {
-        __builtin_amdgcn_s_waitcnt(0x0F70);
-        __syncthreads();
-        if (ks + 2 < nk) issue(ks + 2, s_a0, s_b0);
-        compute(s_a1, s_b1);
-      }
+    // stage 0 (K step 0) must be complete; K step 1 may still be in flight (8 loads per wave per K step)
+    if (L.nk > 1) __builtin_amdgcn_s_waitcnt(0x0F78); else __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();
+    read_frags(s_a0, s_b0, 0, 0);
+    for (int ks = 0; ks < L.nk; ks += 2) {
+      k_step(L, ks, s_a0, s_b0, s_a1, s_b1);
+      if (ks + 1 < L.nk) k_step(L, ks + 1, s_a1, s_b1, s_a0, s_b0);
     }
 
-    // ---- epilogue -----------------------------------------------------------------------------------
-    // accumulator register r of lane l holds row 8*(r/4) + 4*(l/32) + r%4, column l%32 of its 32x32 block
-    const int out_cols = G.n;
-    __bf16* c_base = G.c + static_cast<int64_t>(row0) * G.ldc;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int row = wm * 128 + i * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
-        if (row >= rows_a) continue;
-        __bf16* c_row = c_base + static_cast<int64_t>(row) * G.ldc;
-        if constexpr (SWIGLU) {
-          const int col = col0 + wn * 32 + l32;
-          if (col < out_cols) {
-            // eager bf16 evaluation of act_fn(gate) * up (act.py:80-82): gate, up, silu(gate) and the product are
-            // each rounded to bf16
-            const float g = round_bf16(acc[i][0][r]);
-            const float u = round_bf16(acc[i][1][r]);
-            const float s = round_bf16(g / (1.0f + expf(-g)));
-            c_row[col] = static_cast<__bf16>(s * u);
-          }
-        } else {
-#pragma unroll
-          for (int j = 0; j < 2; ++j) {
-            const int col = col0 + wn * 64 + j * 32 + l32;
-            if (col < out_cols) c_row[col] = static_cast<__bf16>(acc[i][j][r]);
-          }
-        }
-      }
+    // next tile: its first loads fly while this tile's results are stored
+    TileCoord tn;
+    bool more = false;
+    for (t += gridDim.x; t < padded && !more; t += more ? 0 : gridDim.x) more = map_tile(t, total, tiles_m, tiles_n, tn);
+    const Store done = S;
+    __syncthreads();  // every wave holds its last fragments in registers: both stages are free
+    if (more) {
+      setup(tn, L, S);
+      prologue(L);
     }
+    epilogue(done);
+    if (!more) break;
   }
 }
 
