@@ -17,6 +17,8 @@
 // SwiGLU mode: the B tile is 128 gate rows + 128 up rows of the same intermediate columns, so gate and
 // up accumulators of one output element sit in the same lane and register index; the epilogue applies
 // silu(g) * u with eager bf16 rounding and writes the 256 x 128 intermediate tile.
+#include <type_traits>
+
 #include "common.h"
 
 namespace wx {
@@ -25,10 +27,16 @@ namespace {
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
-constexpr int BM = 256, BN = 256, BK = 64;
-constexpr int kThreads = 512;
-constexpr int kRowBytes = BK * 2;              // 128 bytes of K per LDS row
-constexpr int kTileBytes = BM * kRowBytes;     // 32 KiB per operand per stage
+constexpr int BM = 256, BN = 256, BK = 32;
+constexpr int kWavesM = 2, kWavesN = 2;        // wavefront grid over the tile; one wavefront per SIMD
+constexpr int kThreads = kWavesM * kWavesN * 64;
+constexpr int FM = BM / kWavesM / 32;          // 32x32 accumulator blocks per wave along M (4)
+constexpr int FN = BN / kWavesN / 32;          // ... and along N (4): 256 accumulator registers per lane
+constexpr int kLoadRows = BM / (kWavesM * kWavesN);  // LDS rows of each operand one wave loads per K step (64)
+constexpr int kLoads = kLoadRows / 16;         // 16-row load instructions per operand per wave per K step (4)
+constexpr int kStages = 4;                     // ring slots per operand (the tile loop is written out for 4)
+constexpr int kRowBytes = BK * 2;              // 64 bytes of K per LDS row
+constexpr int kSlotBytes = BM * kRowBytes;     // 16 KiB per operand per K step
 constexpr int kXcds = 8;
 constexpr int kGroupM = 8;                     // tile rows per patch in the tile order
 
@@ -58,41 +66,53 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, ui
   return __builtin_amdgcn_make_buffer_rsrc(p, 0, static_cast<int>(__builtin_amdgcn_readfirstlane(bytes)), 0x00020000);
 }
 
+// s_waitcnt immediate for gfx9: vmcnt in bits [3:0] and [15:14], expcnt [6:4] (left at "no wait"), lgkmcnt [11:8]
+constexpr int waitcnt_imm(int vm, int lgkm) { return (vm & 15) | ((vm >> 4) << 14) | (7 << 4) | (lgkm << 8); }
+
 struct TileCoord {
   int group, tm, tn;
 };
 
 // Linear tile id -> coordinates.  Ids are first spread so that each XCD (workgroup id mod 8) walks its own
 // contiguous range of "virtual" ids; virtual ids then sweep patches of kGroupM tile rows column by column.
-__device__ __forceinline__ bool map_tile(int64_t t, int64_t total, const int* tiles_m, const int* tiles_n,
-                                         TileCoord& tc) {
-  const int64_t per = (total + kXcds - 1) / kXcds;
-  int64_t v = (t % kXcds) * per + t / kXcds;
+// Integer division runs on the vector ALU even for uniform operands, so the results are handed back through
+// readfirstlane to keep everything derived from them (descriptors, branches) scalar.
+__device__ __forceinline__ bool map_tile(int t, int total, const int* tiles_m, const int* tiles_n, TileCoord& tc) {
+  const int per = (total + kXcds - 1) / kXcds;
+  int v = (t % kXcds) * per + t / kXcds;
   if (v >= total) return false;
   int g = 0;
-  const int64_t c0 = static_cast<int64_t>(tiles_m[0]) * tiles_n[0];
+  const int c0 = tiles_m[0] * tiles_n[0];
   if (v >= c0) { g = 1; v -= c0; }
   const int tmn = g ? tiles_m[1] : tiles_m[0], tnn = g ? tiles_n[1] : tiles_n[0];
-  const int64_t patch = static_cast<int64_t>(kGroupM) * tnn;
-  const int first_m = static_cast<int>(v / patch) * kGroupM;
+  const int patch = kGroupM * tnn;
+  const int first_m = __builtin_amdgcn_readfirstlane(v / patch) * kGroupM;
   const int rows = tmn - first_m < kGroupM ? tmn - first_m : kGroupM;
-  const int64_t in_patch = v % patch;
+  const int in_patch = v - (first_m / kGroupM) * patch;
+  const int q = __builtin_amdgcn_readfirstlane(in_patch / rows);
   tc.group = g;
-  tc.tm = first_m + static_cast<int>(in_patch % rows);
-  tc.tn = static_cast<int>(in_patch / rows);
+  tc.tm = first_m + (in_patch - q * rows);
+  tc.tn = q;
   return true;
 }
 
 template <bool SWIGLU>
 __global__ __launch_bounds__(kThreads, 1) void dual_gemm_kernel(Params p) {
-  __shared__ __attribute__((aligned(1024))) unsigned char s_a0[kTileBytes];
-  __shared__ __attribute__((aligned(1024))) unsigned char s_b0[kTileBytes];
-  __shared__ __attribute__((aligned(1024))) unsigned char s_a1[kTileBytes];
-  __shared__ __attribute__((aligned(1024))) unsigned char s_b1[kTileBytes];
+#if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stub; the body uses gfx950-only builtins
+  // kStages ring slots per operand, each one K step (256 rows x 32 bf16).  Separate arrays let the compiler
+  // see that a read of one slot never waits for a buffer load that targets another.
+  __shared__ __attribute__((aligned(1024))) unsigned char s_a0[kSlotBytes];
+  __shared__ __attribute__((aligned(1024))) unsigned char s_a1[kSlotBytes];
+  __shared__ __attribute__((aligned(1024))) unsigned char s_a2[kSlotBytes];
+  __shared__ __attribute__((aligned(1024))) unsigned char s_a3[kSlotBytes];
+  __shared__ __attribute__((aligned(1024))) unsigned char s_b0[kSlotBytes];
+  __shared__ __attribute__((aligned(1024))) unsigned char s_b1[kSlotBytes];
+  __shared__ __attribute__((aligned(1024))) unsigned char s_b2[kSlotBytes];
+  __shared__ __attribute__((aligned(1024))) unsigned char s_b3[kSlotBytes];
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keeps descriptors and LDS bases scalar
-  const int wm = wave >> 2, wn = wave & 3;
+  const int wm = wave / kWavesN, wn = wave % kWavesN;
   const int l32 = lane & 31, lhi = lane >> 5;
 
   // ---- problem table (uniform) ------------------------------------------------------------------
@@ -115,153 +135,186 @@ __global__ __launch_bounds__(kThreads, 1) void dual_gemm_kernel(Params p) {
   tiles_m[1] = (g1.m + BM - 1) / BM;
   tiles_n[1] = (g1.n + kTileN - 1) / kTileN;
   if (g1.m <= 0 || g1.n <= 0) tiles_m[1] = tiles_n[1] = 0;
-  const int64_t total = static_cast<int64_t>(tiles_m[0]) * tiles_n[0] + static_cast<int64_t>(tiles_m[1]) * tiles_n[1];
-  const int64_t padded = (total + kXcds - 1) / kXcds * kXcds;
+  const int total = tiles_m[0] * tiles_n[0] + tiles_m[1] * tiles_n[1];  // the host bounds this below 2^31
+  const int padded = (total + kXcds - 1) / kXcds * kXcds;
 
   // ---- per-lane constants -----------------------------------------------------------------------
-  // loader: instruction i of this wave fills LDS rows [wave*32 + 8i, +8); lane -> (row lane/8, slot lane%8)
-  const int ld_row0 = wave * 32 + (lane >> 3);
-  int ld_chunk[4];
+  // loader: one instruction fills 16 LDS rows of 64 bytes; lane -> (row lane/4, slot lane%4).  Instruction i of
+  // this wave covers rows [wave*64 + 16i, +16).  Chunk c of row r lives in slot c ^ ((r >> 2) & 3).
+  const int ld_row0 = wave * kLoadRows + (lane >> 2);
+  const int ld_chunk = (lane & 3) ^ ((lane >> 4) & 3);
+  // fragment reads: row = base + l32, chunk kc = 2*kk + lhi
+  const int sw = (l32 >> 2) & 3;
+  int frag_off[2];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int row = ld_row0 + 8 * i;
-    ld_chunk[i] = (lane & 7) ^ ((row >> 1) & 7);
-  }
-  // fragment reads: row = base + l32, chunk kc = 2*kk + lhi stored at slot kc ^ ((l32 >> 1) & 7)
-  const int sw = (l32 >> 1) & 7;
-  int frag_off[4];
-#pragma unroll
-  for (int kk = 0; kk < 4; ++kk) frag_off[kk] = ((2 * kk + lhi) ^ sw) << 4;
-  const int a_row_off = (wm * 128 + l32) * kRowBytes;
-  const int b_row_off0 = (SWIGLU ? wn * 32 + l32 : wn * 64 + l32) * kRowBytes;
-  const int b_row_off1 = (SWIGLU ? 128 + wn * 32 + l32 : wn * 64 + 32 + l32) * kRowBytes;
+  for (int kk = 0; kk < 2; ++kk) frag_off[kk] = ((2 * kk + lhi) ^ sw) << 4;
+  const int a_row_off = (wm * (FM * 32) + l32) * kRowBytes;
+  // B fragment j of this wave starts at LDS row b_row(j): plain tiles hold 256 weight rows; SwiGLU tiles hold 128
+  // gate rows then the 128 up rows of the same output columns, and fragments [0, FN/2) are gate, [FN/2, FN) up
+  auto b_row = [&](int j) {
+    if constexpr (SWIGLU) return (j < FN / 2 ? 0 : BN / 2) + wn * (FN / 2 * 32) + (j % (FN / 2)) * 32;
+    else return wn * (FN * 32) + j * 32;
+  };
+  const int b_lane_off = l32 * kRowBytes;
 
   // ---- per-tile state ------------------------------------------------------------------------------
-  struct Loader {   // where this thread's eight 16-byte loads per K step come from
+  struct Loader {   // where this thread's four 16-byte loads per K step come from
     const __bf16 *a_base, *b_base;
     uint32_t a_bytes, b_bytes;
-    uint32_t voff_a[4], voff_b[4];
-    int K, nk;
+    uint32_t voff_a[kLoads], voff_b[kLoads];
+    int K, nk;      // nk: K steps of the tile, rounded up to a multiple of kStages (padding steps read zeros)
   };
   struct Store {    // where the finished tile goes
     __bf16* c_base;
-    int rows, cols_left, ldc;  // valid rows / columns from the tile origin
+    int rows, cols_left, ldc, nk;
   };
 
-  auto setup = [&](const TileCoord& tc, Loader& L, Store& S) {
+  auto padded_steps = [](int k) { return ((k + BK - 1) / BK + kStages - 1) / kStages * kStages; };
+  auto setup_store = [&](const TileCoord& tc, Store& S) {
     const Group G = tc.group ? g1 : g0;
     const int row0 = tc.tm * BM, col0 = tc.tn * kTileN;
+    S.c_base = G.c + static_cast<int64_t>(row0) * G.ldc + col0;
+    S.rows = G.m - row0 < BM ? G.m - row0 : BM;
+    S.cols_left = G.n - col0;
+    S.ldc = G.ldc;
+    S.nk = padded_steps(G.k);
+  };
+  auto setup_loader = [&](const TileCoord& tc, Loader& L) {
+    const Group G = tc.group ? g1 : g0;
+#ifdef WX_EXP_SAMETILE
+    const int row0 = 0, col0 = 0;
+#elif defined(WX_EXP_SAMEXCD)
+    const int row0 = (blockIdx.x % 8) * BM, col0 = 0;
+#else
+    const int row0 = tc.tm * BM, col0 = tc.tn * kTileN;
+#endif
     const int rows_a = G.m - row0 < BM ? G.m - row0 : BM;
     const int rows_b = G.n - col0 < kTileN ? G.n - col0 : kTileN;
     L.K = G.k;
-    L.nk = (G.k + BK - 1) / BK;
+    L.nk = padded_steps(G.k);
     L.a_base = G.a + static_cast<int64_t>(row0) * G.lda;
-    const bool up_half = SWIGLU && wave >= 4;
+    constexpr int kHalfWaves = kWavesM * kWavesN / 2;  // SwiGLU: the first half of the waves load gate rows
+    const bool up_half = SWIGLU && wave >= kHalfWaves;
     L.b_base = (up_half ? G.b1 : G.b0) + static_cast<int64_t>(col0) * G.ldb;
     L.a_bytes = static_cast<uint32_t>(rows_a) * G.lda * 2u;
     L.b_bytes = static_cast<uint32_t>(rows_b) * G.ldb * 2u;
-    const int b_ld_row0 = SWIGLU ? (wave & 3) * 32 + (lane >> 3) : ld_row0;  // row inside the gate / up half
+    const int b_ld_row0 = SWIGLU ? (wave % kHalfWaves) * kLoadRows + (lane >> 2) : ld_row0;  // row inside its half
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      L.voff_a[i] = static_cast<uint32_t>(ld_row0 + 8 * i) * G.lda * 2u + ld_chunk[i] * 16u;
-      L.voff_b[i] = static_cast<uint32_t>(b_ld_row0 + 8 * i) * G.ldb * 2u + ld_chunk[i] * 16u;
+    for (int i = 0; i < kLoads; ++i) {
+      L.voff_a[i] = static_cast<uint32_t>(ld_row0 + 16 * i) * G.lda * 2u + ld_chunk * 16u;
+      L.voff_b[i] = static_cast<uint32_t>(b_ld_row0 + 16 * i) * G.ldb * 2u + ld_chunk * 16u;
     }
-    S.c_base = G.c + static_cast<int64_t>(row0) * G.ldc + col0;
-    S.rows = rows_a;
-    S.cols_left = G.n - col0;
-    S.ldc = G.ldc;
   };
 
-  // One K step of global -> LDS for this wave: rows [wave*32, +32) of the A tile and of the B tile.
+  // One K step of global -> LDS for this wave: rows [wave*64, +64) of the A slot and of the B slot.
   auto issue = [&](const Loader& L, int ks, unsigned char* sa, unsigned char* sb) {
     const int k0 = ks * BK;
-    // advancing the base keeps the absolute end of the readable range: rows past the matrix and, through the
-    // per-lane select below, K chunks past the row end read as zero
-    const __amdgpu_buffer_rsrc_t ra = make_rsrc(L.a_base + k0, L.a_bytes - 2u * k0);
-    const __amdgpu_buffer_rsrc_t rb = make_rsrc(L.b_base + k0, L.b_bytes - 2u * k0);
+    // advancing the base keeps the absolute end of the readable range, so rows past the matrix read as zero;
+    // K chunks at or past the row end are pushed out of range per lane (this also zero-fills padding steps)
+    const uint32_t adv = 2u * static_cast<uint32_t>(k0);
+#ifdef WX_EXP_OOB
+    const __amdgpu_buffer_rsrc_t ra = make_rsrc(L.a_base + k0, 0u);
+    const __amdgpu_buffer_rsrc_t rb = make_rsrc(L.b_base + k0, 0u);
+#else
+    const __amdgpu_buffer_rsrc_t ra = make_rsrc(L.a_base + k0, L.a_bytes > adv ? L.a_bytes - adv : 0u);
+    const __amdgpu_buffer_rsrc_t rb = make_rsrc(L.b_base + k0, L.b_bytes > adv ? L.b_bytes - adv : 0u);
+#endif
     const bool k_tail = k0 + BK > L.K;
+    const uint32_t oob = (k_tail && k0 + ld_chunk * 8 >= L.K) ? 0x80000000u : 0u;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      uint32_t va = L.voff_a[i], vb = L.voff_b[i];
-      if (k_tail && k0 + ld_chunk[i] * 8 >= L.K) va = vb = 0x80000000u;
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, LDS_PTR(sa + (wave * 32 + 8 * i) * kRowBytes), 16, va, 0, 0, 0);
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, LDS_PTR(sb + (wave * 32 + 8 * i) * kRowBytes), 16, vb, 0, 0, 0);
+    for (int i = 0; i < kLoads; ++i) {
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, LDS_PTR(sa + (wave * kLoadRows + 16 * i) * kRowBytes), 16,
+                                               L.voff_a[i] | oob, 0, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, LDS_PTR(sb + (wave * kLoadRows + 16 * i) * kRowBytes), 16,
+                                               L.voff_b[i] | oob, 0, 0, 0);
     }
   };
 
-  f32x16 acc[4][2];
-  bf16x8 fa[2][4], fb[2][2];  // two fragment sets: one feeds the MFMAs while the other is being read from LDS
+  f32x16 acc[FM][FN];
+  bf16x8 fa[2][FM], fb[2][FN];  // two fragment sets: one feeds the MFMAs while the other is being read from LDS
 
   auto read_frags = [&](const unsigned char* sa, const unsigned char* sb, int kk, int set) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < FM; ++i)
       fa[set][i] = *reinterpret_cast<const bf16x8*>(sa + a_row_off + i * 32 * kRowBytes + frag_off[kk]);
-    fb[set][0] = *reinterpret_cast<const bf16x8*>(sb + b_row_off0 + frag_off[kk]);
-    fb[set][1] = *reinterpret_cast<const bf16x8*>(sb + b_row_off1 + frag_off[kk]);
+#pragma unroll
+    for (int j = 0; j < FN; ++j)
+      fb[set][j] = *reinterpret_cast<const bf16x8*>(sb + b_row(j) * kRowBytes + b_lane_off + frag_off[kk]);
   };
   auto mma = [&](int set) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < FM; ++i)
 #pragma unroll
-      for (int j = 0; j < 2; ++j)
+      for (int j = 0; j < FN; ++j)
         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[set][i], fb[set][j], acc[i][j], 0, 0, 0);
   };
-  // scheduling hints: interleave the six LDS reads of the next fragment set with the eight MFMAs of this one
-  auto interleave_reads = [&]() {
+  // scheduling hint: the LDS reads of the next fragment set go out early among the MFMAs of this one
+  auto front_load_reads = [&]() {
 #pragma unroll
-    for (int q = 0; q < 6; ++q) {
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one LDS read
+    for (int q = 0; q < (FM + FN) / 2; ++q) {
+      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);  // two LDS reads
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
     }
-    __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+    __builtin_amdgcn_sched_group_barrier(0x008, FM * FN - (FM + FN) / 2, 0);
   };
 
-  // One K step.  On entry fragment set 0 holds kk = 0 of the current stage.  The barrier sits before the last
-  // quarter: by then every wave has its kk = 3 fragments in registers, so the current stage can be refilled
-  // (K step ks + 2) right after it, and the next stage -- issued a whole K step earlier -- is complete.
-  auto k_step = [&](const Loader& L, int ks, unsigned char* sa_cur, unsigned char* sb_cur, unsigned char* sa_nxt,
-                    unsigned char* sb_nxt) {
-    read_frags(sa_cur, sb_cur, 1, 1);
+  // One K step on slot (sa, sb); (sa_n, sb_n) is the next slot of the ring.  On entry fragment set 0 holds kk = 0
+  // of this slot.  After the barrier every wave has finished reading this slot, so it is refilled at once with the
+  // K step kStages ahead in the load stream (step `ld_ks` of tile `L`); the next slot's data was issued
+  // kStages - 1 steps ago.
+  auto k_step = [&](const Loader& L, int ld_ks, unsigned char* sa, unsigned char* sb, unsigned char* sa_n,
+                    unsigned char* sb_n) {
+    read_frags(sa, sb, 1, 1);
     mma(0);
-    interleave_reads();
-    read_frags(sa_cur, sb_cur, 2, 0);
+    front_load_reads();
+    // my LDS reads have returned; of my loads at most the two youngest K steps (2 * kLoads loads each) are still
+    // in flight, i.e. the next slot is complete
+#ifndef WX_EXP_NOWAIT
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(2 * 2 * kLoads, 0));
+#endif
+#ifndef WX_EXP_NOBARRIER
+    __syncthreads();
+#endif
+#ifndef WX_EXP_NOLOAD
+    issue(L, ld_ks, sa, sb);
+#endif
+    __builtin_amdgcn_sched_barrier(0);  // keep the refill right behind the barrier: it has the longest way to go
+    read_frags(sa_n, sb_n, 0, 0);
     mma(1);
-    interleave_reads();
-    read_frags(sa_cur, sb_cur, 3, 1);
-    mma(0);
-    interleave_reads();
-    if (ks + 1 < L.nk) {
-      __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0): my loads for ks+1 landed, my LDS reads returned
-      __syncthreads();
-      if (ks + 2 < L.nk) issue(L, ks + 2, sa_cur, sb_cur);
-      read_frags(sa_nxt, sb_nxt, 0, 0);
-    }
-    mma(1);
+    front_load_reads();
   };
 
   auto epilogue = [&](const Store& S) {
-    // accumulator register r of lane l holds row 8*(r/4) + 4*(l/32) + r%4, column l%32 of its 32x32 block
+    // accumulator register r of lane l holds row 8*(r/4) + 4*(l/32) + r%4, column l%32 of its 32x32 block.
+    // The lane terms are laundered through an empty asm so the per-row address arithmetic is redone here each
+    // tile instead of being hoisted out of the persistent loop and held in registers across the K loop.
+    int lhi_e = lhi, l32_e = l32;
+    asm volatile("" : "+v"(lhi_e), "+v"(l32_e));
+    const int l32 = l32_e;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < FM; ++i) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const int row = wm * 128 + i * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
+        const int row = wm * (FM * 32) + i * 32 + 8 * (r >> 2) + 4 * lhi_e + (r & 3);
         if (row >= S.rows) continue;
         __bf16* c_row = S.c_base + static_cast<int64_t>(row) * S.ldc;
         if constexpr (SWIGLU) {
-          const int col = wn * 32 + l32;
-          if (col < S.cols_left) {
-            // eager bf16 evaluation of act_fn(gate) * up (act.py:80-82): gate, up, silu(gate) and the product are
-            // each rounded to bf16
-            const float g = round_bf16(acc[i][0][r]);
-            const float u = round_bf16(acc[i][1][r]);
-            const float sg = round_bf16(g / (1.0f + expf(-g)));
-            c_row[col] = static_cast<__bf16>(sg * u);
+#pragma unroll
+          for (int j = 0; j < FN / 2; ++j) {
+            const int col = wn * (FN / 2 * 32) + j * 32 + l32;
+            if (col < S.cols_left) {
+              // eager bf16 evaluation of act_fn(gate) * up (act.py:80-82): gate, up, silu(gate) and the product
+              // are each rounded to bf16
+              const float g = round_bf16(acc[i][j][r]);
+              const float u = round_bf16(acc[i][j + FN / 2][r]);
+              const float sg = round_bf16(g / (1.0f + expf(-g)));
+              c_row[col] = static_cast<__bf16>(sg * u);
+            }
           }
         } else {
 #pragma unroll
-          for (int j = 0; j < 2; ++j) {
-            const int col = wn * 64 + j * 32 + l32;
+          for (int j = 0; j < FN; ++j) {
+            const int col = wn * (FN * 32) + j * 32 + l32;
             if (col < S.cols_left) c_row[col] = static_cast<__bf16>(acc[i][j][r]);
           }
         }
@@ -269,53 +322,69 @@ __global__ __launch_bounds__(kThreads, 1) void dual_gemm_kernel(Params p) {
     }
   };
 
-  // first two K steps of a tile go out together; later ones are issued from inside k_step
-  auto prologue = [&](const Loader& L) {
-    issue(L, 0, s_a0, s_b0);
-    if (L.nk > 1) issue(L, 1, s_a1, s_b1);
+  // ---- persistent loop -------------------------------------------------------------------------------
+  // The load stream runs kStages K steps ahead of the MFMAs and crosses tile boundaries: the last kStages steps
+  // of a tile refill the ring with the first kStages steps of the next tile, so the pipeline never drains and
+  // the next tile's data lands while this tile's results are stored.  After the last tile the stream continues
+  // with an empty descriptor (every load out of range, nothing fetched), which keeps the in-flight accounting
+  // of the waits uniform.
+  int next_t = blockIdx.x;
+  auto next_tile = [&](TileCoord& tc) {
+    bool have = false;
+    for (; next_t < padded && !have; next_t += gridDim.x) have = map_tile(next_t, total, tiles_m, tiles_n, tc);
+    return have;
   };
-
-  // ---- persistent tile loop -----------------------------------------------------------------------
-  int64_t t = blockIdx.x;
   TileCoord tc;
-  bool have = false;
-  for (; t < padded && !have; t += have ? 0 : gridDim.x) have = map_tile(t, total, tiles_m, tiles_n, tc);
+  bool have = next_tile(tc);
   if (!have) return;
   Loader L;
   Store S;
-  setup(tc, L, S);
-  prologue(L);
+  setup_loader(tc, L);
+  setup_store(tc, S);
+  issue(L, 0, s_a0, s_b0);
+  issue(L, 1, s_a1, s_b1);
+  issue(L, 2, s_a2, s_b2);
+  issue(L, 3, s_a3, s_b3);
+  // slot 0 must be complete before its first fragments are read: three younger K steps may remain in flight
+  __builtin_amdgcn_s_waitcnt(waitcnt_imm(3 * 2 * kLoads, 15));
+  __syncthreads();
+  read_frags(s_a0, s_b0, 0, 0);
 
-  while (true) {
+  while (have) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < FM; ++i)
 #pragma unroll
-      for (int j = 0; j < 2; ++j)
+      for (int j = 0; j < FN; ++j)
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-    // stage 0 (K step 0) must be complete; K step 1 may still be in flight (8 loads per wave per K step)
-    if (L.nk > 1) __builtin_amdgcn_s_waitcnt(0x0F78); else __builtin_amdgcn_s_waitcnt(0x0F70);
-    __syncthreads();
-    read_frags(s_a0, s_b0, 0, 0);
-    for (int ks = 0; ks < L.nk; ks += 2) {
-      k_step(L, ks, s_a0, s_b0, s_a1, s_b1);
-      if (ks + 1 < L.nk) k_step(L, ks + 1, s_a1, s_b1, s_a0, s_b0);
-    }
-
-    // next tile: its first loads fly while this tile's results are stored
-    TileCoord tn;
-    bool more = false;
-    for (t += gridDim.x; t < padded && !more; t += more ? 0 : gridDim.x) more = map_tile(t, total, tiles_m, tiles_n, tn);
     const Store done = S;
-    __syncthreads();  // every wave holds its last fragments in registers: both stages are free
-    if (more) {
-      setup(tn, L, S);
-      prologue(L);
+    const int nk = S.nk;
+    for (int ks = 0; ks < nk; ks += kStages) {
+      int ld_ks = ks + kStages;
+      if (ld_ks == nk) {  // the loader moves on to the next tile (or to the empty descriptor)
+        have = next_tile(tc);
+        if (have) {
+          setup_loader(tc, L);
+          setup_store(tc, S);
+        } else {
+          L.a_bytes = 0;
+          L.b_bytes = 0;
+        }
+        ld_ks = 0;
+      }
+      k_step(L, ld_ks + 0, s_a0, s_b0, s_a1, s_b1);
+      k_step(L, ld_ks + 1, s_a1, s_b1, s_a2, s_b2);
+      k_step(L, ld_ks + 2, s_a2, s_b2, s_a3, s_b3);
+      k_step(L, ld_ks + 3, s_a3, s_b3, s_a0, s_b0);
     }
+#ifndef WX_EXP_NOEPI
     epilogue(done);
-    if (!more) break;
+#else
+    if (acc[0][0][0] == 123.456f) epilogue(done);
+#endif
   }
+#endif
 }
 
 // ---- generic fallback: any transpose combination, any k; one thread per output element pair -----------

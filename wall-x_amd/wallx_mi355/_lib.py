@@ -9,7 +9,8 @@ import os
 import threading
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libwallx_mi355.so")
+# WALLX_MI355_LIB points at an alternative build of the same library (e.g. one compiled with other tuning flags)
+LIB_PATH = os.environ.get("WALLX_MI355_LIB") or os.path.join(_HERE, "libwallx_mi355.so")
 
 WX_F32, WX_F16, WX_BF16 = 0, 1, 2
 WX_I32, WX_I64, WX_U8 = 0, 1, 2
