@@ -5,7 +5,7 @@
 
 One step = one pass of the hot path over the serving batch of BASELINE config 3: 32 sequences x 912 tokens
 (880 VL + 32 action per sequence, seeded per-token mask), hidden 2048, VL expert 11008, action expert 1024,
-bf16: token partition -> row permute -> gate/up GEMM + SwiGLU (both experts, one launch) -> down GEMM (both
+bf16: token partition -> row permute (into the K-tiled activation layout) -> gate/up GEMM + SwiGLU (both experts, one launch) -> down GEMM (both
 experts, one launch) -> row unpermute.  Inputs are resident in HBM before the timed region.
 
 Prints ONE JSON line.  `value` = algorithmic FFN FLOPs (6*H*(m0*I0 + m1*I1)) / whole-step time, i.e. the
@@ -38,7 +38,7 @@ def parse():
     ap.add_argument("--ops-only", action="store_true", help="skip the side measurements (M-RoPE, index builders)")
     ap.add_argument("--cpu-seqs", type=int, default=4, help="sequences of the batch the CPU baseline runs")
     ap.add_argument("--kernel-loop", default=None,
-                    choices=["gate_up", "down", "permute", "unpermute", "partition", "copy"],
+                    choices=["gate_up", "down", "permute", "permute_plain", "unpermute", "partition", "copy"],
                     help="profiling aid: run only this kernel --steps times (no JSON line); 'copy' is a plain "
                          "device-to-device copy of the [T, H] activations, the known-size yardstick for HBM counters")
     return ap.parse_args()
@@ -93,9 +93,13 @@ def main():
     down_flops = 2.0 * H * (m0 * I0 + m1 * I1)
     row_bytes = 2.0 * T * H * 2 + 8.0 * T  # read + write of [T, H] bf16 plus the index traffic
 
-    hmid = torch.empty(T * max(I0, I1), dtype=torch.bfloat16, device=dev)
+    rows_pad = native.padded_sorted_rows(T)
+    hmid = torch.empty(rows_pad * max(I0, I1), dtype=torch.bfloat16, device=dev)
     x_sorted = torch.empty_like(x)
+    x_tiled = torch.empty(rows_pad * H, dtype=torch.bfloat16, device=dev)
     y_sorted = torch.empty_like(x)
+    # expert weights in the K-tiled layout the MFMA kernels read (packed once, outside the timed region)
+    pg0, pu0, pd0, pg1, pu1, pd1 = (native.pack_weight(w) for w in (g0, u0, d0, g1, u1, d1))
     y = torch.empty_like(x)
     ws = None
     stream = torch.cuda.current_stream().cuda_stream
@@ -106,17 +110,21 @@ def main():
         nonlocal row_id_map, offsets, ws
         row_id_map, offsets, _, ws = native.partition(types, 2, 0, ws)
 
-    def permute():
+    def permute():  # the layer's permute: rows go straight into the K-tiled activation matrix
+        _lib.call("wx_permute_rows_tiled", x.data_ptr(), x_tiled.data_ptr(), row_id_map.data_ptr(),
+                  offsets.data_ptr(), T, H, stream)
+
+    def permute_plain():  # the stand-alone op of the reference API (row-major output)
         _lib.call("wx_permute_rows", x.data_ptr(), x_sorted.data_ptr(), row_id_map.data_ptr(), T, 1, H,
                   _lib.WX_BF16, stream)
 
     def gate_up():
-        _lib.call("wx_dual_swiglu_gate_up", x_sorted.data_ptr(), hmid.data_ptr(), offsets.data_ptr(), g0.data_ptr(),
-                  u0.data_ptr(), g1.data_ptr(), u1.data_ptr(), T, H, I0, I1, stream)
+        _lib.call("wx_dual_swiglu_gate_up", x_tiled.data_ptr(), hmid.data_ptr(), offsets.data_ptr(), pg0.data_ptr(),
+                  pu0.data_ptr(), pg1.data_ptr(), pu1.data_ptr(), T, H, I0, I1, stream)
 
     def down():
-        _lib.call("wx_dual_down_proj", hmid.data_ptr(), y_sorted.data_ptr(), offsets.data_ptr(), d0.data_ptr(),
-                  d1.data_ptr(), T, H, I0, I1, stream)
+        _lib.call("wx_dual_down_proj", hmid.data_ptr(), y_sorted.data_ptr(), offsets.data_ptr(), pd0.data_ptr(),
+                  pd1.data_ptr(), T, H, I0, I1, stream)
 
     def unpermute():
         _lib.call("wx_unpermute_rows", y_sorted.data_ptr(), y.data_ptr(), row_id_map.data_ptr(), None, T, 1, H,
@@ -131,7 +139,8 @@ def main():
 
     if args.kernel_loop:
         permute(); gate_up(); down()
-        fn = {"gate_up": gate_up, "down": down, "permute": permute, "unpermute": unpermute, "partition": partition,
+        fn = {"gate_up": gate_up, "down": down, "permute": permute, "permute_plain": permute_plain,
+              "unpermute": unpermute, "partition": partition,
               "copy": lambda: x_sorted.copy_(x)}[args.kernel_loop]
         for _ in range(args.steps):
             fn()
@@ -155,6 +164,7 @@ def main():
     t_gate_up, t_gate_up_avg = event_ms(gate_up, iters)
     t_down, _ = event_ms(down, iters)
     t_perm, _ = event_ms(permute, iters)
+    t_perm_plain, _ = event_ms(permute_plain, iters)
     t_unperm, _ = event_ms(unpermute, iters)
     t_part, _ = event_ms(partition, iters)
     gate_up_tflops = gate_up_flops / (t_gate_up_avg * 1e-3) / 1e12
@@ -164,6 +174,7 @@ def main():
         "down_ms": round(t_down, 4), "down_tflops": round(down_flops / t_down / 1e9, 1),
         "ffn_kernels_tflops": round(ffn_flops / (t_gate_up + t_down) / 1e9, 1),
         "permute_ms": round(t_perm, 4), "permute_GBps": round(row_bytes / t_perm / 1e6, 1),
+        "permute_rowmajor_ms": round(t_perm_plain, 4), "permute_rowmajor_GBps": round(row_bytes / t_perm_plain / 1e6, 1),
         "unpermute_ms": round(t_unperm, 4), "unpermute_GBps": round(row_bytes / t_unperm / 1e6, 1),
         "permute_frac_hbm_peak": round(row_bytes / t_perm / 1e6 / PEAK_HBM_GBS, 4),
         "partition_us": round(t_part * 1e3, 2),

@@ -87,16 +87,42 @@ int wx_dual_gemm(const void* in0, const void* in1, const void* w0, const void* w
                  void* out1, int64_t m0, int64_t n0, int64_t k0, int64_t m1, int64_t n1, int64_t k1,
                  int trans_a, int trans_b, wx_stream_t stream);
 
+/* ------------------------------------------------------------------------------------------------
+ * K-tiled operands of the fused FFN.  The MFMA kernels read activations and weights from a block layout in
+ * which every 16-row x 32-column block (1 KiB, bank-swizzled for LDS) is contiguous and the 256 x 32 slab a
+ * workgroup consumes per K step is one contiguous run -- the access pattern the memory pipeline serves fastest.
+ * The layout is internal to this library: weights are packed once (wx_pack_tiled), activations are written in
+ * it by wx_permute_rows_tiled, the intermediate never leaves it.  Only bf16; cols must be a multiple of 32.
+ * wx_tiled_bytes: size of a packed [rows, cols] matrix (rows padded to 16).  wx_padded_sorted_rows: rows of the
+ * expert-sorted space for `rows` tokens once each expert's range starts at a multiple of 256 (an upper bound that
+ * depends on `rows` only).  These have no counterpart in the reference (its GEMMs read nn.Linear weights in place). */
+size_t wx_tiled_bytes(int64_t rows, int64_t cols);
+int64_t wx_padded_sorted_rows(int64_t rows);
+int wx_pack_tiled(const void* src_row_major, void* dst_tiled, int64_t rows, int64_t cols,
+                  wx_stream_t stream);
+
+/* Permute straight into the K-tiled activation matrix of the FFN: row t of x goes to sorted row
+ * row_id_map[t], shifted for expert 1 so that its rows start at a multiple of 256.  Replaces
+ * moe_permute_topK_kernel's forward branch (csrc/permute.cu:156-262) for topK == 1 when the consumer is
+ * wx_dual_swiglu_ffn.  out_tiled: wx_tiled_bytes(wx_padded_sorted_rows(T), num_cols) bytes.
+ * expert_offsets: device int32[3] from wx_partition_build. */
+int wx_permute_rows_tiled(const void* x, void* out_tiled, const int32_t* row_id_map,
+                          const int32_t* expert_offsets, int64_t num_tokens, int64_t num_cols,
+                          wx_stream_t stream);
+
 /* Both experts' SwiGLU FFN over expert-sorted rows, two launches (gate/up + SwiGLU, then down), each
- * covering both experts:  out[r, :] = down_e( silu(x[r] @ gate_e^T) * (x[r] @ up_e^T) ) for rows
+ * covering both experts:  out[r, :] = down_e( silu(x[r] @ gate_e^T) * (x[r] @ up_e^T) ) for sorted rows
  * r in [expert_offsets[e], expert_offsets[e+1]).  Replaces the per-expert loop of
  * SparseMoeBlock.forward over BlockSparseMLP (act.py:79-82, 142-154).
- * x, out: [num_rows, hidden] bf16;  gate_e, up_e: [inter_e, hidden];  down_e: [hidden, inter_e].
+ * x_tiled: K-tiled activations from wx_permute_rows_tiled.  out: [num_rows, hidden] bf16 row-major in sorted
+ * order (what wx_unpermute_rows reads).  gate_e, up_e: packed [inter_e, hidden]; down_e: packed
+ * [hidden, inter_e] (wx_pack_tiled of the nn.Linear weights).
  * expert_offsets: DEVICE int32[3] (from wx_partition_build), read by the kernels -- no host sync.
- * hmid: device scratch, num_rows * max(inter0, inter1) bf16.
+ * hmid: device scratch, wx_padded_sorted_rows(num_rows) * max(inter0, inter1) bf16.
+ * hidden, inter0, inter1 must be multiples of 32.
  * Intermediate rounding follows eager bf16 evaluation: gate, up, silu(gate) and the product are each
  * rounded to bf16 (fp32 accumulation inside each contraction). */
-int wx_dual_swiglu_ffn(const void* x, void* out, const int32_t* expert_offsets, const void* gate0,
+int wx_dual_swiglu_ffn(const void* x_tiled, void* out, const int32_t* expert_offsets, const void* gate0,
                        const void* up0, const void* down0, const void* gate1, const void* up1,
                        const void* down1, void* hmid, int64_t num_rows, int64_t hidden,
                        int64_t inter0, int64_t inter1, wx_stream_t stream);
@@ -104,9 +130,10 @@ int wx_dual_swiglu_ffn(const void* x, void* out, const int32_t* expert_offsets, 
 /* The two launches of wx_dual_swiglu_ffn on their own, for callers that put work between them (and for
  * timing each kernel): hmid = silu(x @ gate^T) * (x @ up^T), then out = hmid @ down^T, per expert.
  * Same arguments and layouts as above; they replace the same reference lines (act.py:79-82, 142-154). */
-int wx_dual_swiglu_gate_up(const void* x, void* hmid, const int32_t* expert_offsets, const void* gate0,
-                           const void* up0, const void* gate1, const void* up1, int64_t num_rows,
-                           int64_t hidden, int64_t inter0, int64_t inter1, wx_stream_t stream);
+int wx_dual_swiglu_gate_up(const void* x_tiled, void* hmid, const int32_t* expert_offsets,
+                           const void* gate0, const void* up0, const void* gate1, const void* up1,
+                           int64_t num_rows, int64_t hidden, int64_t inter0, int64_t inter1,
+                           wx_stream_t stream);
 int wx_dual_down_proj(const void* hmid, void* out, const int32_t* expert_offsets, const void* down0,
                       const void* down1, int64_t num_rows, int64_t hidden, int64_t inter0,
                       int64_t inter1, wx_stream_t stream);

@@ -108,7 +108,7 @@ def _moe_weights(hidden, inters, g, std=0.02):
 
 @pytest.mark.parametrize("T,n_act,hidden,inters", [
     (512, 64, 256, (384, 128)),
-    (700, 33, 512, (1000, 136)),
+    (700, 33, 512, (1056, 160)),
     (300, 0, 256, (256, 128)),
     (300, 300, 256, (256, 128)),
     (1, 1, 64, (64, 64)),

@@ -24,11 +24,9 @@ __device__ __forceinline__ int lane_id() { return static_cast<int>(threadIdx.x) 
 // ---- 16-bit float <-> fp32, round-to-nearest-even (NaN kept quiet) -------------------------------
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t b) { return __uint_as_float(b << 16); }
 
+// gfx950 converts fp32 -> bf16 in hardware (round to nearest even, NaN kept quiet): one instruction, no branches
 __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;  // NaN
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return u >> 16;
+  return __builtin_bit_cast(uint16_t, static_cast<__bf16>(f));
 }
 
 __device__ __forceinline__ float round_bf16(float f) { return bf16_bits_to_f32(f32_to_bf16_bits(f)); }

@@ -1,25 +1,31 @@
 // Dual asymmetric grouped GEMM and the fused dual-expert SwiGLU FFN for gfx950 (bf16 MFMA, fp32 accumulate).
 //
-// One persistent launch covers the tiles of BOTH experts: the grid is one workgroup per CU, the tile list
-// is derived on the device from the per-expert row counts (host values or the partition's device-side
-// expert_offsets), and a tile id -> (expert, tile_m, tile_n) map keeps the 32 tiles that run concurrently
-// on one XCD inside a compact patch of the output so they share A/B slabs through that XCD's L2.
-// A skewed pair (thousands of VL rows, tens of action rows, or an empty group) is just a longer or
-// shorter tile list; no CU waits for "its" expert.
+// One persistent launch covers the tiles of BOTH experts: the grid is one workgroup per CU, the tile list is
+// derived on the device from the per-expert row counts (host values, or the partition's device-side
+// expert_offsets), and the tile id -> (expert, tile_m, tile_n) map keeps the 32 tiles that run concurrently on one
+// XCD inside a compact patch of the output so they share operand slabs through that XCD's L2.  A skewed pair
+// (thousands of VL rows next to tens of action rows, or an empty group) is just a longer or shorter tile list.
 //
-// Workgroup tile 256 x 256 x 64, 8 wavefronts as 2 (M) x 4 (N), wave tile 128 x 64 = 4 x 2 MFMA
-// 32x32x16 accumulators.  Operands are K-contiguous ([m,k] activations, [n,k] nn.Linear weights), so both
-// fragments are 16-byte LDS reads.  Global -> LDS goes through buffer loads that write LDS directly
-// (no VGPR staging), double buffered, one barrier per K step; rows past the end of a matrix read as zero
-// through the buffer bounds check.  LDS rows are 128 bytes (64 bf16); the 16-byte chunk c of row r is
-// stored at slot c ^ ((r >> 1) & 7) so that the 16 rows a quarter-wave reads land on distinct banks.
+// Workgroup tile 256 x 256, K step 32, four wavefronts (one per SIMD) as 2 x 2, wave tile 128 x 128 = 4 x 4 MFMA
+// 32x32x16 accumulator blocks (256 accumulator registers per lane).  Operands are K-contiguous, so both MFMA
+// fragments are 16-byte LDS reads.  Global -> LDS uses buffer loads that write LDS directly (no register
+// staging) into a ring of four K-step slots per operand; the load stream runs four K steps ahead of the MFMAs and
+// crosses tile boundaries, with one workgroup barrier per K step.  LDS rows are 64 bytes; chunk c of row r sits
+// in slot c ^ ((r >> 2) & 3), which makes the 16-byte fragment reads bank-conflict free.
 //
-// SwiGLU mode: the B tile is 128 gate rows + 128 up rows of the same intermediate columns, so gate and
-// up accumulators of one output element sit in the same lane and register index; the epilogue applies
-// silu(g) * u with eager bf16 rounding and writes the 256 x 128 intermediate tile.
+// Three operand layouts:
+//   generic  (wx_dual_gemm)            A, B, C row-major; loads touch 16 rows x 64 bytes per instruction.
+//   gate/up  (wx_dual_swiglu_gate_up)  A = K-tiled activations, B = K-tiled gate and up weights (the B tile is 128
+//                                      gate rows + 128 up rows of the same output columns, so gate and up of an
+//                                      output element meet in one lane), C = K-tiled intermediate, SwiGLU epilogue.
+//   down     (wx_dual_down_proj)       A = K-tiled intermediate, B = K-tiled down weights, C row-major.
+// With K-tiled operands every load instruction moves one contiguous KiB (tiled_layout.h).
+// Results leave through a per-wave LDS staging area so that global stores are full 16-byte lanes on contiguous
+// runs (whole 1 KiB blocks for the tiled intermediate, 256-byte row segments for row-major outputs).
 #include <type_traits>
 
 #include "common.h"
+#include "tiled_layout.h"
 
 namespace wx {
 namespace {
@@ -29,29 +35,34 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 constexpr int BM = 256, BN = 256, BK = 32;
 constexpr int kWavesM = 2, kWavesN = 2;        // wavefront grid over the tile; one wavefront per SIMD
-constexpr int kThreads = kWavesM * kWavesN * 64;
+constexpr int kWaves = kWavesM * kWavesN;
+constexpr int kThreads = kWaves * 64;
 constexpr int FM = BM / kWavesM / 32;          // 32x32 accumulator blocks per wave along M (4)
 constexpr int FN = BN / kWavesN / 32;          // ... and along N (4): 256 accumulator registers per lane
-constexpr int kLoadRows = BM / (kWavesM * kWavesN);  // LDS rows of each operand one wave loads per K step (64)
+constexpr int kLoadRows = BM / kWaves;         // LDS rows of each operand one wave loads per K step (64)
 constexpr int kLoads = kLoadRows / 16;         // 16-row load instructions per operand per wave per K step (4)
 constexpr int kStages = 4;                     // ring slots per operand (the tile loop is written out for 4)
 constexpr int kRowBytes = BK * 2;              // 64 bytes of K per LDS row
 constexpr int kSlotBytes = BM * kRowBytes;     // 16 KiB per operand per K step
+constexpr int kStageBytes = 8192;              // per-wave staging for the epilogue
 constexpr int kXcds = 8;
 constexpr int kGroupM = 8;                     // tile rows per patch in the tile order
 
+enum Mode { kGeneric = 0, kGateUp = 1, kDown = 2 };
+
 struct Group {
-  const __bf16* a;    // [m, k] row-major, leading dimension lda
-  const __bf16* b0;   // [n, k] row-major (SwiGLU: gate)
-  const __bf16* b1;   // SwiGLU: up; otherwise unused
-  __bf16* c;          // [m, n] row-major, leading dimension ldc
+  const __bf16* a;   // generic: [m, k] row-major (lda).  tiled: base of the K-tiled matrix
+  const __bf16* b0;  // generic: [n, k] row-major (ldb).  tiled: K-tiled weights (gate for kGateUp)
+  const __bf16* b1;  // kGateUp: K-tiled up weights
+  __bf16* c;         // row-major [m, n] (ldc), or base of the K-tiled intermediate (kGateUp)
   int m, n, k;
-  int lda, ldb, ldc;
+  int lda, ldb, ldc;  // row-major: leading dimension in elements.  tiled: number of 16-row blocks of the matrix
+  int a_row0;         // tiled A: first row of this group inside the tiled matrix (a multiple of 256)
 };
 
 struct Params {
   Group g[2];
-  const int32_t* offsets;  // device int32[3]: rows of expert e are [offsets[e], offsets[e+1]); or null
+  const int32_t* offsets;  // device int32[3]: rows of expert e are [offsets[e], offsets[e+1]); null for kGeneric
 };
 
 #define LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
@@ -96,9 +107,18 @@ __device__ __forceinline__ bool map_tile(int t, int total, const int* tiles_m, c
   return true;
 }
 
-template <bool SWIGLU>
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  const bf16x2 v = {static_cast<__bf16>(lo), static_cast<__bf16>(hi)};  // one packed convert
+  return __builtin_bit_cast(uint32_t, v);
+}
+
+template <int MODE>
 __global__ __launch_bounds__(kThreads, 1) void dual_gemm_kernel(Params p) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stub; the body uses gfx950-only builtins
+  constexpr bool SWIGLU = MODE == kGateUp;
+  constexpr bool TILED_IN = MODE != kGeneric;   // A and B are K-tiled
+  constexpr bool TILED_OUT = MODE == kGateUp;   // C is K-tiled
   // kStages ring slots per operand, each one K step (256 rows x 32 bf16).  Separate arrays let the compiler
   // see that a read of one slot never waits for a buffer load that targets another.
   __shared__ __attribute__((aligned(1024))) unsigned char s_a0[kSlotBytes];
@@ -109,6 +129,7 @@ __global__ __launch_bounds__(kThreads, 1) void dual_gemm_kernel(Params p) {
   __shared__ __attribute__((aligned(1024))) unsigned char s_b1[kSlotBytes];
   __shared__ __attribute__((aligned(1024))) unsigned char s_b2[kSlotBytes];
   __shared__ __attribute__((aligned(1024))) unsigned char s_b3[kSlotBytes];
+  __shared__ __attribute__((aligned(1024))) unsigned char s_out[kWaves * kStageBytes];
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keeps descriptors and LDS bases scalar
@@ -118,14 +139,29 @@ __global__ __launch_bounds__(kThreads, 1) void dual_gemm_kernel(Params p) {
   // ---- problem table (uniform) ------------------------------------------------------------------
   // (kept as two named structs, selected per tile, so everything stays in scalar registers)
   Group g0 = p.g[0], g1 = p.g[1];
-  if (p.offsets != nullptr) {
+  if constexpr (MODE != kGeneric) {
     const int o0 = p.offsets[0], o1 = p.offsets[1], o2 = p.offsets[2];
     g0.m = o1 - o0;
     g1.m = o2 - o1;
-    g0.a += static_cast<int64_t>(o0) * g0.lda;
-    g0.c += static_cast<int64_t>(o0) * g0.ldc;
-    g1.a = g0.a + static_cast<int64_t>(g0.m) * g0.lda;
-    g1.c = g0.c + static_cast<int64_t>(g0.m) * g0.ldc;
+    const int pad0 = static_cast<int>(round_up_256(g0.m)), pad1 = static_cast<int>(round_up_256(g1.m));
+    if constexpr (MODE == kGateUp) {
+      // A: one tiled activation matrix, expert 1 starts at the next multiple of 256 rows.
+      // C: per-expert tiled intermediates, packed one after the other
+      g0.a_row0 = 0;
+      g1.a_row0 = pad0;
+      g0.ldc = pad0 / kBlkRows;
+      g1.ldc = pad1 / kBlkRows;
+      g1.c = g0.c + static_cast<int64_t>(pad0) * g0.n;
+    } else {
+      // A: per-expert tiled intermediates;  C: row-major, expert e's rows start at offsets[e]
+      g0.a_row0 = 0;
+      g1.a_row0 = 0;
+      g0.lda = pad0 / kBlkRows;
+      g1.lda = pad1 / kBlkRows;
+      g1.a = g0.a + static_cast<int64_t>(pad0) * g0.k;
+      g0.c += static_cast<int64_t>(o0) * g0.ldc;
+      g1.c += static_cast<int64_t>(o1) * g1.ldc;
+    }
   }
   constexpr int kTileN = SWIGLU ? BN / 2 : BN;  // output columns per tile
   int tiles_m[2], tiles_n[2];
@@ -139,8 +175,8 @@ __global__ __launch_bounds__(kThreads, 1) void dual_gemm_kernel(Params p) {
   const int padded = (total + kXcds - 1) / kXcds * kXcds;
 
   // ---- per-lane constants -----------------------------------------------------------------------
-  // loader: one instruction fills 16 LDS rows of 64 bytes; lane -> (row lane/4, slot lane%4).  Instruction i of
-  // this wave covers rows [wave*64 + 16i, +16).  Chunk c of row r lives in slot c ^ ((r >> 2) & 3).
+  // row-major loader: one instruction fills 16 LDS rows of 64 bytes; lane -> (row lane/4, slot lane%4).
+  // Instruction i of this wave covers rows [wave*64 + 16i, +16).  Chunk c of row r lives in slot c ^ ((r >> 2) & 3).
   const int ld_row0 = wave * kLoadRows + (lane >> 2);
   const int ld_chunk = (lane & 3) ^ ((lane >> 4) & 3);
   // fragment reads: row = base + l32, chunk kc = 2*kk + lhi
@@ -158,10 +194,11 @@ __global__ __launch_bounds__(kThreads, 1) void dual_gemm_kernel(Params p) {
   const int b_lane_off = l32 * kRowBytes;
 
   // ---- per-tile state ------------------------------------------------------------------------------
-  struct Loader {   // where this thread's four 16-byte loads per K step come from
+  struct Loader {   // where this wave's 2 * kLoads loads per K step come from
     const __bf16 *a_base, *b_base;
-    uint32_t a_bytes, b_bytes;
+    uint32_t a_bytes, b_bytes;        // readable bytes from the base (row-major) / from the current block (tiled)
     uint32_t voff_a[kLoads], voff_b[kLoads];
+    int64_t a_step, b_step;           // tiled: bytes between consecutive K steps
     int K, nk;      // nk: K steps of the tile, rounded up to a multiple of kStages (padding steps read zeros)
   };
   struct Store {    // where the finished tile goes
@@ -173,7 +210,12 @@ __global__ __launch_bounds__(kThreads, 1) void dual_gemm_kernel(Params p) {
   auto setup_store = [&](const TileCoord& tc, Store& S) {
     const Group G = tc.group ? g1 : g0;
     const int row0 = tc.tm * BM, col0 = tc.tn * kTileN;
-    S.c_base = G.c + static_cast<int64_t>(row0) * G.ldc + col0;
+    if constexpr (TILED_OUT) {
+      // block (row block, column block) of the tiled intermediate: [column block][row block], 1 KiB each
+      S.c_base = G.c + ((static_cast<int64_t>(col0 / kBlkCols) * G.ldc + row0 / kBlkRows) << 9);
+    } else {
+      S.c_base = G.c + static_cast<int64_t>(row0) * G.ldc + col0;
+    }
     S.rows = G.m - row0 < BM ? G.m - row0 : BM;
     S.cols_left = G.n - col0;
     S.ldc = G.ldc;
@@ -181,46 +223,74 @@ __global__ __launch_bounds__(kThreads, 1) void dual_gemm_kernel(Params p) {
   };
   auto setup_loader = [&](const TileCoord& tc, Loader& L) {
     const Group G = tc.group ? g1 : g0;
-#ifdef WX_EXP_SAMETILE
-    const int row0 = 0, col0 = 0;
-#elif defined(WX_EXP_SAMEXCD)
-    const int row0 = (blockIdx.x % 8) * BM, col0 = 0;
-#else
     const int row0 = tc.tm * BM, col0 = tc.tn * kTileN;
-#endif
-    const int rows_a = G.m - row0 < BM ? G.m - row0 : BM;
-    const int rows_b = G.n - col0 < kTileN ? G.n - col0 : kTileN;
     L.K = G.k;
     L.nk = padded_steps(G.k);
-    L.a_base = G.a + static_cast<int64_t>(row0) * G.lda;
-    constexpr int kHalfWaves = kWavesM * kWavesN / 2;  // SwiGLU: the first half of the waves load gate rows
+    constexpr int kHalfWaves = kWaves / 2;  // SwiGLU: the first half of the waves load gate rows, the rest up rows
     const bool up_half = SWIGLU && wave >= kHalfWaves;
-    L.b_base = (up_half ? G.b1 : G.b0) + static_cast<int64_t>(col0) * G.ldb;
-    L.a_bytes = static_cast<uint32_t>(rows_a) * G.lda * 2u;
-    L.b_bytes = static_cast<uint32_t>(rows_b) * G.ldb * 2u;
-    const int b_ld_row0 = SWIGLU ? (wave % kHalfWaves) * kLoadRows + (lane >> 2) : ld_row0;  // row inside its half
+    const __bf16* b_src = up_half ? G.b1 : G.b0;
+    const int b_wave = SWIGLU ? wave % kHalfWaves : wave;
+    if constexpr (TILED_IN) {
+      // this wave's kLoads row blocks of the A tile and of the B tile at K step 0; a K step later they sit one
+      // column block further, i.e. (row blocks of the matrix) KiB ahead
+      const int64_t a_blk = (G.a_row0 + row0) / kBlkRows + wave * kLoads;
+      const int64_t b_blk = col0 / kBlkRows + b_wave * kLoads;
+      L.a_base = G.a + (a_blk << 9);
+      L.b_base = b_src + (b_blk << 9);
+      L.a_step = static_cast<int64_t>(G.lda) << 10;
+      L.b_step = static_cast<int64_t>(G.ldb) << 10;
+      const int64_t a_left = (static_cast<int64_t>(G.k / kBlkCols) * G.lda - a_blk) << 10;
+      const int64_t b_left = (static_cast<int64_t>(G.k / kBlkCols) * G.ldb - b_blk) << 10;
+      L.a_bytes = static_cast<uint32_t>(a_left < 0 ? 0 : (a_left > 0x7fffff00ll ? 0x7fffff00ll : a_left));
+      L.b_bytes = static_cast<uint32_t>(b_left < 0 ? 0 : (b_left > 0x7fffff00ll ? 0x7fffff00ll : b_left));
 #pragma unroll
-    for (int i = 0; i < kLoads; ++i) {
-      L.voff_a[i] = static_cast<uint32_t>(ld_row0 + 16 * i) * G.lda * 2u + ld_chunk * 16u;
-      L.voff_b[i] = static_cast<uint32_t>(b_ld_row0 + 16 * i) * G.ldb * 2u + ld_chunk * 16u;
+      for (int i = 0; i < kLoads; ++i) L.voff_a[i] = L.voff_b[i] = static_cast<uint32_t>(i * kBlkBytes + lane * 16);
+    } else {
+      const int rows_a = G.m - row0 < BM ? G.m - row0 : BM;
+      const int rows_b = G.n - col0 < kTileN ? G.n - col0 : kTileN;
+      L.a_base = G.a + static_cast<int64_t>(row0) * G.lda;
+      L.b_base = b_src + static_cast<int64_t>(col0) * G.ldb;
+      L.a_bytes = static_cast<uint32_t>(rows_a) * G.lda * 2u;
+      L.b_bytes = static_cast<uint32_t>(rows_b) * G.ldb * 2u;
+      L.a_step = L.b_step = 0;
+      const int b_ld_row0 = b_wave * kLoadRows + (lane >> 2);
+#pragma unroll
+      for (int i = 0; i < kLoads; ++i) {
+        L.voff_a[i] = static_cast<uint32_t>(ld_row0 + 16 * i) * G.lda * 2u + ld_chunk * 16u;
+        L.voff_b[i] = static_cast<uint32_t>(b_ld_row0 + 16 * i) * G.ldb * 2u + ld_chunk * 16u;
+      }
     }
   };
 
   // One K step of global -> LDS for this wave: rows [wave*64, +64) of the A slot and of the B slot.
   auto issue = [&](const Loader& L, int ks, unsigned char* sa, unsigned char* sb) {
-    const int k0 = ks * BK;
-    // advancing the base keeps the absolute end of the readable range, so rows past the matrix read as zero;
-    // K chunks at or past the row end are pushed out of range per lane (this also zero-fills padding steps)
-    const uint32_t adv = 2u * static_cast<uint32_t>(k0);
+    __amdgpu_buffer_rsrc_t ra, rb;
+    uint32_t oob = 0;
+    if constexpr (TILED_IN) {
+      // steps past K (ring padding) and blocks past the end of the matrix read as zero through the bounds check
+      const bool real = ks * BK < L.K;
+      const int64_t da = L.a_step * ks, db = L.b_step * ks;
+      const int64_t la = static_cast<int64_t>(L.a_bytes) - da, lb = static_cast<int64_t>(L.b_bytes) - db;
+      // the byte counts are clamped for huge matrices; a clamped count is far above what one step reads
+      const uint32_t na = !real ? 0u : (L.a_bytes == 0x7fffff00u ? 0x7fffff00u : static_cast<uint32_t>(la < 0 ? 0 : la));
+      const uint32_t nb = !real ? 0u : (L.b_bytes == 0x7fffff00u ? 0x7fffff00u : static_cast<uint32_t>(lb < 0 ? 0 : lb));
 #ifdef WX_EXP_OOB
-    const __amdgpu_buffer_rsrc_t ra = make_rsrc(L.a_base + k0, 0u);
-    const __amdgpu_buffer_rsrc_t rb = make_rsrc(L.b_base + k0, 0u);
+      ra = make_rsrc(reinterpret_cast<const char*>(L.a_base) + da, 0u);
+      rb = make_rsrc(reinterpret_cast<const char*>(L.b_base) + db, 0u);
 #else
-    const __amdgpu_buffer_rsrc_t ra = make_rsrc(L.a_base + k0, L.a_bytes > adv ? L.a_bytes - adv : 0u);
-    const __amdgpu_buffer_rsrc_t rb = make_rsrc(L.b_base + k0, L.b_bytes > adv ? L.b_bytes - adv : 0u);
+      ra = make_rsrc(reinterpret_cast<const char*>(L.a_base) + da, na);
+      rb = make_rsrc(reinterpret_cast<const char*>(L.b_base) + db, nb);
 #endif
-    const bool k_tail = k0 + BK > L.K;
-    const uint32_t oob = (k_tail && k0 + ld_chunk * 8 >= L.K) ? 0x80000000u : 0u;
+    } else {
+      const int k0 = ks * BK;
+      // advancing the base keeps the absolute end of the readable range, so rows past the matrix read as zero;
+      // K chunks at or past the row end are pushed out of range per lane (this also zero-fills padding steps)
+      const uint32_t adv = 2u * static_cast<uint32_t>(k0);
+      ra = make_rsrc(L.a_base + k0, L.a_bytes > adv ? L.a_bytes - adv : 0u);
+      rb = make_rsrc(L.b_base + k0, L.b_bytes > adv ? L.b_bytes - adv : 0u);
+      const bool k_tail = k0 + BK > L.K;
+      oob = (k_tail && k0 + ld_chunk * 8 >= L.K) ? 0x80000000u : 0u;
+    }
 #pragma unroll
     for (int i = 0; i < kLoads; ++i) {
       __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, LDS_PTR(sa + (wave * kLoadRows + 16 * i) * kRowBytes), 16,
@@ -269,55 +339,114 @@ __global__ __launch_bounds__(kThreads, 1) void dual_gemm_kernel(Params p) {
     front_load_reads();
     // my LDS reads have returned; of my loads at most the two youngest K steps (2 * kLoads loads each) are still
     // in flight, i.e. the next slot is complete
-#ifndef WX_EXP_NOWAIT
     __builtin_amdgcn_s_waitcnt(waitcnt_imm(2 * 2 * kLoads, 0));
-#endif
-#ifndef WX_EXP_NOBARRIER
     __syncthreads();
-#endif
-#ifndef WX_EXP_NOLOAD
     issue(L, ld_ks, sa, sb);
-#endif
     __builtin_amdgcn_sched_barrier(0);  // keep the refill right behind the barrier: it has the longest way to go
     read_frags(sa_n, sb_n, 0, 0);
     mma(1);
     front_load_reads();
   };
 
+  // ---- epilogue ------------------------------------------------------------------------------------------
+  // Accumulator register r of lane l holds row 8*(r/4) + 4*(l/32) + r%4, column l%32 of its 32x32 block.  Values
+  // are rounded to bf16, paired with the neighbouring column through a lane swap (even lanes keep the even
+  // register's row, odd lanes the odd register's row), written to this wave's staging area as dwords, and read
+  // back as 16-byte lanes laid out the way the destination wants them.
+  unsigned char* stage = s_out + wave * kStageBytes;
+  auto swap_adjacent = [](float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));
+  };
+  // Stores register pair (r, r+1) of one 32x32 block -- rows srow and srow + 1, column scol of this lane -- into
+  // the staging area with row pitch `pitch` bytes.
+  auto stage_pair = [&](float v0, float v1, int srow, int scol, int pitch, int odd) {
+    // even lane: (own v0, neighbour's v0) -> row srow; odd lane: (neighbour's v1, own v1) -> row srow + 1
+    const float recv = swap_adjacent(odd ? v0 : v1);
+    const uint32_t packed = odd ? pack_bf16x2(recv, v1) : pack_bf16x2(v0, recv);
+    *reinterpret_cast<uint32_t*>(stage + (srow + odd) * pitch + (scol & ~1) * 2) = packed;
+  };
+
   auto epilogue = [&](const Store& S) {
-    // accumulator register r of lane l holds row 8*(r/4) + 4*(l/32) + r%4, column l%32 of its 32x32 block.
-    // The lane terms are laundered through an empty asm so the per-row address arithmetic is redone here each
-    // tile instead of being hoisted out of the persistent loop and held in registers across the K loop.
-    int lhi_e = lhi, l32_e = l32;
-    asm volatile("" : "+v"(lhi_e), "+v"(l32_e));
-    const int l32 = l32_e;
+    // The lane id is laundered through an empty asm so the address arithmetic is redone here each tile instead
+    // of being hoisted out of the persistent loop and held in registers across the K loop.
+    int lane_e = lane;
+    asm volatile("" : "+v"(lane_e));
+    const int el32 = lane_e & 31, elhi = lane_e >> 5, odd = lane_e & 1;
+    if constexpr (SWIGLU) {
+      // wave output: 128 rows x 64 intermediate columns, staged 64 rows at a time (64 x 64 bf16 = 8 KiB)
+      constexpr int kPitch = 64 * 2;
 #pragma unroll
-    for (int i = 0; i < FM; ++i) {
+      for (int half = 0; half < 2; ++half) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int row = wm * (FM * 32) + i * 32 + 8 * (r >> 2) + 4 * lhi_e + (r & 3);
-        if (row >= S.rows) continue;
-        __bf16* c_row = S.c_base + static_cast<int64_t>(row) * S.ldc;
-        if constexpr (SWIGLU) {
+        for (int ii = 0; ii < 2; ++ii) {
+          const int i = half * 2 + ii;
 #pragma unroll
           for (int j = 0; j < FN / 2; ++j) {
-            const int col = wn * (FN / 2 * 32) + j * 32 + l32;
-            if (col < S.cols_left) {
-              // eager bf16 evaluation of act_fn(gate) * up (act.py:80-82): gate, up, silu(gate) and the product
-              // are each rounded to bf16
-              const float g = round_bf16(acc[i][j][r]);
-              const float u = round_bf16(acc[i][j + FN / 2][r]);
-              const float sg = round_bf16(g / (1.0f + expf(-g)));
-              c_row[col] = static_cast<__bf16>(sg * u);
+#pragma unroll
+            for (int r = 0; r < 16; r += 2) {
+              float h[2];
+#pragma unroll
+              for (int q = 0; q < 2; ++q) {
+                // eager bf16 evaluation of act_fn(gate) * up (act.py:80-82): gate, up, silu(gate) and the
+                // product are each rounded to bf16
+                const float g = round_bf16(acc[i][j][r + q]);
+                const float u = round_bf16(acc[i][j + FN / 2][r + q]);
+                const float sg = round_bf16(g * __builtin_amdgcn_rcpf(1.0f + __expf(-g)));
+                h[q] = sg * u;
+              }
+              const int srow = ii * 32 + 8 * (r >> 2) + 4 * elhi + (r & 3);
+              stage_pair(h[0], h[1], srow, j * 32 + el32, kPitch, odd);
             }
           }
-        } else {
+        }
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, 0));
+        // 64 rows x 64 columns = 4 row blocks x 2 column blocks of the tiled intermediate, 1 KiB each; one store
+        // instruction per block: lane -> (row lane/4, slot lane%4) holding chunk slot ^ ((row >> 2) & 3)
+        const int r16 = lane_e >> 2, slot = lane_e & 3, chunk = slot ^ ((r16 >> 2) & 3);
 #pragma unroll
-          for (int j = 0; j < FN; ++j) {
-            const int col = wn * (FN * 32) + j * 32 + l32;
-            if (col < S.cols_left) c_row[col] = static_cast<__bf16>(acc[i][j][r]);
+        for (int rbl = 0; rbl < 4; ++rbl) {
+#pragma unroll
+          for (int kbl = 0; kbl < 2; ++kbl) {
+            const u32x4 v =
+                *reinterpret_cast<const u32x4*>(stage + (rbl * 16 + r16) * kPitch + (kbl * 32 + chunk * 8) * 2);
+            const int row = wm * (FM * 32) + half * 64 + rbl * 16;  // first row of the block inside the tile
+            const int col = wn * (FN / 2 * 32) + kbl * 32;           // first column of the block inside the tile
+            // rows past the expert's last row are padding of the tiled matrix: harmless to write, never read
+            if (col < S.cols_left) {
+              unsigned char* dst = reinterpret_cast<unsigned char*>(S.c_base) +
+                                   ((static_cast<int64_t>(col / kBlkCols) * S.ldc + row / kBlkRows) << 10);
+              *reinterpret_cast<u32x4*>(dst + lane_e * 16) = v;
+            }
           }
         }
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, 0));  // staging is rewritten by the next half
+      }
+    } else {
+      // wave output: 128 rows x 128 columns row-major, staged 32 rows at a time (32 x 128 bf16 = 8 KiB)
+      constexpr int kPitch = 128 * 2;
+#pragma unroll
+      for (int i = 0; i < FM; ++i) {
+#pragma unroll
+        for (int j = 0; j < FN; ++j) {
+#pragma unroll
+          for (int r = 0; r < 16; r += 2) {
+            const int srow = 8 * (r >> 2) + 4 * elhi + (r & 3);
+            stage_pair(acc[i][j][r], acc[i][j][r + 1], srow, j * 32 + el32, kPitch, odd);
+          }
+        }
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, 0));
+        // a row is 256 bytes = 16 lanes; one store instruction writes 4 rows
+        const int rr = lane_e >> 4, cc = (lane_e & 15) * 8;
+#pragma unroll
+        for (int q = 0; q < 8; ++q) {
+          const int srow = q * 4 + rr;
+          const u32x4 v = *reinterpret_cast<const u32x4*>(stage + srow * kPitch + cc * 2);
+          const int row = wm * (FM * 32) + i * 32 + srow;
+          const int col = wn * (FN * 32) + cc;
+          if (row < S.rows && col < S.cols_left)
+            *reinterpret_cast<u32x4*>(S.c_base + static_cast<int64_t>(row) * S.ldc + col) = v;
+        }
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, 0));
       }
     }
   };
@@ -370,6 +499,7 @@ __global__ __launch_bounds__(kThreads, 1) void dual_gemm_kernel(Params p) {
         } else {
           L.a_bytes = 0;
           L.b_bytes = 0;
+          L.K = 0;
         }
         ld_ks = 0;
       }
@@ -387,7 +517,7 @@ __global__ __launch_bounds__(kThreads, 1) void dual_gemm_kernel(Params p) {
 #endif
 }
 
-// ---- generic fallback: any transpose combination, any k; one thread per output element pair -----------
+// ---- other operand layouts: any transpose combination, any k; plain FMA tiles ------------------------------
 // Used for the layouts the MFMA kernel does not read in place (trans_a, or weights stored [k, n]).
 __global__ __launch_bounds__(256) void dual_gemm_reference_layout_kernel(Params p, int trans_a, int trans_b) {
   __shared__ float s_a[32][33];
@@ -416,7 +546,7 @@ __global__ __launch_bounds__(256) void dual_gemm_reference_layout_kernel(Params 
         for (int kk = 0; kk < 32; ++kk) {
           const float bv = s_b[tx][kk];
 #pragma unroll
-          for (int q = 0; q < 4; ++q) acc[q] += s_a[ty + 8 * q][kk] * bv;
+          for (int q = 0; q < 4; ++q) acc[q] = fmaf(s_a[ty + 8 * q][kk], bv, acc[q]);
         }
         __syncthreads();
       }
@@ -429,6 +559,20 @@ __global__ __launch_bounds__(256) void dual_gemm_reference_layout_kernel(Params 
   }
 }
 
+// Row-major [rows, cols] bf16 -> K-tiled (rows padded to 16 with zeros).  One thread per 16-byte chunk.
+__global__ __launch_bounds__(256) void pack_tiled_kernel(const u32x4* __restrict__ src, unsigned char* __restrict__ dst,
+                                                         int64_t rows, int64_t cols) {
+  const int64_t chunks_per_row = cols / 8;
+  const int64_t row_blocks = tiled_row_blocks(rows);
+  const int64_t n = row_blocks * kBlkRows * chunks_per_row;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n;
+       i += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+    const int64_t row = i / chunks_per_row, c = i - row * chunks_per_row;
+    const u32x4 v = row < rows ? src[i] : u32x4{0, 0, 0, 0};
+    *reinterpret_cast<u32x4*>(dst + tiled_chunk_offset(row, c * 8, row_blocks)) = v;
+  }
+}
+
 int check_dims(const char* who, int64_t m, int64_t n, int64_t k) {
   if (m < 0 || n < 0 || k < 0) return fail(WX_ERR_INVALID_ARGUMENT, "%s: negative dimension", who);
   if (m > INT32_MAX || n > INT32_MAX || k > INT32_MAX) return fail(WX_ERR_UNSUPPORTED, "%s: dimension exceeds int32", who);
@@ -437,12 +581,14 @@ int check_dims(const char* who, int64_t m, int64_t n, int64_t k) {
                 static_cast<long long>(k));
   // 256 rows of one operand must stay addressable through a 31-bit buffer offset
   if (k * 2 * 256 >= (1ll << 31) || n * 2 * 256 >= (1ll << 31)) return fail(WX_ERR_UNSUPPORTED, "%s: row too long", who);
+  // the tile list is indexed with 32-bit integers
+  if (((m + 255) / 256) * ((n + 127) / 128) >= (1ll << 30)) return fail(WX_ERR_UNSUPPORTED, "%s: too many tiles", who);
   return WX_OK;
 }
 
-template <bool SWIGLU>
+template <int MODE>
 int launch_mfma(const Params& p, hipStream_t s, const char* who) {
-  hipLaunchKernelGGL(dual_gemm_kernel<SWIGLU>, dim3(device_cu_count()), dim3(kThreads), 0, s, p);
+  hipLaunchKernelGGL(dual_gemm_kernel<MODE>, dim3(device_cu_count()), dim3(kThreads), 0, s, p);
   return check_launch(who);
 }
 
@@ -476,13 +622,37 @@ extern "C" int wx_dual_gemm(const void* in0, const void* in1, const void* w0, co
     g.lda = static_cast<int>(trans_a ? m : k);
     g.ldb = static_cast<int>(trans_b ? k : n);
     g.ldc = static_cast<int>(n);
+    g.a_row0 = 0;
   }
   p.offsets = nullptr;
   if ((m0 == 0 || n0 == 0) && (m1 == 0 || n1 == 0)) return WX_OK;
   hipStream_t s = as_stream(stream);
-  if (!trans_a && trans_b) return launch_mfma<false>(p, s, "dual_gemm_kernel");
+  if (!trans_a && trans_b) return launch_mfma<kGeneric>(p, s, "dual_gemm_kernel<generic>");
   hipLaunchKernelGGL(dual_gemm_reference_layout_kernel, dim3(device_cu_count() * 4), dim3(256), 0, s, p, trans_a, trans_b);
   return check_launch("dual_gemm_reference_layout_kernel");
+}
+
+extern "C" size_t wx_tiled_bytes(int64_t rows, int64_t cols) {
+  if (rows < 0 || cols < 0) return 0;
+  return static_cast<size_t>(tiled_bytes(rows, (cols + kBlkCols - 1) / kBlkCols * kBlkCols));
+}
+
+extern "C" int64_t wx_padded_sorted_rows(int64_t rows) { return rows < 0 ? 0 : padded_sorted_rows(rows); }
+
+extern "C" int wx_pack_tiled(const void* src, void* dst, int64_t rows, int64_t cols, wx_stream_t stream) {
+  if (rows < 0 || cols < 0) return fail(WX_ERR_INVALID_ARGUMENT, "wx_pack_tiled: negative size");
+  if (cols % kBlkCols != 0)
+    return fail(WX_ERR_UNSUPPORTED, "wx_pack_tiled: cols (%lld) must be a multiple of 32", static_cast<long long>(cols));
+  if (rows == 0 || cols == 0) return WX_OK;
+  if (!src || !dst) return fail(WX_ERR_INVALID_ARGUMENT, "wx_pack_tiled: null pointer");
+  if ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15)
+    return fail(WX_ERR_INVALID_ARGUMENT, "wx_pack_tiled: buffers must be 16-byte aligned");
+  const int64_t chunks = tiled_row_blocks(rows) * kBlkRows * (cols / 8);
+  const int64_t want = (chunks + 255) / 256;
+  const int64_t cap = static_cast<int64_t>(device_cu_count()) * 16;
+  hipLaunchKernelGGL(pack_tiled_kernel, dim3(static_cast<unsigned>(want < cap ? want : cap)), dim3(256), 0,
+                     as_stream(stream), static_cast<const u32x4*>(src), static_cast<unsigned char*>(dst), rows, cols);
+  return check_launch("pack_tiled_kernel");
 }
 
 namespace {
@@ -497,6 +667,8 @@ struct FfnArgs {
 int check_ffn(const char* who, const FfnArgs& a, bool need_gate_up, bool need_down) {
   if (int rc = check_dims(who, a.rows, a.inter[0], a.hidden)) return rc;
   if (int rc = check_dims(who, a.rows, a.hidden, a.inter[1])) return rc;
+  if (a.hidden % kBlkCols != 0 || a.inter[0] % kBlkCols != 0 || a.inter[1] % kBlkCols != 0)
+    return fail(WX_ERR_UNSUPPORTED, "%s: hidden and intermediate sizes must be multiples of 32", who);
   if (a.rows == 0) return WX_OK;
   if (!a.offsets || !a.hmid || (need_gate_up && !a.x) || (need_down && !a.out))
     return fail(WX_ERR_INVALID_ARGUMENT, "%s: null pointer", who);
@@ -506,11 +678,12 @@ int check_ffn(const char* who, const FfnArgs& a, bool need_gate_up, bool need_do
       return fail(WX_ERR_INVALID_ARGUMENT, "%s: null weight pointer for expert %d", who, e);
   }
   const int64_t max_inter = a.inter[0] > a.inter[1] ? a.inter[0] : a.inter[1];
-  if (a.rows * max_inter * 2 >= (1ll << 40)) return fail(WX_ERR_UNSUPPORTED, "%s: intermediate too large", who);
+  if (padded_sorted_rows(a.rows) * max_inter * 2 >= (1ll << 40))
+    return fail(WX_ERR_UNSUPPORTED, "%s: intermediate too large", who);
   return WX_OK;
 }
 
-// hmid_e = silu(x_e @ gate_e^T) * (x_e @ up_e^T); expert e's rows are packed with row length inter_e
+// hmid_e = silu(x_e @ gate_e^T) * (x_e @ up_e^T), K-tiled per expert
 int launch_gate_up(const FfnArgs& a, hipStream_t s) {
   Params p{};
   for (int e = 0; e < 2; ++e) {
@@ -520,13 +693,16 @@ int launch_gate_up(const FfnArgs& a, hipStream_t s) {
     g.b1 = static_cast<const __bf16*>(a.up[e]);
     g.c = static_cast<__bf16*>(a.hmid);
     g.m = 0; g.n = static_cast<int>(a.inter[e]); g.k = static_cast<int>(a.hidden);
-    g.lda = static_cast<int>(a.hidden); g.ldb = static_cast<int>(a.hidden); g.ldc = static_cast<int>(a.inter[e]);
+    g.lda = static_cast<int>(padded_sorted_rows(a.rows) / kBlkRows);  // row blocks of the tiled activations
+    g.ldb = static_cast<int>(tiled_row_blocks(a.inter[e]));           // row blocks of the tiled weights
+    g.ldc = 0;                                                        // set on the device from the row counts
+    g.a_row0 = 0;
   }
   p.offsets = a.offsets;
-  return launch_mfma<true>(p, s, "dual_gemm_kernel<swiglu>");
+  return launch_mfma<kGateUp>(p, s, "dual_gemm_kernel<gate_up>");
 }
 
-// out_e = hmid_e @ down_e^T
+// out_e = hmid_e @ down_e^T, row-major, expert e's rows start at offsets[e]
 int launch_down(const FfnArgs& a, hipStream_t s) {
   Params p{};
   for (int e = 0; e < 2; ++e) {
@@ -536,18 +712,22 @@ int launch_down(const FfnArgs& a, hipStream_t s) {
     g.b1 = nullptr;
     g.c = static_cast<__bf16*>(a.out);
     g.m = 0; g.n = static_cast<int>(a.hidden); g.k = static_cast<int>(a.inter[e]);
-    g.lda = static_cast<int>(a.inter[e]); g.ldb = static_cast<int>(a.inter[e]); g.ldc = static_cast<int>(a.hidden);
+    g.lda = 0;  // set on the device from the row counts
+    g.ldb = static_cast<int>(tiled_row_blocks(a.hidden));
+    g.ldc = static_cast<int>(a.hidden);
+    g.a_row0 = 0;
   }
   p.offsets = a.offsets;
-  return launch_mfma<false>(p, s, "dual_gemm_kernel<down>");
+  return launch_mfma<kDown>(p, s, "dual_gemm_kernel<down>");
 }
 
 }  // namespace
 
-extern "C" int wx_dual_swiglu_gate_up(const void* x, void* hmid, const int32_t* expert_offsets, const void* gate0,
-                                      const void* up0, const void* gate1, const void* up1, int64_t num_rows,
-                                      int64_t hidden, int64_t inter0, int64_t inter1, wx_stream_t stream) {
-  const FfnArgs a{x, {gate0, gate1}, {up0, up1}, {nullptr, nullptr}, nullptr, hmid, expert_offsets,
+extern "C" int wx_dual_swiglu_gate_up(const void* x_tiled, void* hmid, const int32_t* expert_offsets,
+                                      const void* gate0, const void* up0, const void* gate1, const void* up1,
+                                      int64_t num_rows, int64_t hidden, int64_t inter0, int64_t inter1,
+                                      wx_stream_t stream) {
+  const FfnArgs a{x_tiled, {gate0, gate1}, {up0, up1}, {nullptr, nullptr}, nullptr, hmid, expert_offsets,
                   num_rows, hidden, {inter0, inter1}};
   if (int rc = check_ffn("wx_dual_swiglu_gate_up", a, true, false)) return rc;
   if (num_rows == 0) return WX_OK;
@@ -564,11 +744,11 @@ extern "C" int wx_dual_down_proj(const void* hmid, void* out, const int32_t* exp
   return launch_down(a, as_stream(stream));
 }
 
-extern "C" int wx_dual_swiglu_ffn(const void* x, void* out, const int32_t* expert_offsets, const void* gate0,
+extern "C" int wx_dual_swiglu_ffn(const void* x_tiled, void* out, const int32_t* expert_offsets, const void* gate0,
                                   const void* up0, const void* down0, const void* gate1, const void* up1,
                                   const void* down1, void* hmid, int64_t num_rows, int64_t hidden, int64_t inter0,
                                   int64_t inter1, wx_stream_t stream) {
-  const FfnArgs a{x, {gate0, gate1}, {up0, up1}, {down0, down1}, out, hmid, expert_offsets,
+  const FfnArgs a{x_tiled, {gate0, gate1}, {up0, up1}, {down0, down1}, out, hmid, expert_offsets,
                   num_rows, hidden, {inter0, inter1}};
   if (int rc = check_ffn("wx_dual_swiglu_ffn", a, true, true)) return rc;
   if (num_rows == 0) return WX_OK;

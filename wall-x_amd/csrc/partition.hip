@@ -8,6 +8,7 @@
 //   pass 2  partition_scatter  per-block prefix over hist (bins, then earlier segments), then ranks
 // The row movers are pure HBM streams: one wavefront per token row, 16-byte lanes, several rows in flight.
 #include "common.h"
+#include "tiled_layout.h"
 
 namespace wx {
 namespace {
@@ -168,6 +169,41 @@ __global__ __launch_bounds__(kMoverWaves* kWave) void permute_rows_kernel(
         }
       }
     }
+  }
+}
+
+// Row scatter into the K-tiled, expert-padded layout the MFMA kernels read (bf16): row p of the sorted space lands
+// at row p (expert 0) or p + pad (expert 1, which starts at the next multiple of 256 rows), cut into 64-byte
+// column-block segments.  One wavefront per source row; lane q handles 16-byte chunks q, q + 64, ...
+__global__ __launch_bounds__(kMoverWaves* kWave) void permute_rows_tiled_kernel(
+    const u32x4* __restrict__ x, unsigned char* __restrict__ out, const int32_t* __restrict__ row_id_map,
+    const int32_t* __restrict__ expert_offsets, int64_t num_tokens, int64_t chunks_per_row, int64_t row_blocks) {
+  const int lane = lane_id();
+  const int64_t wave = static_cast<int64_t>(blockIdx.x) * kMoverWaves + threadIdx.x / kWave;
+  const int64_t n_waves = static_cast<int64_t>(gridDim.x) * kMoverWaves;
+  const int32_t first1 = expert_offsets[1];                                    // first sorted row of expert 1
+  const int32_t pad = static_cast<int32_t>(round_up_256(first1 - expert_offsets[0])) - (first1 - expert_offsets[0]);
+  for (int64_t t = wave; t < num_tokens; t += n_waves) {
+    int32_t dst_row = row_id_map[t];
+    if (dst_row < 0) continue;
+    if (dst_row >= first1) dst_row += pad;
+    const u32x4* src = x + t * chunks_per_row;
+    const int64_t rb = dst_row >> 4;
+    const int r = dst_row & 15, swz = (r >> 2) & 3;
+    unsigned char* dst = out + (rb << 10) + (r << 6);
+    int64_t q = lane;
+    for (; q + 3 * kWave < chunks_per_row; q += 4 * kWave) {
+      u32x4 v[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) v[u] = ld16(src + q + u * kWave);
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int64_t qq = q + u * kWave;
+        st16(reinterpret_cast<u32x4*>(dst + (((qq >> 2) * row_blocks) << 10) + (((qq & 3) ^ swz) << 4)), v[u]);
+      }
+    }
+    for (; q < chunks_per_row; q += kWave)
+      st16(reinterpret_cast<u32x4*>(dst + (((q >> 2) * row_blocks) << 10) + (((q & 3) ^ swz) << 4)), ld16(src + q));
   }
 }
 
@@ -361,6 +397,21 @@ extern "C" int wx_permute_rows(const void* x, void* out, const int32_t* row_id_m
                      as_stream(stream), static_cast<const u32x4*>(x), static_cast<u32x4*>(out), row_id_map,
                      num_tokens, num_topk, vec);
   return check_launch("permute_rows_kernel");
+}
+
+extern "C" int wx_permute_rows_tiled(const void* x, void* out_tiled, const int32_t* row_id_map,
+                                     const int32_t* expert_offsets, int64_t num_tokens, int64_t num_cols,
+                                     wx_stream_t stream) {
+  if (int rc = check_rows("wx_permute_rows_tiled", x, out_tiled, row_id_map, num_tokens, 1, num_cols, WX_BF16)) return rc;
+  if (num_cols % kBlkCols != 0)
+    return fail(WX_ERR_UNSUPPORTED, "wx_permute_rows_tiled: num_cols (%lld) must be a multiple of 32",
+                static_cast<long long>(num_cols));
+  if (num_tokens == 0) return WX_OK;
+  if (expert_offsets == nullptr) return fail(WX_ERR_INVALID_ARGUMENT, "wx_permute_rows_tiled: null expert_offsets");
+  hipLaunchKernelGGL(permute_rows_tiled_kernel, dim3(mover_grid(num_tokens)), dim3(kMoverWaves * kWave), 0,
+                     as_stream(stream), static_cast<const u32x4*>(x), static_cast<unsigned char*>(out_tiled),
+                     row_id_map, expert_offsets, num_tokens, num_cols / 8, padded_sorted_rows(num_tokens) / kBlkRows);
+  return check_launch("permute_rows_tiled_kernel");
 }
 
 extern "C" int wx_unpermute_rows(const void* y, void* out, const int32_t* row_id_map, const float* probs,

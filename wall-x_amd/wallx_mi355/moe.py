@@ -2,8 +2,9 @@
 
 The reference's SparseMoeBlock permutes the tokens, loops over the experts in Python (six cuBLAS GEMMs,
 four elementwise kernels and two slice copies per layer, bounds read from CPU tensors) and unpermutes.
-Here one layer is: partition (2 small launches, reusable across layers) -> row scatter -> gate/up + SwiGLU
-for both experts (1 launch) -> down for both experts (1 launch) -> row gather.  The per-expert row ranges
+Here one layer is: partition (2 small launches, reusable across layers) -> row scatter into the K-tiled
+activation layout -> gate/up + SwiGLU for both experts (1 launch) -> down for both experts (1 launch) -> row
+gather.  Expert weights are packed into the same K-tiled layout once and cached.  The per-expert row ranges
 stay on the device (expert_offsets from the partition), so nothing synchronises with the host.
 
 Parameter names match the reference (``experts.{e}.{gate,up,down}_proj.weight``), so its checkpoints load.
@@ -49,9 +50,9 @@ class _DualExpertFFN(torch.autograd.Function):
     """Inference-only for now: the fused path has no backward (training falls outside this build's scope)."""
 
     @staticmethod
-    def forward(ctx, x_sorted, expert_offsets, hmid, *weights):
+    def forward(ctx, x_tiled, num_rows, expert_offsets, hmid, *weights):
         w = ((weights[0], weights[1], weights[2]), (weights[3], weights[4], weights[5]))
-        return native.dual_swiglu_ffn(x_sorted, expert_offsets, w, hmid=hmid)
+        return native.dual_swiglu_ffn(x_tiled, num_rows, expert_offsets, w, hmid=hmid)
 
     @staticmethod
     def backward(ctx, grad):
@@ -69,6 +70,7 @@ class SparseMoeBlock(nn.Module):
         self.experts = nn.ModuleList([ExpertMLP(config.experts[i]) for i in range(num_experts)])
         self._partition_ws: Optional[List[torch.Tensor]] = None
         self._hmid: Optional[torch.Tensor] = None
+        self._x_tiled: Optional[torch.Tensor] = None
 
     def route(self, experts_indices: torch.Tensor) -> Routing:
         """Stable partition of the flattened token types; reuse the result for all layers of a forward."""
@@ -93,12 +95,12 @@ class SparseMoeBlock(nn.Module):
             routing = self.route(experts_indices)
         if routing.num_tokens != x.size(0):
             raise RuntimeError(f"routing was built for {routing.num_tokens} tokens, got {x.size(0)}")
-        x_sorted = native.permute_rows(x.contiguous(), routing.row_id_map, 1, x.size(0))
-        need = x.size(0) * max(e.intermediate_size for e in self.experts)
+        self._x_tiled = native.permute_rows_tiled(x, routing.row_id_map, routing.expert_offsets, self._x_tiled)
+        need = native.padded_sorted_rows(x.size(0)) * max(e.intermediate_size for e in self.experts)
         if self._hmid is None or self._hmid.numel() < need or self._hmid.device != x.device:
             self._hmid = torch.empty(need, dtype=torch.bfloat16, device=x.device)
         flat = [w for e in self.experts for w in e.weights()]
-        y_sorted = _DualExpertFFN.apply(x_sorted, routing.expert_offsets, self._hmid, *flat)
+        y_sorted = _DualExpertFFN.apply(self._x_tiled, x.size(0), routing.expert_offsets, self._hmid, *flat)
         y = native.unpermute(y_sorted, routing.row_id_map, torch.tensor([]), x.size(0), 1)
         return y.view(batch, seq, hidden)
 
@@ -112,7 +114,7 @@ def moe_layer_forward(x: torch.Tensor, token_types: torch.Tensor, weights, routi
     if routing is None:
         row_id_map, offsets, _, _ = native.partition(token_types.reshape(-1), 2, 0, workspace)
         routing = Routing(row_id_map, offsets, x.size(0))
-    x_sorted = native.permute_rows(x, routing.row_id_map, 1, x.size(0))
-    y_sorted = native.dual_swiglu_ffn(x_sorted, routing.expert_offsets, weights, hmid=hmid)
+    x_tiled = native.permute_rows_tiled(x, routing.row_id_map, routing.expert_offsets)
+    y_sorted = native.dual_swiglu_ffn(x_tiled, x.size(0), routing.expert_offsets, weights, hmid=hmid)
     y = native.unpermute(y_sorted, routing.row_id_map, torch.tensor([]), x.size(0), 1)
     return y, routing

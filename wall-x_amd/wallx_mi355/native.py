@@ -350,34 +350,83 @@ def get_window_index(grid_thw: torch.Tensor, spatial_merge_size: int, vit_merger
 
 
 # ----------------------------------------------------------------------------- fused dual-expert FFN
-def dual_swiglu_ffn(x: torch.Tensor, expert_offsets: torch.Tensor, weights, hmid: Optional[torch.Tensor] = None,
-                    out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """Both experts' SwiGLU FFN over expert-sorted rows in two launches (act.py:79-82, 142-154).
+import weakref
 
-    x [T, H] bf16 sorted by expert; expert_offsets int32 [3] ON THE DEVICE (from partition());
-    weights = ((gate0, up0, down0), (gate1, up1, down1)) in nn.Linear layout.
+_packed_cache = {}  # id(weight) -> (weakref to weight, version, packed tensor)
+
+
+def padded_sorted_rows(num_tokens: int) -> int:
+    """Rows of the expert-sorted space once each expert's range starts at a multiple of 256."""
+    return int(_lib.load().wx_padded_sorted_rows(int(num_tokens)))
+
+
+def pack_weight(w: torch.Tensor, cache: bool = True) -> torch.Tensor:
+    """nn.Linear weight [out, in] (bf16, CUDA) -> the K-tiled layout the MFMA kernels read (flat bf16 tensor).
+
+    Packed copies are cached per weight tensor and rebuilt when the tensor is modified in place.
     """
+    _need_cuda("weight", w)
+    if w.dtype != torch.bfloat16 or w.dim() != 2:
+        raise RuntimeError("expert weights must be 2-D BFloat16 tensors")
+    key = id(w)
+    if cache:
+        hit = _packed_cache.get(key)
+        if hit is not None and hit[0]() is w and hit[1] == w._version and hit[2].device == w.device:
+            return hit[2]
+    src = w.detach().contiguous()
+    rows, cols = src.shape
+    nbytes = _lib.load().wx_tiled_bytes(rows, cols)
+    packed = torch.empty(nbytes // 2, dtype=torch.bfloat16, device=w.device)
+    with _DeviceGuard(src):
+        _lib.call("wx_pack_tiled", _ptr(src), packed.data_ptr(), rows, cols, _stream(src))
+    if cache:
+        _packed_cache[key] = (weakref.ref(w, lambda _r, k=key: _packed_cache.pop(k, None)), w._version, packed)
+    return packed
+
+
+def permute_rows_tiled(x: torch.Tensor, row_id_map: torch.Tensor, expert_offsets: torch.Tensor,
+                       out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x [T, H] bf16 -> K-tiled, expert-padded activation matrix for dual_swiglu_ffn (flat bf16 tensor)."""
     _need_cuda("x", x)
     if x.dtype != torch.bfloat16:
         raise RuntimeError("All tensors must be BFloat16 for this kernel")
-    (g0, u0, d0), (g1, u1, d1) = weights
-    for w in (g0, u0, d0, g1, u1, d1):
-        if w.dtype != torch.bfloat16 or not w.is_cuda or not w.is_contiguous():
-            raise RuntimeError("expert weights must be contiguous BFloat16 CUDA tensors")
+    x = x.contiguous()
     T, H = x.shape
+    need = _lib.load().wx_tiled_bytes(padded_sorted_rows(T), H) // 2
+    if out is None or out.numel() < need or out.dtype != torch.bfloat16 or out.device != x.device:
+        out = torch.empty(need, dtype=torch.bfloat16, device=x.device)
+    with _DeviceGuard(x):
+        _lib.call("wx_permute_rows_tiled", _ptr(x), out.data_ptr(), _ptr(row_id_map), expert_offsets.data_ptr(), T, H,
+                  _stream(x))
+    return out
+
+
+def dual_swiglu_ffn(x_tiled: torch.Tensor, num_rows: int, expert_offsets: torch.Tensor, weights,
+                    hmid: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Both experts' SwiGLU FFN over expert-sorted rows in two launches (act.py:79-82, 142-154).
+
+    x_tiled: result of permute_rows_tiled for num_rows tokens; expert_offsets int32 [3] ON THE DEVICE (from
+    partition()); weights = ((gate0, up0, down0), (gate1, up1, down1)) in nn.Linear layout (packed and cached
+    here).  Returns out [num_rows, hidden] bf16 in sorted order.
+    """
+    _need_cuda("x_tiled", x_tiled)
+    (g0, u0, d0), (g1, u1, d1) = weights
+    H = g0.size(1)
     I0, I1 = g0.size(0), g1.size(0)
     if tuple(g0.shape) != (I0, H) or tuple(u0.shape) != (I0, H) or tuple(d0.shape) != (H, I0) or \
             tuple(g1.shape) != (I1, H) or tuple(u1.shape) != (I1, H) or tuple(d1.shape) != (H, I1):
         raise RuntimeError("expert weight shapes are inconsistent with hidden size")
     if expert_offsets.dtype != torch.int32 or expert_offsets.numel() < 3 or not expert_offsets.is_cuda:
         raise RuntimeError("expert_offsets must be an int32 CUDA tensor with 3 entries")
-    x = x.contiguous()
-    need = T * max(I0, I1)
+    packed = [pack_weight(w) for w in (g0, u0, d0, g1, u1, d1)]
+    dev = x_tiled.device
+    need = padded_sorted_rows(num_rows) * max(I0, I1)
     if hmid is None or hmid.numel() < need or hmid.dtype != torch.bfloat16:
-        hmid = torch.empty(need, dtype=torch.bfloat16, device=x.device)
+        hmid = torch.empty(need, dtype=torch.bfloat16, device=dev)
     if out is None:
-        out = torch.empty_like(x)
-    with _DeviceGuard(x):
-        _lib.call("wx_dual_swiglu_ffn", _ptr(x), _ptr(out), expert_offsets.data_ptr(), _ptr(g0), _ptr(u0), _ptr(d0),
-                  _ptr(g1), _ptr(u1), _ptr(d1), hmid.data_ptr(), T, H, I0, I1, _stream(x))
+        out = torch.empty((num_rows, H), dtype=torch.bfloat16, device=dev)
+    with _DeviceGuard(x_tiled):
+        _lib.call("wx_dual_swiglu_ffn", x_tiled.data_ptr(), _ptr(out), expert_offsets.data_ptr(), _ptr(packed[0]),
+                  _ptr(packed[1]), _ptr(packed[2]), _ptr(packed[3]), _ptr(packed[4]), _ptr(packed[5]),
+                  hmid.data_ptr(), int(num_rows), H, I0, I1, _stream(x_tiled))
     return out
