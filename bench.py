@@ -213,13 +213,26 @@ def main():
             "frac": round(gate_up_tflops / PEAK_BF16_TFLOPS, 4),
             "flops_per_launch": gate_up_flops,
             "avg_launch_ms": round(t_gate_up_avg, 4),
-            "traffic": None,
+            "traffic": measured_traffic("gate_up"),
         },
         "extra": extra,
     }
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(x_cpu, types_cpu, w_cpu, args.cpu_seqs, H, I0, I1)
     print(json.dumps(result), flush=True)
+
+
+def measured_traffic(kernel):
+    """HBM-side bytes per launch of `kernel` from the committed rocprofv3 --pmc summary (FETCH_SIZE + WRITE_SIZE,
+    each scaled by what the same counter reads for a plain copy of known size); None when the summary is absent.
+    Counters need their own profiler runs, so this figure is read, not measured, by a bench.py run."""
+    path = os.path.join(ROOT, "profiles", "config3_hbm_traffic.json")
+    try:
+        with open(path) as f:
+            k = json.load(f)["kernels"][kernel]
+        return round(k["read_bytes"] + k["write_bytes"])
+    except (OSError, KeyError, ValueError):
+        return None
 
 
 def side_measurements(dev, iters):

@@ -274,13 +274,8 @@ __global__ __launch_bounds__(kThreads, 1) void dual_gemm_kernel(Params p) {
       // the byte counts are clamped for huge matrices; a clamped count is far above what one step reads
       const uint32_t na = !real ? 0u : (L.a_bytes == 0x7fffff00u ? 0x7fffff00u : static_cast<uint32_t>(la < 0 ? 0 : la));
       const uint32_t nb = !real ? 0u : (L.b_bytes == 0x7fffff00u ? 0x7fffff00u : static_cast<uint32_t>(lb < 0 ? 0 : lb));
-#ifdef WX_EXP_OOB
-      ra = make_rsrc(reinterpret_cast<const char*>(L.a_base) + da, 0u);
-      rb = make_rsrc(reinterpret_cast<const char*>(L.b_base) + db, 0u);
-#else
       ra = make_rsrc(reinterpret_cast<const char*>(L.a_base) + da, na);
       rb = make_rsrc(reinterpret_cast<const char*>(L.b_base) + db, nb);
-#endif
     } else {
       const int k0 = ks * BK;
       // advancing the base keeps the absolute end of the readable range, so rows past the matrix read as zero;
@@ -508,11 +503,7 @@ __global__ __launch_bounds__(kThreads, 1) void dual_gemm_kernel(Params p) {
       k_step(L, ld_ks + 2, s_a2, s_b2, s_a3, s_b3);
       k_step(L, ld_ks + 3, s_a3, s_b3, s_a0, s_b0);
     }
-#ifndef WX_EXP_NOEPI
     epilogue(done);
-#else
-    if (acc[0][0][0] == 123.456f) epilogue(done);
-#endif
   }
 #endif
 }
