@@ -44,8 +44,9 @@ def parse():
     return ap.parse_args()
 
 
-def event_ms(fn, iters, warm=3):
-    """Median duration of fn() in ms from HIP events on the current stream."""
+def event_ms(fn, iters, warm=3, batch=1):
+    """(median, mean) duration of one fn() in ms from HIP events on the current stream.  batch > 1 times that many
+    back-to-back calls per event pair, which keeps launch gaps out of the figure for kernels of a few tens of us."""
     import torch
 
     for _ in range(warm):
@@ -54,10 +55,11 @@ def event_ms(fn, iters, warm=3):
     for _ in range(iters):
         a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         a.record()
-        fn()
+        for _ in range(batch):
+            fn()
         b.record()
         b.synchronize()
-        times.append(a.elapsed_time(b))
+        times.append(a.elapsed_time(b) / batch)
     return statistics.median(times), sum(times) / len(times)
 
 
@@ -104,15 +106,15 @@ def main():
     ws = None
     stream = torch.cuda.current_stream().cuda_stream
 
-    row_id_map, offsets, _, ws = native.partition(types, 2, 0, ws)
+    row_id_map, offsets, inverse, ws = native.partition(types, 2, 0, ws, want_sorted=True)
 
     def partition():
-        nonlocal row_id_map, offsets, ws
-        row_id_map, offsets, _, ws = native.partition(types, 2, 0, ws)
+        nonlocal row_id_map, offsets, inverse, ws
+        row_id_map, offsets, inverse, ws = native.partition(types, 2, 0, ws, want_sorted=True)
 
     def permute():  # the layer's permute: rows go straight into the K-tiled activation matrix
         _lib.call("wx_permute_rows_tiled", x.data_ptr(), x_tiled.data_ptr(), row_id_map.data_ptr(),
-                  offsets.data_ptr(), T, H, stream)
+                  inverse.data_ptr(), offsets.data_ptr(), T, H, stream)
 
     def permute_plain():  # the stand-alone op of the reference API (row-major output)
         _lib.call("wx_permute_rows", x.data_ptr(), x_sorted.data_ptr(), row_id_map.data_ptr(), T, 1, H,
@@ -163,9 +165,9 @@ def main():
     iters = max(10, args.steps)
     t_gate_up, t_gate_up_avg = event_ms(gate_up, iters)
     t_down, _ = event_ms(down, iters)
-    t_perm, _ = event_ms(permute, iters)
-    t_perm_plain, _ = event_ms(permute_plain, iters)
-    t_unperm, _ = event_ms(unpermute, iters)
+    t_perm, _ = event_ms(permute, iters, batch=10)
+    t_perm_plain, _ = event_ms(permute_plain, iters, batch=10)
+    t_unperm, _ = event_ms(unpermute, iters, batch=10)
     t_part, _ = event_ms(partition, iters)
     gate_up_tflops = gate_up_flops / (t_gate_up_avg * 1e-3) / 1e12
 
@@ -266,7 +268,7 @@ def side_measurements(dev, iters):
     qo = torch.empty(B, wl.N_Q_HEADS, S, D, dtype=torch.bfloat16, device=dev)
     ko = torch.empty(B, wl.N_KV_HEADS, S, D, dtype=torch.bfloat16, device=dev)
     sec2 = [2 * v for v in wl.MROPE_SECTION]
-    t, _ = event_ms(lambda: native.rope(q, k, cos, sin, qo, ko, sec2), iters)
+    t, _ = event_ms(lambda: native.rope(q, k, cos, sin, qo, ko, sec2), iters, batch=10)
     tokens = B * S
     rope_bytes = 2.0 * 2 * tokens * D * (wl.N_Q_HEADS + wl.N_KV_HEADS) + 2.0 * 2 * tokens * D
     out["mrope_us"] = round(t * 1e3, 2)

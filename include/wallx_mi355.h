@@ -105,10 +105,12 @@ int wx_pack_tiled(const void* src_row_major, void* dst_tiled, int64_t rows, int6
  * row_id_map[t], shifted for expert 1 so that its rows start at a multiple of 256.  Replaces
  * moe_permute_topK_kernel's forward branch (csrc/permute.cu:156-262) for topK == 1 when the consumer is
  * wx_dual_swiglu_ffn.  out_tiled: wx_tiled_bytes(wx_padded_sorted_rows(T), num_cols) bytes.
- * expert_offsets: device int32[3] from wx_partition_build. */
+ * expert_offsets: device int32[3] from wx_partition_build.  Either map may be NULL, not both: with
+ * sorted_row_id (the partition's inverse map) rows are gathered block by block and every store is a whole
+ * contiguous KiB (the faster form; padding rows are zero-filled); with row_id_map alone rows are scattered. */
 int wx_permute_rows_tiled(const void* x, void* out_tiled, const int32_t* row_id_map,
-                          const int32_t* expert_offsets, int64_t num_tokens, int64_t num_cols,
-                          wx_stream_t stream);
+                          const int32_t* sorted_row_id, const int32_t* expert_offsets,
+                          int64_t num_tokens, int64_t num_cols, wx_stream_t stream);
 
 /* Both experts' SwiGLU FFN over expert-sorted rows, two launches (gate/up + SwiGLU, then down), each
  * covering both experts:  out[r, :] = down_e( silu(x[r] @ gate_e^T) * (x[r] @ up_e^T) ) for sorted rows

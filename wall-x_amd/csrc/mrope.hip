@@ -3,8 +3,8 @@
 // HBM-bound elementwise kernel.  A thread owns one rotation group of a token: the 8 channels
 // [8j, 8j+8) of the low half together with their partners in the high half, so both operands of every
 // rotation are in registers and each access is a full 16-byte lane (32 bytes for fp32).  The thread
-// loads the selected cos/sin values for its channels once and then walks the heads of q and k that
-// its head group covers, which amortises the table over the heads.  q/k/outputs are addressed
+// loads the selected cos/sin values for its channels once and applies them to three heads of q / k; all
+// loads of the three heads are in flight before the first result is needed.  q/k/outputs are addressed
 // through (batch, head, seq) strides so the projection's [B, S, H, D] memory is read in place.
 #include "common.h"
 
@@ -26,6 +26,17 @@ template <int DT>
 __device__ __forceinline__ void load8(const void* base, int64_t elem_off, float* f) {
   if constexpr (DT == WX_F32) {
     const u32x4* p = reinterpret_cast<const u32x4*>(static_cast<const float*>(base) + elem_off);
+    unpack16<DT>(__builtin_nontemporal_load(p), f);
+    unpack16<DT>(__builtin_nontemporal_load(p + 1), f + 4);
+  } else {
+    unpack16<DT>(__builtin_nontemporal_load(reinterpret_cast<const u32x4*>(static_cast<const uint16_t*>(base) + elem_off)), f);
+  }
+}
+// same as load8 with a regular (cached) load: the cos/sin chunks are re-read by every head group
+template <int DT>
+__device__ __forceinline__ void load8_cached(const void* base, int64_t elem_off, float* f) {
+  if constexpr (DT == WX_F32) {
+    const u32x4* p = reinterpret_cast<const u32x4*>(static_cast<const float*>(base) + elem_off);
     unpack16<DT>(p[0], f);
     unpack16<DT>(p[1], f + 4);
   } else {
@@ -36,10 +47,10 @@ template <int DT>
 __device__ __forceinline__ void store8(void* base, int64_t elem_off, const float* f) {
   if constexpr (DT == WX_F32) {
     u32x4* p = reinterpret_cast<u32x4*>(static_cast<float*>(base) + elem_off);
-    p[0] = pack16<DT>(f);
-    p[1] = pack16<DT>(f + 4);
+    __builtin_nontemporal_store(pack16<DT>(f), p);
+    __builtin_nontemporal_store(pack16<DT>(f + 4), p + 1);
   } else {
-    *reinterpret_cast<u32x4*>(static_cast<uint16_t*>(base) + elem_off) = pack16<DT>(f);
+    __builtin_nontemporal_store(pack16<DT>(f), reinterpret_cast<u32x4*>(static_cast<uint16_t*>(base) + elem_off));
   }
 }
 template <int DT>
@@ -53,64 +64,80 @@ template <int DT>
 __device__ __forceinline__ void load_selected(const void* table, const AxisTable& ax, int64_t plane_stride,
                                               int64_t token_off, int d0, float* f) {
   if (ax.uniform[d0 >> 3]) {
-    load8<DT>(table, ax.axis[d0] * plane_stride + token_off + d0, f);
+    load8_cached<DT>(table, ax.axis[d0] * plane_stride + token_off + d0, f);
   } else {
 #pragma unroll
     for (int e = 0; e < 8; ++e) f[e] = load1<DT>(table, ax.axis[d0 + e] * plane_stride + token_off + d0 + e);
   }
 }
 
+// Heads per thread: the loads of all of them are issued before the first result is needed.
+constexpr int kHeadsPerThread = 3;
+
 template <int DT, bool BWD>
 __global__ __launch_bounds__(256) void mrope_kernel(
     const void* __restrict__ q, const void* __restrict__ k, const void* __restrict__ cos_t,
     const void* __restrict__ sin_t, void* __restrict__ q_out, void* __restrict__ k_out, int64_t n_tokens,
     int64_t seq, int n_q_heads, int n_kv_heads, int head_dim, Strides sq, Strides sk, Strides sqo, Strides sko,
-    AxisTable ax, int head_groups) {
+    AxisTable ax) {
   const int groups = head_dim / 16;  // rotation groups per head
+  // blockIdx.y = head group (uniform per workgroup), blockIdx.x walks (token, rotation group)
   const int64_t gid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   const int j = static_cast<int>(gid % groups);
-  const int hg = static_cast<int>((gid / groups) % head_groups);
-  const int64_t token = gid / (static_cast<int64_t>(groups) * head_groups);
+  const int64_t token = gid / groups;
   if (token >= n_tokens) return;
+  const int h0 = blockIdx.y * kHeadsPerThread;
   const int64_t b = token / seq, s = token - b * seq;
   const int half = head_dim / 2;
   const int d_lo = 8 * j, d_hi = half + 8 * j;
   const int64_t plane = n_tokens * head_dim, tok_off = token * head_dim;
+  const int n_heads = n_q_heads + n_kv_heads;
 
+  float x_lo[kHeadsPerThread][8], x_hi[kHeadsPerThread][8];
+#pragma unroll
+  for (int u = 0; u < kHeadsPerThread; ++u) {
+    const int h = h0 + u;
+    if (h < n_heads) {
+      const bool is_q = h < n_q_heads;
+      const int hh = is_q ? h : h - n_q_heads;
+      const Strides& si = is_q ? sq : sk;
+      const void* in = is_q ? q : k;
+      const int64_t in_off = b * si.b + hh * si.h + s * si.s;
+      load8<DT>(in, in_off + d_lo, x_lo[u]);
+      load8<DT>(in, in_off + d_hi, x_hi[u]);
+    }
+  }
   float c_lo[8], c_hi[8], s_lo[8], s_hi[8];
   load_selected<DT>(cos_t, ax, plane, tok_off, d_lo, c_lo);
   load_selected<DT>(cos_t, ax, plane, tok_off, d_hi, c_hi);
   load_selected<DT>(sin_t, ax, plane, tok_off, d_lo, s_lo);
   load_selected<DT>(sin_t, ax, plane, tok_off, d_hi, s_hi);
 
-  const int n_heads = n_q_heads + n_kv_heads;
-  for (int h = hg; h < n_heads; h += head_groups) {
+#pragma unroll
+  for (int u = 0; u < kHeadsPerThread; ++u) {
+    const int h = h0 + u;
+    if (h >= n_heads) break;
     const bool is_q = h < n_q_heads;
     const int hh = is_q ? h : h - n_q_heads;
-    const Strides& si = is_q ? sq : sk;
     const Strides& so = is_q ? sqo : sko;
-    const void* in = is_q ? q : k;
     void* out = is_q ? q_out : k_out;
-    const int64_t in_off = b * si.b + hh * si.h + s * si.s;
     const int64_t out_off = b * so.b + hh * so.h + s * so.s;
-    float x_lo[8], x_hi[8], o_lo[8], o_hi[8];
-    load8<DT>(in, in_off + d_lo, x_lo);
-    load8<DT>(in, in_off + d_hi, x_hi);
+    float o_lo[8], o_hi[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       if constexpr (!BWD) {
         // eager evaluation order of (x * cos) + (rotate_half(x) * sin): every product and the sum are
         // rounded to the storage type; rotate_half(x) = (-x_hi, x_lo)
-        const float p1 = Elem<DT>::round(__fmul_rn(x_lo[e], c_lo[e]));
-        const float p2 = Elem<DT>::round(__fmul_rn(-x_hi[e], s_lo[e]));
+        const float p1 = Elem<DT>::round(__fmul_rn(x_lo[u][e], c_lo[e]));
+        const float p2 = Elem<DT>::round(__fmul_rn(-x_hi[u][e], s_lo[e]));
         o_lo[e] = __fadd_rn(p1, p2);
-        const float p3 = Elem<DT>::round(__fmul_rn(x_hi[e], c_hi[e]));
-        const float p4 = Elem<DT>::round(__fmul_rn(x_lo[e], s_hi[e]));
+        const float p3 = Elem<DT>::round(__fmul_rn(x_hi[u][e], c_hi[e]));
+        const float p4 = Elem<DT>::round(__fmul_rn(x_lo[u][e], s_hi[e]));
         o_hi[e] = __fadd_rn(p3, p4);
       } else {
         // adjoint: g*cos + rotate_half^T(g*sin), rotate_half^T(y) = (y_hi, -y_lo)
-        o_lo[e] = x_lo[e] * c_lo[e] + x_hi[e] * s_hi[e];
-        o_hi[e] = x_hi[e] * c_hi[e] - x_lo[e] * s_lo[e];
+        o_lo[e] = x_lo[u][e] * c_lo[e] + x_hi[u][e] * s_hi[e];
+        o_hi[e] = x_hi[u][e] * c_hi[e] - x_lo[u][e] * s_lo[e];
       }
     }
     store8<DT>(out, out_off + d_lo, o_lo);
@@ -165,17 +192,16 @@ int launch(const void* q, const void* k, const void* cos_t, const void* sin_t, v
   AxisTable ax{};
   if (int rc = build_axis_table(sec, head_dim, layout, ax)) return rc;
   const Strides a{sq[0], sq[1], sq[2]}, b{sk[0], sk[1], sk[2]}, c{sqo[0], sqo[1], sqo[2]}, d{sko[0], sko[1], sko[2]};
-  // spread heads over a few threads per rotation group when there are few tokens to fill the chip
+  // grid.x walks (token, rotation group); grid.y walks groups of kHeadsPerThread heads
   const int groups = head_dim / 16;
-  int head_groups = 1;
-  const int64_t target_threads = static_cast<int64_t>(device_cu_count()) * 2048;
-  while (head_groups * 2 <= n_q + n_kv && n_tokens * groups * head_groups < target_threads) head_groups *= 2;
-  const int64_t threads = n_tokens * groups * head_groups;
-  const dim3 grid(static_cast<unsigned>((threads + 255) / 256)), block(256);
+  const int head_groups = (n_q + n_kv + kHeadsPerThread - 1) / kHeadsPerThread;
+  const int64_t threads = n_tokens * groups;
+  if ((threads + 255) / 256 > 0x7fffffffll) return fail(WX_ERR_UNSUPPORTED, "%s: too many tokens", who);
+  const dim3 grid(static_cast<unsigned>((threads + 255) / 256), static_cast<unsigned>(head_groups)), block(256);
   hipStream_t s = as_stream(stream);
 #define WX_LAUNCH(DT)                                                                                             \
   hipLaunchKernelGGL((mrope_kernel<DT, BWD>), grid, block, 0, s, q, k, cos_t, sin_t, q_out, k_out, n_tokens, seq, \
-                     n_q, n_kv, head_dim, a, b, c, d, ax, head_groups)
+                     n_q, n_kv, head_dim, a, b, c, d, ax)
   switch (dtype) {
     case WX_F32: WX_LAUNCH(WX_F32); break;
     case WX_F16: WX_LAUNCH(WX_F16); break;

@@ -207,6 +207,45 @@ __global__ __launch_bounds__(kMoverWaves* kWave) void permute_rows_tiled_kernel(
   }
 }
 
+// Same result, driven from the destination side: a wavefront owns one 16-row block of the tiled matrix and a
+// range of column blocks; lane -> (row lane/4, slot lane%4) reads 16 bytes of its source row and the 64 lanes
+// write one whole contiguous KiB block.  Needs the inverse map (sorted position -> source token).
+constexpr int kGatherSplit = 4;  // wavefronts per 16-row block, each takes a quarter of the column blocks
+__global__ __launch_bounds__(kMoverWaves* kWave) void permute_rows_tiled_gather_kernel(
+    const u32x4* __restrict__ x, unsigned char* __restrict__ out, const int32_t* __restrict__ sorted_row_id,
+    const int32_t* __restrict__ expert_offsets, int64_t num_tokens, int64_t col_blocks, int64_t row_blocks) {
+  const int lane = lane_id();
+  const int64_t wave = static_cast<int64_t>(blockIdx.x) * kMoverWaves + threadIdx.x / kWave;
+  const int64_t rb = wave / kGatherSplit;
+  const int part = static_cast<int>(wave % kGatherSplit);
+  if (rb >= row_blocks) return;
+  const int32_t o0 = expert_offsets[0], o1 = expert_offsets[1], o2 = expert_offsets[2];
+  const int64_t pad0 = round_up_256(o1 - o0);
+  // padded row -> sorted position (or none for the padding rows of either expert)
+  const int r = lane >> 2, slot = lane & 3, chunk = slot ^ ((r >> 2) & 3);
+  const int64_t prow = rb * kBlkRows + r;
+  int64_t pos = -1;
+  if (prow < pad0) { if (prow < o1 - o0) pos = o0 + prow; }
+  else if (prow - pad0 < o2 - o1) pos = o1 + (prow - pad0);
+  const int64_t src_tok = (pos >= 0 && pos < num_tokens) ? sorted_row_id[pos] : -1;
+  const int64_t chunks_per_row = col_blocks * 4;
+  const u32x4* src = x + (src_tok < 0 ? 0 : src_tok) * chunks_per_row + chunk;
+  const int64_t kb_per = (col_blocks + kGatherSplit - 1) / kGatherSplit;
+  const int64_t kb0 = part * kb_per, kb1 = kb0 + kb_per < col_blocks ? kb0 + kb_per : col_blocks;
+  unsigned char* dst = out + (rb << 10) + lane * 16;
+  const u32x4 zero = {0, 0, 0, 0};
+  int64_t kb = kb0;
+  for (; kb + 3 < kb1; kb += 4) {
+    u32x4 v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) v[u] = src_tok < 0 ? zero : ld16(src + (kb + u) * 4);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) st16(reinterpret_cast<u32x4*>(dst + (((kb + u) * row_blocks) << 10)), v[u]);
+  }
+  for (; kb < kb1; ++kb)
+    st16(reinterpret_cast<u32x4*>(dst + ((kb * row_blocks) << 10)), src_tok < 0 ? zero : ld16(src + kb * 4));
+}
+
 // out[t] = y[row_id_map[t]] (zeros when the map entry is -1); one wavefront per destination row.
 __global__ __launch_bounds__(kMoverWaves* kWave) void gather_rows_kernel(
     const u32x4* __restrict__ y, u32x4* __restrict__ out, const int32_t* __restrict__ row_id_map,
@@ -400,14 +439,24 @@ extern "C" int wx_permute_rows(const void* x, void* out, const int32_t* row_id_m
 }
 
 extern "C" int wx_permute_rows_tiled(const void* x, void* out_tiled, const int32_t* row_id_map,
-                                     const int32_t* expert_offsets, int64_t num_tokens, int64_t num_cols,
-                                     wx_stream_t stream) {
-  if (int rc = check_rows("wx_permute_rows_tiled", x, out_tiled, row_id_map, num_tokens, 1, num_cols, WX_BF16)) return rc;
+                                     const int32_t* sorted_row_id, const int32_t* expert_offsets,
+                                     int64_t num_tokens, int64_t num_cols, wx_stream_t stream) {
+  const int32_t* any_map = row_id_map != nullptr ? row_id_map : sorted_row_id;
+  if (int rc = check_rows("wx_permute_rows_tiled", x, out_tiled, any_map, num_tokens, 1, num_cols, WX_BF16)) return rc;
   if (num_cols % kBlkCols != 0)
     return fail(WX_ERR_UNSUPPORTED, "wx_permute_rows_tiled: num_cols (%lld) must be a multiple of 32",
                 static_cast<long long>(num_cols));
   if (num_tokens == 0) return WX_OK;
   if (expert_offsets == nullptr) return fail(WX_ERR_INVALID_ARGUMENT, "wx_permute_rows_tiled: null expert_offsets");
+  const int64_t row_blocks = padded_sorted_rows(num_tokens) / kBlkRows;
+  if (sorted_row_id != nullptr) {
+    const int64_t waves = row_blocks * kGatherSplit;
+    hipLaunchKernelGGL(permute_rows_tiled_gather_kernel, dim3(static_cast<unsigned>((waves + kMoverWaves - 1) / kMoverWaves)),
+                       dim3(kMoverWaves * kWave), 0, as_stream(stream), static_cast<const u32x4*>(x),
+                       static_cast<unsigned char*>(out_tiled), sorted_row_id, expert_offsets, num_tokens,
+                       num_cols / kBlkCols, row_blocks);
+    return check_launch("permute_rows_tiled_gather_kernel");
+  }
   hipLaunchKernelGGL(permute_rows_tiled_kernel, dim3(mover_grid(num_tokens)), dim3(kMoverWaves * kWave), 0,
                      as_stream(stream), static_cast<const u32x4*>(x), static_cast<unsigned char*>(out_tiled),
                      row_id_map, expert_offsets, num_tokens, num_cols / 8, padded_sorted_rows(num_tokens) / kBlkRows);

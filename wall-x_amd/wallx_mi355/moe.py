@@ -44,6 +44,7 @@ class Routing:
     row_id_map: torch.Tensor      # int32 [T]: sorted position of each token
     expert_offsets: torch.Tensor  # int32 [E + 1] on the device
     num_tokens: int
+    sorted_row_id: Optional[torch.Tensor] = None  # int32 [T]: token at each sorted position (inverse map)
 
 
 class _DualExpertFFN(torch.autograd.Function):
@@ -75,8 +76,9 @@ class SparseMoeBlock(nn.Module):
     def route(self, experts_indices: torch.Tensor) -> Routing:
         """Stable partition of the flattened token types; reuse the result for all layers of a forward."""
         ids = experts_indices.reshape(-1)
-        row_id_map, offsets, _, self._partition_ws = native.partition(ids, self.num_experts, 0, self._partition_ws)
-        return Routing(row_id_map, offsets, ids.numel())
+        row_id_map, offsets, inverse, self._partition_ws = native.partition(ids, self.num_experts, 0,
+                                                                            self._partition_ws, want_sorted=True)
+        return Routing(row_id_map, offsets, ids.numel(), inverse)
 
     def forward(self, hidden_states: torch.Tensor, experts_indices: torch.Tensor,
                 start_indices: Optional[torch.Tensor] = None, end_indices: Optional[torch.Tensor] = None,
@@ -95,7 +97,8 @@ class SparseMoeBlock(nn.Module):
             routing = self.route(experts_indices)
         if routing.num_tokens != x.size(0):
             raise RuntimeError(f"routing was built for {routing.num_tokens} tokens, got {x.size(0)}")
-        self._x_tiled = native.permute_rows_tiled(x, routing.row_id_map, routing.expert_offsets, self._x_tiled)
+        self._x_tiled = native.permute_rows_tiled(x, routing.row_id_map, routing.expert_offsets, self._x_tiled,
+                                                  routing.sorted_row_id)
         need = native.padded_sorted_rows(x.size(0)) * max(e.intermediate_size for e in self.experts)
         if self._hmid is None or self._hmid.numel() < need or self._hmid.device != x.device:
             self._hmid = torch.empty(need, dtype=torch.bfloat16, device=x.device)
@@ -112,9 +115,9 @@ def moe_layer_forward(x: torch.Tensor, token_types: torch.Tensor, weights, routi
     x [T, H] bf16, token_types [T] (bool / int), weights ((g0,u0,d0),(g1,u1,d1)).  Returns (y [T, H], routing).
     """
     if routing is None:
-        row_id_map, offsets, _, _ = native.partition(token_types.reshape(-1), 2, 0, workspace)
-        routing = Routing(row_id_map, offsets, x.size(0))
-    x_tiled = native.permute_rows_tiled(x, routing.row_id_map, routing.expert_offsets)
+        row_id_map, offsets, inverse, _ = native.partition(token_types.reshape(-1), 2, 0, workspace, want_sorted=True)
+        routing = Routing(row_id_map, offsets, x.size(0), inverse)
+    x_tiled = native.permute_rows_tiled(x, routing.row_id_map, routing.expert_offsets, None, routing.sorted_row_id)
     y_sorted = native.dual_swiglu_ffn(x_tiled, x.size(0), routing.expert_offsets, weights, hmid=hmid)
     y = native.unpermute(y_sorted, routing.row_id_map, torch.tensor([]), x.size(0), 1)
     return y, routing

@@ -384,9 +384,11 @@ def pack_weight(w: torch.Tensor, cache: bool = True) -> torch.Tensor:
     return packed
 
 
-def permute_rows_tiled(x: torch.Tensor, row_id_map: torch.Tensor, expert_offsets: torch.Tensor,
-                       out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """x [T, H] bf16 -> K-tiled, expert-padded activation matrix for dual_swiglu_ffn (flat bf16 tensor)."""
+def permute_rows_tiled(x: torch.Tensor, row_id_map: Optional[torch.Tensor], expert_offsets: torch.Tensor,
+                       out: Optional[torch.Tensor] = None, sorted_row_id: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x [T, H] bf16 -> K-tiled, expert-padded activation matrix for dual_swiglu_ffn (flat bf16 tensor).
+
+    With sorted_row_id (partition(..., want_sorted=True)) the rows are gathered block by block, the faster form."""
     _need_cuda("x", x)
     if x.dtype != torch.bfloat16:
         raise RuntimeError("All tensors must be BFloat16 for this kernel")
@@ -396,8 +398,8 @@ def permute_rows_tiled(x: torch.Tensor, row_id_map: torch.Tensor, expert_offsets
     if out is None or out.numel() < need or out.dtype != torch.bfloat16 or out.device != x.device:
         out = torch.empty(need, dtype=torch.bfloat16, device=x.device)
     with _DeviceGuard(x):
-        _lib.call("wx_permute_rows_tiled", _ptr(x), out.data_ptr(), _ptr(row_id_map), expert_offsets.data_ptr(), T, H,
-                  _stream(x))
+        _lib.call("wx_permute_rows_tiled", _ptr(x), out.data_ptr(), _ptr(row_id_map), _ptr(sorted_row_id),
+                  expert_offsets.data_ptr(), T, H, _stream(x))
     return out
 
 
