@@ -72,7 +72,10 @@ __device__ __forceinline__ void load_selected(const void* table, const AxisTable
 }
 
 // Heads per thread: the loads of all of them are issued before the first result is needed.
-constexpr int kHeadsPerThread = 3;
+#ifndef WX_MROPE_HPT
+#define WX_MROPE_HPT 3
+#endif
+constexpr int kHeadsPerThread = WX_MROPE_HPT;
 
 template <int DT, bool BWD>
 __global__ __launch_bounds__(256) void mrope_kernel(

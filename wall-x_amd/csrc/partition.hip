@@ -210,7 +210,10 @@ __global__ __launch_bounds__(kMoverWaves* kWave) void permute_rows_tiled_kernel(
 // Same result, driven from the destination side: a wavefront owns one 16-row block of the tiled matrix and a
 // range of column blocks; lane -> (row lane/4, slot lane%4) reads 16 bytes of its source row and the 64 lanes
 // write one whole contiguous KiB block.  Needs the inverse map (sorted position -> source token).
-constexpr int kGatherSplit = 4;  // wavefronts per 16-row block, each takes a quarter of the column blocks
+#ifndef WX_GATHER_SPLIT
+#define WX_GATHER_SPLIT 4
+#endif
+constexpr int kGatherSplit = WX_GATHER_SPLIT;  // wavefronts per 16-row block, each takes a quarter of the column blocks
 __global__ __launch_bounds__(kMoverWaves* kWave) void permute_rows_tiled_gather_kernel(
     const u32x4* __restrict__ x, unsigned char* __restrict__ out, const int32_t* __restrict__ sorted_row_id,
     const int32_t* __restrict__ expert_offsets, int64_t num_tokens, int64_t col_blocks, int64_t row_blocks) {
