@@ -36,6 +36,8 @@ def parse():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--ops-only", action="store_true", help="skip the side measurements (M-RoPE, index builders)")
+    ap.add_argument("--no-prefill", action="store_true", help="skip the config 5 prefill measurement (36-layer decoder)")
+    ap.add_argument("--prefill-mask", default="causal", choices=["causal", "action_block"])
     ap.add_argument("--cpu-seqs", type=int, default=4, help="sequences of the batch the CPU baseline runs")
     ap.add_argument("--kernel-loop", default=None,
                     choices=["gate_up", "down", "permute", "permute_plain", "unpermute", "partition", "copy"],
@@ -184,6 +186,9 @@ def main():
 
     if not args.ops_only:
         extra.update(side_measurements(dev, iters))
+    if not args.ops_only and not args.no_prefill:
+        del x_tiled, hmid, x_sorted, y_sorted, y
+        extra["prefill"] = prefill_measurement(dev, args.prefill_mask)
 
     result = {
         "metric": "dual_expert_ffn_tflops",
@@ -275,6 +280,38 @@ def side_measurements(dev, iters):
     out["mrope_GBps"] = round(rope_bytes / t / 1e6, 1)
     out["mrope_frac_hbm_peak"] = round(rope_bytes / t / 1e6 / PEAK_HBM_GBS, 4)
     return out
+
+
+def prefill_measurement(dev, mask):
+    """BASELINE config 5: one prefill of 16 x 912 tokens through a randomly initialised 36-layer decoder of the
+    Qwen2.5-VL-3B shape with the dual-expert FFN in every layer; attention, projections and norms on PyTorch."""
+    import torch
+    from wallx_mi355 import harness
+
+    model = harness.PrefillHarness(device=dev, mask=mask)
+    ids, grid, types = harness.config5_inputs(16, dev)
+    for _ in range(2):
+        model.forward(ids, grid, types)
+    torch.cuda.synchronize()
+    reps = 5
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        model.forward(ids, grid, types)
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / reps
+    timer = harness.OpTimer()
+    model.forward(ids, grid, types, timer)
+    split = timer.report_ms()
+    total = sum(split.values())
+    return {
+        "workload": "config 5 (BASELINE.json configs[4]): 36 layers, hidden 2048, 16 q / 2 kv heads x 128, experts "
+                    "11008 / 1024, 16 x 912 tokens (32 action each), bf16, random init, rms eps 1e-6, mask " + mask,
+        "tokens_per_s": round(ids.numel() / dt, 1),
+        "ms_per_forward": round(dt * 1e3, 3),
+        "op_split_ms": {k: round(v, 3) for k, v in sorted(split.items(), key=lambda kv: -kv[1])},
+        "op_split_total_ms": round(total, 3),
+        "ours_ms": round(sum(v for k, v in split.items() if not k.endswith("_torch")), 3),
+    }
 
 
 def cpu_baseline(x_cpu, types_cpu, w_cpu, n_seq, H, I0, I1):

@@ -1,0 +1,173 @@
+"""Prefill harness for BASELINE config 5: a randomly initialised decoder with the Qwen2.5-VL-3B shape and the
+dual VL / action expert FFN in every layer (act.py:172-273, 397-530), with every layer's permute, grouped GEMM,
+M-RoPE and the position builder replaced by the MI355X kernels.  RMSNorm, the QKV / O projections and attention
+stay on PyTorch-ROCm (attention = F.scaled_dot_product_attention), as the configuration prescribes.
+
+This is a measurement harness, not a model port: no KV cache, no generation, no losses; one forward over a
+batch of full sequences (prefill).  What it states explicitly:
+  * RMSNorm eps 1e-6 (the Qwen2.5-VL-3B value; the reference's config default is 1e-5, cfg.py:179),
+  * q/k/v projections with bias, o projection without (vl.py:821-832),
+  * attention mask: plain causal by default (`mask="causal"`); `mask="action_block"` adds the reference's
+    bidirectional block among action tokens (act.py:616-637) through a dense boolean mask,
+  * rotary base 1e6, mrope_section [16, 24, 24], cos/sin built in fp32 and cast to bf16 (vl.py:679-712).
+"""
+
+from contextlib import contextmanager
+from typing import Dict, List, Optional
+
+import torch
+import torch.nn.functional as F
+
+from . import moe, native, workloads as wl
+from .fusions import ops
+
+
+class OpTimer:
+    """Accumulates HIP-event durations per op name; events are resolved once, at report time."""
+
+    def __init__(self, enabled: bool = True):
+        self.enabled = enabled
+        self.pairs: List = []
+
+    @contextmanager
+    def section(self, name: str):
+        if not self.enabled:
+            yield
+            return
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        yield
+        b.record()
+        self.pairs.append((name, a, b))
+
+    def report_ms(self) -> Dict[str, float]:
+        torch.cuda.synchronize()
+        out: Dict[str, float] = {}
+        for name, a, b in self.pairs:
+            out[name] = out.get(name, 0.0) + a.elapsed_time(b)
+        self.pairs = []
+        return out
+
+
+def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    v = x.float()
+    v = v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps)
+    return weight * v.to(x.dtype)
+
+
+class PrefillHarness:
+    def __init__(self, n_layers: int = 36, hidden: int = wl.HIDDEN, n_q: int = wl.N_Q_HEADS, n_kv: int = wl.N_KV_HEADS,
+                 head_dim: int = wl.HEAD_DIM, inter=(wl.INTER_VL, wl.INTER_ACT), vocab: int = 151936,
+                 eps: float = 1e-6, device="cuda:0", seed: int = 0, mask: str = "causal", keep_dense: bool = False):
+        self.dev = torch.device(device)
+        self.n_layers, self.hidden, self.n_q, self.n_kv, self.head_dim = n_layers, hidden, n_q, n_kv, head_dim
+        self.inter, self.eps, self.mask_mode = inter, eps, mask
+        g = torch.Generator(device=self.dev).manual_seed(seed)
+
+        def w(*shape):
+            return (torch.randn(*shape, device=self.dev, generator=g, dtype=torch.float32) * 0.02).to(torch.bfloat16)
+
+        self.embed = w(vocab, hidden)
+        self.layers = []
+        for _ in range(n_layers):
+            layer = {
+                "ln1": torch.ones(hidden, dtype=torch.bfloat16, device=self.dev),
+                "ln2": torch.ones(hidden, dtype=torch.bfloat16, device=self.dev),
+                "wqkv": w((n_q + 2 * n_kv) * head_dim, hidden),  # q, k, v projections in one matrix
+                "bqkv": w((n_q + 2 * n_kv) * head_dim),
+                "wo": w(hidden, n_q * head_dim),
+                "experts": [(w(i, hidden), w(i, hidden), w(hidden, i)) for i in inter],
+            }
+            # the FFN kernels read K-tiled weights; pack now (static weights) and drop the nn.Linear copies
+            layer["packed"] = [tuple(native.pack_weight(t, cache=False) for t in e) for e in layer["experts"]]
+            if not keep_dense:  # tests keep the nn.Linear-layout copies to run a plain PyTorch forward beside this one
+                layer["experts"] = None
+            self.layers.append(layer)
+        self.final_ln = torch.ones(hidden, dtype=torch.bfloat16, device=self.dev)
+        self.inv_freq = wl.text_inv_freq(head_dim).to(self.dev)
+        self._hmid: Optional[torch.Tensor] = None
+        self._x_tiled: Optional[torch.Tensor] = None
+        self._ws = None
+
+    # ------------------------------------------------------------------------------------------------
+    def _ffn(self, x: torch.Tensor, routing: moe.Routing, packed, timer: OpTimer) -> torch.Tensor:
+        from . import _lib
+
+        T, H = x.shape
+        I0, I1 = self.inter
+        stream = torch.cuda.current_stream().cuda_stream
+        rows_pad = native.padded_sorted_rows(T)
+        if self._hmid is None or self._hmid.numel() < rows_pad * max(I0, I1):
+            self._hmid = torch.empty(rows_pad * max(I0, I1), dtype=torch.bfloat16, device=self.dev)
+        with timer.section("permute"):
+            self._x_tiled = native.permute_rows_tiled(x, routing.row_id_map, routing.expert_offsets, self._x_tiled,
+                                                      routing.sorted_row_id)
+        y_sorted = torch.empty_like(x)
+        (g0, u0, d0), (g1, u1, d1) = packed
+        with timer.section("ffn_gate_up_swiglu"):
+            _lib.call("wx_dual_swiglu_gate_up", self._x_tiled.data_ptr(), self._hmid.data_ptr(),
+                      routing.expert_offsets.data_ptr(), g0.data_ptr(), u0.data_ptr(), g1.data_ptr(), u1.data_ptr(),
+                      T, H, I0, I1, stream)
+        with timer.section("ffn_down"):
+            _lib.call("wx_dual_down_proj", self._hmid.data_ptr(), y_sorted.data_ptr(), routing.expert_offsets.data_ptr(),
+                      d0.data_ptr(), d1.data_ptr(), T, H, I0, I1, stream)
+        with timer.section("unpermute"):
+            y = native.unpermute(y_sorted, routing.row_id_map, torch.tensor([]), T, 1)
+        return y
+
+    @torch.no_grad()
+    def forward(self, input_ids: torch.Tensor, image_grid_thw: torch.Tensor, moe_token_types: torch.Tensor,
+                timer: Optional[OpTimer] = None) -> torch.Tensor:
+        """input_ids [B, S] int64, image_grid_thw [n_img, 3], moe_token_types [B, S] bool -> logits of the last
+        position [B, vocab]."""
+        timer = timer or OpTimer(False)
+        B, S = input_ids.shape
+        H, D, nq, nkv = self.hidden, self.head_dim, self.n_q, self.n_kv
+        with timer.section("rope_index"):
+            pos, _ = ops.get_rope_index(input_ids, 2, wl.IMAGE_TOKEN_ID, wl.VIDEO_TOKEN_ID, wl.VISION_START_TOKEN_ID, 2,
+                                        image_grid_thw=image_grid_thw)
+        with timer.section("cos_sin_torch"):
+            freqs = pos.float()[..., None] * self.inv_freq
+            emb = torch.cat((freqs, freqs), -1)
+            cos, sin = emb.cos().to(torch.bfloat16), emb.sin().to(torch.bfloat16)
+        with timer.section("partition"):
+            ids = moe_token_types.reshape(-1)
+            rmap, off, inv, self._ws = native.partition(ids, 2, 0, self._ws, want_sorted=True)
+            routing = moe.Routing(rmap, off, ids.numel(), inv)
+        attn_mask = None
+        if self.mask_mode == "action_block":
+            causal = torch.ones(S, S, dtype=torch.bool, device=self.dev).tril()
+            act = moe_token_types[:, None, :, None] & moe_token_types[:, None, None, :]
+            attn_mask = causal[None, None] | act
+        with timer.section("embed_torch"):
+            h = self.embed[input_ids]
+        for layer in self.layers:
+            with timer.section("rmsnorm_torch"):
+                x = rms_norm(h, layer["ln1"], self.eps)
+            with timer.section("qkv_proj_torch"):
+                qkv = F.linear(x, layer["wqkv"], layer["bqkv"])
+                q, k, v = qkv.split([nq * D, nkv * D, nkv * D], dim=-1)
+                q = q.view(B, S, nq, D).transpose(1, 2)
+                k = k.view(B, S, nkv, D).transpose(1, 2)
+                v = v.view(B, S, nkv, D).transpose(1, 2)
+            with timer.section("mrope"):
+                q, k = ops.multimodal_rope(q, k, cos, sin, list(wl.MROPE_SECTION))
+            with timer.section("sdpa_torch"):
+                a = F.scaled_dot_product_attention(q, k, v, attn_mask=attn_mask, is_causal=attn_mask is None,
+                                                   enable_gqa=True)
+            with timer.section("o_proj_torch"):
+                h = h + F.linear(a.transpose(1, 2).reshape(B, S, nq * D), layer["wo"])
+            with timer.section("rmsnorm_torch"):
+                x = rms_norm(h, layer["ln2"], self.eps)
+            h = h + self._ffn(x.view(B * S, H), routing, layer["packed"], timer).view(B, S, H)
+        with timer.section("lm_head_torch"):
+            last = rms_norm(h[:, -1], self.final_ln, self.eps)
+            logits = F.linear(last, self.embed)
+        return logits
+
+
+def config5_inputs(batch: int = 16, device="cuda:0"):
+    """16 sequences x 912 tokens: 768 vision, 112 text-class, 32 action (tail_text = 96 in the config 2 row layout)."""
+    ids, grid = wl.config2_tokens(batch=batch, tail_text=96)
+    types = ids == wl.ACTION_TOKEN_ID  # load_lerobot_dataset.py:406-409
+    return ids.to(device), grid.to(device), types.to(device)
