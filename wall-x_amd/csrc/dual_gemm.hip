@@ -107,6 +107,16 @@ __device__ __forceinline__ bool map_tile(int t, int total, const int* tiles_m, c
   return true;
 }
 
+// Workgroup barrier without the fences of __syncthreads().  Those fences make the compiler wait for EVERY
+// outstanding LDS-direct load (vmcnt(0)) at the barrier, which drains the prefetch ring on each K step; the waits
+// the data flow needs (own LDS reads returned, own loads of the next slot landed) are written out before each call.
+// The empty asm statements keep the compiler from moving memory accesses across the barrier.
+__device__ __forceinline__ void barrier_no_fence() {
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}
+
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
   const bf16x2 v = {static_cast<__bf16>(lo), static_cast<__bf16>(hi)};  // one packed convert
@@ -335,7 +345,7 @@ __global__ __launch_bounds__(kThreads, 1) void dual_gemm_kernel(Params p) {
     // my LDS reads have returned; of my loads at most the two youngest K steps (2 * kLoads loads each) are still
     // in flight, i.e. the next slot is complete
     __builtin_amdgcn_s_waitcnt(waitcnt_imm(2 * 2 * kLoads, 0));
-    __syncthreads();
+    barrier_no_fence();
     issue(L, ld_ks, sa, sb);
     __builtin_amdgcn_sched_barrier(0);  // keep the refill right behind the barrier: it has the longest way to go
     read_frags(sa_n, sb_n, 0, 0);
