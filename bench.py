@@ -186,6 +186,8 @@ def main():
 
     if not args.ops_only:
         extra.update(side_measurements(dev, iters))
+    if not args.ops_only:
+        extra["ceilings"] = ceiling_measurements(dev, x, weights, m0)
     if not args.ops_only and not args.no_prefill:
         del x_tiled, hmid, x_sorted, y_sorted, y
         extra["prefill"] = prefill_measurement(dev, args.prefill_mask)
@@ -279,6 +281,48 @@ def side_measurements(dev, iters):
     out["mrope_us"] = round(t * 1e3, 2)
     out["mrope_GBps"] = round(rope_bytes / t / 1e6, 1)
     out["mrope_frac_hbm_peak"] = round(rope_bytes / t / 1e6 / PEAK_HBM_GBS, 4)
+    return out
+
+
+def ceiling_measurements(dev, x, weights, m0):
+    """What bounds an MFMA kernel on THIS data, measured on the same GPU in the same run (reported, not part of
+    `value`): (1) back-to-back bf16 MFMA instructions with operands held in registers, on zeros and on values
+    drawn like the benchmark's activations and weights -- the sustained MFMA rate depends on the operand values
+    (switching activity moves the clock the chip holds), so the nominal 2.5 PFLOP/s is not reachable on random
+    data; (2) the vendor GEMM (torch.matmul -> hipBLASLt) on the VL expert's two GEMM shapes with the benchmark's
+    own tensors, without the SwiGLU epilogue or the second expert."""
+    import ctypes
+    import torch
+    from wallx_mi355 import _lib
+
+    out = {}
+    lib = _lib.load()
+    n = lib.wx_probe_mfma_operand_bytes() // 2
+    sink = torch.zeros(1, dtype=torch.float32, device=dev)
+    flops = ctypes.c_double(0.0)
+    stream = torch.cuda.current_stream().cuda_stream
+    g = torch.Generator(device=dev).manual_seed(1)
+    data = torch.randn(n, device=dev, generator=g)
+    data[n // 2:] *= 0.02  # half the fragments look like activations N(0, 1), half like weights N(0, 0.02)
+    for name, ops in (("zeros", torch.zeros(n, dtype=torch.bfloat16, device=dev)), ("normal", data.to(torch.bfloat16))):
+        def run():
+            _lib.call("wx_probe_mfma_rate", ops.data_ptr(), 4000, sink.data_ptr(), ctypes.byref(flops), stream)
+        t, _ = event_ms(run, 5, warm=2)
+        out[f"mfma_only_{name}_operands_tflops"] = round(flops.value / t / 1e9, 1)
+    (g0, u0, d0) = weights[0]
+    H, I0 = g0.shape[1], g0.shape[0]
+    xv = x[:m0]
+    wgu = torch.cat((g0, u0), 0)
+    o = torch.empty(m0, 2 * I0, dtype=torch.bfloat16, device=dev)
+    t, _ = event_ms(lambda: torch.matmul(xv, wgu.t(), out=o), 10)
+    out["hipblaslt_gate_up_shape_tflops"] = round(4.0 * m0 * I0 * H / t / 1e9, 1)
+    hm = o[:, :I0].contiguous()
+    del o
+    o2 = torch.empty(m0, H, dtype=torch.bfloat16, device=dev)
+    t, _ = event_ms(lambda: torch.matmul(hm, d0.t(), out=o2), 10)
+    out["hipblaslt_down_shape_tflops"] = round(2.0 * m0 * I0 * H / t / 1e9, 1)
+    out["note"] = ("same GPU, same run; hipBLASLt numbers are plain GEMMs of the VL expert on the benchmark's tensors "
+                   "(no SwiGLU, no second expert, rows already contiguous)")
     return out
 
 

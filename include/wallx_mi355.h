@@ -203,6 +203,16 @@ int wx_window_index(const void* grid_thw, int grid_type, int64_t n_grid, int spa
                     int64_t total_windows, int32_t* window_index, int32_t* cu_window_seqlens,
                     wx_stream_t stream);
 
+/* ---- measurement probe (no counterpart in the reference; used by bench.py) --------------------------------
+ * Runs bf16 32x32x16 MFMA instructions back to back on every CU, operands taken from `operands`
+ * (wx_probe_mfma_operand_bytes() bytes of bf16 values, device memory, 16-byte aligned) and held in registers:
+ * no LDS or memory traffic inside the loop.  The sustained MFMA rate depends on the operand VALUES (switching
+ * activity moves the clock the chip can hold), so timing this on the same kind of data as a GEMM gives the
+ * ceiling an MFMA-bound kernel can reach on that data.  *flops_per_launch receives the flops one launch performs
+ * (host pointer, may be NULL); sink is one float of device memory that is practically never written. */
+size_t wx_probe_mfma_operand_bytes(void);
+int wx_probe_mfma_rate(const void* operands, int iters, float* sink, double* flops_per_launch, wx_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -7,11 +7,13 @@
 // (thousands of VL rows next to tens of action rows, or an empty group) is just a longer or shorter tile list.
 //
 // Workgroup tile 256 x 256, K step 32, four wavefronts (one per SIMD) as 2 x 2, wave tile 128 x 128 = 4 x 4 MFMA
-// 32x32x16 accumulator blocks (256 accumulator registers per lane).  Operands are K-contiguous, so both MFMA
-// fragments are 16-byte LDS reads.  Global -> LDS uses buffer loads that write LDS directly (no register
-// staging) into a ring of four K-step slots per operand; the load stream runs four K steps ahead of the MFMAs and
-// crosses tile boundaries, with one workgroup barrier per K step.  LDS rows are 64 bytes; chunk c of row r sits
-// in slot c ^ ((r >> 2) & 3), which makes the 16-byte fragment reads bank-conflict free.
+// 32x32x16 accumulator blocks (256 accumulator registers per lane), one workgroup per CU.  (WX_GEMM_BN=128 builds
+// a 256 x 128 tile with two resident workgroups per CU, three ring slots and 128 accumulator registers; it
+// measures a few percent slower on both FFN GEMMs and is kept as a build option.)  Operands are K-contiguous, so
+// both MFMA fragments are 16-byte LDS reads.  Global -> LDS uses buffer loads that write LDS directly (no
+// register staging) into a ring of four K-step slots per operand; the load stream runs four K steps ahead of
+// the MFMAs and crosses tile boundaries, with one workgroup barrier per K step.  LDS rows are 64 bytes; chunk c
+// of row r sits in slot c ^ ((r >> 2) & 3), which makes the 16-byte fragment reads bank-conflict free.
 //
 // Three operand layouts:
 //   generic  (wx_dual_gemm)            A, B, C row-major; loads touch 16 rows x 64 bytes per instruction.
@@ -33,18 +35,33 @@ namespace {
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
-constexpr int BM = 256, BN = 256, BK = 32;
+#ifndef WX_GEMM_BN
+#define WX_GEMM_BN 256
+#endif
+#if WX_GEMM_BN == 256
+#define WX_GEMM_STAGES 4
+#else
+#define WX_GEMM_STAGES 3
+#endif
+constexpr int BM = 256, BN = WX_GEMM_BN, BK = 32;
+static_assert(BN == 128 || BN == 256, "tile width");
+constexpr int kWgPerCu = BN == 256 ? 1 : 2;    // resident workgroups per CU (LDS and registers are sized for this)
 constexpr int kWavesM = 2, kWavesN = 2;        // wavefront grid over the tile; one wavefront per SIMD
 constexpr int kWaves = kWavesM * kWavesN;
 constexpr int kThreads = kWaves * 64;
 constexpr int FM = BM / kWavesM / 32;          // 32x32 accumulator blocks per wave along M (4)
-constexpr int FN = BN / kWavesN / 32;          // ... and along N (4): 256 accumulator registers per lane
-constexpr int kLoadRows = BM / kWaves;         // LDS rows of each operand one wave loads per K step (64)
-constexpr int kLoads = kLoadRows / 16;         // 16-row load instructions per operand per wave per K step (4)
-constexpr int kStages = 4;                     // ring slots per operand (the tile loop is written out for 4)
+constexpr int FN = BN / kWavesN / 32;          // ... and along N (4, or 2 for the 128-wide tile)
+constexpr int kLoadRowsA = BM / kWaves;        // LDS rows of A one wave loads per K step (64)
+constexpr int kLoadRowsB = BN / kWaves;        // ... and of B (64 / 32)
+constexpr int kLoadsA = kLoadRowsA / 16;       // 16-row load instructions per wave per K step: A (4)
+constexpr int kLoadsB = kLoadRowsB / 16;       // ... and B (4 / 2)
+constexpr int kLoadsPerStep = kLoadsA + kLoadsB;
+constexpr int kStages = WX_GEMM_STAGES;        // ring slots per operand
 constexpr int kRowBytes = BK * 2;              // 64 bytes of K per LDS row
-constexpr int kSlotBytes = BM * kRowBytes;     // 16 KiB per operand per K step
-constexpr int kStageBytes = 8192;              // per-wave staging for the epilogue
+constexpr int kSlotBytesA = BM * kRowBytes;    // 16 KiB of A per K step
+constexpr int kSlotBytesB = BN * kRowBytes;    // 16 / 8 KiB of B per K step
+constexpr int kStageBytes = BN == 256 ? 8192 : 2048;  // per-wave staging for the epilogue
+static_assert(kStages * (kSlotBytesA + kSlotBytesB) + kWaves * kStageBytes <= 160 * 1024 / kWgPerCu, "LDS budget");
 constexpr int kXcds = 8;
 constexpr int kGroupM = 8;                     // tile rows per patch in the tile order
 
@@ -124,22 +141,37 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
 }
 
 template <int MODE>
-__global__ __launch_bounds__(kThreads, 1) void dual_gemm_kernel(Params p) {
+__global__ __launch_bounds__(kThreads, kWgPerCu) void dual_gemm_kernel(Params p) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stub; the body uses gfx950-only builtins
   constexpr bool SWIGLU = MODE == kGateUp;
   constexpr bool TILED_IN = MODE != kGeneric;   // A and B are K-tiled
   constexpr bool TILED_OUT = MODE == kGateUp;   // C is K-tiled
   // kStages ring slots per operand, each one K step (256 rows x 32 bf16).  Separate arrays let the compiler
   // see that a read of one slot never waits for a buffer load that targets another.
-  __shared__ __attribute__((aligned(1024))) unsigned char s_a0[kSlotBytes];
-  __shared__ __attribute__((aligned(1024))) unsigned char s_a1[kSlotBytes];
-  __shared__ __attribute__((aligned(1024))) unsigned char s_a2[kSlotBytes];
-  __shared__ __attribute__((aligned(1024))) unsigned char s_a3[kSlotBytes];
-  __shared__ __attribute__((aligned(1024))) unsigned char s_b0[kSlotBytes];
-  __shared__ __attribute__((aligned(1024))) unsigned char s_b1[kSlotBytes];
-  __shared__ __attribute__((aligned(1024))) unsigned char s_b2[kSlotBytes];
-  __shared__ __attribute__((aligned(1024))) unsigned char s_b3[kSlotBytes];
+  __shared__ __attribute__((aligned(1024))) unsigned char s_a0[kSlotBytesA];
+  __shared__ __attribute__((aligned(1024))) unsigned char s_a1[kSlotBytesA];
+  __shared__ __attribute__((aligned(1024))) unsigned char s_a2[kSlotBytesA];
+  __shared__ __attribute__((aligned(1024))) unsigned char s_b0[kSlotBytesB];
+  __shared__ __attribute__((aligned(1024))) unsigned char s_b1[kSlotBytesB];
+  __shared__ __attribute__((aligned(1024))) unsigned char s_b2[kSlotBytesB];
+#if WX_GEMM_STAGES == 4
+  __shared__ __attribute__((aligned(1024))) unsigned char s_a3[kSlotBytesA];
+  __shared__ __attribute__((aligned(1024))) unsigned char s_b3[kSlotBytesB];
+#endif
   __shared__ __attribute__((aligned(1024))) unsigned char s_out[kWaves * kStageBytes];
+  // ring slot s of each operand (s is a constant after unrolling)
+  auto slot_a = [&](int s) -> unsigned char* {
+#if WX_GEMM_STAGES == 4
+    if (s == 3) return s_a3;
+#endif
+    return s == 0 ? s_a0 : (s == 1 ? s_a1 : s_a2);
+  };
+  auto slot_b = [&](int s) -> unsigned char* {
+#if WX_GEMM_STAGES == 4
+    if (s == 3) return s_b3;
+#endif
+    return s == 0 ? s_b0 : (s == 1 ? s_b1 : s_b2);
+  };
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keeps descriptors and LDS bases scalar
@@ -186,8 +218,8 @@ __global__ __launch_bounds__(kThreads, 1) void dual_gemm_kernel(Params p) {
 
   // ---- per-lane constants -----------------------------------------------------------------------
   // row-major loader: one instruction fills 16 LDS rows of 64 bytes; lane -> (row lane/4, slot lane%4).
-  // Instruction i of this wave covers rows [wave*64 + 16i, +16).  Chunk c of row r lives in slot c ^ ((r >> 2) & 3).
-  const int ld_row0 = wave * kLoadRows + (lane >> 2);
+  // Instruction i of this wave covers rows [wave*64 + 16i, +16) of A.  Chunk c of row r lives in slot c ^ ((r >> 2) & 3).
+  const int ld_row0 = wave * kLoadRowsA + (lane >> 2);
   const int ld_chunk = (lane & 3) ^ ((lane >> 4) & 3);
   // fragment reads: row = base + l32, chunk kc = 2*kk + lhi
   const int sw = (l32 >> 2) & 3;
@@ -204,10 +236,10 @@ __global__ __launch_bounds__(kThreads, 1) void dual_gemm_kernel(Params p) {
   const int b_lane_off = l32 * kRowBytes;
 
   // ---- per-tile state ------------------------------------------------------------------------------
-  struct Loader {   // where this wave's 2 * kLoads loads per K step come from
+  struct Loader {   // where this wave's kLoadsA + kLoadsB loads per K step come from
     const __bf16 *a_base, *b_base;
     uint32_t a_bytes, b_bytes;        // readable bytes from the base (row-major) / from the current block (tiled)
-    uint32_t voff_a[kLoads], voff_b[kLoads];
+    uint32_t voff_a[kLoadsA], voff_b[kLoadsB];
     int64_t a_step, b_step;           // tiled: bytes between consecutive K steps
     int K, nk;      // nk: K steps of the tile, rounded up to a multiple of kStages (padding steps read zeros)
   };
@@ -241,10 +273,10 @@ __global__ __launch_bounds__(kThreads, 1) void dual_gemm_kernel(Params p) {
     const __bf16* b_src = up_half ? G.b1 : G.b0;
     const int b_wave = SWIGLU ? wave % kHalfWaves : wave;
     if constexpr (TILED_IN) {
-      // this wave's kLoads row blocks of the A tile and of the B tile at K step 0; a K step later they sit one
-      // column block further, i.e. (row blocks of the matrix) KiB ahead
-      const int64_t a_blk = (G.a_row0 + row0) / kBlkRows + wave * kLoads;
-      const int64_t b_blk = col0 / kBlkRows + b_wave * kLoads;
+      // this wave's row blocks of the A tile and of the B tile at K step 0; a K step later they sit one column
+      // block further, i.e. (row blocks of the matrix) KiB ahead
+      const int64_t a_blk = (G.a_row0 + row0) / kBlkRows + wave * kLoadsA;
+      const int64_t b_blk = col0 / kBlkRows + b_wave * kLoadsB;
       L.a_base = G.a + (a_blk << 9);
       L.b_base = b_src + (b_blk << 9);
       L.a_step = static_cast<int64_t>(G.lda) << 10;
@@ -254,7 +286,9 @@ __global__ __launch_bounds__(kThreads, 1) void dual_gemm_kernel(Params p) {
       L.a_bytes = static_cast<uint32_t>(a_left < 0 ? 0 : (a_left > 0x7fffff00ll ? 0x7fffff00ll : a_left));
       L.b_bytes = static_cast<uint32_t>(b_left < 0 ? 0 : (b_left > 0x7fffff00ll ? 0x7fffff00ll : b_left));
 #pragma unroll
-      for (int i = 0; i < kLoads; ++i) L.voff_a[i] = L.voff_b[i] = static_cast<uint32_t>(i * kBlkBytes + lane * 16);
+      for (int i = 0; i < kLoadsA; ++i) L.voff_a[i] = static_cast<uint32_t>(i * kBlkBytes + lane * 16);
+#pragma unroll
+      for (int i = 0; i < kLoadsB; ++i) L.voff_b[i] = static_cast<uint32_t>(i * kBlkBytes + lane * 16);
     } else {
       const int rows_a = G.m - row0 < BM ? G.m - row0 : BM;
       const int rows_b = G.n - col0 < kTileN ? G.n - col0 : kTileN;
@@ -263,16 +297,15 @@ __global__ __launch_bounds__(kThreads, 1) void dual_gemm_kernel(Params p) {
       L.a_bytes = static_cast<uint32_t>(rows_a) * G.lda * 2u;
       L.b_bytes = static_cast<uint32_t>(rows_b) * G.ldb * 2u;
       L.a_step = L.b_step = 0;
-      const int b_ld_row0 = b_wave * kLoadRows + (lane >> 2);
+      const int b_ld_row0 = b_wave * kLoadRowsB + (lane >> 2);
 #pragma unroll
-      for (int i = 0; i < kLoads; ++i) {
-        L.voff_a[i] = static_cast<uint32_t>(ld_row0 + 16 * i) * G.lda * 2u + ld_chunk * 16u;
-        L.voff_b[i] = static_cast<uint32_t>(b_ld_row0 + 16 * i) * G.ldb * 2u + ld_chunk * 16u;
-      }
+      for (int i = 0; i < kLoadsA; ++i) L.voff_a[i] = static_cast<uint32_t>(ld_row0 + 16 * i) * G.lda * 2u + ld_chunk * 16u;
+#pragma unroll
+      for (int i = 0; i < kLoadsB; ++i) L.voff_b[i] = static_cast<uint32_t>(b_ld_row0 + 16 * i) * G.ldb * 2u + ld_chunk * 16u;
     }
   };
 
-  // One K step of global -> LDS for this wave: rows [wave*64, +64) of the A slot and of the B slot.
+  // One K step of global -> LDS for this wave: rows [wave*64, +64) of the A slot, [wave*kLoadRowsB, +kLoadRowsB) of B.
   auto issue = [&](const Loader& L, int ks, unsigned char* sa, unsigned char* sb) {
     __amdgpu_buffer_rsrc_t ra, rb;
     uint32_t oob = 0;
@@ -297,11 +330,12 @@ __global__ __launch_bounds__(kThreads, 1) void dual_gemm_kernel(Params p) {
       oob = (k_tail && k0 + ld_chunk * 8 >= L.K) ? 0x80000000u : 0u;
     }
 #pragma unroll
-    for (int i = 0; i < kLoads; ++i) {
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, LDS_PTR(sa + (wave * kLoadRows + 16 * i) * kRowBytes), 16,
+    for (int i = 0; i < kLoadsA; ++i) {
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, LDS_PTR(sa + (wave * kLoadRowsA + 16 * i) * kRowBytes), 16,
                                                L.voff_a[i] | oob, 0, 0, 0);
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, LDS_PTR(sb + (wave * kLoadRows + 16 * i) * kRowBytes), 16,
-                                               L.voff_b[i] | oob, 0, 0, 0);
+      if (i < kLoadsB)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, LDS_PTR(sb + (wave * kLoadRowsB + 16 * i) * kRowBytes), 16,
+                                                 L.voff_b[i] | oob, 0, 0, 0);
     }
   };
 
@@ -323,14 +357,29 @@ __global__ __launch_bounds__(kThreads, 1) void dual_gemm_kernel(Params p) {
       for (int j = 0; j < FN; ++j)
         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[set][i], fb[set][j], acc[i][j], 0, 0, 0);
   };
-  // scheduling hint: the LDS reads of the next fragment set go out early among the MFMAs of this one
-  auto front_load_reads = [&]() {
+  // Scheduling hints.  Before the barrier: the LDS reads of the next fragment set go out among the first MFMAs
+  // of this one and the remaining MFMAs cover their latency, so the wait in front of the barrier finds them done.
+  auto schedule_reads_then_mfma = [&]() {
 #pragma unroll
     for (int q = 0; q < (FM + FN) / 2; ++q) {
       __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);  // two LDS reads
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
     }
     __builtin_amdgcn_sched_group_barrier(0x008, FM * FN - (FM + FN) / 2, 0);
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  // After the barrier: the refill loads and the next slot's fragment reads are spread over the MFMAs.
+  auto schedule_loads_reads_mfma = [&]() {
+    constexpr int kPairs = (FM + FN) / 2;
+    constexpr int kMixed = kLoadsPerStep > kPairs ? kLoadsPerStep : kPairs;
+#pragma unroll
+    for (int q = 0; q < kMixed; ++q) {
+      if (q < kLoadsPerStep) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // one buffer load
+      if (q < kPairs) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);         // two LDS reads
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                         // one MFMA
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, FM * FN - kMixed, 0);
+    __builtin_amdgcn_sched_barrier(0);
   };
 
   // One K step on slot (sa, sb); (sa_n, sb_n) is the next slot of the ring.  On entry fragment set 0 holds kk = 0
@@ -341,16 +390,15 @@ __global__ __launch_bounds__(kThreads, 1) void dual_gemm_kernel(Params p) {
                     unsigned char* sb_n) {
     read_frags(sa, sb, 1, 1);
     mma(0);
-    front_load_reads();
-    // my LDS reads have returned; of my loads at most the two youngest K steps (2 * kLoads loads each) are still
-    // in flight, i.e. the next slot is complete
-    __builtin_amdgcn_s_waitcnt(waitcnt_imm(2 * 2 * kLoads, 0));
+    schedule_reads_then_mfma();
+    // my LDS reads have returned; of my loads at most the kStages - 2 youngest K steps are still in flight, i.e.
+    // the next slot is complete
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm((kStages - 2) * kLoadsPerStep, 0));
     barrier_no_fence();
     issue(L, ld_ks, sa, sb);
-    __builtin_amdgcn_sched_barrier(0);  // keep the refill right behind the barrier: it has the longest way to go
     read_frags(sa_n, sb_n, 0, 0);
     mma(1);
-    front_load_reads();
+    schedule_loads_reads_mfma();
   };
 
   // ---- epilogue ------------------------------------------------------------------------------------------
@@ -378,13 +426,17 @@ __global__ __launch_bounds__(kThreads, 1) void dual_gemm_kernel(Params p) {
     asm volatile("" : "+v"(lane_e));
     const int el32 = lane_e & 31, elhi = lane_e >> 5, odd = lane_e & 1;
     if constexpr (SWIGLU) {
-      // wave output: 128 rows x 64 intermediate columns, staged 64 rows at a time (64 x 64 bf16 = 8 KiB)
-      constexpr int kPitch = 64 * 2;
+      // wave output: 128 rows x kOutCols intermediate columns, staged kRound rows at a time
+      constexpr int kOutCols = FN / 2 * 32;
+      constexpr int kPitch = kOutCols * 2;
+      constexpr int kRound = kStageBytes / kPitch;  // rows per round (64 / 32)
+      constexpr int kIPerRound = kRound / 32;       // 32-row accumulator blocks per round
+      static_assert(kIPerRound >= 1 && FM % kIPerRound == 0, "staging holds whole accumulator blocks");
 #pragma unroll
-      for (int half = 0; half < 2; ++half) {
+      for (int round = 0; round < FM / kIPerRound; ++round) {
 #pragma unroll
-        for (int ii = 0; ii < 2; ++ii) {
-          const int i = half * 2 + ii;
+        for (int ii = 0; ii < kIPerRound; ++ii) {
+          const int i = round * kIPerRound + ii;
 #pragma unroll
           for (int j = 0; j < FN / 2; ++j) {
 #pragma unroll
@@ -405,17 +457,18 @@ __global__ __launch_bounds__(kThreads, 1) void dual_gemm_kernel(Params p) {
           }
         }
         __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, 0));
-        // 64 rows x 64 columns = 4 row blocks x 2 column blocks of the tiled intermediate, 1 KiB each; one store
-        // instruction per block: lane -> (row lane/4, slot lane%4) holding chunk slot ^ ((row >> 2) & 3)
+        // kRound rows x kOutCols columns = (kRound / 16) row blocks x (kOutCols / 32) column blocks of the tiled
+        // intermediate, 1 KiB each; one store instruction per block: lane -> (row lane/4, slot lane%4) holding
+        // chunk slot ^ ((row >> 2) & 3)
         const int r16 = lane_e >> 2, slot = lane_e & 3, chunk = slot ^ ((r16 >> 2) & 3);
 #pragma unroll
-        for (int rbl = 0; rbl < 4; ++rbl) {
+        for (int rbl = 0; rbl < kRound / 16; ++rbl) {
 #pragma unroll
-          for (int kbl = 0; kbl < 2; ++kbl) {
+          for (int kbl = 0; kbl < kOutCols / 32; ++kbl) {
             const u32x4 v =
                 *reinterpret_cast<const u32x4*>(stage + (rbl * 16 + r16) * kPitch + (kbl * 32 + chunk * 8) * 2);
-            const int row = wm * (FM * 32) + half * 64 + rbl * 16;  // first row of the block inside the tile
-            const int col = wn * (FN / 2 * 32) + kbl * 32;           // first column of the block inside the tile
+            const int row = wm * (FM * 32) + round * kRound + rbl * 16;  // first row of the block inside the tile
+            const int col = wn * kOutCols + kbl * 32;                     // first column of the block inside the tile
             // rows past the expert's last row are padding of the tiled matrix: harmless to write, never read
             if (col < S.cols_left) {
               unsigned char* dst = reinterpret_cast<unsigned char*>(S.c_base) +
@@ -424,34 +477,43 @@ __global__ __launch_bounds__(kThreads, 1) void dual_gemm_kernel(Params p) {
             }
           }
         }
-        __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, 0));  // staging is rewritten by the next half
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, 0));  // staging is rewritten by the next round
       }
     } else {
-      // wave output: 128 rows x 128 columns row-major, staged 32 rows at a time (32 x 128 bf16 = 8 KiB)
-      constexpr int kPitch = 128 * 2;
+      // wave output: 128 rows x kOutCols columns row-major, staged kRound rows at a time
+      constexpr int kOutCols = FN * 32;
+      constexpr int kPitch = kOutCols * 2;
+      constexpr int kRound = kStageBytes / kPitch;  // 32 / 16 rows
+      constexpr int kParts = 32 / kRound;           // rounds per 32-row accumulator block
+      static_assert(kParts == 1 || kParts == 2, "a round is a whole or half accumulator block");
+      constexpr int kLanesPerRow = kPitch / 16, kRowsPerStore = 64 / kLanesPerRow;
 #pragma unroll
       for (int i = 0; i < FM; ++i) {
 #pragma unroll
-        for (int j = 0; j < FN; ++j) {
+        for (int part = 0; part < kParts; ++part) {
 #pragma unroll
-          for (int r = 0; r < 16; r += 2) {
-            const int srow = 8 * (r >> 2) + 4 * elhi + (r & 3);
-            stage_pair(acc[i][j][r], acc[i][j][r + 1], srow, j * 32 + el32, kPitch, odd);
+          for (int j = 0; j < FN; ++j) {
+#pragma unroll
+            for (int rr = 0; rr < 16 / kParts; rr += 2) {
+              const int r = part * (16 / kParts) + rr;  // half blocks: registers 0..7 are rows 0..15, 8..15 rows 16..31
+              const int srow = 8 * (r >> 2) + 4 * elhi + (r & 3) - part * kRound;
+              stage_pair(acc[i][j][r], acc[i][j][r + 1], srow, j * 32 + el32, kPitch, odd);
+            }
           }
-        }
-        __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, 0));
-        // a row is 256 bytes = 16 lanes; one store instruction writes 4 rows
-        const int rr = lane_e >> 4, cc = (lane_e & 15) * 8;
+          __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, 0));
+          // a row is kPitch bytes = kLanesPerRow lanes; one store instruction writes kRowsPerStore rows
+          const int rl = lane_e / kLanesPerRow, cc = (lane_e % kLanesPerRow) * 8;
 #pragma unroll
-        for (int q = 0; q < 8; ++q) {
-          const int srow = q * 4 + rr;
-          const u32x4 v = *reinterpret_cast<const u32x4*>(stage + srow * kPitch + cc * 2);
-          const int row = wm * (FM * 32) + i * 32 + srow;
-          const int col = wn * (FN * 32) + cc;
-          if (row < S.rows && col < S.cols_left)
-            *reinterpret_cast<u32x4*>(S.c_base + static_cast<int64_t>(row) * S.ldc + col) = v;
+          for (int q = 0; q < kRound / kRowsPerStore; ++q) {
+            const int srow = q * kRowsPerStore + rl;
+            const u32x4 v = *reinterpret_cast<const u32x4*>(stage + srow * kPitch + cc * 2);
+            const int row = wm * (FM * 32) + i * 32 + part * kRound + srow;
+            const int col = wn * kOutCols + cc;
+            if (row < S.rows && col < S.cols_left)
+              *reinterpret_cast<u32x4*>(S.c_base + static_cast<int64_t>(row) * S.ldc + col) = v;
+          }
+          __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, 0));
         }
-        __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, 0));
       }
     }
   };
@@ -475,12 +537,10 @@ __global__ __launch_bounds__(kThreads, 1) void dual_gemm_kernel(Params p) {
   Store S;
   setup_loader(tc, L);
   setup_store(tc, S);
-  issue(L, 0, s_a0, s_b0);
-  issue(L, 1, s_a1, s_b1);
-  issue(L, 2, s_a2, s_b2);
-  issue(L, 3, s_a3, s_b3);
-  // slot 0 must be complete before its first fragments are read: three younger K steps may remain in flight
-  __builtin_amdgcn_s_waitcnt(waitcnt_imm(3 * 2 * kLoads, 15));
+#pragma unroll
+  for (int s = 0; s < kStages; ++s) issue(L, s, slot_a(s), slot_b(s));
+  // slot 0 must be complete before its first fragments are read: the younger K steps may remain in flight
+  __builtin_amdgcn_s_waitcnt(waitcnt_imm((kStages - 1) * kLoadsPerStep, 15));
   __syncthreads();
   read_frags(s_a0, s_b0, 0, 0);
 
@@ -508,10 +568,9 @@ __global__ __launch_bounds__(kThreads, 1) void dual_gemm_kernel(Params p) {
         }
         ld_ks = 0;
       }
-      k_step(L, ld_ks + 0, s_a0, s_b0, s_a1, s_b1);
-      k_step(L, ld_ks + 1, s_a1, s_b1, s_a2, s_b2);
-      k_step(L, ld_ks + 2, s_a2, s_b2, s_a3, s_b3);
-      k_step(L, ld_ks + 3, s_a3, s_b3, s_a0, s_b0);
+#pragma unroll
+      for (int s = 0; s < kStages; ++s)
+        k_step(L, ld_ks + s, slot_a(s), slot_b(s), slot_a((s + 1) % kStages), slot_b((s + 1) % kStages));
     }
     epilogue(done);
   }
@@ -583,13 +642,13 @@ int check_dims(const char* who, int64_t m, int64_t n, int64_t k) {
   // 256 rows of one operand must stay addressable through a 31-bit buffer offset
   if (k * 2 * 256 >= (1ll << 31) || n * 2 * 256 >= (1ll << 31)) return fail(WX_ERR_UNSUPPORTED, "%s: row too long", who);
   // the tile list is indexed with 32-bit integers
-  if (((m + 255) / 256) * ((n + 127) / 128) >= (1ll << 30)) return fail(WX_ERR_UNSUPPORTED, "%s: too many tiles", who);
+  if (((m + BM - 1) / BM) * ((n + BN / 2 - 1) / (BN / 2)) >= (1ll << 30)) return fail(WX_ERR_UNSUPPORTED, "%s: too many tiles", who);
   return WX_OK;
 }
 
 template <int MODE>
 int launch_mfma(const Params& p, hipStream_t s, const char* who) {
-  hipLaunchKernelGGL(dual_gemm_kernel<MODE>, dim3(device_cu_count()), dim3(kThreads), 0, s, p);
+  hipLaunchKernelGGL(dual_gemm_kernel<MODE>, dim3(device_cu_count() * kWgPerCu), dim3(kThreads), 0, s, p);
   return check_launch(who);
 }
 
