@@ -187,6 +187,8 @@ def main():
     if not args.ops_only:
         extra.update(side_measurements(dev, iters))
     if not args.ops_only:
+        extra["cold_hbm"] = cold_measurements(dev, x, row_id_map, T, H, row_bytes, iters)
+        extra["config4"] = config4_measurement(dev, weights)
         extra["ceilings"] = ceiling_measurements(dev, x, weights, m0)
     if not args.ops_only and not args.no_prefill:
         del x_tiled, hmid, x_sorted, y_sorted, y
@@ -281,6 +283,69 @@ def side_measurements(dev, iters):
     out["mrope_us"] = round(t * 1e3, 2)
     out["mrope_GBps"] = round(rope_bytes / t / 1e6, 1)
     out["mrope_frac_hbm_peak"] = round(rope_bytes / t / 1e6 / PEAK_HBM_GBS, 4)
+    return out
+
+
+def cold_measurements(dev, x, row_id_map, T, H, row_bytes, iters):
+    """The bandwidth kernels with operands that are NOT resident in the 256 MB memory-side cache: each call works
+    on the next of several buffer sets whose total size is above 1 GB, so every byte comes from and goes to HBM.
+    (The per-kernel figures elsewhere in this report reuse one buffer set, which that cache largely holds.)  A
+    plain device copy of the same size, timed the same way, is the reference for what HBM sustains."""
+    import torch
+    from wallx_mi355 import _lib
+
+    stream = torch.cuda.current_stream().cuda_stream
+    sets = 5
+    xs = [x.clone() for _ in range(sets)]
+    outs = [torch.empty_like(x) for _ in range(sets)]
+    state = {"i": 0}
+
+    def nxt():
+        state["i"] = (state["i"] + 1) % sets
+        return state["i"]
+
+    def permute_cold():
+        i = nxt()
+        _lib.call("wx_permute_rows", xs[i].data_ptr(), outs[i].data_ptr(), row_id_map.data_ptr(), T, 1, H,
+                  _lib.WX_BF16, stream)
+
+    def unpermute_cold():
+        i = nxt()
+        _lib.call("wx_unpermute_rows", xs[i].data_ptr(), outs[i].data_ptr(), row_id_map.data_ptr(), None, T, 1, H,
+                  _lib.WX_BF16, stream)
+
+    def copy_cold():
+        i = nxt()
+        outs[i].copy_(xs[i])
+
+    out = {}
+    for name, fn in (("permute_rowmajor", permute_cold), ("unpermute", unpermute_cold), ("device_copy", copy_cold)):
+        t, _ = event_ms(fn, iters, warm=sets, batch=sets)
+        out[f"{name}_GBps"] = round(row_bytes / t / 1e6, 1)
+    out["note"] = f"{sets} buffer sets of {2 * T * H * 2 / 1e6:.0f} MB each, used round-robin; bytes counted as for the warm figures"
+    return out
+
+
+def config4_measurement(dev, weights):
+    """BASELINE config 4, the skewed / empty-group regime, through the layer entry point (partition, tiled permute,
+    both FFN launches, unpermute) with no retuning between shapes: (i) a denoise step of 2048 action tokens with the
+    VL group empty, (ii) a prefill of 4096 VL tokens plus n action tokens.  Activations N(0, 1); the weights are
+    the benchmark's N(0, 0.02) tensors (timing does not depend on the weight scale)."""
+    import torch
+    from wallx_mi355 import moe
+
+    H = weights[0][0].shape[1]
+    I0, I1 = weights[0][0].shape[0], weights[1][0].shape[0]
+    g = torch.Generator(device=dev).manual_seed(4)
+    out = {}
+    cases = [("denoise_2048_action", 0, 2048)] + [(f"prefill_4096_vl_plus_{n}_action", 4096, n) for n in (0, 1, 8, 32, 64)]
+    for name, n_vl, n_act in cases:
+        T = n_vl + n_act
+        x = torch.randn(T, H, device=dev, generator=g).to(torch.bfloat16)
+        types = torch.cat([torch.zeros(n_vl, dtype=torch.bool), torch.ones(n_act, dtype=torch.bool)]).to(dev)
+        t, _ = event_ms(lambda: moe.moe_layer_forward(x, types, weights), 20, warm=5)
+        flops = 6.0 * H * (n_vl * I0 + n_act * I1)
+        out[name] = {"us": round(t * 1e3, 1), "tflops": round(flops / t / 1e9, 1)}
     return out
 
 

@@ -1,11 +1,21 @@
 // 3D multimodal RoPE apply (forward and adjoint) for gfx950.
 //
-// HBM-bound elementwise kernel.  A thread owns one rotation group of a token: the 8 channels
-// [8j, 8j+8) of the low half together with their partners in the high half, so both operands of every
-// rotation are in registers and each access is a full 16-byte lane (32 bytes for fp32).  The thread
-// loads the selected cos/sin values for its channels once and applies them to three heads of q / k; all
-// loads of the three heads are in flight before the first result is needed.  q/k/outputs are addressed
-// through (batch, head, seq) strides so the projection's [B, S, H, D] memory is read in place.
+// HBM-bound elementwise kernels.
+//
+// mrope_rows_kernel (the one the model shapes use): a thread owns one 16-byte chunk position of the head
+// (channels [8c, 8c+8) for 2-byte types) of one token and walks over ALL heads of q and k.  It loads the selected
+// cos/sin values of its channels once, gets the partner chunk of every rotation (the same channels in the other
+// half of the head) from the lane that owns it through a lane exchange, and writes its own 16 bytes.  The lanes
+// of a token cover a whole head, so a wavefront reads whole 256-byte heads and writes runs of consecutive tokens
+// (1 KiB for head_dim 128) of the head-major output; the loads of several heads are in flight before the first
+// result is needed.
+//
+// mrope_kernel (general fallback: head sizes whose chunk count is not a power of two, sections that cut through
+// a chunk): a thread owns the 8 channels [8j, 8j+8) of the low half together with their partners in the high
+// half and applies them to a few heads.
+//
+// q/k/outputs are addressed through (batch, head, seq) strides so the projection's [B, S, H, D] memory is read
+// in place.
 #include "common.h"
 
 namespace wx {
@@ -148,6 +158,110 @@ __global__ __launch_bounds__(256) void mrope_kernel(
   }
 }
 
+// Heads whose loads are issued together in mrope_rows_kernel.
+#ifndef WX_MROPE_BATCH
+#define WX_MROPE_BATCH 6
+#endif
+constexpr int kRowsHeadBatch = WX_MROPE_BATCH;
+
+// The chunk held by the lane `half_lanes` away (lane ^ half_lanes): the other half of the same head.
+template <int L>
+__device__ __forceinline__ u32x4 partner_chunk(const u32x4& v, int half_lanes) {
+  u32x4 r;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    if constexpr (L == 16) {
+      // rotate by 8 inside each row of 16 lanes
+      r[i] = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v[i]), 0x128, 0xF, 0xF, true));
+    } else {
+      r[i] = static_cast<uint32_t>(__shfl_xor(static_cast<int>(v[i]), half_lanes));
+    }
+  }
+  return r;
+}
+
+// L = lanes per head when known at compile time (16), 0 = any power of two up to 64 (runtime).
+template <int DT, bool BWD, int L>
+__global__ __launch_bounds__(256) void mrope_rows_kernel(
+    const void* __restrict__ q, const void* __restrict__ k, const void* __restrict__ cos_t,
+    const void* __restrict__ sin_t, void* __restrict__ q_out, void* __restrict__ k_out, int64_t n_tokens,
+    int64_t seq, int n_q_heads, int n_kv_heads, int head_dim, Strides sq, Strides sk, Strides sqo, Strides sko,
+    AxisTable ax) {
+  constexpr int kEpc = 16 / Elem<DT>::kBytes;  // elements per 16-byte chunk
+  const int lanes = L ? L : head_dim / kEpc;   // lanes per (token, head)
+  const int64_t gid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const int chunk = static_cast<int>(gid % lanes);
+  int64_t token = gid / lanes;
+  const bool live = token < n_tokens;
+  if (!live) token = n_tokens - 1;  // lanes past the end keep taking part in the lane exchanges, and store nothing
+  const int64_t b = token / seq, s = token - b * seq;
+  const int d0 = chunk * kEpc;
+  const bool hi = chunk >= lanes / 2;
+  const int n_heads = n_q_heads + n_kv_heads;
+  const u32x4* qc = reinterpret_cast<const u32x4*>(static_cast<const char*>(q) + (b * sq.b + s * sq.s + d0) * Elem<DT>::kBytes);
+  const u32x4* kc = reinterpret_cast<const u32x4*>(static_cast<const char*>(k) + (b * sk.b + s * sk.s + d0) * Elem<DT>::kBytes);
+  u32x4* qo = reinterpret_cast<u32x4*>(static_cast<char*>(q_out) + (b * sqo.b + s * sqo.s + d0) * Elem<DT>::kBytes);
+  u32x4* ko = reinterpret_cast<u32x4*>(static_cast<char*>(k_out) + (b * sko.b + s * sko.s + d0) * Elem<DT>::kBytes);
+  const int64_t hq_in = sq.h * Elem<DT>::kBytes, hk_in = sk.h * Elem<DT>::kBytes;
+  const int64_t hq_out = sqo.h * Elem<DT>::kBytes, hk_out = sko.h * Elem<DT>::kBytes;
+
+  // selected cos / sin of my channels (regular loads: other workgroups never need them, later heads do not either,
+  // but the three position planes are small next to q)
+  const int64_t tab_off = (ax.axis[d0] * (n_tokens * head_dim) + token * head_dim + d0) * Elem<DT>::kBytes;
+  const u32x4 c_raw = *reinterpret_cast<const u32x4*>(static_cast<const char*>(cos_t) + tab_off);
+  u32x4 s_raw = *reinterpret_cast<const u32x4*>(static_cast<const char*>(sin_t) + tab_off);
+  if constexpr (BWD) s_raw = partner_chunk<L>(s_raw, lanes / 2);  // the adjoint multiplies by the partner's sin
+  float c[kEpc], sn[kEpc];
+  unpack16<DT>(c_raw, c);
+  unpack16<DT>(s_raw, sn);
+  // forward: out = x*cos + rotate_half(x)*sin with rotate_half(x) = (-x_hi, x_lo): the low half takes -partner
+  // adjoint: out = g*cos + rotate_half^T(g*sin) with rotate_half^T(y) = (y_hi, -y_lo): the high half takes -partner
+  const float sign = (hi != BWD) ? 1.0f : -1.0f;
+#pragma unroll
+  for (int e = 0; e < kEpc; ++e) sn[e] *= sign;  // exact
+
+  for (int h0 = 0; h0 < n_heads; h0 += kRowsHeadBatch) {
+    u32x4 raw[kRowsHeadBatch];
+#pragma unroll
+    for (int u = 0; u < kRowsHeadBatch; ++u) {
+      const int h = h0 + u;
+      if (h < n_heads) {
+        const u32x4* src = h < n_q_heads
+            ? reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(qc) + h * hq_in)
+            : reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(kc) + (h - n_q_heads) * hk_in);
+        raw[u] = __builtin_nontemporal_load(src);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < kRowsHeadBatch; ++u) {
+      const int h = h0 + u;
+      if (h < n_heads) {  // uniform over the workgroup
+        const u32x4 other = partner_chunk<L>(raw[u], lanes / 2);
+        float x[kEpc], xp[kEpc], o[kEpc];
+        unpack16<DT>(raw[u], x);
+        unpack16<DT>(other, xp);
+#pragma unroll
+        for (int e = 0; e < kEpc; ++e) {
+          if constexpr (!BWD) {
+            // eager evaluation order of (x * cos) + (rotate_half(x) * sin): every product and the sum are rounded
+            // to the storage type (the sum by the final pack)
+            const float p1 = Elem<DT>::round(__fmul_rn(x[e], c[e]));
+            const float p2 = Elem<DT>::round(__fmul_rn(xp[e], sn[e]));
+            o[e] = __fadd_rn(p1, p2);
+          } else {
+            o[e] = __fadd_rn(__fmul_rn(x[e], c[e]), __fmul_rn(xp[e], sn[e]));
+          }
+        }
+        if (live) {
+          u32x4* dst = h < n_q_heads ? reinterpret_cast<u32x4*>(reinterpret_cast<char*>(qo) + h * hq_out)
+                                     : reinterpret_cast<u32x4*>(reinterpret_cast<char*>(ko) + (h - n_q_heads) * hk_out);
+          __builtin_nontemporal_store(pack16<DT>(o), dst);
+        }
+      }
+    }
+  }
+}
+
 int build_axis_table(const int sec[3], int head_dim, int layout, AxisTable& ax) {
   int d = 0;
   auto put = [&](int axis, int n) {
@@ -195,13 +309,35 @@ int launch(const void* q, const void* k, const void* cos_t, const void* sin_t, v
   AxisTable ax{};
   if (int rc = build_axis_table(sec, head_dim, layout, ax)) return rc;
   const Strides a{sq[0], sq[1], sq[2]}, b{sk[0], sk[1], sk[2]}, c{sqo[0], sqo[1], sqo[2]}, d{sko[0], sko[1], sko[2]};
+  hipStream_t s = as_stream(stream);
+  // Row form: 16-byte chunks per head must be a power of two that divides the workgroup, and no section boundary
+  // may cut through a chunk.
+  const int epc = dtype == WX_F32 ? 4 : 8;
+  const int lanes = head_dim / epc;
+  bool rows_ok = lanes >= 2 && lanes <= 64 && (lanes & (lanes - 1)) == 0;
+  for (int cidx = 0; cidx < head_dim / 8 && rows_ok; ++cidx) rows_ok = ax.uniform[cidx] != 0;
+  if (rows_ok) {
+    const int64_t threads = n_tokens * lanes;
+    if ((threads + 255) / 256 > 0x7fffffffll) return fail(WX_ERR_UNSUPPORTED, "%s: too many tokens", who);
+    const dim3 grid(static_cast<unsigned>((threads + 255) / 256)), block(256);
+#define WX_LAUNCH_ROWS(DT, L)                                                                                       \
+  hipLaunchKernelGGL((mrope_rows_kernel<DT, BWD, L>), grid, block, 0, s, q, k, cos_t, sin_t, q_out, k_out, n_tokens, \
+                     seq, n_q, n_kv, head_dim, a, b, c, d, ax)
+    switch (dtype) {
+      case WX_F32: WX_LAUNCH_ROWS(WX_F32, 0); break;
+      case WX_F16: if (lanes == 16) WX_LAUNCH_ROWS(WX_F16, 16); else WX_LAUNCH_ROWS(WX_F16, 0); break;
+      case WX_BF16: if (lanes == 16) WX_LAUNCH_ROWS(WX_BF16, 16); else WX_LAUNCH_ROWS(WX_BF16, 0); break;
+      default: return fail(WX_ERR_UNSUPPORTED, "%s: dtype %d", who, dtype);
+    }
+#undef WX_LAUNCH_ROWS
+    return check_launch(who);
+  }
   // grid.x walks (token, rotation group); grid.y walks groups of kHeadsPerThread heads
   const int groups = head_dim / 16;
   const int head_groups = (n_q + n_kv + kHeadsPerThread - 1) / kHeadsPerThread;
   const int64_t threads = n_tokens * groups;
   if ((threads + 255) / 256 > 0x7fffffffll) return fail(WX_ERR_UNSUPPORTED, "%s: too many tokens", who);
   const dim3 grid(static_cast<unsigned>((threads + 255) / 256), static_cast<unsigned>(head_groups)), block(256);
-  hipStream_t s = as_stream(stream);
 #define WX_LAUNCH(DT)                                                                                             \
   hipLaunchKernelGGL((mrope_kernel<DT, BWD>), grid, block, 0, s, q, k, cos_t, sin_t, q_out, k_out, n_tokens, seq, \
                      n_q, n_kv, head_dim, a, b, c, d, ax)
