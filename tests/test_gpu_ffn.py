@@ -34,6 +34,7 @@ GEMM_SHAPES = [
     (0, 256, 64, 77, 520, 72),           # empty VL group, K not a multiple of 64
     (129, 136, 200, 0, 64, 64),          # empty action group, K tail
     (0, 64, 64, 0, 64, 64),              # nothing to do
+    (3000, 3080, 96, 200, 264, 160),     # enough 256 x 256 tiles to take the large-tile kernel, ragged everywhere
 ]
 
 
@@ -207,6 +208,11 @@ def test_config4_skewed_and_empty_groups(dev):
     assert r.expert_offsets.cpu().tolist() == [0, 0, 2048]
     rows = torch.arange(0, 2048, 37)
     _close(y[rows.to(dev)], oracle.swiglu_ffn_ref(x[rows], *ws[1].as_tuple()), what="denoise step")
+    # the same step next to a wide VL expert: the host cannot tell which tile shape fits (the row split is on the
+    # device), so both are launched and the device picks
+    ws_wide = _moe_weights(2048, (4096, 1024), g, 0.02)
+    y2, _ = moe.moe_layer_forward(x.to(dev), types.to(dev), [w.to(dev).as_tuple() for w in ws_wide])
+    _close(y2[rows.to(dev)], oracle.swiglu_ffn_ref(x[rows], *ws_wide[1].as_tuple()), what="denoise step, wide VL expert")
     # (ii) prefill: 4096 VL tokens + n action tokens, alternating with (i) without re-tuning
     for n_act in (0, 1, 8, 64):
         x = _bf((4096 + n_act, 2048), g)

@@ -7,13 +7,13 @@
 // (thousands of VL rows next to tens of action rows, or an empty group) is just a longer or shorter tile list.
 //
 // Workgroup tile 256 x 256, K step 32, four wavefronts (one per SIMD) as 2 x 2, wave tile 128 x 128 = 4 x 4 MFMA
-// 32x32x16 accumulator blocks (256 accumulator registers per lane), one workgroup per CU.  (WX_GEMM_BN=128 builds
-// a 256 x 128 tile with two resident workgroups per CU, three ring slots and 128 accumulator registers; it
-// measures a few percent slower on both FFN GEMMs and is kept as a build option.)  Operands are K-contiguous, so
-// both MFMA fragments are 16-byte LDS reads.  Global -> LDS uses buffer loads that write LDS directly (no
-// register staging) into a ring of four K-step slots per operand; the load stream runs four K steps ahead of
-// the MFMAs and crosses tile boundaries, with one workgroup barrier per K step.  LDS rows are 64 bytes; chunk c
-// of row r sits in slot c ^ ((r >> 2) & 3), which makes the 16-byte fragment reads bank-conflict free.
+// 32x32x16 accumulator blocks (256 accumulator registers per lane), one workgroup per CU.  Problems whose 256 x 256
+// tiles would leave most CUs idle (a denoise step of a few thousand action tokens) run the same kernel with a
+// 128 x 128 tile, two workgroups per CU.  Operands are K-contiguous, so both MFMA fragments are 16-byte LDS reads.
+// Global -> LDS uses buffer loads that write LDS directly (no register staging) into a ring of four K-step slots
+// per operand; the load stream runs four K steps ahead of the MFMAs and crosses tile boundaries, with one
+// workgroup barrier per K step.  LDS rows are 64 bytes; chunk c of row r sits in slot c ^ ((r >> 2) & 3), which
+// makes the 16-byte fragment reads bank-conflict free.
 //
 // Three operand layouts:
 //   generic  (wx_dual_gemm)            A, B, C row-major; loads touch 16 rows x 64 bytes per instruction.
@@ -35,33 +35,35 @@ namespace {
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
-#ifndef WX_GEMM_BN
-#define WX_GEMM_BN 256
-#endif
-#if WX_GEMM_BN == 256
-#define WX_GEMM_STAGES 4
-#else
-#define WX_GEMM_STAGES 3
-#endif
-constexpr int BM = 256, BN = WX_GEMM_BN, BK = 32;
-static_assert(BN == 128 || BN == 256, "tile width");
-constexpr int kWgPerCu = BN == 256 ? 1 : 2;    // resident workgroups per CU (LDS and registers are sized for this)
+constexpr int BK = 32;
 constexpr int kWavesM = 2, kWavesN = 2;        // wavefront grid over the tile; one wavefront per SIMD
 constexpr int kWaves = kWavesM * kWavesN;
 constexpr int kThreads = kWaves * 64;
-constexpr int FM = BM / kWavesM / 32;          // 32x32 accumulator blocks per wave along M (4)
-constexpr int FN = BN / kWavesN / 32;          // ... and along N (4, or 2 for the 128-wide tile)
-constexpr int kLoadRowsA = BM / kWaves;        // LDS rows of A one wave loads per K step (64)
-constexpr int kLoadRowsB = BN / kWaves;        // ... and of B (64 / 32)
-constexpr int kLoadsA = kLoadRowsA / 16;       // 16-row load instructions per wave per K step: A (4)
-constexpr int kLoadsB = kLoadRowsB / 16;       // ... and B (4 / 2)
-constexpr int kLoadsPerStep = kLoadsA + kLoadsB;
-constexpr int kStages = WX_GEMM_STAGES;        // ring slots per operand
+constexpr int kStages = 4;                     // ring slots per operand
 constexpr int kRowBytes = BK * 2;              // 64 bytes of K per LDS row
-constexpr int kSlotBytesA = BM * kRowBytes;    // 16 KiB of A per K step
-constexpr int kSlotBytesB = BN * kRowBytes;    // 16 / 8 KiB of B per K step
-constexpr int kStageBytes = BN == 256 ? 8192 : 2048;  // per-wave staging for the epilogue
-static_assert(kStages * (kSlotBytesA + kSlotBytesB) + kWaves * kStageBytes <= 160 * 1024 / kWgPerCu, "LDS budget");
+
+// Workgroup tile shapes.  Everything else (wave tile, loads per step, LDS footprint, resident workgroups per CU)
+// follows from the two numbers.
+template <int BM_, int BN_>
+struct TileShape {
+  static constexpr int BM = BM_, BN = BN_;
+  static constexpr int FM = BM / kWavesM / 32;        // 32x32 accumulator blocks per wave along M
+  static constexpr int FN = BN / kWavesN / 32;        // ... and along N
+  static constexpr int kLoadRowsA = BM / kWaves;      // LDS rows of A one wave loads per K step
+  static constexpr int kLoadRowsB = BN / kWaves;      // ... and of B
+  static constexpr int kLoadsA = kLoadRowsA / 16;     // 16-row load instructions per wave per K step: A
+  static constexpr int kLoadsB = kLoadRowsB / 16;     // ... and B
+  static constexpr int kSlotBytesA = BM * kRowBytes;  // bytes of A per K step
+  static constexpr int kSlotBytesB = BN * kRowBytes;
+  static constexpr int kStageBytes = FN >= 4 ? 8192 : 2048;  // per-wave staging for the epilogue
+  static constexpr int kLdsBytes = kStages * (kSlotBytesA + kSlotBytesB) + kWaves * kStageBytes;
+  static constexpr int kWgPerCu = kLdsBytes <= 80 * 1024 && FM * FN * 16 <= 128 ? 2 : 1;
+  static_assert(kLdsBytes <= 160 * 1024, "LDS budget");
+  static_assert(FM >= 1 && FN >= 2 && FN % 2 == 0 && kLoadsA >= 1 && kLoadsB >= 1 && kLoadsB <= kLoadsA, "tile shape");
+};
+using BigTile = TileShape<256, 256>;    // one workgroup per CU, 256 accumulator registers per lane
+using SmallTile = TileShape<128, 128>;  // two workgroups per CU; for problems with too few big tiles to fill the chip
+
 constexpr int kXcds = 8;
 constexpr int kGroupM = 8;                     // tile rows per patch in the tile order
 
@@ -80,6 +82,11 @@ struct Group {
 struct Params {
   Group g[2];
   const int32_t* offsets;  // device int32[3]: rows of expert e are [offsets[e], offsets[e+1]); null for kGeneric
+  // Tile-shape choice made on the device, for launches where the host cannot tell (the split of the rows between
+  // the experts lives in `offsets`): both tile shapes are launched and each kernel returns at once unless the
+  // number of 256 x 256 tiles is on its side of `gate_tiles`.  0 = always run, 1 = run if at most gate_tiles,
+  // 2 = run if more.
+  int gate, gate_tiles;
 };
 
 #define LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
@@ -140,9 +147,13 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
   return __builtin_bit_cast(uint32_t, v);
 }
 
-template <int MODE>
-__global__ __launch_bounds__(kThreads, kWgPerCu) void dual_gemm_kernel(Params p) {
+template <int MODE, typename TS>
+__global__ __launch_bounds__(kThreads, TS::kWgPerCu) void dual_gemm_kernel(Params p) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stub; the body uses gfx950-only builtins
+  constexpr int BM = TS::BM, BN = TS::BN, FM = TS::FM, FN = TS::FN;
+  constexpr int kLoadRowsA = TS::kLoadRowsA, kLoadRowsB = TS::kLoadRowsB, kLoadsA = TS::kLoadsA, kLoadsB = TS::kLoadsB;
+  constexpr int kLoadsPerStep = kLoadsA + kLoadsB;
+  constexpr int kSlotBytesA = TS::kSlotBytesA, kSlotBytesB = TS::kSlotBytesB, kStageBytes = TS::kStageBytes;
   constexpr bool SWIGLU = MODE == kGateUp;
   constexpr bool TILED_IN = MODE != kGeneric;   // A and B are K-tiled
   constexpr bool TILED_OUT = MODE == kGateUp;   // C is K-tiled
@@ -154,24 +165,13 @@ __global__ __launch_bounds__(kThreads, kWgPerCu) void dual_gemm_kernel(Params p)
   __shared__ __attribute__((aligned(1024))) unsigned char s_b0[kSlotBytesB];
   __shared__ __attribute__((aligned(1024))) unsigned char s_b1[kSlotBytesB];
   __shared__ __attribute__((aligned(1024))) unsigned char s_b2[kSlotBytesB];
-#if WX_GEMM_STAGES == 4
   __shared__ __attribute__((aligned(1024))) unsigned char s_a3[kSlotBytesA];
   __shared__ __attribute__((aligned(1024))) unsigned char s_b3[kSlotBytesB];
-#endif
   __shared__ __attribute__((aligned(1024))) unsigned char s_out[kWaves * kStageBytes];
   // ring slot s of each operand (s is a constant after unrolling)
-  auto slot_a = [&](int s) -> unsigned char* {
-#if WX_GEMM_STAGES == 4
-    if (s == 3) return s_a3;
-#endif
-    return s == 0 ? s_a0 : (s == 1 ? s_a1 : s_a2);
-  };
-  auto slot_b = [&](int s) -> unsigned char* {
-#if WX_GEMM_STAGES == 4
-    if (s == 3) return s_b3;
-#endif
-    return s == 0 ? s_b0 : (s == 1 ? s_b1 : s_b2);
-  };
+  static_assert(kStages == 4, "ring slots are declared one by one");
+  auto slot_a = [&](int s) -> unsigned char* { return s == 0 ? s_a0 : (s == 1 ? s_a1 : (s == 2 ? s_a2 : s_a3)); };
+  auto slot_b = [&](int s) -> unsigned char* { return s == 0 ? s_b0 : (s == 1 ? s_b1 : (s == 2 ? s_b2 : s_b3)); };
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keeps descriptors and LDS bases scalar
@@ -213,6 +213,12 @@ __global__ __launch_bounds__(kThreads, kWgPerCu) void dual_gemm_kernel(Params p)
   tiles_m[1] = (g1.m + BM - 1) / BM;
   tiles_n[1] = (g1.n + kTileN - 1) / kTileN;
   if (g1.m <= 0 || g1.n <= 0) tiles_m[1] = tiles_n[1] = 0;
+  if (p.gate != 0) {
+    constexpr int kBigN = SWIGLU ? BigTile::BN / 2 : BigTile::BN;
+    auto big = [](int m, int n) { return (m <= 0 || n <= 0) ? 0 : ((m + BigTile::BM - 1) / BigTile::BM) * ((n + kBigN - 1) / kBigN); };
+    const bool few = big(g0.m, g0.n) + big(g1.m, g1.n) <= p.gate_tiles;
+    if (few != (p.gate == 1)) return;  // uniform: the other tile shape's launch does this problem
+  }
   const int total = tiles_m[0] * tiles_n[0] + tiles_m[1] * tiles_n[1];  // the host bounds this below 2^31
   const int padded = (total + kXcds - 1) / kXcds * kXcds;
 
@@ -642,15 +648,33 @@ int check_dims(const char* who, int64_t m, int64_t n, int64_t k) {
   // 256 rows of one operand must stay addressable through a 31-bit buffer offset
   if (k * 2 * 256 >= (1ll << 31) || n * 2 * 256 >= (1ll << 31)) return fail(WX_ERR_UNSUPPORTED, "%s: row too long", who);
   // the tile list is indexed with 32-bit integers
-  if (((m + BM - 1) / BM) * ((n + BN / 2 - 1) / (BN / 2)) >= (1ll << 30)) return fail(WX_ERR_UNSUPPORTED, "%s: too many tiles", who);
+  if (((m + SmallTile::BM - 1) / SmallTile::BM) * ((n + SmallTile::BN / 2 - 1) / (SmallTile::BN / 2)) >= (1ll << 30))
+    return fail(WX_ERR_UNSUPPORTED, "%s: too many tiles", who);
   return WX_OK;
 }
 
+// The problem has between `tiles_lo` and `tiles_hi` 256 x 256 tiles (equal when the host knows the row counts).
+// When they would occupy at most half of the CUs, the 128 x 128 tile gives four times as many workgroups to spread
+// over the chip.  If the bounds fall on both sides of that threshold the choice is made on the device: both
+// shapes are launched and the one on the wrong side returns immediately.
 template <int MODE>
-int launch_mfma(const Params& p, hipStream_t s, const char* who) {
-  hipLaunchKernelGGL(dual_gemm_kernel<MODE>, dim3(device_cu_count() * kWgPerCu), dim3(kThreads), 0, s, p);
+int launch_mfma(Params p, int64_t tiles_lo, int64_t tiles_hi, hipStream_t s, const char* who) {
+  const int cus = device_cu_count();
+  const int threshold = cus / 2;
+  const bool small = tiles_lo <= threshold, big = tiles_hi > threshold;
+  p.gate_tiles = threshold;
+  if (small) {
+    p.gate = big ? 1 : 0;
+    hipLaunchKernelGGL((dual_gemm_kernel<MODE, SmallTile>), dim3(cus * SmallTile::kWgPerCu), dim3(kThreads), 0, s, p);
+  }
+  if (big) {
+    p.gate = small ? 2 : 0;
+    hipLaunchKernelGGL((dual_gemm_kernel<MODE, BigTile>), dim3(cus * BigTile::kWgPerCu), dim3(kThreads), 0, s, p);
+  }
   return check_launch(who);
 }
+
+int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
 }  // namespace
 }  // namespace wx
@@ -687,7 +711,10 @@ extern "C" int wx_dual_gemm(const void* in0, const void* in1, const void* w0, co
   p.offsets = nullptr;
   if ((m0 == 0 || n0 == 0) && (m1 == 0 || n1 == 0)) return WX_OK;
   hipStream_t s = as_stream(stream);
-  if (!trans_a && trans_b) return launch_mfma<kGeneric>(p, s, "dual_gemm_kernel<generic>");
+  if (!trans_a && trans_b) {
+    const int64_t tiles = ceil_div(m0, BigTile::BM) * ceil_div(n0, BigTile::BN) + ceil_div(m1, BigTile::BM) * ceil_div(n1, BigTile::BN);
+    return launch_mfma<kGeneric>(p, tiles, tiles, s, "dual_gemm_kernel<generic>");
+  }
   hipLaunchKernelGGL(dual_gemm_reference_layout_kernel, dim3(device_cu_count() * 4), dim3(256), 0, s, p, trans_a, trans_b);
   return check_launch("dual_gemm_reference_layout_kernel");
 }
@@ -759,7 +786,11 @@ int launch_gate_up(const FfnArgs& a, hipStream_t s) {
     g.a_row0 = 0;
   }
   p.offsets = a.offsets;
-  return launch_mfma<kGateUp>(p, s, "dual_gemm_kernel<gate_up>");
+  // the split of the rows between the experts is only known on the device: bound the tile count from the total
+  const int64_t t0 = ceil_div(a.inter[0], BigTile::BN / 2), t1 = ceil_div(a.inter[1], BigTile::BN / 2);
+  const int64_t row_tiles = ceil_div(a.rows, BigTile::BM);
+  return launch_mfma<kGateUp>(p, row_tiles * (t0 < t1 ? t0 : t1), (row_tiles + 1) * (t0 > t1 ? t0 : t1), s,
+                              "dual_gemm_kernel<gate_up>");
 }
 
 // out_e = hmid_e @ down_e^T, row-major, expert e's rows start at offsets[e]
@@ -778,7 +809,8 @@ int launch_down(const FfnArgs& a, hipStream_t s) {
     g.a_row0 = 0;
   }
   p.offsets = a.offsets;
-  return launch_mfma<kDown>(p, s, "dual_gemm_kernel<down>");
+  const int64_t row_tiles = ceil_div(a.rows, BigTile::BM), col_tiles = ceil_div(a.hidden, BigTile::BN);
+  return launch_mfma<kDown>(p, row_tiles * col_tiles, (row_tiles + 1) * col_tiles, s, "dual_gemm_kernel<down>");
 }
 
 }  // namespace
