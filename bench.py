@@ -189,6 +189,7 @@ def main():
     if not args.ops_only:
         extra["cold_hbm"] = cold_measurements(dev, x, row_id_map, T, H, row_bytes, iters)
         extra["config4"] = config4_measurement(dev, weights)
+        extra["backward_gemms"] = backward_measurement(dev, x, weights, m0)
         extra["ceilings"] = ceiling_measurements(dev, x, weights, m0)
     if not args.ops_only and not args.no_prefill:
         del x_tiled, hmid, x_sorted, y_sorted, y
@@ -347,6 +348,30 @@ def config4_measurement(dev, weights):
         flops = 6.0 * H * (n_vl * I0 + n_act * I1)
         out[name] = {"us": round(t * 1e3, 1), "tflops": round(flops / t / 1e9, 1)}
     return out
+
+
+def backward_measurement(dev, x, weights, m0):
+    """The two backward GEMMs of `asym_dual_gmm` (ops.py:78-144) at the gate projection's config 3 shapes:
+    dX = dY @ W (both experts) and dW = dY^T @ X, each as transposed copies + the MFMA kernel; the times include
+    the transposes."""
+    import torch
+    from wallx_mi355 import native
+
+    H = x.shape[1]
+    (g0, _, _), (g1, _, _) = weights
+    I0, I1 = g0.shape[0], g1.shape[0]
+    m1 = x.shape[0] - m0
+    gen = torch.Generator(device=dev).manual_seed(2)
+    dy0 = torch.randn(m0, I0, device=dev, generator=gen).to(torch.bfloat16)
+    dy1 = torch.randn(m1, I1, device=dev, generator=gen).to(torch.bfloat16)
+    x0, x1 = x[:m0].contiguous(), x[m0:].contiguous()
+    dx0, dx1 = torch.empty_like(x0), torch.empty_like(x1)
+    dw0, dw1 = torch.empty_like(g0), torch.empty_like(g1)
+    flops = 2.0 * H * (m0 * I0 + m1 * I1)
+    t_dx, _ = event_ms(lambda: native.asym_dual_gmm(dy0, dy1, g0, g1, dx0, dx1, False, False), 5, warm=2)
+    t_dw, _ = event_ms(lambda: native.asym_dual_gmm(dy0, dy1, x0, x1, dw0, dw1, True, False), 5, warm=2)
+    return {"dx_ms": round(t_dx, 3), "dx_tflops": round(flops / t_dx / 1e9, 1),
+            "dw_ms": round(t_dw, 3), "dw_tflops": round(flops / t_dw / 1e9, 1)}
 
 
 def ceiling_measurements(dev, x, weights, m0):

@@ -203,6 +203,13 @@ int wx_window_index(const void* grid_thw, int grid_type, int64_t n_grid, int spa
                     int64_t total_windows, int32_t* window_index, int32_t* cu_window_seqlens,
                     wx_stream_t stream);
 
+/* dst [cols, rows] = transpose of src [rows, cols], both row-major and contiguous, 2-byte elements (bf16 / fp16),
+ * rows and cols multiples of 8.  Feeds the backward of asym_dual_gmm (ops.py:78-144: dX uses (F, not trans_b), dW
+ * uses (T, F)): the MFMA kernel reads both operands with the contraction index contiguous, so the Python layer
+ * hands it transposed copies; the reference gets the same effect from CUTLASS layout tags
+ * (csrc/dual_asym_grouped_gemm.cu:286-305). */
+int wx_transpose_2d(const void* src, void* dst, int64_t rows, int64_t cols, int elem_bytes, wx_stream_t stream);
+
 /* ---- measurement probe (no counterpart in the reference; used by bench.py) --------------------------------
  * Runs bf16 32x32x16 MFMA instructions back to back on every CU, operands taken from `operands`
  * (wx_probe_mfma_operand_bytes() bytes of bf16 values, device memory, 16-byte aligned) and held in registers:
