@@ -203,6 +203,18 @@ int wx_window_index(const void* grid_thw, int grid_type, int64_t n_grid, int spa
                     int64_t total_windows, int32_t* window_index, int32_t* cu_window_seqlens,
                     wx_stream_t stream);
 
+/* Caller fusions around the FFN (act.py:256-265: residual; post_attention_layernorm; moe; residual add), bf16:
+ * wx_rmsnorm_permute_rows_tiled = RMSNorm (the module at act.py:190-193: fp32 variance, x * rsqrt(var + eps) rounded
+ * to bf16, times the bf16 weight) followed by wx_permute_rows_tiled in its gather form, in one pass;
+ * sorted_row_id is the inverse map from wx_partition_build.  num_cols: a multiple of 128, at most 4096.
+ * wx_unpermute_rows_add = wx_unpermute_rows at topK 1 followed by `residual + .` (one rounding), in one pass.
+ * The reference runs these as separate PyTorch ops; listed as the next step after the ops themselves. */
+int wx_rmsnorm_permute_rows_tiled(const void* x, const void* weight, float eps, void* out_tiled,
+                                  const int32_t* sorted_row_id, const int32_t* expert_offsets,
+                                  int64_t num_tokens, int64_t num_cols, wx_stream_t stream);
+int wx_unpermute_rows_add(const void* y, const void* residual, void* out, const int32_t* row_id_map,
+                          int64_t num_tokens, int64_t num_cols, wx_stream_t stream);
+
 /* dst [cols, rows] = transpose of src [rows, cols], both row-major and contiguous, 2-byte elements (bf16 / fp16),
  * rows and cols multiples of 8.  Feeds the backward of asym_dual_gmm (ops.py:78-144: dX uses (F, not trans_b), dW
  * uses (T, F)): the MFMA kernel reads both operands with the contraction index contiguous, so the Python layer

@@ -32,6 +32,9 @@ How each function is pinned (tests/test_oracle_*.py):
                                    brute force over small grids
   window_index_ref                 permutation / window-size invariants, brute
                                    force enumeration of windows on small grids
+  rms_norm_ref                     torch.nn.functional.rms_norm in fp32, the
+                                   closed form for constant rows, transformers'
+                                   Qwen2RMSNorm where it is importable
 
   unpermute_ref with topK > 1 and probs, unpermute_bwd_ref, mrope_apply_ref in
   its "csrc" channel layout and rope_index_ref's "csrc" padding mode follow
@@ -56,3 +59,4 @@ from .mrope import (  # noqa: F401
 from .rope_index import rope_index_ref  # noqa: F401
 from .rot_pos import rot_pos_ids_ref, rot_pos_emb_ref  # noqa: F401
 from .window_index import window_index_ref, window_index_dedup_ref  # noqa: F401
+from .norm import rms_norm_ref  # noqa: F401

@@ -1,0 +1,87 @@
+"""RMSNorm + tiled permute and unpermute + residual add (the caller fusions around the FFN) against the oracle."""
+
+import pytest
+import torch
+
+import oracle
+from wallx_mi355 import moe, native
+
+pytestmark = pytest.mark.gpu
+
+
+def _bf(shape, g, std=1.0):
+    return (torch.randn(shape, generator=g) * std).to(torch.bfloat16)
+
+
+def _untile(tiled, rows_pad, H):
+    """K-tiled [rows_pad, H] (16 x 32 blocks, [column block][row block], swizzled 16-byte chunks) -> row-major."""
+    rb, kb = rows_pad // 16, H // 32
+    t = tiled[: rows_pad * H].view(kb, rb, 16, 4, 8)
+    out = torch.empty(rows_pad, H, dtype=tiled.dtype)
+    for r in range(16):
+        for c in range(4):
+            slot = c ^ ((r >> 2) & 3)
+            out.view(rb, 16, kb, 4, 8)[:, r, :, c, :] = t[:, :, r, slot, :].transpose(0, 1)
+    return out
+
+
+@pytest.mark.parametrize("T,H,n_act", [(300, 256, 37), (912, 2048, 32), (64, 128, 0), (50, 4096, 50), (1000, 1536, 999)])
+def test_rmsnorm_permute_tiled(dev, T, H, n_act):
+    g = torch.Generator().manual_seed(T + H)
+    x = _bf((T, H), g, 3.0)
+    w = (1.0 + 0.1 * torch.randn(H, generator=g)).to(torch.bfloat16)
+    types = torch.zeros(T, dtype=torch.bool)
+    types[torch.randperm(T, generator=g)[:n_act]] = True
+    rmap, off, inv, _ = native.partition(types.to(dev), 2, 0, None, want_sorted=True)
+    fused = native.rmsnorm_permute_rows_tiled(x.to(dev), w.to(dev), 1e-6, off, inv)
+    # the same layout from the unfused pair, fed with the oracle's norm: equal up to one bf16 step where the
+    # fp32 sum of squares (accumulated in a different order) moves a value across a rounding boundary
+    normed = oracle.rms_norm_ref(x, w, 1e-6)
+    plain = native.permute_rows_tiled(normed.to(dev), rmap, off, None, inv)
+    rows_pad = native.padded_sorted_rows(T)
+    a = _untile(fused.cpu(), rows_pad, H).float()
+    b = _untile(plain.cpu(), rows_pad, H).float()
+    o = off.cpu().tolist()
+    pad0 = (o[1] + 255) // 256 * 256
+    live = torch.zeros(rows_pad, dtype=torch.bool)
+    live[: o[1]] = True
+    live[pad0: pad0 + (o[2] - o[1])] = True
+    a, b = a[live], b[live]
+    assert a.shape[0] == T
+    tol = 2.0 ** -7 * b.abs() + 1e-6  # one bf16 step
+    bad = (a - b).abs() > tol
+    assert not bad.any(), f"{int(bad.sum())} of {bad.numel()} differ by more than a bf16 step"
+    assert float((a != b).float().mean()) < 0.02  # and almost all values are identical
+
+
+@pytest.mark.parametrize("T,H", [(300, 256), (912, 2048), (7, 8), (33, 1000)])
+def test_unpermute_add(dev, T, H):
+    g = torch.Generator().manual_seed(T * H)
+    y, resid = _bf((T, H), g), _bf((T, H), g)
+    types = torch.rand(T, generator=g) < 0.2
+    _, rmap_ref, _ = oracle.permute_ref(y, types)
+    rmap, _, _, _ = native.partition(types.to(dev), 2, 0, None, want_sorted=False)
+    got = native.unpermute_add(y.to(dev), resid.to(dev), rmap)
+    ref = resid + oracle.unpermute_ref(y, rmap_ref)  # eager bf16 add: one rounding
+    assert torch.equal(got.cpu(), ref)
+
+
+def test_moe_block_with_both_fusions(dev):
+    """h + block(RMSNorm(h)) through the module's fused path against the same module fed by separate PyTorch ops."""
+    from types import SimpleNamespace
+
+    g = torch.Generator().manual_seed(11)
+    cfg = SimpleNamespace(experts=[dict(hidden_size=256, intermediate_size=512, hidden_act="silu"),
+                                   dict(hidden_size=256, intermediate_size=128, hidden_act="silu")])
+    block = moe.SparseMoeBlock(cfg, 2).to(dev).to(torch.bfloat16)
+    with torch.no_grad():
+        for prm in block.parameters():
+            prm.copy_((torch.randn(prm.shape, generator=g) * 0.05).to(torch.bfloat16))
+    h = _bf((2, 150, 256), g, 2.0).to(dev)
+    w = (1.0 + 0.1 * torch.randn(256, generator=g)).to(torch.bfloat16).to(dev)
+    types = (torch.rand(2, 150, generator=g) < 0.1).to(dev)
+    with torch.no_grad():
+        fused = block(h, types, pre_norm=(w, 1e-6), residual=True)
+        plain = h + block(oracle.rms_norm_ref(h.cpu(), w.cpu(), 1e-6).to(dev), types)
+    err = (fused.float() - plain.float()).abs()
+    assert not (err > 2e-2 + 1e-2 * plain.float().abs()).any(), float(err.max())

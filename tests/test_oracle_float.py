@@ -189,3 +189,35 @@ def test_mrope_backward_is_the_adjoint():
         bq, bk = oracle.mrope_apply_bwd_ref(gq, gk, cos, sin, list(wl.MROPE_SECTION), layout)
         assert torch.allclose(bq, qq.grad.to(bq.dtype), atol=1e-5)
         assert torch.allclose(bk, kk.grad.to(bk.dtype), atol=1e-5)
+
+
+# ----------------------------------------------------------------------------- RMSNorm (caller fusion)
+def test_rms_norm_against_library_routine_and_closed_form():
+    g = torch.Generator().manual_seed(8)
+    x = torch.randn(5, 33, 64, generator=g)
+    w = torch.randn(64, generator=g)
+    ref = torch.nn.functional.rms_norm(x, (64,), w, 1e-6)
+    assert torch.allclose(oracle.rms_norm_ref(x, w, 1e-6), ref, rtol=1e-6, atol=1e-7)
+    # a constant row c normalises to sign(c) (up to eps), so the output is sign(c) * weight
+    c = torch.full((3, 64), -2.5)
+    assert torch.allclose(oracle.rms_norm_ref(c, w, 0.0), -w.expand(3, 64), rtol=1e-6, atol=1e-7)
+    # scaling the input leaves the output unchanged when eps = 0
+    assert torch.allclose(oracle.rms_norm_ref(7.0 * x, w, 0.0), oracle.rms_norm_ref(x, w, 0.0), rtol=1e-5, atol=1e-6)
+    # a dropped eps or a sum in place of the mean would fail this: one-hot row of magnitude a -> a / sqrt(a^2/n + eps)
+    e = torch.zeros(1, 64); e[0, 3] = 0.01
+    want = 0.01 / (0.01 ** 2 / 64 + 1e-3) ** 0.5
+    assert abs(float(oracle.rms_norm_ref(e, torch.ones(64), 1e-3)[0, 3]) - want) < 1e-6
+
+
+def test_rms_norm_against_transformers_module():
+    try:
+        from transformers.models.qwen2.modeling_qwen2 import Qwen2RMSNorm
+    except Exception:
+        pytest.skip("transformers' Qwen2RMSNorm is not importable")
+    g = torch.Generator().manual_seed(9)
+    x = torch.randn(4, 17, 128, generator=g).to(torch.bfloat16)
+    m = Qwen2RMSNorm(128, eps=1e-6).to(torch.bfloat16)
+    with torch.no_grad():
+        m.weight.copy_(torch.randn(128, generator=g).to(torch.bfloat16))
+        got = m(x)
+    assert torch.equal(got, oracle.rms_norm_ref(x, m.weight.detach(), 1e-6))

@@ -1,0 +1,169 @@
+// The row movers fused with their neighbours in the decoder layer (act.py:256-265):
+//   rmsnorm_permute_tiled   post-attention RMSNorm + permute into the K-tiled activation matrix of the FFN
+//   unpermute_add           unpermute + residual add
+// Each replaces two passes over [T, H] by one.  bf16 only (the FFN kernels' type).
+//
+// RMSNorm follows the reference module op by op: x in fp32, variance = mean(x^2), x * rsqrt(variance + eps),
+// rounded to bf16, times the bf16 weight, rounded to bf16 (Qwen2RMSNorm as used at act.py:190-193).  The sum of
+// squares is accumulated in fp32 in this kernel's own order, so results can differ from eager PyTorch in the last
+// bf16 bit where a value sits on a rounding boundary.
+#include "common.h"
+#include "tiled_layout.h"
+
+namespace wx {
+namespace {
+
+constexpr int kSplit = 4;        // wavefronts per 16-row block = one workgroup; each takes a quarter of the columns
+constexpr int kMaxChunks = 32;   // column blocks per wavefront held in registers (hidden <= 4096)
+
+__device__ __forceinline__ u32x4 ld16(const u32x4* p) { return __builtin_nontemporal_load(p); }
+__device__ __forceinline__ void st16(u32x4* p, const u32x4& v) { __builtin_nontemporal_store(v, p); }
+
+// NCH = column blocks per wavefront (compile-time so the row stays in registers)
+template <int NCH>
+__global__ __launch_bounds__(kSplit * 64) void rmsnorm_permute_tiled_kernel(
+    const u32x4* __restrict__ x, const u32x4* __restrict__ weight, float eps, unsigned char* __restrict__ out,
+    const int32_t* __restrict__ sorted_row_id, const int32_t* __restrict__ expert_offsets, int64_t num_tokens,
+    int64_t row_blocks) {
+  __shared__ float s_part[kSplit][kBlkRows];
+  const int lane = threadIdx.x & 63, part = threadIdx.x >> 6;
+  const int64_t rb = blockIdx.x;
+  const int32_t o0 = expert_offsets[0], o1 = expert_offsets[1], o2 = expert_offsets[2];
+  const int64_t pad0 = round_up_256(o1 - o0);
+  // lane -> (row of the block, 16-byte slot); the slot holds chunk slot ^ ((row >> 2) & 3) of the 32 columns
+  const int r = lane >> 2, slot = lane & 3, chunk = slot ^ ((r >> 2) & 3);
+  const int64_t prow = rb * kBlkRows + r;
+  int64_t pos = -1;  // padded row -> sorted position (none for the padding rows of either expert)
+  if (prow < pad0) { if (prow < o1 - o0) pos = o0 + prow; }
+  else if (prow - pad0 < o2 - o1) pos = o1 + (prow - pad0);
+  const int64_t src_tok = (pos >= 0 && pos < num_tokens) ? sorted_row_id[pos] : -1;
+  constexpr int64_t kChunksPerRow = static_cast<int64_t>(NCH) * kSplit * 4;
+  const int kb0 = part * NCH;  // first column block of this wavefront
+  const u32x4* src = x + (src_tok < 0 ? 0 : src_tok) * kChunksPerRow + kb0 * 4 + chunk;
+  u32x4 v[NCH];
+#pragma unroll
+  for (int u = 0; u < NCH; ++u) v[u] = src_tok < 0 ? u32x4{0, 0, 0, 0} : ld16(src + u * 4);
+  float ss = 0.f;
+#pragma unroll
+  for (int u = 0; u < NCH; ++u) {
+    float f[8];
+    unpack16<WX_BF16>(v[u], f);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) ss += f[e] * f[e];
+  }
+  // the 4 lanes of a row, then the 4 wavefronts of the workgroup
+  ss += __shfl_xor(ss, 1);
+  ss += __shfl_xor(ss, 2);
+  if (slot == 0) s_part[part][r] = ss;
+  __syncthreads();
+  const float total = s_part[0][r] + s_part[1][r] + s_part[2][r] + s_part[3][r];
+  const float inv = __frsqrt_rn(total / static_cast<float>(kChunksPerRow * 8) + eps);
+  unsigned char* dst = out + (rb << 10) + lane * 16;
+#pragma unroll
+  for (int u = 0; u < NCH; ++u) {
+    float f[8], w[8];
+    unpack16<WX_BF16>(v[u], f);
+    unpack16<WX_BF16>(weight[(kb0 + u) * 4 + chunk], w);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) f[e] = w[e] * round_bf16(f[e] * inv);  // pack16 rounds the product
+    st16(reinterpret_cast<u32x4*>(dst + ((static_cast<int64_t>(kb0 + u) * row_blocks) << 10)), pack16<WX_BF16>(f));
+  }
+}
+
+// out[t] = resid[t] + y[row_id_map[t]] (resid[t] alone when the map entry is -1); one wavefront per destination row.
+__global__ __launch_bounds__(256) void unpermute_add_kernel(const u32x4* __restrict__ y, const u32x4* __restrict__ resid,
+                                                            u32x4* __restrict__ out, const int32_t* __restrict__ row_id_map,
+                                                            int64_t num_tokens, int64_t vec_per_row) {
+  const int lane = threadIdx.x & 63;
+  const int64_t wave = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
+  const int64_t n_waves = static_cast<int64_t>(gridDim.x) * 4;
+  for (int64_t t = wave; t < num_tokens; t += n_waves) {
+    const int32_t src_row = row_id_map[t];
+    const u32x4* src = y + static_cast<int64_t>(src_row < 0 ? 0 : src_row) * vec_per_row;
+    const u32x4* res = resid + t * vec_per_row;
+    u32x4* dst = out + t * vec_per_row;
+    for (int64_t c = lane; c < vec_per_row; c += 4 * 64) {
+      u32x4 a[4], b[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int64_t cc = c + u * 64;
+        if (cc < vec_per_row) {
+          a[u] = ld16(res + cc);
+          b[u] = src_row < 0 ? u32x4{0, 0, 0, 0} : ld16(src + cc);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int64_t cc = c + u * 64;
+        if (cc < vec_per_row) {
+          float fa[8], fb[8];
+          unpack16<WX_BF16>(a[u], fa);
+          unpack16<WX_BF16>(b[u], fb);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) fa[e] += fb[e];
+          st16(dst + cc, pack16<WX_BF16>(fa));
+        }
+      }
+    }
+  }
+}
+
+}  // namespace
+}  // namespace wx
+
+using namespace wx;
+
+extern "C" int wx_rmsnorm_permute_rows_tiled(const void* x, const void* weight, float eps, void* out_tiled,
+                                             const int32_t* sorted_row_id, const int32_t* expert_offsets,
+                                             int64_t num_tokens, int64_t num_cols, wx_stream_t stream) {
+  const char* who = "wx_rmsnorm_permute_rows_tiled";
+  if (num_tokens < 0 || num_cols <= 0) return fail(WX_ERR_INVALID_ARGUMENT, "%s: bad sizes", who);
+  if (num_cols % (kBlkCols * kSplit) != 0 || num_cols / (kBlkCols * kSplit) > kMaxChunks)
+    return fail(WX_ERR_UNSUPPORTED, "%s: num_cols (%lld) must be a multiple of %d and at most %d", who,
+                static_cast<long long>(num_cols), kBlkCols * kSplit, kBlkCols * kSplit * kMaxChunks);
+  if (!(eps >= 0.f)) return fail(WX_ERR_INVALID_ARGUMENT, "%s: eps must be non-negative", who);
+  if (num_tokens == 0) return WX_OK;
+  if (num_tokens > INT32_MAX) return fail(WX_ERR_UNSUPPORTED, "%s: more than 2^31-1 rows", who);
+  if (!x || !weight || !out_tiled || !sorted_row_id || !expert_offsets)
+    return fail(WX_ERR_INVALID_ARGUMENT, "%s: null pointer", who);
+  if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(weight) | reinterpret_cast<uintptr_t>(out_tiled)) & 15)
+    return fail(WX_ERR_INVALID_ARGUMENT, "%s: buffers must be 16-byte aligned", who);
+  const int64_t row_blocks = padded_sorted_rows(num_tokens) / kBlkRows;
+  const int nch = static_cast<int>(num_cols / (kBlkCols * kSplit));
+  const dim3 grid(static_cast<unsigned>(row_blocks)), block(kSplit * 64);
+  hipStream_t s = as_stream(stream);
+#define WX_CASE(N)                                                                                                  \
+  case N:                                                                                                           \
+    hipLaunchKernelGGL(rmsnorm_permute_tiled_kernel<N>, grid, block, 0, s, static_cast<const u32x4*>(x),            \
+                       static_cast<const u32x4*>(weight), eps, static_cast<unsigned char*>(out_tiled), sorted_row_id, \
+                       expert_offsets, num_tokens, row_blocks);                                                     \
+    break;
+  switch (nch) {
+    WX_CASE(1) WX_CASE(2) WX_CASE(3) WX_CASE(4) WX_CASE(5) WX_CASE(6) WX_CASE(7) WX_CASE(8)
+    WX_CASE(9) WX_CASE(10) WX_CASE(11) WX_CASE(12) WX_CASE(13) WX_CASE(14) WX_CASE(15) WX_CASE(16)
+    WX_CASE(20) WX_CASE(24) WX_CASE(28) WX_CASE(32)
+    default:
+      return fail(WX_ERR_UNSUPPORTED, "%s: num_cols %lld has no built kernel (hidden / 128 must be 1..16, 20, 24, 28 or 32)",
+                  who, static_cast<long long>(num_cols));
+  }
+#undef WX_CASE
+  return check_launch("rmsnorm_permute_tiled_kernel");
+}
+
+extern "C" int wx_unpermute_rows_add(const void* y, const void* residual, void* out, const int32_t* row_id_map,
+                                     int64_t num_tokens, int64_t num_cols, wx_stream_t stream) {
+  const char* who = "wx_unpermute_rows_add";
+  if (num_tokens < 0 || num_cols <= 0) return fail(WX_ERR_INVALID_ARGUMENT, "%s: bad sizes", who);
+  if (num_cols % 8 != 0) return fail(WX_ERR_UNSUPPORTED, "%s: num_cols must be a multiple of 8", who);
+  if (num_tokens == 0) return WX_OK;
+  if (num_tokens > INT32_MAX) return fail(WX_ERR_UNSUPPORTED, "%s: more than 2^31-1 rows", who);
+  if (!y || !residual || !out || !row_id_map) return fail(WX_ERR_INVALID_ARGUMENT, "%s: null pointer", who);
+  if ((reinterpret_cast<uintptr_t>(y) | reinterpret_cast<uintptr_t>(residual) | reinterpret_cast<uintptr_t>(out)) & 15)
+    return fail(WX_ERR_INVALID_ARGUMENT, "%s: buffers must be 16-byte aligned", who);
+  const int64_t want = (num_tokens + 3) / 4;
+  const int64_t cap = static_cast<int64_t>(device_cu_count()) * 8;  // 8 workgroups of 4 wavefronts per CU cover HBM latency
+  hipLaunchKernelGGL(unpermute_add_kernel, dim3(static_cast<unsigned>(want < cap ? want : cap)), dim3(256), 0,
+                     as_stream(stream), static_cast<const u32x4*>(y), static_cast<const u32x4*>(residual),
+                     static_cast<u32x4*>(out), row_id_map, num_tokens, num_cols / 8);
+  return check_launch("unpermute_add_kernel");
+}

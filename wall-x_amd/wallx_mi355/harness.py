@@ -9,7 +9,9 @@ batch of full sequences (prefill).  What it states explicitly:
   * q/k/v projections with bias, o projection without (vl.py:821-832),
   * attention mask: plain causal by default (`mask="causal"`); `mask="action_block"` adds the reference's
     bidirectional block among action tokens (act.py:616-637) through a dense boolean mask,
-  * rotary base 1e6, mrope_section [16, 24, 24], cos/sin built in fp32 and cast to bf16 (vl.py:679-712).
+  * rotary base 1e6, mrope_section [16, 24, 24], cos/sin built in fp32 and cast to bf16 (vl.py:679-712),
+  * `fuse=True` (default) runs the post-attention RMSNorm inside the permute and the residual add inside the
+    unpermute (one pass over [T, H] each instead of two); `fuse=False` keeps them as separate PyTorch ops.
 """
 
 from contextlib import contextmanager
@@ -50,18 +52,17 @@ class OpTimer:
 
 
 def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
-    v = x.float()
-    v = v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps)
-    return weight * v.to(x.dtype)
+    return F.rms_norm(x, (x.shape[-1],), weight, eps)
 
 
 class PrefillHarness:
     def __init__(self, n_layers: int = 36, hidden: int = wl.HIDDEN, n_q: int = wl.N_Q_HEADS, n_kv: int = wl.N_KV_HEADS,
                  head_dim: int = wl.HEAD_DIM, inter=(wl.INTER_VL, wl.INTER_ACT), vocab: int = 151936,
-                 eps: float = 1e-6, device="cuda:0", seed: int = 0, mask: str = "causal", keep_dense: bool = False):
+                 eps: float = 1e-6, device="cuda:0", seed: int = 0, mask: str = "causal", keep_dense: bool = False,
+                 fuse: bool = True):
         self.dev = torch.device(device)
         self.n_layers, self.hidden, self.n_q, self.n_kv, self.head_dim = n_layers, hidden, n_q, n_kv, head_dim
-        self.inter, self.eps, self.mask_mode = inter, eps, mask
+        self.inter, self.eps, self.mask_mode, self.fuse = inter, eps, mask, fuse
         g = torch.Generator(device=self.dev).manual_seed(seed)
 
         def w(*shape):
@@ -90,19 +91,27 @@ class PrefillHarness:
         self._ws = None
 
     # ------------------------------------------------------------------------------------------------
-    def _ffn(self, x: torch.Tensor, routing: moe.Routing, packed, timer: OpTimer) -> torch.Tensor:
+    def _ffn(self, h: torch.Tensor, ln_weight: torch.Tensor, routing: moe.Routing, packed, timer: OpTimer) -> torch.Tensor:
+        """h [T, H] (the residual stream after attention) -> h + FFN(RMSNorm(h))."""
         from . import _lib
 
-        T, H = x.shape
+        T, H = h.shape
         I0, I1 = self.inter
         stream = torch.cuda.current_stream().cuda_stream
         rows_pad = native.padded_sorted_rows(T)
         if self._hmid is None or self._hmid.numel() < rows_pad * max(I0, I1):
             self._hmid = torch.empty(rows_pad * max(I0, I1), dtype=torch.bfloat16, device=self.dev)
-        with timer.section("permute"):
-            self._x_tiled = native.permute_rows_tiled(x, routing.row_id_map, routing.expert_offsets, self._x_tiled,
-                                                      routing.sorted_row_id)
-        y_sorted = torch.empty_like(x)
+        if self.fuse:
+            with timer.section("rmsnorm+permute"):
+                self._x_tiled = native.rmsnorm_permute_rows_tiled(h, ln_weight, self.eps, routing.expert_offsets,
+                                                                  routing.sorted_row_id, self._x_tiled)
+        else:
+            with timer.section("rmsnorm_torch"):
+                x = rms_norm(h, ln_weight, self.eps)
+            with timer.section("permute"):
+                self._x_tiled = native.permute_rows_tiled(x, routing.row_id_map, routing.expert_offsets, self._x_tiled,
+                                                          routing.sorted_row_id)
+        y_sorted = torch.empty_like(h)
         (g0, u0, d0), (g1, u1, d1) = packed
         with timer.section("ffn_gate_up_swiglu"):
             _lib.call("wx_dual_swiglu_gate_up", self._x_tiled.data_ptr(), self._hmid.data_ptr(),
@@ -111,9 +120,13 @@ class PrefillHarness:
         with timer.section("ffn_down"):
             _lib.call("wx_dual_down_proj", self._hmid.data_ptr(), y_sorted.data_ptr(), routing.expert_offsets.data_ptr(),
                       d0.data_ptr(), d1.data_ptr(), T, H, I0, I1, stream)
+        if self.fuse:
+            with timer.section("unpermute+residual"):
+                return native.unpermute_add(y_sorted, h, routing.row_id_map)
         with timer.section("unpermute"):
             y = native.unpermute(y_sorted, routing.row_id_map, torch.tensor([]), T, 1)
-        return y
+        with timer.section("residual_torch"):
+            return h + y
 
     @torch.no_grad()
     def forward(self, input_ids: torch.Tensor, image_grid_thw: torch.Tensor, moe_token_types: torch.Tensor,
@@ -157,9 +170,7 @@ class PrefillHarness:
                                                    enable_gqa=True)
             with timer.section("o_proj_torch"):
                 h = h + F.linear(a.transpose(1, 2).reshape(B, S, nq * D), layer["wo"])
-            with timer.section("rmsnorm_torch"):
-                x = rms_norm(h, layer["ln2"], self.eps)
-            h = h + self._ffn(x.view(B * S, H), routing, layer["packed"], timer).view(B, S, H)
+            h = self._ffn(h.view(B * S, H), layer["ln2"], routing, layer["packed"], timer).view(B, S, H)
         with timer.section("lm_head_torch"):
             last = rms_norm(h[:, -1], self.final_ln, self.eps)
             logits = F.linear(last, self.embed)

@@ -82,11 +82,16 @@ class SparseMoeBlock(nn.Module):
 
     def forward(self, hidden_states: torch.Tensor, experts_indices: torch.Tensor,
                 start_indices: Optional[torch.Tensor] = None, end_indices: Optional[torch.Tensor] = None,
-                routing: Optional[Routing] = None) -> torch.Tensor:
+                routing: Optional[Routing] = None, pre_norm=None, residual: bool = False) -> torch.Tensor:
         """hidden_states [B, S, H] bf16; experts_indices [B, S] (bool or integer expert id).
 
         start_indices / end_indices are accepted for signature parity and not read: the row ranges come from
         the partition on the device.
+
+        Two optional caller fusions (the decoder layer around this block, act.py:256-265):
+        pre_norm=(weight, eps) applies the post-attention RMSNorm to hidden_states inside the permute, and
+        residual=True returns hidden_states + block(...) with the add done inside the unpermute.  With both, the
+        layer's `residual = h; h = norm(h); h = moe(h); h = residual + h` is `h = moe(h, ..., pre_norm, True)`.
         """
         del start_indices, end_indices
         batch, seq, hidden = hidden_states.shape
@@ -97,14 +102,22 @@ class SparseMoeBlock(nn.Module):
             routing = self.route(experts_indices)
         if routing.num_tokens != x.size(0):
             raise RuntimeError(f"routing was built for {routing.num_tokens} tokens, got {x.size(0)}")
-        self._x_tiled = native.permute_rows_tiled(x, routing.row_id_map, routing.expert_offsets, self._x_tiled,
-                                                  routing.sorted_row_id)
+        if pre_norm is not None:
+            norm_weight, eps = pre_norm
+            self._x_tiled = native.rmsnorm_permute_rows_tiled(x, norm_weight, eps, routing.expert_offsets,
+                                                              routing.sorted_row_id, self._x_tiled)
+        else:
+            self._x_tiled = native.permute_rows_tiled(x, routing.row_id_map, routing.expert_offsets, self._x_tiled,
+                                                      routing.sorted_row_id)
         need = native.padded_sorted_rows(x.size(0)) * max(e.intermediate_size for e in self.experts)
         if self._hmid is None or self._hmid.numel() < need or self._hmid.device != x.device:
             self._hmid = torch.empty(need, dtype=torch.bfloat16, device=x.device)
         flat = [w for e in self.experts for w in e.weights()]
         y_sorted = _DualExpertFFN.apply(self._x_tiled, x.size(0), routing.expert_offsets, self._hmid, *flat)
-        y = native.unpermute(y_sorted, routing.row_id_map, torch.tensor([]), x.size(0), 1)
+        if residual:
+            y = native.unpermute_add(y_sorted, x, routing.row_id_map)
+        else:
+            y = native.unpermute(y_sorted, routing.row_id_map, torch.tensor([]), x.size(0), 1)
         return y.view(batch, seq, hidden)
 
 

@@ -430,6 +430,41 @@ def permute_rows_tiled(x: torch.Tensor, row_id_map: Optional[torch.Tensor], expe
     return out
 
 
+def rmsnorm_permute_rows_tiled(x: torch.Tensor, weight: torch.Tensor, eps: float, expert_offsets: torch.Tensor,
+                               sorted_row_id: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """RMSNorm(x) * weight written straight into the K-tiled, expert-padded activation matrix (one pass)."""
+    _need_cuda("x", x)
+    if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
+        raise RuntimeError("All tensors must be BFloat16 for this kernel")
+    x, weight = x.contiguous(), weight.contiguous()
+    T, H = x.shape
+    if weight.numel() != H:
+        raise RuntimeError("weight size must equal the hidden size")
+    need = _lib.load().wx_tiled_bytes(padded_sorted_rows(T), H) // 2
+    if out is None or out.numel() < need or out.dtype != torch.bfloat16 or out.device != x.device:
+        out = torch.empty(need, dtype=torch.bfloat16, device=x.device)
+    with _DeviceGuard(x):
+        _lib.call("wx_rmsnorm_permute_rows_tiled", _ptr(x), _ptr(weight), float(eps), out.data_ptr(),
+                  _ptr(sorted_row_id), expert_offsets.data_ptr(), T, H, _stream(x))
+    return out
+
+
+def unpermute_add(y_sorted: torch.Tensor, residual: torch.Tensor, row_id_map: torch.Tensor) -> torch.Tensor:
+    """residual + y_sorted[row_id_map] in one pass (topK 1, bf16)."""
+    _need_cuda("y_sorted", y_sorted)
+    if y_sorted.dtype != torch.bfloat16 or residual.dtype != torch.bfloat16:
+        raise RuntimeError("All tensors must be BFloat16 for this kernel")
+    y_sorted, residual = y_sorted.contiguous(), residual.contiguous()
+    T, H = residual.shape
+    if y_sorted.shape[1] != H or row_id_map.numel() < T:
+        raise RuntimeError("shape mismatch between residual, sorted rows and row_id_map")
+    out = torch.empty_like(residual)
+    with _DeviceGuard(residual):
+        _lib.call("wx_unpermute_rows_add", _ptr(y_sorted), _ptr(residual), _ptr(out), _ptr(row_id_map), T, H,
+                  _stream(residual))
+    return out
+
+
 def dual_swiglu_ffn(x_tiled: torch.Tensor, num_rows: int, expert_offsets: torch.Tensor, weights,
                     hmid: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Both experts' SwiGLU FFN over expert-sorted rows in two launches (act.py:79-82, 142-154).
