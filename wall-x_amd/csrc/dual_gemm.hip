@@ -312,8 +312,15 @@ __global__ __launch_bounds__(kThreads, TS::kWgPerCu) void dual_gemm_kernel(Param
   };
 
   // One K step of global -> LDS for this wave: rows [wave*64, +64) of the A slot, [wave*kLoadRowsB, +kLoadRowsB) of B.
-  auto issue = [&](const Loader& L, int ks, unsigned char* sa, unsigned char* sb) {
-    __amdgpu_buffer_rsrc_t ra, rb;
+  // The A half goes out right after the barrier that frees the slot, the B half one MFMA group later (spreading
+  // the loads keeps the CU's L2 port, 64 bytes per clock, from backing up into the wave's in-order issue);
+  // `Pending` carries what the B half needs across that gap, which may include a change of tile.
+  struct Pending {
+    __amdgpu_buffer_rsrc_t rb;
+    uint32_t voff_b[kLoadsB];
+  };
+  auto issue_a = [&](const Loader& L, int ks, unsigned char* sa, Pending& P) {
+    __amdgpu_buffer_rsrc_t ra;
     uint32_t oob = 0;
     if constexpr (TILED_IN) {
       // steps past K (ring padding) and blocks past the end of the matrix read as zero through the bounds check
@@ -324,87 +331,105 @@ __global__ __launch_bounds__(kThreads, TS::kWgPerCu) void dual_gemm_kernel(Param
       const uint32_t na = !real ? 0u : (L.a_bytes == 0x7fffff00u ? 0x7fffff00u : static_cast<uint32_t>(la < 0 ? 0 : la));
       const uint32_t nb = !real ? 0u : (L.b_bytes == 0x7fffff00u ? 0x7fffff00u : static_cast<uint32_t>(lb < 0 ? 0 : lb));
       ra = make_rsrc(reinterpret_cast<const char*>(L.a_base) + da, na);
-      rb = make_rsrc(reinterpret_cast<const char*>(L.b_base) + db, nb);
+      P.rb = make_rsrc(reinterpret_cast<const char*>(L.b_base) + db, nb);
     } else {
       const int k0 = ks * BK;
       // advancing the base keeps the absolute end of the readable range, so rows past the matrix read as zero;
       // K chunks at or past the row end are pushed out of range per lane (this also zero-fills padding steps)
       const uint32_t adv = 2u * static_cast<uint32_t>(k0);
       ra = make_rsrc(L.a_base + k0, L.a_bytes > adv ? L.a_bytes - adv : 0u);
-      rb = make_rsrc(L.b_base + k0, L.b_bytes > adv ? L.b_bytes - adv : 0u);
+      P.rb = make_rsrc(L.b_base + k0, L.b_bytes > adv ? L.b_bytes - adv : 0u);
       const bool k_tail = k0 + BK > L.K;
       oob = (k_tail && k0 + ld_chunk * 8 >= L.K) ? 0x80000000u : 0u;
     }
 #pragma unroll
-    for (int i = 0; i < kLoadsA; ++i) {
+    for (int i = 0; i < kLoadsB; ++i) P.voff_b[i] = L.voff_b[i] | oob;
+#pragma unroll
+    for (int i = 0; i < kLoadsA; ++i)
       __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, LDS_PTR(sa + (wave * kLoadRowsA + 16 * i) * kRowBytes), 16,
                                                L.voff_a[i] | oob, 0, 0, 0);
-      if (i < kLoadsB)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, LDS_PTR(sb + (wave * kLoadRowsB + 16 * i) * kRowBytes), 16,
-                                                 L.voff_b[i] | oob, 0, 0, 0);
-    }
+  };
+  auto issue_b = [&](const Pending& P, unsigned char* sb) {
+#pragma unroll
+    for (int i = 0; i < kLoadsB; ++i)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(P.rb, LDS_PTR(sb + (wave * kLoadRowsB + 16 * i) * kRowBytes), 16,
+                                               P.voff_b[i], 0, 0, 0);
   };
 
   f32x16 acc[FM][FN];
   bf16x8 fa[2][FM], fb[2][FN];  // two fragment sets: one feeds the MFMAs while the other is being read from LDS
 
+  // Fragments are read in the order the MFMAs (A-major: all B blocks for A block 0, then A block 1, ...) first
+  // need them: A0, every B, then the other A blocks.
   auto read_frags = [&](const unsigned char* sa, const unsigned char* sb, int kk, int set) {
-#pragma unroll
-    for (int i = 0; i < FM; ++i)
-      fa[set][i] = *reinterpret_cast<const bf16x8*>(sa + a_row_off + i * 32 * kRowBytes + frag_off[kk]);
+    fa[set][0] = *reinterpret_cast<const bf16x8*>(sa + a_row_off + frag_off[kk]);
 #pragma unroll
     for (int j = 0; j < FN; ++j)
       fb[set][j] = *reinterpret_cast<const bf16x8*>(sb + b_row(j) * kRowBytes + b_lane_off + frag_off[kk]);
+#pragma unroll
+    for (int i = 1; i < FM; ++i)
+      fa[set][i] = *reinterpret_cast<const bf16x8*>(sa + a_row_off + i * 32 * kRowBytes + frag_off[kk]);
   };
   auto mma = [&](int set) {
 #pragma unroll
     for (int i = 0; i < FM; ++i)
 #pragma unroll
-      for (int j = 0; j < FN; ++j)
+      for (int jj = 0; jj < FN; ++jj) {
+        const int j = jj;
         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[set][i], fb[set][j], acc[i][j], 0, 0, 0);
+      }
   };
-  // Scheduling hints.  Before the barrier: the LDS reads of the next fragment set go out among the first MFMAs
-  // of this one and the remaining MFMAs cover their latency, so the wait in front of the barrier finds them done.
-  auto schedule_reads_then_mfma = [&]() {
+  // Scheduling hints.  Before the barrier: the LDS reads of the other fragment set and the B half of the previous
+  // slot's refill go out among the first half of this group's MFMAs; the second half covers the read latency, so
+  // the wait in front of the barrier finds the reads done.
+  auto schedule_before_barrier = [&]() {
+    constexpr int kMfma = FM * FN, kReads = FM + FN;
+    constexpr int kCarry = kMfma / 2;                              // MFMAs that carry other instructions
+    constexpr int kReadsPer = (kReads + kCarry - 1) / kCarry;      // LDS reads per carrying MFMA
+    constexpr int kLoadEvery = kCarry / kLoadsB > 0 ? kCarry / kLoadsB : 1;
 #pragma unroll
-    for (int q = 0; q < (FM + FN) / 2; ++q) {
-      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);  // two LDS reads
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
+    for (int m = 0; m < kCarry; ++m) {
+      __builtin_amdgcn_sched_group_barrier(0x100, kReadsPer, 0);
+      if (m % kLoadEvery == 0 && m / kLoadEvery < kLoadsB) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
     }
-    __builtin_amdgcn_sched_group_barrier(0x008, FM * FN - (FM + FN) / 2, 0);
+    __builtin_amdgcn_sched_group_barrier(0x008, kMfma - kCarry, 0);
     __builtin_amdgcn_sched_barrier(0);
   };
-  // After the barrier: the refill loads and the next slot's fragment reads are spread over the MFMAs.
-  auto schedule_loads_reads_mfma = [&]() {
-    constexpr int kPairs = (FM + FN) / 2;
-    constexpr int kMixed = kLoadsPerStep > kPairs ? kLoadsPerStep : kPairs;
+  // After the barrier: the A half of the refill and the next slot's fragment reads are spread over the whole group.
+  auto schedule_after_barrier = [&]() {
+    constexpr int kMfma = FM * FN, kReads = FM + FN;
+    constexpr int kReadEvery = kMfma / kReads > 0 ? kMfma / kReads : 1;
+    constexpr int kReadsPer = kReads * kReadEvery > kMfma ? (kReads + kMfma - 1) / kMfma : 1;
+    constexpr int kLoadEvery = kMfma / kLoadsA > 0 ? kMfma / kLoadsA : 1;
 #pragma unroll
-    for (int q = 0; q < kMixed; ++q) {
-      if (q < kLoadsPerStep) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // one buffer load
-      if (q < kPairs) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);         // two LDS reads
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                         // one MFMA
+    for (int m = 0; m < kMfma; ++m) {
+      if (m % kLoadEvery == 0 && m / kLoadEvery < kLoadsA) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+      if (m % kReadEvery == 0 && m / kReadEvery * kReadsPer < kReads) __builtin_amdgcn_sched_group_barrier(0x100, kReadsPer, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
     }
-    __builtin_amdgcn_sched_group_barrier(0x008, FM * FN - kMixed, 0);
     __builtin_amdgcn_sched_barrier(0);
   };
 
-  // One K step on slot (sa, sb); (sa_n, sb_n) is the next slot of the ring.  On entry fragment set 0 holds kk = 0
-  // of this slot.  After the barrier every wave has finished reading this slot, so it is refilled at once with the
-  // K step kStages ahead in the load stream (step `ld_ks` of tile `L`); the next slot's data was issued
-  // kStages - 1 steps ago.
+  // One K step on slot (sa, sb); (sa_n, sb_n) is the next slot of the ring and sb_p the previous one.  On entry
+  // fragment set 0 holds kk = 0 of this slot.  After the barrier every wave has finished reading this slot, so its
+  // refill with the K step kStages ahead in the load stream (step `ld_ks` of tile `L`) starts at once: the A half
+  // here, the B half in the next step's first group.  The next slot's data was issued kStages - 1 steps ago.
+  Pending pend;
   auto k_step = [&](const Loader& L, int ld_ks, unsigned char* sa, unsigned char* sb, unsigned char* sa_n,
-                    unsigned char* sb_n) {
+                    unsigned char* sb_n, unsigned char* sb_p) {
     read_frags(sa, sb, 1, 1);
+    issue_b(pend, sb_p);
     mma(0);
-    schedule_reads_then_mfma();
-    // my LDS reads have returned; of my loads at most the kStages - 2 youngest K steps are still in flight, i.e.
-    // the next slot is complete
+    schedule_before_barrier();
+    // my LDS reads have returned; of my loads at most the kStages - 2 youngest K steps' worth are still in flight,
+    // i.e. the next slot is complete
     __builtin_amdgcn_s_waitcnt(waitcnt_imm((kStages - 2) * kLoadsPerStep, 0));
     barrier_no_fence();
-    issue(L, ld_ks, sa, sb);
+    issue_a(L, ld_ks, sa, pend);
     read_frags(sa_n, sb_n, 0, 0);
     mma(1);
-    schedule_loads_reads_mfma();
+    schedule_after_barrier();
   };
 
   // ---- epilogue ------------------------------------------------------------------------------------------
@@ -544,9 +569,12 @@ __global__ __launch_bounds__(kThreads, TS::kWgPerCu) void dual_gemm_kernel(Param
   setup_loader(tc, L);
   setup_store(tc, S);
 #pragma unroll
-  for (int s = 0; s < kStages; ++s) issue(L, s, slot_a(s), slot_b(s));
-  // slot 0 must be complete before its first fragments are read: the younger K steps may remain in flight
-  __builtin_amdgcn_s_waitcnt(waitcnt_imm((kStages - 1) * kLoadsPerStep, 15));
+  for (int s = 0; s < kStages; ++s) {
+    issue_a(L, s, slot_a(s), pend);
+    if (s + 1 < kStages) issue_b(pend, slot_b(s));  // the last slot's B half goes out in the first K step
+  }
+  // slot 0 must be complete before its first fragments are read: the younger loads may remain in flight
+  __builtin_amdgcn_s_waitcnt(waitcnt_imm((kStages - 2) * kLoadsPerStep + kLoadsA, 15));
   __syncthreads();
   read_frags(s_a0, s_b0, 0, 0);
 
@@ -576,7 +604,8 @@ __global__ __launch_bounds__(kThreads, TS::kWgPerCu) void dual_gemm_kernel(Param
       }
 #pragma unroll
       for (int s = 0; s < kStages; ++s)
-        k_step(L, ld_ks + s, slot_a(s), slot_b(s), slot_a((s + 1) % kStages), slot_b((s + 1) % kStages));
+        k_step(L, ld_ks + s, slot_a(s), slot_b(s), slot_a((s + 1) % kStages), slot_b((s + 1) % kStages),
+               slot_b((s + kStages - 1) % kStages));
     }
     epilogue(done);
   }
