@@ -189,7 +189,7 @@ def main():
     if not args.ops_only:
         extra["cold_hbm"] = cold_measurements(dev, x, row_id_map, T, H, row_bytes, iters)
         extra["config4"] = config4_measurement(dev, weights)
-        extra["backward_gemms"] = backward_measurement(dev, x, weights, m0)
+        extra["asym_dual_gmm_op"] = backward_measurement(dev, x, weights, m0)
         extra["ceilings"] = ceiling_measurements(dev, x, weights, m0)
     if not args.ops_only and not args.no_prefill:
         del x_tiled, hmid, x_sorted, y_sorted, y
@@ -351,9 +351,10 @@ def config4_measurement(dev, weights):
 
 
 def backward_measurement(dev, x, weights, m0):
-    """The two backward GEMMs of `asym_dual_gmm` (ops.py:78-144) at the gate projection's config 3 shapes:
-    dX = dY @ W (both experts) and dW = dY^T @ X, each as transposed copies + the MFMA kernel; the times include
-    the transposes."""
+    """The reference's own op, `asym_dual_gmm` on row-major operands (ops.py:6-165), at the gate projection's
+    config 3 shapes: the forward (x @ W^T for both experts in one launch, nn.Linear weights read in place) and the
+    two backward GEMMs of ops.py:78-144, dX = dY @ W and dW = dY^T @ X, each as transposed copies + the MFMA
+    kernel (times include the transposes)."""
     import torch
     from wallx_mi355 import native
 
@@ -368,9 +369,12 @@ def backward_measurement(dev, x, weights, m0):
     dx0, dx1 = torch.empty_like(x0), torch.empty_like(x1)
     dw0, dw1 = torch.empty_like(g0), torch.empty_like(g1)
     flops = 2.0 * H * (m0 * I0 + m1 * I1)
+    y0, y1 = torch.empty_like(dy0), torch.empty_like(dy1)
+    t_fw, _ = event_ms(lambda: native.asym_dual_gmm(x0, x1, g0, g1, y0, y1, False, True), 5, warm=2)
     t_dx, _ = event_ms(lambda: native.asym_dual_gmm(dy0, dy1, g0, g1, dx0, dx1, False, False), 5, warm=2)
     t_dw, _ = event_ms(lambda: native.asym_dual_gmm(dy0, dy1, x0, x1, dw0, dw1, True, False), 5, warm=2)
-    return {"dx_ms": round(t_dx, 3), "dx_tflops": round(flops / t_dx / 1e9, 1),
+    return {"forward_nt_ms": round(t_fw, 3), "forward_nt_tflops": round(flops / t_fw / 1e9, 1),
+            "dx_ms": round(t_dx, 3), "dx_tflops": round(flops / t_dx / 1e9, 1),
             "dw_ms": round(t_dw, 3), "dw_tflops": round(flops / t_dw / 1e9, 1)}
 
 
