@@ -57,6 +57,18 @@ def test_argument_errors_without_a_gpu():
     assert lib.wx_partition_build(None, 0, 4, 1, 300, 0, None, None, None, None, None, 0, None) == -2
     assert lib.wx_partition_build(None, 0, 4, 200, 2, 0, None, None, None, None, None, 0, None) == -2
     assert b"num_topK cannot exceed 128" in lib.wx_last_error_string()
+    # the fused movers, the transpose and the probe check their arguments the same way
+    assert lib.wx_rmsnorm_permute_rows_tiled(None, None, 1e-6, None, None, None, 4, 100, None) == -2  # cols % 128
+    assert lib.wx_rmsnorm_permute_rows_tiled(None, None, 1e-6, None, None, None, 4, 8192, None) == -2  # cols > 4096
+    assert lib.wx_rmsnorm_permute_rows_tiled(None, None, 1e-6, None, None, None, 4, 2048, None) == -1  # null pointers
+    assert lib.wx_rmsnorm_permute_rows_tiled(None, None, 1e-6, None, None, None, 0, 2048, None) == 0   # nothing to do
+    assert lib.wx_unpermute_rows_add(None, None, None, None, 4, 12, None) == -2  # cols % 8
+    assert lib.wx_unpermute_rows_add(None, None, None, None, 4, 16, None) == -1
+    assert lib.wx_transpose_2d(None, None, 12, 16, 2, None) == -2  # rows % 8
+    assert lib.wx_transpose_2d(None, None, 16, 16, 4, None) == -2  # element size
+    assert lib.wx_transpose_2d(None, None, 16, 16, 2, None) == -1
+    assert lib.wx_probe_mfma_rate(None, 10, None, None, None) == -1
+    assert lib.wx_probe_mfma_operand_bytes() == 4 * 8 * 64 * 16
 
 
 def test_op_layer_validation_matches_reference_behaviour():
