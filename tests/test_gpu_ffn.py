@@ -35,6 +35,7 @@ GEMM_SHAPES = [
     (129, 136, 200, 0, 64, 64),          # empty action group, K tail
     (0, 64, 64, 0, 64, 64),              # nothing to do
     (3000, 3080, 96, 200, 264, 160),     # enough 256 x 256 tiles to take the large-tile kernel, ragged everywhere
+    (40, 64, 0, 24, 72, 64),             # empty contraction: the output is zeros
 ]
 
 

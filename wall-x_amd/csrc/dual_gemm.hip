@@ -263,7 +263,12 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
     int rows, cols_left, ldc, nk;
   };
 
-  auto padded_steps = [](int k) { return ((k + BK - 1) / BK + kStages - 1) / kStages * kStages; };
+  // K steps of a tile rounded up to whole ring rounds (padding steps read zeros); at least one round, so that a
+  // problem with k == 0 still walks the tile loop (and stores zeros)
+  auto padded_steps = [](int k) {
+    const int n = ((k + BK - 1) / BK + kStages - 1) / kStages * kStages;
+    return n < kStages ? kStages : n;
+  };
   auto setup_store = [&](const TileCoord& tc, Store& S) {
     const Group G = tc.group ? g1 : g0;
     const int row0 = tc.tm * BM, col0 = tc.tn * kTileN;
