@@ -47,10 +47,32 @@ def _newer(target: str, deps) -> bool:
     return all(os.path.getmtime(d) <= t for d in deps)
 
 
+# The large-tile GEMM kernels use every register a wave can have; a small source change can push values of the K
+# loop into scratch memory, which costs a factor of three and shows in no test.  Their compile prints the
+# resource-usage remarks and this limit on "ScratchSize [bytes/lane]" turns a spill into a loud warning.
+RESOURCE_CHECKED = {"dual_gemm.hip": ("dual_gemm_kernel", 64)}
+
+
+def _check_resources(src, stderr):
+    name_part, limit = RESOURCE_CHECKED[src]
+    current = None
+    for line in stderr.splitlines():
+        if "Function Name:" in line:
+            current = line.split("Function Name:")[1].split()[0]
+        elif "ScratchSize [bytes/lane]:" in line and current and name_part in current:
+            size = int(line.split("ScratchSize [bytes/lane]:")[1].split()[0])
+            if size > limit:
+                sys.stderr.write(f"[wallx_mi355] WARNING: {current} spills {size} bytes per lane to scratch "
+                                 f"(limit {limit}): check that no spill sits inside the K loop\n")
+
+
 def _run(cmd):
     proc = subprocess.run(cmd, capture_output=True, text=True)
-    noise = "is not a recognized feature for this target"
-    err = "\n".join(line for line in proc.stderr.splitlines() if noise not in line)
+    noise = ("is not a recognized feature for this target", "-Rpass-analysis=kernel-resource-usage")
+    src = os.path.basename(cmd[-3]) if len(cmd) > 3 else ""
+    if proc.returncode == 0 and src in RESOURCE_CHECKED:
+        _check_resources(src, proc.stderr)
+    err = "\n".join(line for line in proc.stderr.splitlines() if not any(n in line for n in noise))
     if proc.returncode != 0:
         raise RuntimeError(f"command failed: {' '.join(cmd)}\n{proc.stdout}\n{err}")
     if err.strip():
@@ -67,7 +89,8 @@ def build(force: bool = False, verbose: bool = True) -> str:
         obj = os.path.join(OBJ_DIR, src.replace(".hip", ".o"))
         objs.append(obj)
         if force or not _newer(obj, [path] + headers):
-            jobs.append([hipcc] + FLAGS + ["-c", path, "-o", obj])
+            extra = ["-Rpass-analysis=kernel-resource-usage", "-fno-caret-diagnostics"] if src in RESOURCE_CHECKED else []
+            jobs.append([hipcc] + FLAGS + extra + ["-c", path, "-o", obj])
     if jobs:
         if verbose:
             print(f"[wallx_mi355] compiling {len(jobs)} source(s) for gfx950", flush=True)

@@ -263,12 +263,9 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
     int rows, cols_left, ldc, nk;
   };
 
-  // K steps of a tile rounded up to whole ring rounds (padding steps read zeros); at least one round, so that a
-  // problem with k == 0 still walks the tile loop (and stores zeros)
-  auto padded_steps = [](int k) {
-    const int n = ((k + BK - 1) / BK + kStages - 1) / kStages * kStages;
-    return n < kStages ? kStages : n;
-  };
+  // K steps of a tile rounded up to whole ring rounds (padding steps read zeros).  The host never launches this
+  // kernel with k == 0 and a non-empty output: the tile loop below advances only from inside the K loop.
+  auto padded_steps = [](int k) { return ((k + BK - 1) / BK + kStages - 1) / kStages * kStages; };
   auto setup_store = [&](const TileCoord& tc, Store& S) {
     const Group G = tc.group ? g1 : g0;
     const int row0 = tc.tm * BM, col0 = tc.tn * kTileN;
@@ -755,7 +752,9 @@ extern "C" int wx_dual_gemm(const void* in0, const void* in1, const void* w0, co
   p.offsets = nullptr;
   if ((m0 == 0 || n0 == 0) && (m1 == 0 || n1 == 0)) return WX_OK;
   hipStream_t s = as_stream(stream);
-  if (!trans_a && trans_b) {
+  // an empty contraction (k == 0) has zeros as its result: the plain kernel below writes them
+  const bool empty_k = (k0 == 0 && m0 > 0 && n0 > 0) || (k1 == 0 && m1 > 0 && n1 > 0);
+  if (!trans_a && trans_b && !empty_k) {
     const int64_t tiles = ceil_div(m0, BigTile::BM) * ceil_div(n0, BigTile::BN) + ceil_div(m1, BigTile::BM) * ceil_div(n1, BigTile::BN);
     return launch_mfma<kGeneric>(p, tiles, tiles, s, "dual_gemm_kernel<generic>");
   }
@@ -800,6 +799,8 @@ int check_ffn(const char* who, const FfnArgs& a, bool need_gate_up, bool need_do
   if (int rc = check_dims(who, a.rows, a.hidden, a.inter[1])) return rc;
   if (a.hidden % kBlkCols != 0 || a.inter[0] % kBlkCols != 0 || a.inter[1] % kBlkCols != 0)
     return fail(WX_ERR_UNSUPPORTED, "%s: hidden and intermediate sizes must be multiples of 32", who);
+  if (a.hidden == 0 || a.inter[0] == 0 || a.inter[1] == 0)
+    return fail(WX_ERR_UNSUPPORTED, "%s: hidden and both intermediate sizes must be positive", who);
   if (a.rows == 0) return WX_OK;
   if (!a.offsets || !a.hmid || (need_gate_up && !a.x) || (need_down && !a.out))
     return fail(WX_ERR_INVALID_ARGUMENT, "%s: null pointer", who);
