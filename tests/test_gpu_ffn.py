@@ -250,3 +250,44 @@ def test_config4_skewed_and_empty_groups(dev):
         rows = torch.cat([torch.arange(0, 4096, 173), torch.arange(4096, 4096 + n_act)])
         ref = oracle.sparse_moe_block_ref(x[rows][None], types[rows][None], [w.as_tuple() for w in ws])[0]
         _close(y[rows.to(dev)], ref, what=f"prefill + {n_act} action")
+
+
+@pytest.mark.parametrize("fused_extras", [False, True])
+def test_moe_block_backward_matches_autograd_of_the_plain_forward(dev, fused_extras):
+    """Gradients of the block (inputs and all six weights) against torch autograd through the oracle's fp32
+    forward; with fused_extras the layer's RMSNorm and residual ride along (PyTorch ops under autograd)."""
+    class Cfg:
+        experts = [{"hidden_size": 128, "intermediate_size": 256, "hidden_act": "silu"},
+                   {"hidden_size": 128, "intermediate_size": 64, "hidden_act": "silu"}]
+
+    g = torch.Generator().manual_seed(12)
+    block = moe.SparseMoeBlock(Cfg(), 2).to(torch.bfloat16)
+    with torch.no_grad():
+        for prm in block.parameters():
+            prm.copy_(_bf(prm.shape, g, 0.08))
+    x = _bf((1, 203, 128), g)
+    types = torch.rand(1, 203, generator=g) > 0.7
+    dy = _bf((1, 203, 128), g)
+    nw = (1.0 + 0.1 * torch.randn(128, generator=g)).to(torch.bfloat16)
+    # reference: fp32 leaves, oracle forward, torch autograd
+    xr = x.float().requires_grad_(True)
+    wr = [tuple(w.detach().float().requires_grad_(True) for w in e.weights()) for e in block.experts]
+    hin = oracle.rms_norm_ref(xr, nw.float(), 1e-6) if fused_extras else xr
+    yr = oracle.sparse_moe_block_ref(hin, types, wr, eager_rounding=False)
+    if fused_extras:
+        yr = xr + yr
+    yr.backward(dy.float())
+    # kernels
+    block = block.to(dev)
+    xd = x.to(dev).requires_grad_(True)
+    kw = dict(pre_norm=(nw.to(dev), 1e-6), residual=True) if fused_extras else {}
+    yd = block(xd, types.to(dev), **kw)
+    _close(yd, yr.detach(), atol=3e-2, rtol=2e-2, what="forward under autograd")
+    yd.backward(dy.to(dev))
+    _close(xd.grad, xr.grad, atol=3e-2, rtol=3e-2, what="grad of the input")
+    for e in range(2):
+        for name, wref in zip(("gate", "up", "down"), wr[e]):
+            got = getattr(block.experts[e], f"{name}_proj").weight.grad
+            scale = float(wref.grad.abs().max())
+            err = float((got.float().cpu() - wref.grad).abs().max())
+            assert err <= 0.03 * scale + 1e-3, f"expert {e} {name}: max err {err} at scale {scale}"

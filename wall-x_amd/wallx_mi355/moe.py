@@ -48,7 +48,7 @@ class Routing:
 
 
 class _DualExpertFFN(torch.autograd.Function):
-    """Inference-only for now: the fused path has no backward (training falls outside this build's scope)."""
+    """The fused forward (tiled activations in, sorted rows out); used when nothing needs a gradient."""
 
     @staticmethod
     def forward(ctx, x_tiled, num_rows, expert_offsets, hmid, *weights):
@@ -57,7 +57,83 @@ class _DualExpertFFN(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, grad):
-        raise NotImplementedError("wallx_mi355.moe: the fused dual-expert FFN implements the forward pass only")
+        raise NotImplementedError("wallx_mi355.moe: gradients go through _MoeBlockFunction, not the fused forward")
+
+
+def _pad_rows8(t: torch.Tensor) -> torch.Tensor:
+    """Zero rows up to a multiple of 8 (the transposed GEMM layouts want 16-byte rows after transposition)."""
+    extra = (-t.size(0)) % 8
+    return t if extra == 0 else torch.cat((t, t.new_zeros(extra, t.size(1))))
+
+
+def _dual(a0, a1, w0, w1, n0, n1, trans_a, trans_b):
+    m0 = a0.size(1) if trans_a else a0.size(0)
+    m1 = a1.size(1) if trans_a else a1.size(0)
+    o0 = torch.empty(m0, n0, dtype=torch.bfloat16, device=a0.device)
+    o1 = torch.empty(m1, n1, dtype=torch.bfloat16, device=a0.device)
+    native.asym_dual_gmm(a0, a1, w0, w1, o0, o1, trans_a, trans_b)
+    return o0, o1
+
+
+class _MoeBlockFunction(torch.autograd.Function):
+    """permute -> both experts' SwiGLU FFN -> unpermute with a backward (act.py:105-162 under autograd).
+
+    Forward is the fused path.  Backward recomputes gate and up (they are not kept by the fused kernels) and runs
+    every contraction of both experts as one dual GEMM: dHm = dY Wd, dWd = dY^T Hm, dX = dG Wg + dU Wu,
+    dWg = dG^T X, dWu = dU^T X, with the SwiGLU derivative elementwise in fp32.  The per-expert row counts are
+    read back from the device once per backward (the forward never synchronises)."""
+
+    @staticmethod
+    def forward(ctx, x, row_id_map, expert_offsets, sorted_row_id, scratch, *weights):
+        T = x.size(0)
+        scratch["x_tiled"] = native.permute_rows_tiled(x, row_id_map, expert_offsets, scratch.get("x_tiled"),
+                                                       sorted_row_id)
+        w = ((weights[0], weights[1], weights[2]), (weights[3], weights[4], weights[5]))
+        y_sorted = native.dual_swiglu_ffn(scratch["x_tiled"], T, expert_offsets, w, hmid=scratch.get("hmid"))
+        ctx.save_for_backward(x, row_id_map, expert_offsets, *weights)
+        return native.unpermute(y_sorted, row_id_map, torch.tensor([]), T, 1)
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, row_id_map, expert_offsets, g0, u0, d0, g1, u1, d1 = ctx.saved_tensors
+        T, H = x.shape
+        o = expert_offsets.cpu().tolist()
+        m0, m1 = o[1] - o[0], o[2] - o[1]
+        xs = native.permute_rows(x.detach(), row_id_map, 1, T)
+        dys = native.permute_rows(dy.contiguous().to(torch.bfloat16), row_id_map, 1, T)
+        x0, x1 = _pad_rows8(xs[:m0]), _pad_rows8(xs[m0:m0 + m1])
+        dy0, dy1 = _pad_rows8(dys[:m0]), _pad_rows8(dys[m0:m0 + m1])
+        I0, I1 = g0.size(0), g1.size(0)
+        ga0, ga1 = _dual(x0, x1, g0, g1, I0, I1, False, True)
+        up0, up1 = _dual(x0, x1, u0, u1, I0, I1, False, True)
+        dh0, dh1 = _dual(dy0, dy1, d0, d1, I0, I1, False, False)
+
+        def swiglu_grads(ga, up, dh):
+            g, u, d = ga.float(), up.float(), dh.float()
+            sig = torch.sigmoid(g)
+            silu = g * sig
+            hm = (silu.to(torch.bfloat16).float() * u).to(torch.bfloat16)  # what the forward fed to the down GEMM
+            dg = (d * u * sig * (1.0 + g * (1.0 - sig))).to(torch.bfloat16)
+            du = (d * silu).to(torch.bfloat16)
+            return hm, dg, du
+
+        hm0, dg0, du0 = swiglu_grads(ga0, up0, dh0)
+        hm1, dg1, du1 = swiglu_grads(ga1, up1, dh1)
+        need = ctx.needs_input_grad
+        grads = [None] * 6
+        if need[5] or need[8]:  # gate weights
+            grads[0], grads[3] = _dual(dg0, dg1, x0, x1, H, H, True, False)
+        if need[6] or need[9]:  # up weights
+            grads[1], grads[4] = _dual(du0, du1, x0, x1, H, H, True, False)
+        if need[7] or need[10]:  # down weights
+            grads[2], grads[5] = _dual(dy0, dy1, hm0, hm1, I0, I1, True, False)
+        dx = None
+        if need[0]:
+            a0, a1 = _dual(dg0, dg1, g0, g1, H, H, False, False)
+            b0, b1 = _dual(du0, du1, u0, u1, H, H, False, False)
+            dxs = torch.cat(((a0.float() + b0.float())[:m0], (a1.float() + b1.float())[:m1])).to(torch.bfloat16)
+            dx = native.unpermute(dxs, row_id_map, torch.tensor([]), T, 1)
+        return (dx, None, None, None, None, *grads)
 
 
 class SparseMoeBlock(nn.Module):
@@ -102,6 +178,24 @@ class SparseMoeBlock(nn.Module):
             routing = self.route(experts_indices)
         if routing.num_tokens != x.size(0):
             raise RuntimeError(f"routing was built for {routing.num_tokens} tokens, got {x.size(0)}")
+        flat = [w for e in self.experts for w in e.weights()]
+        need = native.padded_sorted_rows(x.size(0)) * max(e.intermediate_size for e in self.experts)
+        if self._hmid is None or self._hmid.numel() < need or self._hmid.device != x.device:
+            self._hmid = torch.empty(need, dtype=torch.bfloat16, device=x.device)
+        if torch.is_grad_enabled() and (x.requires_grad or any(w.requires_grad for w in flat)):
+            # training: norm and residual stay PyTorch ops (autograd differentiates them), the block itself has
+            # its own backward
+            xin = x
+            if pre_norm is not None:
+                norm_weight, eps = pre_norm
+                xin = torch.nn.functional.rms_norm(x, (hidden,), norm_weight, eps)
+            scratch = {"x_tiled": self._x_tiled, "hmid": self._hmid}
+            y = _MoeBlockFunction.apply(xin, routing.row_id_map, routing.expert_offsets, routing.sorted_row_id,
+                                        scratch, *flat)
+            self._x_tiled = scratch["x_tiled"]
+            if residual:
+                y = x + y
+            return y.view(batch, seq, hidden)
         if pre_norm is not None:
             norm_weight, eps = pre_norm
             self._x_tiled = native.rmsnorm_permute_rows_tiled(x, norm_weight, eps, routing.expert_offsets,
@@ -109,10 +203,6 @@ class SparseMoeBlock(nn.Module):
         else:
             self._x_tiled = native.permute_rows_tiled(x, routing.row_id_map, routing.expert_offsets, self._x_tiled,
                                                       routing.sorted_row_id)
-        need = native.padded_sorted_rows(x.size(0)) * max(e.intermediate_size for e in self.experts)
-        if self._hmid is None or self._hmid.numel() < need or self._hmid.device != x.device:
-            self._hmid = torch.empty(need, dtype=torch.bfloat16, device=x.device)
-        flat = [w for e in self.experts for w in e.weights()]
         y_sorted = _DualExpertFFN.apply(self._x_tiled, x.size(0), routing.expert_offsets, self._hmid, *flat)
         if residual:
             y = native.unpermute_add(y_sorted, x, routing.row_id_map)
