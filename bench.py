@@ -38,7 +38,7 @@ def parse():
     ap.add_argument("--ops-only", action="store_true", help="skip the side measurements (M-RoPE, index builders)")
     ap.add_argument("--no-prefill", action="store_true", help="skip the config 5 prefill measurement (36-layer decoder)")
     ap.add_argument("--prefill-mask", default="causal", choices=["causal", "action_block"])
-    ap.add_argument("--cpu-seqs", type=int, default=4, help="sequences of the batch the CPU baseline runs")
+    ap.add_argument("--cpu-seqs", type=int, default=16, help="sequences of the batch the CPU baseline runs")
     ap.add_argument("--kernel-loop", default=None,
                     choices=["gate_up", "down", "permute", "permute_plain", "unpermute", "partition", "copy"],
                     help="profiling aid: run only this kernel --steps times (no JSON line); 'copy' is a plain "
