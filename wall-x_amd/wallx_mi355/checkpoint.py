@@ -1,0 +1,85 @@
+"""Expert weights of a wall-x checkpoint -> `wallx_mi355.moe.SparseMoeBlock` modules.
+
+The reference stores its weights as safetensors files in the model directory and loads every tensor into one
+state dict (act.py:785-794).  Expert e of decoder layer L lives under
+``model.layers.{L}.moe.experts.{e}.{gate,up,down}_proj.weight``; when training starts from a dense Qwen2.5-VL
+checkpoint, the trainer renames ``model.layers.{L}.mlp.*`` to ``...moe.experts.0.*`` and leaves the action expert at
+its initialisation (qwen_vl_act_trainer.py:657-671).  Both conventions are handled here.
+
+Only safetensors are read (no pickles are ever loaded), one tensor at a time, so a multi-file checkpoint never
+sits in host memory as a whole.
+"""
+
+import glob
+import os
+import re
+from typing import Dict, Iterable, Mapping, Optional
+
+import torch
+
+_EXPERT_KEY = re.compile(r"(?:^|\.)layers\.(\d+)\.moe\.experts\.(\d+)\.(gate|up|down)_proj\.weight$")
+_DENSE_KEY = re.compile(r"(?:^|\.)layers\.(\d+)\.mlp\.(gate|up|down)_proj\.weight$")
+
+
+def expert_weight_key(layer: int, expert: int, proj: str, prefix: str = "model.") -> str:
+    return f"{prefix}layers.{layer}.moe.experts.{expert}.{proj}_proj.weight"
+
+
+def classify_key(key: str, dense_as_expert0: bool = True):
+    """(layer, expert, proj) for a key that holds an expert projection weight, else None."""
+    m = _EXPERT_KEY.search(key)
+    if m:
+        return int(m.group(1)), int(m.group(2)), m.group(3)
+    if dense_as_expert0:
+        m = _DENSE_KEY.search(key)
+        if m:
+            return int(m.group(1)), 0, m.group(2)
+    return None
+
+
+def iter_safetensors(path: str) -> Iterable:
+    """Yields (key, tensor) over every *.safetensors file of a directory (or over one file)."""
+    from safetensors import safe_open
+
+    files = [path] if os.path.isfile(path) else sorted(glob.glob(os.path.join(path, "*.safetensors")))
+    if not files:
+        raise FileNotFoundError(f"no safetensors files under {path}")
+    for f in files:
+        with safe_open(f, framework="pt", device="cpu") as handle:
+            for key in handle.keys():
+                yield key, handle.get_tensor(key)
+
+
+def load_expert_weights(source, blocks: Mapping[int, torch.nn.Module], dense_as_expert0: bool = True,
+                        strict: bool = True) -> Dict[int, int]:
+    """Copies expert projection weights into `blocks` (decoder layer index -> SparseMoeBlock).
+
+    source: a checkpoint directory / safetensors file, or an already loaded state dict.
+    Returns {layer: number of tensors loaded}.  With strict=True every block must receive all six tensors unless
+    the checkpoint is a dense one (then expert 0's three).  Shapes and the bf16 requirement of the kernels are
+    checked; the packed copies the kernels read are rebuilt lazily because the parameters are modified in place.
+    """
+    items = source.items() if isinstance(source, Mapping) else iter_safetensors(source)
+    loaded: Dict[int, set] = {layer: set() for layer in blocks}
+    for key, tensor in items:
+        hit = classify_key(key, dense_as_expert0)
+        if hit is None:
+            continue
+        layer, expert, proj = hit
+        block = blocks.get(layer)
+        if block is None or expert >= len(block.experts):
+            continue
+        param = getattr(block.experts[expert], f"{proj}_proj").weight
+        if tuple(param.shape) != tuple(tensor.shape):
+            raise ValueError(f"{key}: checkpoint shape {tuple(tensor.shape)} != module shape {tuple(param.shape)}")
+        with torch.no_grad():
+            param.copy_(tensor.to(device=param.device, dtype=param.dtype))
+        loaded[layer].add((expert, proj))
+    if strict:
+        for layer, got in loaded.items():
+            experts_seen = {e for e, _ in got}
+            for e in experts_seen or {0}:
+                missing = {"gate", "up", "down"} - {p for ee, p in got if ee == e}
+                if missing:
+                    raise KeyError(f"layer {layer}, expert {e}: missing {sorted(missing)} projection weights")
+    return {layer: len(got) for layer, got in loaded.items()}
