@@ -171,6 +171,20 @@ def main():
     t_perm_plain, _ = event_ms(permute_plain, iters, batch=10)
     t_unperm, _ = event_ms(unpermute, iters, batch=10)
     t_part, _ = event_ms(partition, iters)
+    # the caller fusions: RMSNorm inside the tiled permute, residual add inside the unpermute
+    norm_w = torch.ones(H, dtype=torch.bfloat16, device=dev)
+
+    def norm_permute():
+        _lib.call("wx_rmsnorm_permute_rows_tiled", x.data_ptr(), norm_w.data_ptr(), 1e-6, x_tiled.data_ptr(),
+                  inverse.data_ptr(), offsets.data_ptr(), T, H, stream)
+
+    def unpermute_add():
+        _lib.call("wx_unpermute_rows_add", y_sorted.data_ptr(), x.data_ptr(), y.data_ptr(), row_id_map.data_ptr(), T, H,
+                  stream)
+
+    t_np, _ = event_ms(norm_permute, iters, batch=10)
+    t_ua, _ = event_ms(unpermute_add, iters, batch=10)
+    permute()  # x_tiled back to the plain permute's contents for anything that runs after this
     gate_up_tflops = gate_up_flops / (t_gate_up_avg * 1e-3) / 1e12
 
     extra = {
@@ -182,6 +196,9 @@ def main():
         "unpermute_ms": round(t_unperm, 4), "unpermute_GBps": round(row_bytes / t_unperm / 1e6, 1),
         "permute_frac_hbm_peak": round(row_bytes / t_perm / 1e6 / PEAK_HBM_GBS, 4),
         "partition_us": round(t_part * 1e3, 2),
+        "rmsnorm_permute_ms": round(t_np, 4), "rmsnorm_permute_GBps": round(row_bytes / t_np / 1e6, 1),
+        "unpermute_residual_ms": round(t_ua, 4),
+        "unpermute_residual_GBps": round((row_bytes + 2.0 * T * H) / t_ua / 1e6, 1),  # one more [T, H] read
     }
 
     if not args.ops_only:

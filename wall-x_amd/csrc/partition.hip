@@ -80,8 +80,20 @@ __global__ __launch_bounds__(kBlock) void partition_scatter(
   const int64_t first_seg = static_cast<int64_t>(blockIdx.x) * kWavesPerBlock;
 
   // bin `tid`: rows of this bin in all segments (total) and in segments before this block (before)
+  // (eight independent loads per trip: with one load per trip the loop costs a memory latency per segment)
   int32_t total = 0, before = 0;
-  for (int64_t s = 0; s < num_seg; ++s) {
+  int64_t s = 0;
+  for (; s + 8 <= num_seg; s += 8) {
+    int32_t v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = hist[(s + u) * kBins + tid];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      total += v[u];
+      if (s + u < first_seg) before += v[u];
+    }
+  }
+  for (; s < num_seg; ++s) {
     const int32_t v = hist[s * kBins + tid];
     total += v;
     if (s < first_seg) before += v;
