@@ -127,7 +127,8 @@ int wx_permute_rows_tiled(const void* x, void* out_tiled, const int32_t* row_id_
 int wx_dual_swiglu_ffn(const void* x_tiled, void* out, const int32_t* expert_offsets, const void* gate0,
                        const void* up0, const void* down0, const void* gate1, const void* up1,
                        const void* down1, void* hmid, int64_t num_rows, int64_t hidden,
-                       int64_t inter0, int64_t inter1, wx_stream_t stream);
+                       int64_t inter0, int64_t inter1, const int64_t* host_rows_per_expert,
+                       wx_stream_t stream);
 
 /* The two launches of wx_dual_swiglu_ffn on their own, for callers that put work between them (and for
  * timing each kernel): hmid = silu(x @ gate^T) * (x @ up^T), then out = hmid @ down^T, per expert.
@@ -135,10 +136,15 @@ int wx_dual_swiglu_ffn(const void* x_tiled, void* out, const int32_t* expert_off
 int wx_dual_swiglu_gate_up(const void* x_tiled, void* hmid, const int32_t* expert_offsets,
                            const void* gate0, const void* up0, const void* gate1, const void* up1,
                            int64_t num_rows, int64_t hidden, int64_t inter0, int64_t inter1,
-                           wx_stream_t stream);
+                           const int64_t* host_rows_per_expert, wx_stream_t stream);
 int wx_dual_down_proj(const void* hmid, void* out, const int32_t* expert_offsets, const void* down0,
                       const void* down1, int64_t num_rows, int64_t hidden, int64_t inter0,
-                      int64_t inter1, wx_stream_t stream);
+                      int64_t inter1, const int64_t* host_rows_per_expert, wx_stream_t stream);
+/* host_rows_per_expert (optional, may be NULL): HOST int64[2], the rows of each expert when the caller already
+ * has them on the host (the reference computes them there, act.py:1274-1283).  They only steer the choice between
+ * the two tile shapes: without them, a call whose bounds on the tile count straddle the threshold launches both
+ * shapes and the device decides (one of the launches returns at once).  The kernels always take the row ranges
+ * from expert_offsets on the device; a hint that disagrees with them costs speed, never correctness. */
 
 /* ------------------------------------------------------------------------------------------------
  * 3D multimodal RoPE:  out = x * cos_sel + rotate_half(x) * sin_sel for q and k, where channel d of

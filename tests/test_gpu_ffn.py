@@ -237,6 +237,10 @@ def test_config4_skewed_and_empty_groups(dev):
     assert r.expert_offsets.cpu().tolist() == [0, 0, 2048]
     rows = torch.arange(0, 2048, 37)
     _close(y[rows.to(dev)], oracle.swiglu_ffn_ref(x[rows], *ws[1].as_tuple()), what="denoise step")
+    # row counts handed over from the host only pick the tile shape: same result, right or wrong
+    for hint in ((0, 2048), (2048, 0)):
+        yh, _ = moe.moe_layer_forward(x.to(dev), types.to(dev), wd, host_rows=hint)
+        assert int((yh != y).sum()) == 0
     # the same step next to a wide VL expert: the host cannot tell which tile shape fits (the row split is on the
     # device), so both are launched and the device picks
     ws_wide = _moe_weights(2048, (4096, 1024), g, 0.02)

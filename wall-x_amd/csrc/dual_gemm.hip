@@ -790,6 +790,7 @@ namespace {
 struct FfnArgs {
   const void *x, *gate[2], *up[2], *down[2];
   void *out, *hmid;
+  const int64_t* host_rows;  // optional: rows of each expert as the caller knows them on the host
   const int32_t* offsets;
   int64_t rows, hidden, inter[2];
 };
@@ -799,6 +800,8 @@ int check_ffn(const char* who, const FfnArgs& a, bool need_gate_up, bool need_do
   if (int rc = check_dims(who, a.rows, a.hidden, a.inter[1])) return rc;
   if (a.hidden % kBlkCols != 0 || a.inter[0] % kBlkCols != 0 || a.inter[1] % kBlkCols != 0)
     return fail(WX_ERR_UNSUPPORTED, "%s: hidden and intermediate sizes must be multiples of 32", who);
+  if (a.host_rows != nullptr && (a.host_rows[0] < 0 || a.host_rows[1] < 0 || a.host_rows[0] + a.host_rows[1] != a.rows))
+    return fail(WX_ERR_INVALID_ARGUMENT, "%s: host_rows_per_expert must be non-negative and sum to num_rows", who);
   if (a.hidden == 0 || a.inter[0] == 0 || a.inter[1] == 0)
     return fail(WX_ERR_UNSUPPORTED, "%s: hidden and both intermediate sizes must be positive", who);
   if (a.rows == 0) return WX_OK;
@@ -831,8 +834,12 @@ int launch_gate_up(const FfnArgs& a, hipStream_t s) {
     g.a_row0 = 0;
   }
   p.offsets = a.offsets;
-  // the split of the rows between the experts is only known on the device: bound the tile count from the total
   const int64_t t0 = ceil_div(a.inter[0], BigTile::BN / 2), t1 = ceil_div(a.inter[1], BigTile::BN / 2);
+  if (a.host_rows != nullptr) {  // the caller knows the split: one launch of the right tile shape
+    const int64_t tiles = ceil_div(a.host_rows[0], BigTile::BM) * t0 + ceil_div(a.host_rows[1], BigTile::BM) * t1;
+    return launch_mfma<kGateUp>(p, tiles, tiles, s, "dual_gemm_kernel<gate_up>");
+  }
+  // the split of the rows between the experts is only known on the device: bound the tile count from the total
   const int64_t row_tiles = ceil_div(a.rows, BigTile::BM);
   return launch_mfma<kGateUp>(p, row_tiles * (t0 < t1 ? t0 : t1), (row_tiles + 1) * (t0 > t1 ? t0 : t1), s,
                               "dual_gemm_kernel<gate_up>");
@@ -854,7 +861,12 @@ int launch_down(const FfnArgs& a, hipStream_t s) {
     g.a_row0 = 0;
   }
   p.offsets = a.offsets;
-  const int64_t row_tiles = ceil_div(a.rows, BigTile::BM), col_tiles = ceil_div(a.hidden, BigTile::BN);
+  const int64_t col_tiles = ceil_div(a.hidden, BigTile::BN);
+  if (a.host_rows != nullptr) {
+    const int64_t tiles = (ceil_div(a.host_rows[0], BigTile::BM) + ceil_div(a.host_rows[1], BigTile::BM)) * col_tiles;
+    return launch_mfma<kDown>(p, tiles, tiles, s, "dual_gemm_kernel<down>");
+  }
+  const int64_t row_tiles = ceil_div(a.rows, BigTile::BM);
   return launch_mfma<kDown>(p, row_tiles * col_tiles, (row_tiles + 1) * col_tiles, s, "dual_gemm_kernel<down>");
 }
 
@@ -863,8 +875,8 @@ int launch_down(const FfnArgs& a, hipStream_t s) {
 extern "C" int wx_dual_swiglu_gate_up(const void* x_tiled, void* hmid, const int32_t* expert_offsets,
                                       const void* gate0, const void* up0, const void* gate1, const void* up1,
                                       int64_t num_rows, int64_t hidden, int64_t inter0, int64_t inter1,
-                                      wx_stream_t stream) {
-  const FfnArgs a{x_tiled, {gate0, gate1}, {up0, up1}, {nullptr, nullptr}, nullptr, hmid, expert_offsets,
+                                      const int64_t* host_rows_per_expert, wx_stream_t stream) {
+  const FfnArgs a{x_tiled, {gate0, gate1}, {up0, up1}, {nullptr, nullptr}, nullptr, hmid, host_rows_per_expert, expert_offsets,
                   num_rows, hidden, {inter0, inter1}};
   if (int rc = check_ffn("wx_dual_swiglu_gate_up", a, true, false)) return rc;
   if (num_rows == 0) return WX_OK;
@@ -873,9 +885,9 @@ extern "C" int wx_dual_swiglu_gate_up(const void* x_tiled, void* hmid, const int
 
 extern "C" int wx_dual_down_proj(const void* hmid, void* out, const int32_t* expert_offsets, const void* down0,
                                  const void* down1, int64_t num_rows, int64_t hidden, int64_t inter0,
-                                 int64_t inter1, wx_stream_t stream) {
+                                 int64_t inter1, const int64_t* host_rows_per_expert, wx_stream_t stream) {
   const FfnArgs a{nullptr, {nullptr, nullptr}, {nullptr, nullptr}, {down0, down1}, out, const_cast<void*>(hmid),
-                  expert_offsets, num_rows, hidden, {inter0, inter1}};
+                  host_rows_per_expert, expert_offsets, num_rows, hidden, {inter0, inter1}};
   if (int rc = check_ffn("wx_dual_down_proj", a, false, true)) return rc;
   if (num_rows == 0) return WX_OK;
   return launch_down(a, as_stream(stream));
@@ -884,8 +896,8 @@ extern "C" int wx_dual_down_proj(const void* hmid, void* out, const int32_t* exp
 extern "C" int wx_dual_swiglu_ffn(const void* x_tiled, void* out, const int32_t* expert_offsets, const void* gate0,
                                   const void* up0, const void* down0, const void* gate1, const void* up1,
                                   const void* down1, void* hmid, int64_t num_rows, int64_t hidden, int64_t inter0,
-                                  int64_t inter1, wx_stream_t stream) {
-  const FfnArgs a{x_tiled, {gate0, gate1}, {up0, up1}, {down0, down1}, out, hmid, expert_offsets,
+                                  int64_t inter1, const int64_t* host_rows_per_expert, wx_stream_t stream) {
+  const FfnArgs a{x_tiled, {gate0, gate1}, {up0, up1}, {down0, down1}, out, hmid, host_rows_per_expert, expert_offsets,
                   num_rows, hidden, {inter0, inter1}};
   if (int rc = check_ffn("wx_dual_swiglu_ffn", a, true, true)) return rc;
   if (num_rows == 0) return WX_OK;

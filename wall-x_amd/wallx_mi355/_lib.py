@@ -33,9 +33,9 @@ PROTOTYPES = {
     "wx_padded_sorted_rows": (_i64, [_i64]),
     "wx_pack_tiled": (_i32, [_vp, _vp, _i64, _i64, _vp]),
     "wx_permute_rows_tiled": (_i32, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _vp]),
-    "wx_dual_swiglu_ffn": (_i32, [_vp] * 10 + [_i64] * 4 + [_vp]),
-    "wx_dual_swiglu_gate_up": (_i32, [_vp] * 7 + [_i64] * 4 + [_vp]),
-    "wx_dual_down_proj": (_i32, [_vp] * 5 + [_i64] * 4 + [_vp]),
+    "wx_dual_swiglu_ffn": (_i32, [_vp] * 10 + [_i64] * 4 + [_vp, _vp]),
+    "wx_dual_swiglu_gate_up": (_i32, [_vp] * 7 + [_i64] * 4 + [_vp, _vp]),
+    "wx_dual_down_proj": (_i32, [_vp] * 5 + [_i64] * 4 + [_vp, _vp]),
     "wx_mrope_apply": (_i32, [_vp] * 6 + [_i64, _i64, _i32, _i32, _i32] + [_c.POINTER(_i64)] * 4
                        + [_c.POINTER(_i32), _i32, _i32, _vp]),
     "wx_mrope_apply_bwd": (_i32, [_vp] * 6 + [_i64, _i64, _i32, _i32, _i32] + [_c.POINTER(_i64)] * 4
@@ -88,6 +88,11 @@ def check(rc: int, exc=RuntimeError):
 
 def call(name: str, *args, exc=RuntimeError):
     check(getattr(load(), name)(*args), exc)
+
+
+def i64x2(vals):
+    """Host int64[2] for the optional per-expert row counts of the FFN entry points; None stays NULL."""
+    return None if vals is None else (_i64 * 2)(int(vals[0]), int(vals[1]))
 
 
 def i64x3(vals):

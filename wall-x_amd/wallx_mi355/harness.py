@@ -116,10 +116,10 @@ class PrefillHarness:
         with timer.section("ffn_gate_up_swiglu"):
             _lib.call("wx_dual_swiglu_gate_up", self._x_tiled.data_ptr(), self._hmid.data_ptr(),
                       routing.expert_offsets.data_ptr(), g0.data_ptr(), u0.data_ptr(), g1.data_ptr(), u1.data_ptr(),
-                      T, H, I0, I1, stream)
+                      T, H, I0, I1, None, stream)
         with timer.section("ffn_down"):
             _lib.call("wx_dual_down_proj", self._hmid.data_ptr(), y_sorted.data_ptr(), routing.expert_offsets.data_ptr(),
-                      d0.data_ptr(), d1.data_ptr(), T, H, I0, I1, stream)
+                      d0.data_ptr(), d1.data_ptr(), T, H, I0, I1, None, stream)
         if self.fuse:
             with timer.section("unpermute+residual"):
                 return native.unpermute_add(y_sorted, h, routing.row_id_map)

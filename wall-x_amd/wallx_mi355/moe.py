@@ -51,9 +51,9 @@ class _DualExpertFFN(torch.autograd.Function):
     """The fused forward (tiled activations in, sorted rows out); used when nothing needs a gradient."""
 
     @staticmethod
-    def forward(ctx, x_tiled, num_rows, expert_offsets, hmid, *weights):
+    def forward(ctx, x_tiled, num_rows, expert_offsets, hmid, host_rows, *weights):
         w = ((weights[0], weights[1], weights[2]), (weights[3], weights[4], weights[5]))
-        return native.dual_swiglu_ffn(x_tiled, num_rows, expert_offsets, w, hmid=hmid)
+        return native.dual_swiglu_ffn(x_tiled, num_rows, expert_offsets, w, hmid=hmid, host_rows=host_rows)
 
     @staticmethod
     def backward(ctx, grad):
@@ -161,15 +161,20 @@ class SparseMoeBlock(nn.Module):
                 routing: Optional[Routing] = None, pre_norm=None, residual: bool = False) -> torch.Tensor:
         """hidden_states [B, S, H] bf16; experts_indices [B, S] (bool or integer expert id).
 
-        start_indices / end_indices are accepted for signature parity and not read: the row ranges come from
-        the partition on the device.
+        start_indices / end_indices (the reference's CPU tensors of per-expert row ranges, act.py:1274-1283) are
+        optional: the kernels take the row ranges from the partition on the device; when the caller passes them
+        anyway, their lengths tell the library which tile shape fits without a second launch.
 
         Two optional caller fusions (the decoder layer around this block, act.py:256-265):
         pre_norm=(weight, eps) applies the post-attention RMSNorm to hidden_states inside the permute, and
         residual=True returns hidden_states + block(...) with the add done inside the unpermute.  With both, the
         layer's `residual = h; h = norm(h); h = moe(h); h = residual + h` is `h = moe(h, ..., pre_norm, True)`.
         """
-        del start_indices, end_indices
+        host_rows = None
+        if start_indices is not None and end_indices is not None and not start_indices.is_cuda:
+            counts = (end_indices - start_indices).tolist()
+            if len(counts) == 2 and min(counts) >= 0 and sum(counts) == hidden_states.numel() // hidden_states.shape[-1]:
+                host_rows = counts
         batch, seq, hidden = hidden_states.shape
         x = hidden_states.reshape(-1, hidden)
         if x.dtype != torch.bfloat16:
@@ -203,7 +208,7 @@ class SparseMoeBlock(nn.Module):
         else:
             self._x_tiled = native.permute_rows_tiled(x, routing.row_id_map, routing.expert_offsets, self._x_tiled,
                                                       routing.sorted_row_id)
-        y_sorted = _DualExpertFFN.apply(self._x_tiled, x.size(0), routing.expert_offsets, self._hmid, *flat)
+        y_sorted = _DualExpertFFN.apply(self._x_tiled, x.size(0), routing.expert_offsets, self._hmid, host_rows, *flat)
         if residual:
             y = native.unpermute_add(y_sorted, x, routing.row_id_map)
         else:
@@ -212,7 +217,7 @@ class SparseMoeBlock(nn.Module):
 
 
 def moe_layer_forward(x: torch.Tensor, token_types: torch.Tensor, weights, routing: Optional[Routing] = None,
-                      hmid: Optional[torch.Tensor] = None, workspace=None):
+                      hmid: Optional[torch.Tensor] = None, workspace=None, host_rows=None):
     """Functional form of one layer: permute -> dual-expert SwiGLU FFN -> unpermute.
 
     x [T, H] bf16, token_types [T] (bool / int), weights ((g0,u0,d0),(g1,u1,d1)).  Returns (y [T, H], routing).
@@ -221,6 +226,7 @@ def moe_layer_forward(x: torch.Tensor, token_types: torch.Tensor, weights, routi
         row_id_map, offsets, inverse, _ = native.partition(token_types.reshape(-1), 2, 0, workspace, want_sorted=True)
         routing = Routing(row_id_map, offsets, x.size(0), inverse)
     x_tiled = native.permute_rows_tiled(x, routing.row_id_map, routing.expert_offsets, None, routing.sorted_row_id)
-    y_sorted = native.dual_swiglu_ffn(x_tiled, x.size(0), routing.expert_offsets, weights, hmid=hmid)
+    y_sorted = native.dual_swiglu_ffn(x_tiled, x.size(0), routing.expert_offsets, weights, hmid=hmid,
+                                      host_rows=host_rows)
     y = native.unpermute(y_sorted, routing.row_id_map, torch.tensor([]), x.size(0), 1)
     return y, routing

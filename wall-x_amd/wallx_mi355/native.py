@@ -466,12 +466,15 @@ def unpermute_add(y_sorted: torch.Tensor, residual: torch.Tensor, row_id_map: to
 
 
 def dual_swiglu_ffn(x_tiled: torch.Tensor, num_rows: int, expert_offsets: torch.Tensor, weights,
-                    hmid: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                    hmid: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
+                    host_rows=None) -> torch.Tensor:
     """Both experts' SwiGLU FFN over expert-sorted rows in two launches (act.py:79-82, 142-154).
 
     x_tiled: result of permute_rows_tiled for num_rows tokens; expert_offsets int32 [3] ON THE DEVICE (from
     partition()); weights = ((gate0, up0, down0), (gate1, up1, down1)) in nn.Linear layout (packed and cached
-    here).  Returns out [num_rows, hidden] bf16 in sorted order.
+    here).  host_rows: optional (rows of expert 0, rows of expert 1) as host integers, when the caller has them
+    anyway; they only spare the library a second, empty launch when it cannot tell which tile shape fits.
+    Returns out [num_rows, hidden] bf16 in sorted order.
     """
     _need_cuda("x_tiled", x_tiled)
     (g0, u0, d0), (g1, u1, d1) = weights
@@ -492,5 +495,5 @@ def dual_swiglu_ffn(x_tiled: torch.Tensor, num_rows: int, expert_offsets: torch.
     with _DeviceGuard(x_tiled):
         _lib.call("wx_dual_swiglu_ffn", x_tiled.data_ptr(), _ptr(out), expert_offsets.data_ptr(), _ptr(packed[0]),
                   _ptr(packed[1]), _ptr(packed[2]), _ptr(packed[3]), _ptr(packed[4]), _ptr(packed[5]),
-                  hmid.data_ptr(), int(num_rows), H, I0, I1, _stream(x_tiled))
+                  hmid.data_ptr(), int(num_rows), H, I0, I1, _lib.i64x2(host_rows), _stream(x_tiled))
     return out
