@@ -449,15 +449,16 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
   // register's row, odd lanes the odd register's row), written to this wave's staging area as dwords, and read
   // back as 16-byte lanes laid out the way the destination wants them.
   unsigned char* stage = s_out + wave * kStageBytes;
-  auto swap_adjacent = [](float v) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));
-  };
   // Stores register pair (r, r+1) of one 32x32 block -- rows srow and srow + 1, column scol of this lane -- into
   // the staging area with row pitch `pitch` bytes.
   auto stage_pair = [&](float v0, float v1, int srow, int scol, int pitch, int odd) {
-    // even lane: (own v0, neighbour's v0) -> row srow; odd lane: (neighbour's v1, own v1) -> row srow + 1
-    const float recv = swap_adjacent(odd ? v0 : v1);
-    const uint32_t packed = odd ? pack_bf16x2(recv, v1) : pack_bf16x2(v0, recv);
+    // both values are converted at once (low half v0, high half v1) and the pair is swapped with the neighbour;
+    // even lane keeps (own v0, neighbour's v0) -> row srow; odd lane (neighbour's v1, own v1) -> row srow + 1.
+    // One byte permute picks the two halves: selector bytes 0-3 address `theirs`, 4-7 address `mine`.
+    const uint32_t mine = pack_bf16x2(v0, v1);
+    const uint32_t theirs = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(mine), 0xB1, 0xF, 0xF, true));
+    const uint32_t sel = odd ? 0x07060302u : 0x01000504u;
+    const uint32_t packed = __builtin_amdgcn_perm(mine, theirs, sel);
     *reinterpret_cast<uint32_t*>(stage + (srow + odd) * pitch + (scol & ~1) * 2) = packed;
   };
 
@@ -488,8 +489,9 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
               for (int q = 0; q < 2; ++q) {
                 // eager bf16 evaluation of act_fn(gate) * up (act.py:80-82): gate, up, silu(gate) and the
                 // product are each rounded to bf16
-                const float g = round_bf16(acc[i][j][r + q]);
-                const float u = round_bf16(acc[i][j + FN / 2][r + q]);
+                const uint32_t gu = pack_bf16x2(acc[i][j][r + q], acc[i][j + FN / 2][r + q]);  // one convert for both
+                const float g = __uint_as_float(gu << 16);
+                const float u = __uint_as_float(gu & 0xffff0000u);
                 const float sg = round_bf16(g * __builtin_amdgcn_rcpf(1.0f + __expf(-g)));
                 h[q] = sg * u;
               }
