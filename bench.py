@@ -367,6 +367,30 @@ def config4_measurement(dev, weights):
         flops = 6.0 * H * (n_vl * I0 + n_act * I1)
         out[name] = {"us": round(t * 1e3, 1), "tflops": round(flops / t / 1e9, 1),
                      "us_with_host_row_counts": round(th * 1e3, 1)}
+        if n_vl == 0:
+            # the denoise loop repeats this shape 10 x 36 times per action chunk: record 36 layers once into a HIP
+            # graph (the entry points neither allocate nor synchronise) and time its replays
+            layers = 36
+            routing = moe.moe_layer_forward(x, types, weights, host_rows=(n_vl, n_act))[1]
+
+            def stack():
+                h = x
+                for _ in range(layers):
+                    h = moe.moe_layer_forward(h, types, weights, routing=routing, host_rows=(n_vl, n_act))[0]
+                return h
+
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                stack()
+            torch.cuda.current_stream().wait_stream(side)
+            te, _ = event_ms(stack, 5, warm=2)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                stack()
+            tg, _ = event_ms(graph.replay, 10, warm=3)
+            out[name]["us_per_layer_eager_shared_routing"] = round(te * 1e3 / layers, 1)
+            out[name]["us_per_layer_hip_graph_replay"] = round(tg * 1e3 / layers, 1)
     return out
 
 
