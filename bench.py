@@ -301,6 +301,21 @@ def side_measurements(dev, iters):
     out["mrope_us"] = round(t * 1e3, 2)
     out["mrope_GBps"] = round(rope_bytes / t / 1e6, 1)
     out["mrope_frac_hbm_peak"] = round(rope_bytes / t / 1e6 / PEAK_HBM_GBS, 4)
+    # the same rotation with cos/sin evaluated in the kernel from position_ids and inv_freq: no tables are read
+    # (algorithmic bytes: q and k in and out plus the three int64 position planes), and the PyTorch ops that build
+    # the tables once per forward disappear
+    t, _ = event_ms(lambda: native.rope_from_positions(q, k, pos, inv, qo, ko, sec2), iters, batch=10)
+    pos_bytes = 2.0 * 2 * tokens * D * (wl.N_Q_HEADS + wl.N_KV_HEADS) + 3.0 * 8 * tokens
+    out["mrope_from_positions_us"] = round(t * 1e3, 2)
+    out["mrope_from_positions_GBps"] = round(pos_bytes / t / 1e6, 1)
+
+    def build_tables():
+        fr = pos.float()[..., None] * inv
+        e = torch.cat((fr, fr), -1)
+        return e.cos().to(torch.bfloat16), e.sin().to(torch.bfloat16)
+
+    t, _ = event_ms(build_tables, iters)
+    out["cos_sin_tables_torch_us"] = round(t * 1e3, 2)
     return out
 
 

@@ -171,6 +171,23 @@ int wx_mrope_apply_bwd(const void* gq_out, const void* gk_out, const void* cos, 
                        const int64_t gk_strides[3], const int mrope_section[3], int layout,
                        int dtype, wx_stream_t stream);
 
+/* The same rotation with the cos/sin builder folded in: instead of the two [3, B, S, D] tables the call takes
+ * what they are built from, position_ids [3, B, S] int64 (contiguous) and inv_freq [D/2] fp32, and every thread
+ * evaluates cos/sin of its own channels like Qwen2_5_VLRotaryEmbedding.forward does (vl.py:679-712): angle =
+ * fp32(position) * inv_freq[d mod D/2] in fp32, cos and sin in fp32, rounded to the dtype of q (attention_scaling
+ * is 1 for the default rope type, vl.py:635-678).  Replaces that builder plus apply_multimodal_rotary_pos_emb
+ * (vl.py:731-773) / the rope op (ops.py:402-497) in one pass; backward != 0 gives the adjoint (arguments as in
+ * wx_mrope_apply_bwd).  Results equal wx_mrope_apply on tables built in fp32 up to the last-place difference of
+ * the device's sincosf against the table builder's (a rounded bf16 cos/sin then differs in well under 1e-4 of the
+ * entries).  Heads must be 2..64 16-byte chunks, a power of two, with section ends on chunk boundaries;
+ * other shapes return WX_ERR_UNSUPPORTED (build the tables and call wx_mrope_apply). */
+int wx_mrope_apply_positions(const void* q, const void* k, const int64_t* position_ids, const float* inv_freq,
+                             void* q_out, void* k_out, int64_t batch, int64_t seq, int n_q_heads, int n_kv_heads,
+                             int head_dim, const int64_t q_strides[3], const int64_t k_strides[3],
+                             const int64_t qo_strides[3], const int64_t ko_strides[3],
+                             const int mrope_section[3], int layout, int dtype, int backward,
+                             wx_stream_t stream);
+
 /* ------------------------------------------------------------------------------------------------
  * 3D position ids.  Replaces get_rope_index (csrc/rope_index.cu:464-569) with the semantics of the
  * PyTorch path (act.py:929-1149), exact integer arithmetic.

@@ -74,6 +74,15 @@ def test_argument_errors_without_a_gpu():
     assert lib.wx_transpose_2d(None, None, 16, 16, 4, None) == -2  # element size
     assert lib.wx_transpose_2d(None, None, 16, 16, 2, None) == -1
     assert lib.wx_probe_mfma_rate(None, 10, None, None, None) == -1
+    # M-RoPE from positions: shapes the row kernel cannot take are refused, not routed elsewhere
+    st = _lib.i64x3((128 * 4, 128, 128 * 4))
+    assert lib.wx_mrope_apply_positions(None, None, None, None, None, None, 1, 4, 2, 1, 128, st, st, st, st,
+                                        _lib.i32x3((10, 27, 27)), 0, _lib.WX_BF16, 0, None) == -1  # null pointers
+    q = torch.zeros(8)
+    p_ = q.data_ptr()  # never dereferenced: the call fails on the host
+    assert lib.wx_mrope_apply_positions(p_, p_, p_, p_, p_, p_, 1, 4, 2, 1, 128, st, st, st, st,
+                                        _lib.i32x3((10, 27, 27)), 0, _lib.WX_BF16, 0, None) == -2
+    assert b"chunk boundaries" in lib.wx_last_error_string()
     assert lib.wx_probe_mfma_operand_bytes() == 4 * 8 * 64 * 16
 
 

@@ -114,3 +114,93 @@ def test_mrope_backward(dev, layout):
     rq, rk = oracle.mrope_apply_bwd_ref(gq, gk, cos, sin, list(wl.MROPE_SECTION), layout)
     assert torch.allclose(qd.grad.cpu(), rq, rtol=1e-5, atol=1e-5)
     assert torch.allclose(kd.grad.cpu(), rk, rtol=1e-5, atol=1e-5)
+
+
+# ----------------------------------------------------------------------------- cos/sin evaluated in the kernel
+def _pos_inputs(B, S, dtype, seed, hq=4, hk=2, max_pos=2000):
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn(B, S, hq, 128, generator=g).to(dtype)
+    k = torch.randn(B, S, hk, 128, generator=g).to(dtype)
+    pos = torch.randint(0, max_pos, (3, B, S), generator=g)
+    return q, k, pos
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("layout", ["hf", "csrc"])
+def test_mrope_from_positions_matches_the_table_path(dev, dtype, layout):
+    """The oracle builds the tables (fp32 angle, fp32 cos/sin, cast: vl.py:679-712) and rotates; the kernel gets
+    only position_ids and inv_freq.  The device's sincosf and the host's differ in the last place now and then, so a
+    rounded table entry may differ by one unit of the storage type: stated tolerance everywhere, and all but a
+    sliver of the outputs bit-equal."""
+    q, k, pos = _pos_inputs(2, 61, dtype, 21)
+    inv_freq = wl.text_inv_freq()
+    cos, sin = oracle.rotary_cos_sin_ref(pos, inv_freq, dtype)
+    qt, kt = q.transpose(1, 2), k.transpose(1, 2)
+    rq, rk = oracle.mrope_apply_ref(qt, kt, cos, sin, list(wl.MROPE_SECTION), layout, eager_rounding=True)
+    native.set_mrope_layout(layout)
+    try:
+        gq, gk = ops.multimodal_rope_from_positions(qt.to(dev), kt.to(dev), pos.to(dev), inv_freq.to(dev),
+                                                    list(wl.MROPE_SECTION))
+    finally:
+        native.set_mrope_layout("hf")
+    assert gq.is_contiguous() and gk.is_contiguous()
+    if dtype == torch.float32:
+        # fp32 tables keep the full last-place difference; angles reach 2000 rad, where one ulp of the angle is 1e-4
+        _close(gq, rq, atol=1e-3, rtol=1e-3)
+        _close(gk, rk, atol=1e-3, rtol=1e-3)
+    else:
+        _close(gq, rq)
+        _close(gk, rk)
+        assert _n_diff(gq, rq) <= 2e-3 * rq.numel() and _n_diff(gk, rk) <= 2e-3 * rk.numel()
+
+
+def test_mrope_from_positions_config2_full_size(dev):
+    ids, grid = wl.config2_tokens()
+    pos, _ = oracle.rope_index_ref(ids, 2, wl.IMAGE_TOKEN_ID, wl.VIDEO_TOKEN_ID, wl.VISION_START_TOKEN_ID, 2,
+                                   image_grid_thw=grid)
+    inv_freq = wl.text_inv_freq()
+    cos, sin = oracle.rotary_cos_sin_ref(pos, inv_freq, torch.bfloat16)
+    q, k = wl.qk_inputs(16, 896)
+    qt, kt = q.transpose(1, 2), k.transpose(1, 2)
+    rq, rk = oracle.mrope_apply_ref(qt, kt, cos, sin, list(wl.MROPE_SECTION), "hf")
+    gq, gk = ops.multimodal_rope_from_positions(qt.to(dev), kt.to(dev), pos.to(dev), inv_freq.to(dev),
+                                                list(wl.MROPE_SECTION))
+    _close(gq, rq)
+    _close(gk, rk)
+    assert _n_diff(gq, rq) <= 1e-3 * rq.numel() and _n_diff(gk, rk) <= 1e-3 * rk.numel()
+    # position 0 on every axis is the identity whatever the frequencies: cos = 1, sin = 0 exactly
+    zero = torch.zeros_like(pos)
+    iq, ik = ops.multimodal_rope_from_positions(qt.to(dev), kt.to(dev), zero.to(dev), inv_freq.to(dev),
+                                                list(wl.MROPE_SECTION))
+    assert _n_diff(iq, qt.contiguous()) == 0 and _n_diff(ik, kt.contiguous()) == 0
+
+
+def test_mrope_from_positions_backward_is_the_adjoint(dev):
+    q, k, pos = _pos_inputs(2, 11, torch.float32, 23, max_pos=300)
+    inv_freq = wl.text_inv_freq()
+    cos, sin = oracle.rotary_cos_sin_ref(pos, inv_freq, torch.float32)
+    qd = q.transpose(1, 2).to(dev).requires_grad_(True)
+    kd = k.transpose(1, 2).to(dev).requires_grad_(True)
+    oq, ok = ops.multimodal_rope_from_positions(qd, kd, pos.to(dev), inv_freq.to(dev), list(wl.MROPE_SECTION))
+    g = torch.Generator().manual_seed(3)
+    gq, gk = torch.randn(oq.shape, generator=g), torch.randn(ok.shape, generator=g)
+    torch.autograd.backward([oq, ok], [gq.to(dev), gk.to(dev)])
+    rq, rk = oracle.mrope_apply_bwd_ref(gq, gk, cos, sin, list(wl.MROPE_SECTION), "hf")
+    assert torch.allclose(qd.grad.cpu(), rq, rtol=1e-4, atol=1e-4)
+    assert torch.allclose(kd.grad.cpu(), rk, rtol=1e-4, atol=1e-4)
+    # <forward(x), g> == <x, backward(g)>
+    lhs = float((oq.detach().cpu().double() * gq.double()).sum() + (ok.detach().cpu().double() * gk.double()).sum())
+    rhs = float((qd.grad.cpu().double() * q.transpose(1, 2).double()).sum()
+                + (kd.grad.cpu().double() * k.transpose(1, 2).double()).sum())
+    assert abs(lhs - rhs) <= 1e-3 * max(1.0, abs(lhs))
+
+
+def test_mrope_from_positions_refuses_what_it_cannot_do(dev):
+    q, k, pos = _pos_inputs(1, 9, torch.bfloat16, 9)
+    inv_freq = wl.text_inv_freq().to(dev)
+    with pytest.raises(RuntimeError, match="chunk boundaries"):
+        ops.multimodal_rope_from_positions(q.transpose(1, 2).to(dev), k.transpose(1, 2).to(dev), pos.to(dev), inv_freq,
+                                           [10, 27, 27])
+    with pytest.raises(RuntimeError, match="position_ids"):
+        ops.multimodal_rope_from_positions(q.transpose(1, 2).to(dev), k.transpose(1, 2).to(dev),
+                                           pos[:, :, :5].to(dev), inv_freq, [16, 24, 24])

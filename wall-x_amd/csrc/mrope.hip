@@ -181,7 +181,11 @@ __device__ __forceinline__ u32x4 partner_chunk(const u32x4& v, int half_lanes) {
 }
 
 // L = lanes per head when known at compile time (16), 0 = any power of two up to 64 (runtime).
-template <int DT, bool BWD, int L>
+// POS: no cos/sin tables; `cos_t` is position_ids int64 [3, n_tokens] and `sin_t` is inv_freq fp32 [head_dim / 2].
+// The thread evaluates cos/sin of its channels itself, the way the table builder does (vl.py:679-712): the angle
+// is the fp32 product position * inv_freq (channels d and d + head_dim/2 share a frequency), cos and sin are
+// taken in fp32 and rounded to the storage type.
+template <int DT, bool BWD, int L, bool POS>
 __global__ __launch_bounds__(256) void mrope_rows_kernel(
     const void* __restrict__ q, const void* __restrict__ k, const void* __restrict__ cos_t,
     const void* __restrict__ sin_t, void* __restrict__ q_out, void* __restrict__ k_out, int64_t n_tokens,
@@ -205,11 +209,23 @@ __global__ __launch_bounds__(256) void mrope_rows_kernel(
   const int64_t hq_in = sq.h * Elem<DT>::kBytes, hk_in = sk.h * Elem<DT>::kBytes;
   const int64_t hq_out = sqo.h * Elem<DT>::kBytes, hk_out = sko.h * Elem<DT>::kBytes;
 
-  // selected cos / sin of my channels (regular loads: other workgroups never need them, later heads do not either,
-  // but the three position planes are small next to q)
-  const int64_t tab_off = (ax.axis[d0] * (n_tokens * head_dim) + token * head_dim + d0) * Elem<DT>::kBytes;
-  const u32x4 c_raw = *reinterpret_cast<const u32x4*>(static_cast<const char*>(cos_t) + tab_off);
-  u32x4 s_raw = *reinterpret_cast<const u32x4*>(static_cast<const char*>(sin_t) + tab_off);
+  u32x4 c_raw, s_raw;
+  if constexpr (POS) {
+    const int64_t pos = static_cast<const int64_t*>(cos_t)[ax.axis[d0] * n_tokens + token];
+    const float* inv_freq = static_cast<const float*>(sin_t) + (hi ? d0 - head_dim / 2 : d0);
+    const float pf = static_cast<float>(pos);
+    float cv[kEpc], sv[kEpc];
+#pragma unroll
+    for (int e = 0; e < kEpc; ++e) sincosf(__fmul_rn(pf, inv_freq[e]), &sv[e], &cv[e]);
+    c_raw = pack16<DT>(cv);
+    s_raw = pack16<DT>(sv);
+  } else {
+    // selected cos / sin of my channels (regular loads: other workgroups never need them, later heads do not
+    // either, but the three position planes are small next to q)
+    const int64_t tab_off = (ax.axis[d0] * (n_tokens * head_dim) + token * head_dim + d0) * Elem<DT>::kBytes;
+    c_raw = *reinterpret_cast<const u32x4*>(static_cast<const char*>(cos_t) + tab_off);
+    s_raw = *reinterpret_cast<const u32x4*>(static_cast<const char*>(sin_t) + tab_off);
+  }
   if constexpr (BWD) s_raw = partner_chunk<L>(s_raw, lanes / 2);  // the adjoint multiplies by the partner's sin
   float c[kEpc], sn[kEpc];
   unpack16<DT>(c_raw, c);
@@ -288,11 +304,13 @@ int build_axis_table(const int sec[3], int head_dim, int layout, AxisTable& ax) 
   return WX_OK;
 }
 
-template <bool BWD>
+// POS: cos_t / sin_t carry position_ids / inv_freq (see mrope_rows_kernel)
+template <bool BWD, bool POS = false>
 int launch(const void* q, const void* k, const void* cos_t, const void* sin_t, void* q_out, void* k_out,
            int64_t batch, int64_t seq, int n_q, int n_kv, int head_dim, const int64_t* sq, const int64_t* sk,
            const int64_t* sqo, const int64_t* sko, const int sec[3], int layout, int dtype, wx_stream_t stream) {
-  const char* who = BWD ? "wx_mrope_apply_bwd" : "wx_mrope_apply";
+  const char* who = POS ? (BWD ? "wx_mrope_apply_positions(backward)" : "wx_mrope_apply_positions")
+                        : (BWD ? "wx_mrope_apply_bwd" : "wx_mrope_apply");
   if (batch < 0 || seq < 0 || n_q < 0 || n_kv < 0) return fail(WX_ERR_INVALID_ARGUMENT, "%s: negative size", who);
   if (head_dim <= 0 || head_dim % 16 != 0 || head_dim > kMaxHeadDim)
     return fail(WX_ERR_UNSUPPORTED, "%s: head_dim %d must be a multiple of 16 and <= %d", who, head_dim, kMaxHeadDim);
@@ -321,7 +339,7 @@ int launch(const void* q, const void* k, const void* cos_t, const void* sin_t, v
     if ((threads + 255) / 256 > 0x7fffffffll) return fail(WX_ERR_UNSUPPORTED, "%s: too many tokens", who);
     const dim3 grid(static_cast<unsigned>((threads + 255) / 256)), block(256);
 #define WX_LAUNCH_ROWS(DT, L)                                                                                       \
-  hipLaunchKernelGGL((mrope_rows_kernel<DT, BWD, L>), grid, block, 0, s, q, k, cos_t, sin_t, q_out, k_out, n_tokens, \
+  hipLaunchKernelGGL((mrope_rows_kernel<DT, BWD, L, POS>), grid, block, 0, s, q, k, cos_t, sin_t, q_out, k_out, n_tokens, \
                      seq, n_q, n_kv, head_dim, a, b, c, d, ax)
     switch (dtype) {
       case WX_F32: WX_LAUNCH_ROWS(WX_F32, 0); break;
@@ -332,6 +350,11 @@ int launch(const void* q, const void* k, const void* cos_t, const void* sin_t, v
 #undef WX_LAUNCH_ROWS
     return check_launch(who);
   }
+  if constexpr (POS) {
+    return fail(WX_ERR_UNSUPPORTED,
+                "%s: needs a head of 2..64 16-byte chunks (a power of two) and sections that end on chunk boundaries; "
+                "build the cos/sin tables and call wx_mrope_apply instead", who);
+  } else {
   // grid.x walks (token, rotation group); grid.y walks groups of kHeadsPerThread heads
   const int groups = head_dim / 16;
   const int head_groups = (n_q + n_kv + kHeadsPerThread - 1) / kHeadsPerThread;
@@ -349,6 +372,7 @@ int launch(const void* q, const void* k, const void* cos_t, const void* sin_t, v
   }
 #undef WX_LAUNCH
   return check_launch(who);
+  }
 }
 
 }  // namespace
@@ -370,4 +394,19 @@ extern "C" int wx_mrope_apply_bwd(const void* gq_out, const void* gk_out, const 
                                   const int mrope_section[3], int layout, int dtype, wx_stream_t stream) {
   return wx::launch<true>(gq_out, gk_out, cos, sin, gq, gk, batch, seq, n_q_heads, n_kv_heads, head_dim, gqo_strides,
                           gko_strides, gq_strides, gk_strides, mrope_section, layout, dtype, stream);
+}
+
+extern "C" int wx_mrope_apply_positions(const void* q, const void* k, const int64_t* position_ids,
+                                        const float* inv_freq, void* q_out, void* k_out, int64_t batch, int64_t seq,
+                                        int n_q_heads, int n_kv_heads, int head_dim, const int64_t q_strides[3],
+                                        const int64_t k_strides[3], const int64_t qo_strides[3],
+                                        const int64_t ko_strides[3], const int mrope_section[3], int layout,
+                                        int dtype, int backward, wx_stream_t stream) {
+  if (backward)
+    return wx::launch<true, true>(q, k, position_ids, inv_freq, q_out, k_out, batch, seq, n_q_heads, n_kv_heads,
+                                  head_dim, q_strides, k_strides, qo_strides, ko_strides, mrope_section, layout, dtype,
+                                  stream);
+  return wx::launch<false, true>(q, k, position_ids, inv_freq, q_out, k_out, batch, seq, n_q_heads, n_kv_heads,
+                                 head_dim, q_strides, k_strides, qo_strides, ko_strides, mrope_section, layout, dtype,
+                                 stream);
 }

@@ -60,6 +60,11 @@ def rope_bwd(grad_q_out, grad_k_out, q, k, cos, sin, grad_q, grad_k, mrope_secti
     return native.rope_bwd(grad_q_out, grad_k_out, q, k, cos, sin, grad_q, grad_k, mrope_section_doubled)
 
 
+def rope_from_positions(q, k, position_ids, inv_freq, q_out, k_out, mrope_section_doubled, backward=False) -> None:
+    """No counterpart in backend.py: the rope op with the cos/sin builder (vl.py:679-712) folded in."""
+    return native.rope_from_positions(q, k, position_ids, inv_freq, q_out, k_out, mrope_section_doubled, backward)
+
+
 def get_rope_index(input_ids, image_grid_thw, video_grid_thw, second_per_grid_ts, attention_mask,
                    spatial_merge_size, image_token_id, video_token_id, vision_start_token_id, tokens_per_second):
     """backend.py:302-352 (forwards to the native op named rope_index)."""

@@ -242,6 +242,55 @@ def multimodal_rope(q, k, cos, sin, mrope_section):
     return MultimodalRoPE.apply(q, k, cos, sin, mrope_section)
 
 
+class MultimodalRoPEFromPositions(torch.autograd.Function):
+    """Not in the reference's op set: `multimodal_rope` with Qwen2_5_VLRotaryEmbedding.forward (vl.py:679-712)
+    folded in.  Takes position_ids [3, B, S] int64 and inv_freq [D/2] fp32 instead of the cos/sin tables
+    [3, B, S, D] built from them, so neither table is ever written or read.  q [B, Hq, S, D], k [B, Hkv, S, D]
+    through their strides, contiguous outputs, gradients for q and k only."""
+
+    @staticmethod
+    def forward(ctx, q, k, position_ids, inv_freq, mrope_section):
+        for name, t in (("q", q), ("k", k), ("position_ids", position_ids), ("inv_freq", inv_freq)):
+            if t.is_cpu:
+                raise RuntimeError(f"[Error] The input `{name}` of multimodal_rope op is on the device: CPU!")
+        if len(mrope_section) != 3:
+            raise RuntimeError("[Error] The input `mrope_section` of multimodal_rope op must be a list of 3 integers!")
+        if q.stride(-1) != 1:
+            warnings.warn("The input `q` of multimodal_rope op is discontiguous!")
+            q = q.contiguous()
+        if k.stride(-1) != 1:
+            warnings.warn("The input `k` of multimodal_rope op is discontiguous!")
+            k = k.contiguous()
+        doubled = [2 * int(v) for v in mrope_section]
+        inv_freq = inv_freq.to(torch.float32)
+        q_out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+        k_out = torch.empty(k.shape, dtype=k.dtype, device=k.device)
+        backend.rope_from_positions(q, k, position_ids, inv_freq, q_out, k_out, doubled)
+        ctx.save_for_backward(position_ids, inv_freq)
+        ctx.mrope_section_doubled = doubled
+        return q_out, k_out
+
+    @staticmethod
+    def backward(ctx, grad_q_out, grad_k_out):
+        position_ids, inv_freq = ctx.saved_tensors
+        want_q, want_k = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+        if not (want_q or want_k):
+            return None, None, None, None, None
+        if grad_q_out.stride(-1) != 1:
+            grad_q_out = grad_q_out.contiguous()
+        if grad_k_out.stride(-1) != 1:
+            grad_k_out = grad_k_out.contiguous()
+        gq = torch.empty(grad_q_out.shape, dtype=grad_q_out.dtype, device=grad_q_out.device)
+        gk = torch.empty(grad_k_out.shape, dtype=grad_k_out.dtype, device=grad_k_out.device)
+        backend.rope_from_positions(grad_q_out, grad_k_out, position_ids, inv_freq, gq, gk,
+                                    ctx.mrope_section_doubled, backward=True)
+        return (gq if want_q else None), (gk if want_k else None), None, None, None
+
+
+def multimodal_rope_from_positions(q, k, position_ids, inv_freq, mrope_section):
+    return MultimodalRoPEFromPositions.apply(q, k, position_ids, inv_freq, mrope_section)
+
+
 # ----------------------------------------------------------------------------- index builders
 def get_rope_index(input_ids, spatial_merge_size, image_token_id, video_token_id, vision_start_token_id,
                    tokens_per_second, image_grid_thw=None, video_grid_thw=None, second_per_grid_ts=None,

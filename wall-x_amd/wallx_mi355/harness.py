@@ -11,7 +11,8 @@ batch of full sequences (prefill).  What it states explicitly:
     bidirectional block among action tokens (act.py:616-637) through a dense boolean mask,
   * rotary base 1e6, mrope_section [16, 24, 24], cos/sin built in fp32 and cast to bf16 (vl.py:679-712),
   * `fuse=True` (default) runs the post-attention RMSNorm inside the permute and the residual add inside the
-    unpermute (one pass over [T, H] each instead of two); `fuse=False` keeps them as separate PyTorch ops.
+    unpermute (one pass over [T, H] each instead of two), and M-RoPE evaluates cos/sin from the position ids in
+    the kernel (no [3, B, S, D] tables); `fuse=False` keeps them as separate PyTorch ops.
 """
 
 from contextlib import contextmanager
@@ -139,10 +140,11 @@ class PrefillHarness:
         with timer.section("rope_index"):
             pos, _ = ops.get_rope_index(input_ids, 2, wl.IMAGE_TOKEN_ID, wl.VIDEO_TOKEN_ID, wl.VISION_START_TOKEN_ID, 2,
                                         image_grid_thw=image_grid_thw)
-        with timer.section("cos_sin_torch"):
-            freqs = pos.float()[..., None] * self.inv_freq
-            emb = torch.cat((freqs, freqs), -1)
-            cos, sin = emb.cos().to(torch.bfloat16), emb.sin().to(torch.bfloat16)
+        if not self.fuse:
+            with timer.section("cos_sin_torch"):
+                freqs = pos.float()[..., None] * self.inv_freq
+                emb = torch.cat((freqs, freqs), -1)
+                cos, sin = emb.cos().to(torch.bfloat16), emb.sin().to(torch.bfloat16)
         with timer.section("partition"):
             ids = moe_token_types.reshape(-1)
             rmap, off, inv, self._ws = native.partition(ids, 2, 0, self._ws, want_sorted=True)
@@ -164,7 +166,10 @@ class PrefillHarness:
                 k = k.view(B, S, nkv, D).transpose(1, 2)
                 v = v.view(B, S, nkv, D).transpose(1, 2)
             with timer.section("mrope"):
-                q, k = ops.multimodal_rope(q, k, cos, sin, list(wl.MROPE_SECTION))
+                if self.fuse:
+                    q, k = ops.multimodal_rope_from_positions(q, k, pos, self.inv_freq, list(wl.MROPE_SECTION))
+                else:
+                    q, k = ops.multimodal_rope(q, k, cos, sin, list(wl.MROPE_SECTION))
             with timer.section("sdpa_torch"):
                 a = F.scaled_dot_product_attention(q, k, v, attn_mask=attn_mask, is_causal=attn_mask is None,
                                                    enable_gqa=True)

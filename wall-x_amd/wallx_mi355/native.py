@@ -277,6 +277,34 @@ def rope_bwd(grad_q_out, grad_k_out, q, k, cos, sin, grad_q, grad_k, mrope_secti
     _rope_common("wx_mrope_apply_bwd", grad_q_out, grad_k_out, cos, sin, grad_q, grad_k, mrope_section_doubled)
 
 
+def rope_from_positions(q, k, position_ids, inv_freq, q_out, k_out, mrope_section_doubled, backward: bool = False) -> None:
+    """M-RoPE with cos/sin evaluated in the kernel (vl.py:679-712 folded into vl.py:731-773): position_ids
+    [3, B, S] int64, inv_freq [D/2] fp32.  With backward=True, q/k carry the output gradients and q_out/k_out
+    receive the input gradients."""
+    for name, t in (("q", q), ("k", k), ("position_ids", position_ids), ("inv_freq", inv_freq), ("q_out", q_out),
+                    ("k_out", k_out)):
+        _need_cuda(name, t)
+    if len(mrope_section_doubled) != 3:
+        raise RuntimeError("mrope_section_doubled must have 3 entries")
+    B, Hq, S, D = q.shape
+    Hk = k.size(1)
+    if tuple(k.shape) != (B, Hk, S, D) or tuple(q_out.shape) != tuple(q.shape) or tuple(k_out.shape) != tuple(k.shape):
+        raise RuntimeError("q/k/q_out/k_out shapes are inconsistent")
+    if tuple(position_ids.shape) != (3, B, S) or position_ids.dtype != torch.int64:
+        raise RuntimeError(f"position_ids must be int64 [3, {B}, {S}]")
+    if tuple(inv_freq.shape) != (D // 2,) or inv_freq.dtype != torch.float32:
+        raise RuntimeError(f"inv_freq must be fp32 [{D // 2}]")
+    if not (q.dtype == k.dtype == q_out.dtype == k_out.dtype):
+        raise RuntimeError("q, k and the outputs must share one dtype")
+    position_ids = position_ids.contiguous()
+    inv_freq = inv_freq.contiguous()
+    section = _lib.i32x3([int(v) // 2 for v in mrope_section_doubled])
+    with _DeviceGuard(q):
+        _lib.call("wx_mrope_apply_positions", _ptr(q), _ptr(k), _ptr(position_ids), _ptr(inv_freq), _ptr(q_out),
+                  _ptr(k_out), B, S, Hq, Hk, D, _bhsd_strides(q), _bhsd_strides(k), _bhsd_strides(q_out),
+                  _bhsd_strides(k_out), section, _mrope_layout, _dtype_code(q), int(bool(backward)), _stream(q))
+
+
 # ----------------------------------------------------------------------------- index builders
 def rope_index(input_ids, image_grid_thw, video_grid_thw, second_per_grid_ts, attention_mask,
                spatial_merge_size: int, image_token_id: int, video_token_id: int, vision_start_token_id: int,
