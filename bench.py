@@ -412,8 +412,8 @@ def config4_measurement(dev, weights):
 def backward_measurement(dev, x, weights, m0):
     """The reference's own op, `asym_dual_gmm` on row-major operands (ops.py:6-165), at the gate projection's
     config 3 shapes: the forward (x @ W^T for both experts in one launch, nn.Linear weights read in place) and the
-    two backward GEMMs of ops.py:78-144, dX = dY @ W and dW = dY^T @ X, each as transposed copies + the MFMA
-    kernel (times include the transposes)."""
+    two backward GEMMs of ops.py:78-144, dX = dY @ W and dW = dY^T @ X, whose K-major operands the same kernel
+    transposes between LDS and the registers (no transposed copies)."""
     import torch
     from wallx_mi355 import native
 

@@ -82,7 +82,11 @@ int wx_unpermute_rows_bwd(const void* grad_out, const void* y_fwd, void* act_gra
  * Dual asymmetric grouped GEMM: out_e = op(in_e) @ op(w_e), e in {0, 1}, in ONE launch; bf16 in/out,
  * fp32 accumulate.  Replaces AsymmetricDualExpertGemm (csrc/dual_asym_grouped_gemm.cu:308-366,
  * ops.py:6-165).  trans_a: in_e stored [k_e, m_e]; trans_b: w_e stored [n_e, k_e] (nn.Linear layout).
- * All matrices packed row-major; k_e and n_e multiples of 8 (16-byte rows).  m_e == 0 is allowed. */
+ * All matrices packed row-major.  Every layout is read in place by the same MFMA kernel (an operand whose slow
+ * dimension is K is transposed on its way from LDS to the registers), which covers the forward (trans_b) and
+ * both backward GEMMs of ops.py:78-144 (dX: neither flag; dW: trans_a only).  n_e multiples of 8; m_e multiples
+ * of 8 under trans_a; k_e multiples of 8 unless both operands are stored [k, .] (trans_a without trans_b), where
+ * k_e -- the token count of a weight gradient -- is free.  m_e == 0 is allowed. */
 int wx_dual_gemm(const void* in0, const void* in1, const void* w0, const void* w1, void* out0,
                  void* out1, int64_t m0, int64_t n0, int64_t k0, int64_t m1, int64_t n1, int64_t k1,
                  int trans_a, int trans_b, wx_stream_t stream);
@@ -239,10 +243,8 @@ int wx_unpermute_rows_add(const void* y, const void* residual, void* out, const 
                           int64_t num_tokens, int64_t num_cols, wx_stream_t stream);
 
 /* dst [cols, rows] = transpose of src [rows, cols], both row-major and contiguous, 2-byte elements (bf16 / fp16),
- * rows and cols multiples of 8.  Feeds the backward of asym_dual_gmm (ops.py:78-144: dX uses (F, not trans_b), dW
- * uses (T, F)): the MFMA kernel reads both operands with the contraction index contiguous, so the Python layer
- * hands it transposed copies; the reference gets the same effect from CUTLASS layout tags
- * (csrc/dual_asym_grouped_gemm.cu:286-305). */
+ * rows and cols multiples of 8.  A utility without a counterpart in the reference; wx_dual_gemm does not need it
+ * (it reads every layout of ops.py:78-144 in place). */
 int wx_transpose_2d(const void* src, void* dst, int64_t rows, int64_t cols, int elem_bytes, wx_stream_t stream);
 
 /* ---- measurement probe (no counterpart in the reference; used by bench.py) --------------------------------

@@ -102,22 +102,31 @@ def test_transpose_2d_is_exact(dev, shape):
     assert torch.equal(native.transpose_2d(t), t.t().contiguous())
 
 
-def test_dual_gemm_plain_layout_kernel_through_the_c_abi(dev):
-    """The Python layer feeds the MFMA kernel transposed copies; the library's own kernel for the other three
-    layouts stays reachable for C callers and is checked here directly."""
+@pytest.mark.parametrize("shape", [
+    # m0, n0, k0, m1, n1, k1
+    (72, 96, 64, 40, 56, 128),            # small tiles
+    (3000, 3080, 96, 200, 264, 160),      # large tiles, ragged everywhere
+    (264, 520, 2048, 0, 64, 64),          # long contraction, empty second problem
+])
+def test_dual_gemm_k_major_layouts_through_the_c_abi(dev, shape):
+    """Operands stored with K as the slow dimension (A as [k, m], B as [k, n]: the layouts of the backward GEMMs,
+    ops.py:78-144) are read in place and transposed between LDS and the registers; straight through the C ABI."""
     from wallx_mi355 import _lib
 
+    m0, n0, k0, m1, n1, k1 = shape
     g = torch.Generator().manual_seed(5)
-    a0, a1 = _bf((72, 64), g), _bf((40, 128), g)
-    w0, w1 = _bf((96, 64), g, 0.1), _bf((56, 128), g, 0.1)
     for ta, tb in ((False, False), (True, False), (True, True)):
+        kk0, kk1 = (k0 + 13, k1 + 3) if (ta and not tb) else (k0, k1)  # K rows need no alignment when both are K-major
+        a0, a1 = _bf((m0 // 8 * 8 if ta else m0, kk0), g), _bf((m1 // 8 * 8 if ta else m1, kk1), g)
+        w0, w1 = _bf((n0, kk0), g, 0.1), _bf((n1, kk1), g, 0.1)
         x0, x1 = (a0.t().contiguous(), a1.t().contiguous()) if ta else (a0, a1)
         v0, v1 = (w0, w1) if tb else (w0.t().contiguous(), w1.t().contiguous())
         d = [t.to(dev) for t in (x0, x1, v0, v1)]
-        o0 = torch.empty(72, 96, dtype=torch.bfloat16, device=dev)
-        o1 = torch.empty(40, 56, dtype=torch.bfloat16, device=dev)
+        o0 = torch.full((a0.size(0), n0), 7.0, dtype=torch.bfloat16, device=dev)
+        o1 = torch.full((a1.size(0), n1), 7.0, dtype=torch.bfloat16, device=dev)
         _lib.call("wx_dual_gemm", d[0].data_ptr(), d[1].data_ptr(), d[2].data_ptr(), d[3].data_ptr(), o0.data_ptr(),
-                  o1.data_ptr(), 72, 96, 64, 40, 56, 128, int(ta), int(tb), torch.cuda.current_stream().cuda_stream)
+                  o1.data_ptr(), a0.size(0), n0, kk0, a1.size(0), n1, kk1, int(ta), int(tb),
+                  torch.cuda.current_stream().cuda_stream)
         r0, r1 = oracle.dual_gemm_ref(x0, x1, v0, v1, ta, tb)
         _close(o0, r0, what=f"C ABI ta={ta} tb={tb}")
         _close(o1, r1, what=f"C ABI ta={ta} tb={tb}")

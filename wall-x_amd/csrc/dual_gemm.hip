@@ -17,7 +17,10 @@
 // makes the 16-byte fragment reads bank-conflict free.
 //
 // Three operand layouts:
-//   generic  (wx_dual_gemm)            A, B, C row-major; loads touch 16 rows x 64 bytes per instruction.
+//   generic  (wx_dual_gemm)            A, B, C row-major; loads touch 16 rows x 64 bytes per instruction.  An
+//                                      operand stored with K as its slow dimension (A as [k, m], B as [k, n]: the
+//                                      backward GEMMs) is loaded as K rows of 256 columns and transposed by the LDS
+//                                      reads (ds_read_b64_tr_b16), so no layout needs a transposed copy.
 //   gate/up  (wx_dual_swiglu_gate_up)  A = K-tiled activations, B = K-tiled gate and up weights (the B tile is 128
 //                                      gate rows + 128 up rows of the same output columns, so gate and up of an
 //                                      output element meet in one lane), C = K-tiled intermediate, SwiGLU epilogue.
@@ -34,6 +37,7 @@ namespace wx {
 namespace {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 constexpr int BK = 32;
@@ -98,6 +102,7 @@ struct Params {
 };
 
 #define LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
+#define LDS_TR_PTR(p) ((__attribute__((address_space(3))) bf16x4*)(p))
 
 // Buffer descriptor for `bytes` readable bytes at `base`.  Both are wave-uniform by construction; passing them
 // through readfirstlane pins the descriptor to scalar registers.
@@ -155,7 +160,9 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
   return __builtin_bit_cast(uint32_t, v);
 }
 
-template <int MODE, typename TS>
+// KA / KB (generic mode only): the operand is stored with K as its slow dimension -- A as [k, m], B as [k, n] --
+// and is transposed on the way from LDS to the MFMA registers.
+template <int MODE, typename TS, bool KA = false, bool KB = false>
 __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(Params p) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stub; the body uses gfx950-only builtins
   constexpr int BM = TS::BM, BN = TS::BN, FM = TS::FM, FN = TS::FN;
@@ -166,6 +173,7 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
   constexpr bool SWIGLU = MODE == kGateUp;
   constexpr bool TILED_IN = MODE != kGeneric;   // A and B are K-tiled
   constexpr bool TILED_OUT = MODE == kGateUp;   // C is K-tiled
+  static_assert(MODE == kGeneric || (!KA && !KB), "K-major operands exist in the generic mode only");
   // kStages ring slots per operand, each one K step (256 rows x 32 bf16).  Separate arrays let the compiler
   // see that a read of one slot never waits for a buffer load that targets another.
   __shared__ __attribute__((aligned(1024))) unsigned char s_a0[kSlotBytesA];
@@ -249,6 +257,18 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
     else return wn * (FN * 32) + j * 32;
   };
   const int b_lane_off = l32 * kRowBytes;
+  // K-major operand (KA / KB): a slot holds BK rows of K, each a run of BM (BN) columns, as whole 16-byte chunks;
+  // the 64-byte segment s of row k sits at segment position s ^ (k & 3), so that the four rows one transposing
+  // read touches fall into different banks.  ds_read_b64_tr_b16 works on groups of 16 lanes: lane j of a group
+  // supplies the address of 4 consecutive columns of row (j >> 2), and receives column j of the 4 rows.  A group
+  // covers 16 columns; the two groups of a half-wave cover a 32-column block, the half-waves rows k and k + 8.
+  const int tr_j = lane & 15, tr_grp = (lane >> 4) & 1;
+  const int tr_in = (2 * tr_grp + ((tr_j >> 1) & 1)) * 16 + 8 * (tr_j & 1);  // bytes inside the 64-byte segment
+  auto tr_lane_base = [&](int row_bytes, int first_block) {  // first_block: this wave's first 32-column block
+    return (8 * lhi + (tr_j >> 2)) * row_bytes + ((first_block ^ (tr_j >> 2)) << 6) + tr_in;
+  };
+  const int tr_base_a = KA ? tr_lane_base(BM * 2, wm * FM) : 0;
+  const int tr_base_b = KB ? tr_lane_base(BN * 2, wn * FN) : 0;
 
   // ---- per-tile state ------------------------------------------------------------------------------
   struct Loader {   // where this wave's kLoadsA + kLoadsB loads per K step come from
@@ -309,16 +329,45 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
     } else {
       const int rows_a = G.m - row0 < BM ? G.m - row0 : BM;
       const int rows_b = G.n - col0 < kTileN ? G.n - col0 : kTileN;
-      L.a_base = G.a + static_cast<int64_t>(row0) * G.lda;
-      L.b_base = b_src + static_cast<int64_t>(col0) * G.ldb;
-      L.a_bytes = static_cast<uint32_t>(rows_a) * G.lda * 2u;
-      L.b_bytes = static_cast<uint32_t>(rows_b) * G.ldb * 2u;
       L.a_step = L.b_step = 0;
-      const int b_ld_row0 = b_wave * kLoadRowsB + (lane >> 2);
+      // K-major operand: load instruction q of the slot (1 KiB of LDS) holds 1024 / row_bytes rows of K; the lane's
+      // 16-byte LDS position p = 64 q + lane is chunk p % chunks of row p / chunks, which takes the matrix chunk
+      // whose 64-byte segment index is XORed with (row & 3).  Columns past the matrix edge read whatever follows
+      // (the next row, or zero past the end): they only reach output rows / columns that are never stored.
+      // Rows past K are out of the descriptor's range and read as zero.
+      auto k_major_voff = [&](int q, int chunks, int ld) {
+        const int pos = 64 * q + lane;
+        const int krow = pos / chunks, c = pos % chunks;
+        const int src_chunk = ((((c >> 2) ^ (krow & 3)) << 2) | (c & 3));
+        return static_cast<uint32_t>(krow) * static_cast<uint32_t>(ld) * 2u + static_cast<uint32_t>(src_chunk) * 16u;
+      };
+      if constexpr (KA) {
+        L.a_base = G.a + row0;
+        const int64_t left = (static_cast<int64_t>(G.k) * G.lda - row0) * 2;
+        L.a_bytes = static_cast<uint32_t>(left < 0 ? 0 : left);
+        L.a_step = static_cast<int64_t>(G.lda) * 2;  // bytes per K row
 #pragma unroll
-      for (int i = 0; i < kLoadsA; ++i) L.voff_a[i] = static_cast<uint32_t>(ld_row0 + 16 * i) * G.lda * 2u + ld_chunk * 16u;
+        for (int i = 0; i < kLoadsA; ++i) L.voff_a[i] = k_major_voff(wave * kLoadsA + i, BM / 8, G.lda);
+      } else {
+        L.a_base = G.a + static_cast<int64_t>(row0) * G.lda;
+        L.a_bytes = static_cast<uint32_t>(rows_a) * G.lda * 2u;
 #pragma unroll
-      for (int i = 0; i < kLoadsB; ++i) L.voff_b[i] = static_cast<uint32_t>(b_ld_row0 + 16 * i) * G.ldb * 2u + ld_chunk * 16u;
+        for (int i = 0; i < kLoadsA; ++i) L.voff_a[i] = static_cast<uint32_t>(ld_row0 + 16 * i) * G.lda * 2u + ld_chunk * 16u;
+      }
+      if constexpr (KB) {
+        L.b_base = b_src + col0;
+        const int64_t left = (static_cast<int64_t>(G.k) * G.ldb - col0) * 2;
+        L.b_bytes = static_cast<uint32_t>(left < 0 ? 0 : left);
+        L.b_step = static_cast<int64_t>(G.ldb) * 2;
+#pragma unroll
+        for (int i = 0; i < kLoadsB; ++i) L.voff_b[i] = k_major_voff(b_wave * kLoadsB + i, BN / 8, G.ldb);
+      } else {
+        L.b_base = b_src + static_cast<int64_t>(col0) * G.ldb;
+        L.b_bytes = static_cast<uint32_t>(rows_b) * G.ldb * 2u;
+        const int b_ld_row0 = b_wave * kLoadRowsB + (lane >> 2);
+#pragma unroll
+        for (int i = 0; i < kLoadsB; ++i) L.voff_b[i] = static_cast<uint32_t>(b_ld_row0 + 16 * i) * G.ldb * 2u + ld_chunk * 16u;
+      }
     }
   };
 
@@ -346,19 +395,31 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
     } else {
       const int k0 = ks * BK;
       // advancing the base keeps the absolute end of the readable range, so rows past the matrix read as zero;
-      // K chunks at or past the row end are pushed out of range per lane (this also zero-fills padding steps)
+      // K chunks at or past the row end are pushed out of range per lane (this also zero-fills padding steps).
+      // A K-major operand advances by whole rows of K instead, and its rows past K are past the end by themselves.
       const uint32_t adv = 2u * static_cast<uint32_t>(k0);
-      ra = make_rsrc(L.a_base + k0, L.a_bytes > adv ? L.a_bytes - adv : 0u);
-      P.rb = make_rsrc(L.b_base + k0, L.b_bytes > adv ? L.b_bytes - adv : 0u);
+      if constexpr (KA) {
+        const int64_t da = L.a_step * k0;
+        ra = make_rsrc(reinterpret_cast<const char*>(L.a_base) + da, L.a_bytes > da ? static_cast<uint32_t>(L.a_bytes - da) : 0u);
+      } else {
+        ra = make_rsrc(L.a_base + k0, L.a_bytes > adv ? L.a_bytes - adv : 0u);
+      }
+      if constexpr (KB) {
+        const int64_t db = L.b_step * k0;
+        P.rb = make_rsrc(reinterpret_cast<const char*>(L.b_base) + db, L.b_bytes > db ? static_cast<uint32_t>(L.b_bytes - db) : 0u);
+      } else {
+        P.rb = make_rsrc(L.b_base + k0, L.b_bytes > adv ? L.b_bytes - adv : 0u);
+      }
       const bool k_tail = k0 + BK > L.K;
       oob = (k_tail && k0 + ld_chunk * 8 >= L.K) ? 0x80000000u : 0u;
     }
+    const uint32_t oob_a = KA ? 0u : oob, oob_b = KB ? 0u : oob;
 #pragma unroll
-    for (int i = 0; i < kLoadsB; ++i) P.voff_b[i] = L.voff_b[i] | oob;
+    for (int i = 0; i < kLoadsB; ++i) P.voff_b[i] = L.voff_b[i] | oob_b;
 #pragma unroll
     for (int i = 0; i < kLoadsA; ++i)
       __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, LDS_PTR(sa + (wave * kLoadRowsA + 16 * i) * kRowBytes), 16,
-                                               L.voff_a[i] | oob, 0, 0, 0);
+                                               L.voff_a[i] | oob_a, 0, 0, 0);
   };
   auto issue_b = [&](const Pending& P, unsigned char* sb) {
 #pragma unroll
@@ -372,14 +433,28 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
 
   // Fragments are read in the order the MFMAs (A-major: all B blocks for A block 0, then A block 1, ...) first
   // need them: A0, every B, then the other A blocks.
+  // K-major slot: K values [8 lhi, +8) of step half kk for the lane's column of 32-column block `blk` (counted
+  // from the wave's first block): two transposing reads of four rows each.
+  auto read_k_major = [&](const unsigned char* slot, int lane_base, int row_bytes, int blk, int kk) {
+    const unsigned char* at = slot + (lane_base ^ (blk << 6)) + 16 * kk * row_bytes;
+    const bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(LDS_TR_PTR(at));
+    const bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(LDS_TR_PTR(at + 4 * row_bytes));
+    return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  };
+  auto read_a = [&](const unsigned char* sa, int i, int kk) {
+    if constexpr (KA) return read_k_major(sa, tr_base_a, BM * 2, i, kk);
+    else return *reinterpret_cast<const bf16x8*>(sa + a_row_off + i * 32 * kRowBytes + frag_off[kk]);
+  };
+  auto read_b = [&](const unsigned char* sb, int j, int kk) {
+    if constexpr (KB) return read_k_major(sb, tr_base_b, BN * 2, j, kk);
+    else return *reinterpret_cast<const bf16x8*>(sb + b_row(j) * kRowBytes + b_lane_off + frag_off[kk]);
+  };
   auto read_frags = [&](const unsigned char* sa, const unsigned char* sb, int kk, int set) {
-    fa[set][0] = *reinterpret_cast<const bf16x8*>(sa + a_row_off + frag_off[kk]);
+    fa[set][0] = read_a(sa, 0, kk);
 #pragma unroll
-    for (int j = 0; j < FN; ++j)
-      fb[set][j] = *reinterpret_cast<const bf16x8*>(sb + b_row(j) * kRowBytes + b_lane_off + frag_off[kk]);
+    for (int j = 0; j < FN; ++j) fb[set][j] = read_b(sb, j, kk);
 #pragma unroll
-    for (int i = 1; i < FM; ++i)
-      fa[set][i] = *reinterpret_cast<const bf16x8*>(sa + a_row_off + i * 32 * kRowBytes + frag_off[kk]);
+    for (int i = 1; i < FM; ++i) fa[set][i] = read_a(sa, i, kk);
   };
   auto mma = [&](int set) {
 #pragma unroll
@@ -394,7 +469,7 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
   // slot's refill go out among the first half of this group's MFMAs; the second half covers the read latency, so
   // the wait in front of the barrier finds the reads done.
   auto schedule_before_barrier = [&]() {
-    constexpr int kMfma = FM * FN, kReads = FM + FN;
+    constexpr int kMfma = FM * FN, kReads = FM * (KA ? 2 : 1) + FN * (KB ? 2 : 1);
     constexpr int kCarry = kMfma / 2;                              // MFMAs that carry other instructions
     constexpr int kReadsPer = (kReads + kCarry - 1) / kCarry;      // LDS reads per carrying MFMA
     constexpr int kLoadEvery = kCarry / kLoadsB > 0 ? kCarry / kLoadsB : 1;
@@ -409,7 +484,7 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
   };
   // After the barrier: the A half of the refill and the next slot's fragment reads are spread over the whole group.
   auto schedule_after_barrier = [&]() {
-    constexpr int kMfma = FM * FN, kReads = FM + FN;
+    constexpr int kMfma = FM * FN, kReads = FM * (KA ? 2 : 1) + FN * (KB ? 2 : 1);
     constexpr int kReadEvery = kMfma / kReads > 0 ? kMfma / kReads : 1;
     constexpr int kReadsPer = kReads * kReadEvery > kMfma ? (kReads + kMfma - 1) / kMfma : 1;
     constexpr int kLoadEvery = kMfma / kLoadsA > 0 ? kMfma / kLoadsA : 1;
@@ -625,8 +700,8 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
 #endif
 }
 
-// ---- other operand layouts: any transpose combination, any k; plain FMA tiles ------------------------------
-// Used for the layouts the MFMA kernel does not read in place (trans_a, or weights stored [k, n]).
+// ---- plain FMA tiles: any transpose combination, any k --------------------------------------------------------
+// Used for what the MFMA kernel does not take: an empty contraction, K-major operands of 4 GiB or more.
 __global__ __launch_bounds__(256) void dual_gemm_reference_layout_kernel(Params p, int trans_a, int trans_b) {
   __shared__ float s_a[32][33];
   __shared__ float s_b[32][33];
@@ -681,10 +756,11 @@ __global__ __launch_bounds__(256) void pack_tiled_kernel(const u32x4* __restrict
   }
 }
 
-int check_dims(const char* who, int64_t m, int64_t n, int64_t k) {
+// k_in_rows: both operands are stored with K as the slow dimension, so K needs no alignment
+int check_dims(const char* who, int64_t m, int64_t n, int64_t k, bool k_in_rows = false) {
   if (m < 0 || n < 0 || k < 0) return fail(WX_ERR_INVALID_ARGUMENT, "%s: negative dimension", who);
   if (m > INT32_MAX || n > INT32_MAX || k > INT32_MAX) return fail(WX_ERR_UNSUPPORTED, "%s: dimension exceeds int32", who);
-  if (n % 8 != 0 || k % 8 != 0)
+  if (n % 8 != 0 || (k % 8 != 0 && !k_in_rows))
     return fail(WX_ERR_UNSUPPORTED, "%s: n (%lld) and k (%lld) must be multiples of 8", who, static_cast<long long>(n),
                 static_cast<long long>(k));
   // 256 rows of one operand must stay addressable through a 31-bit buffer offset
@@ -699,7 +775,7 @@ int check_dims(const char* who, int64_t m, int64_t n, int64_t k) {
 // When they would occupy at most half of the CUs, the 128 x 128 tile gives four times as many workgroups to spread
 // over the chip.  If the bounds fall on both sides of that threshold the choice is made on the device: both
 // shapes are launched and the one on the wrong side returns immediately.
-template <int MODE>
+template <int MODE, bool KA = false, bool KB = false>
 int launch_mfma(Params p, int64_t tiles_lo, int64_t tiles_hi, hipStream_t s, const char* who) {
   const int cus = device_cu_count();
   const int threshold = cus / 2;
@@ -707,12 +783,13 @@ int launch_mfma(Params p, int64_t tiles_lo, int64_t tiles_hi, hipStream_t s, con
   p.gate_tiles = threshold;
   if (small) {
     p.gate = big ? 1 : 0;
-    hipLaunchKernelGGL((dual_gemm_kernel<MODE, SmallTile>), dim3(cus * SmallTile::kWgPerCu), dim3(SmallTile::kThreads), 0, s, p);
+    hipLaunchKernelGGL((dual_gemm_kernel<MODE, SmallTile, KA, KB>), dim3(cus * SmallTile::kWgPerCu),
+                       dim3(SmallTile::kThreads), 0, s, p);
   }
   if (big) {
     p.gate = small ? 2 : 0;
     using Big = BigTileFor<MODE>;
-    hipLaunchKernelGGL((dual_gemm_kernel<MODE, Big>), dim3(cus * Big::kWgPerCu), dim3(Big::kThreads), 0, s, p);
+    hipLaunchKernelGGL((dual_gemm_kernel<MODE, Big, KA, KB>), dim3(cus * Big::kWgPerCu), dim3(Big::kThreads), 0, s, p);
   }
   return check_launch(who);
 }
@@ -727,8 +804,9 @@ using namespace wx;
 extern "C" int wx_dual_gemm(const void* in0, const void* in1, const void* w0, const void* w1, void* out0, void* out1,
                             int64_t m0, int64_t n0, int64_t k0, int64_t m1, int64_t n1, int64_t k1, int trans_a,
                             int trans_b, wx_stream_t stream) {
-  if (int rc = check_dims("wx_dual_gemm", m0, n0, k0)) return rc;
-  if (int rc = check_dims("wx_dual_gemm", m1, n1, k1)) return rc;
+  const bool k_in_rows = trans_a && !trans_b;  // A [k, m] and B [k, n]
+  if (int rc = check_dims("wx_dual_gemm", m0, n0, k0, k_in_rows)) return rc;
+  if (int rc = check_dims("wx_dual_gemm", m1, n1, k1, k_in_rows)) return rc;
   const void* ptrs[2][3] = {{in0, w0, out0}, {in1, w1, out1}};
   const int64_t dims[2][3] = {{m0, n0, k0}, {m1, n1, k1}};
   Params p{};
@@ -754,11 +832,22 @@ extern "C" int wx_dual_gemm(const void* in0, const void* in1, const void* w0, co
   p.offsets = nullptr;
   if ((m0 == 0 || n0 == 0) && (m1 == 0 || n1 == 0)) return WX_OK;
   hipStream_t s = as_stream(stream);
-  // an empty contraction (k == 0) has zeros as its result: the plain kernel below writes them
+  // an empty contraction (k == 0) has zeros as its result: the plain kernel below writes them (it also takes
+  // K-major operands too large for the MFMA kernel's 32-bit byte counts)
   const bool empty_k = (k0 == 0 && m0 > 0 && n0 > 0) || (k1 == 0 && m1 > 0 && n1 > 0);
-  if (!trans_a && trans_b && !empty_k) {
+  // K-major operands (A stored [k, m], B stored [k, n]) advance by whole rows of K through a 32-bit byte count
+  bool fits = true;
+  for (int e = 0; e < 2; ++e) {
+    if (trans_a && dims[e][2] * dims[e][0] * 2 >= (1ll << 32)) fits = false;
+    if (!trans_b && dims[e][2] * dims[e][1] * 2 >= (1ll << 32)) fits = false;
+  }
+  if (!empty_k && fits) {
     const int64_t tiles = ceil_div(m0, BigTile::BM) * ceil_div(n0, BigTile::BN) + ceil_div(m1, BigTile::BM) * ceil_div(n1, BigTile::BN);
-    return launch_mfma<kGeneric>(p, tiles, tiles, s, "dual_gemm_kernel<generic>");
+    const char* who = "dual_gemm_kernel<generic>";
+    if (!trans_a && trans_b) return launch_mfma<kGeneric, false, false>(p, tiles, tiles, s, who);
+    if (!trans_a && !trans_b) return launch_mfma<kGeneric, false, true>(p, tiles, tiles, s, who);
+    if (trans_a && trans_b) return launch_mfma<kGeneric, true, false>(p, tiles, tiles, s, who);
+    return launch_mfma<kGeneric, true, true>(p, tiles, tiles, s, who);
   }
   hipLaunchKernelGGL(dual_gemm_reference_layout_kernel, dim3(device_cu_count() * 4), dim3(256), 0, s, p, trans_a, trans_b);
   return check_launch("dual_gemm_reference_layout_kernel");

@@ -60,12 +60,6 @@ class _DualExpertFFN(torch.autograd.Function):
         raise NotImplementedError("wallx_mi355.moe: gradients go through _MoeBlockFunction, not the fused forward")
 
 
-def _pad_rows8(t: torch.Tensor) -> torch.Tensor:
-    """Zero rows up to a multiple of 8 (the transposed GEMM layouts want 16-byte rows after transposition)."""
-    extra = (-t.size(0)) % 8
-    return t if extra == 0 else torch.cat((t, t.new_zeros(extra, t.size(1))))
-
-
 def _dual(a0, a1, w0, w1, n0, n1, trans_a, trans_b):
     m0 = a0.size(1) if trans_a else a0.size(0)
     m1 = a1.size(1) if trans_a else a1.size(0)
@@ -101,8 +95,8 @@ class _MoeBlockFunction(torch.autograd.Function):
         m0, m1 = o[1] - o[0], o[2] - o[1]
         xs = native.permute_rows(x.detach(), row_id_map, 1, T)
         dys = native.permute_rows(dy.contiguous().to(torch.bfloat16), row_id_map, 1, T)
-        x0, x1 = _pad_rows8(xs[:m0]), _pad_rows8(xs[m0:m0 + m1])
-        dy0, dy1 = _pad_rows8(dys[:m0]), _pad_rows8(dys[m0:m0 + m1])
+        x0, x1 = xs[:m0], xs[m0:m0 + m1]
+        dy0, dy1 = dys[:m0], dys[m0:m0 + m1]
         I0, I1 = g0.size(0), g1.size(0)
         ga0, ga1 = _dual(x0, x1, g0, g1, I0, I1, False, True)
         up0, up1 = _dual(x0, x1, u0, u1, I0, I1, False, True)
@@ -131,7 +125,7 @@ class _MoeBlockFunction(torch.autograd.Function):
         if need[0]:
             a0, a1 = _dual(dg0, dg1, g0, g1, H, H, False, False)
             b0, b1 = _dual(du0, du1, u0, u1, H, H, False, False)
-            dxs = torch.cat(((a0.float() + b0.float())[:m0], (a1.float() + b1.float())[:m1])).to(torch.bfloat16)
+            dxs = torch.cat((a0.float() + b0.float(), a1.float() + b1.float())).to(torch.bfloat16)
             dx = native.unpermute(dxs, row_id_map, torch.tensor([]), T, 1)
         return (dx, None, None, None, None, *grads)
 

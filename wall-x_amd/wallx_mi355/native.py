@@ -98,26 +98,12 @@ def asym_dual_gmm(input_expert0, input_expert1, weight_expert0, weight_expert1, 
     m1, n1, k1 = dims(a1, w1)
     if tuple(output_expert0.shape) != (m0, n0) or tuple(output_expert1.shape) != (m1, n1):
         raise RuntimeError("output shape mismatch")
-    # The MFMA kernel contracts over the contiguous index of both operands (A [m, k], B [n, k]).  Other layouts get
-    # transposed copies first (one pass over HBM each); shapes the transpose kernel does not take (an edge that is
-    # not a multiple of 8) go to the library's plain kernel for that layout.
-    def transposable(t):
-        return t.size(0) % 8 == 0 and t.size(1) % 8 == 0
-
-    if (trans_a and not (transposable(a0) and transposable(a1))) or \
-            (not trans_b and not (transposable(w0) and transposable(w1))):
-        with _DeviceGuard(a0):
-            _lib.call("wx_dual_gemm", _ptr(a0), _ptr(a1), _ptr(w0), _ptr(w1), _ptr(output_expert0),
-                      _ptr(output_expert1), m0, n0, k0, m1, n1, k1, int(bool(trans_a)), int(bool(trans_b)),
-                      _stream(a0))
-        return
-    if trans_a:
-        a0, a1 = transpose_2d(a0), transpose_2d(a1)
-    if not trans_b:
-        w0, w1 = transpose_2d(w0), transpose_2d(w1)
+    # Every layout runs on the MFMA kernel: operands stored with K as the slow dimension (trans_a, or weights kept
+    # [k, n]) are transposed between LDS and the registers, so no transposed copy is made.
     with _DeviceGuard(a0):
         _lib.call("wx_dual_gemm", _ptr(a0), _ptr(a1), _ptr(w0), _ptr(w1), _ptr(output_expert0),
-                  _ptr(output_expert1), m0, n0, k0, m1, n1, k1, 0, 1, _stream(a0))
+                  _ptr(output_expert1), m0, n0, k0, m1, n1, k1, int(bool(trans_a)), int(bool(trans_b)),
+                  _stream(a0))
 
 
 def transpose_2d(t: torch.Tensor) -> torch.Tensor:
