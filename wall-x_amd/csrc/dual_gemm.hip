@@ -276,6 +276,10 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
     uint32_t a_bytes, b_bytes;        // readable bytes from the base (row-major) / from the current block (tiled)
     uint32_t voff_a[kLoadsA], voff_b[kLoadsB];
     int64_t a_step, b_step;           // tiled: bytes between consecutive K steps
+    // tiled: the load stream walks a tile's K steps in order, so the step's base and the bytes readable from it are
+    // kept as running values (one add and one saturating subtract per step) instead of products with the step index
+    const char *a_cur, *b_cur;
+    uint32_t a_left, b_left, a_dec, b_dec;
     int K, nk;      // nk: K steps of the tile, rounded up to a multiple of kStages (padding steps read zeros)
   };
   struct Store {    // where the finished tile goes
@@ -322,6 +326,12 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
       const int64_t b_left = (static_cast<int64_t>(G.k / kBlkCols) * G.ldb - b_blk) << 10;
       L.a_bytes = static_cast<uint32_t>(a_left < 0 ? 0 : (a_left > 0x7fffff00ll ? 0x7fffff00ll : a_left));
       L.b_bytes = static_cast<uint32_t>(b_left < 0 ? 0 : (b_left > 0x7fffff00ll ? 0x7fffff00ll : b_left));
+      L.a_cur = reinterpret_cast<const char*>(L.a_base);
+      L.b_cur = reinterpret_cast<const char*>(L.b_base);
+      L.a_left = L.a_bytes;
+      L.b_left = L.b_bytes;
+      L.a_dec = static_cast<uint32_t>(L.a_step > 0x7fffff00ll ? 0x7fffff00ll : L.a_step);
+      L.b_dec = static_cast<uint32_t>(L.b_step > 0x7fffff00ll ? 0x7fffff00ll : L.b_step);
 #pragma unroll
       for (int i = 0; i < kLoadsA; ++i) L.voff_a[i] = static_cast<uint32_t>(i * kBlkBytes + lane * 16);
 #pragma unroll
@@ -379,19 +389,20 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
     __amdgpu_buffer_rsrc_t rb;
     uint32_t voff_b[kLoadsB];
   };
-  auto issue_a = [&](const Loader& L, int ks, unsigned char* sa, Pending& P) {
+  auto issue_a = [&](Loader& L, int ks, unsigned char* sa, Pending& P) {
     __amdgpu_buffer_rsrc_t ra;
     uint32_t oob = 0;
     if constexpr (TILED_IN) {
       // steps past K (ring padding) and blocks past the end of the matrix read as zero through the bounds check
       const bool real = ks * BK < L.K;
-      const int64_t da = L.a_step * ks, db = L.b_step * ks;
-      const int64_t la = static_cast<int64_t>(L.a_bytes) - da, lb = static_cast<int64_t>(L.b_bytes) - db;
-      // the byte counts are clamped for huge matrices; a clamped count is far above what one step reads
-      const uint32_t na = !real ? 0u : (L.a_bytes == 0x7fffff00u ? 0x7fffff00u : static_cast<uint32_t>(la < 0 ? 0 : la));
-      const uint32_t nb = !real ? 0u : (L.b_bytes == 0x7fffff00u ? 0x7fffff00u : static_cast<uint32_t>(lb < 0 ? 0 : lb));
-      ra = make_rsrc(reinterpret_cast<const char*>(L.a_base) + da, na);
-      P.rb = make_rsrc(reinterpret_cast<const char*>(L.b_base) + db, nb);
+      ra = make_rsrc(L.a_cur, real ? L.a_left : 0u);
+      P.rb = make_rsrc(L.b_cur, real ? L.b_left : 0u);
+      // on to the next K step.  The byte counts are clamped for huge matrices; a clamped count is far above what
+      // one step reads and stays as it is.
+      L.a_cur += L.a_step;
+      L.b_cur += L.b_step;
+      if (L.a_left != 0x7fffff00u) L.a_left = L.a_left > L.a_dec ? L.a_left - L.a_dec : 0u;
+      if (L.b_left != 0x7fffff00u) L.b_left = L.b_left > L.b_dec ? L.b_left - L.b_dec : 0u;
     } else {
       const int k0 = ks * BK;
       // advancing the base keeps the absolute end of the readable range, so rows past the matrix read as zero;
@@ -502,7 +513,7 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
   // refill with the K step kStages ahead in the load stream (step `ld_ks` of tile `L`) starts at once: the A half
   // here, the B half in the next step's first group.  The next slot's data was issued kStages - 1 steps ago.
   Pending pend;
-  auto k_step = [&](const Loader& L, int ld_ks, unsigned char* sa, unsigned char* sb, unsigned char* sa_n,
+  auto k_step = [&](Loader& L, int ld_ks, unsigned char* sa, unsigned char* sb, unsigned char* sa_n,
                     unsigned char* sb_n, unsigned char* sb_p) {
     read_frags(sa, sb, 1, 1);
     issue_b(pend, sb_p);
@@ -684,8 +695,8 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
           setup_loader(tc, L);
           setup_store(tc, S);
         } else {
-          L.a_bytes = 0;
-          L.b_bytes = 0;
+          L.a_bytes = L.a_left = 0;
+          L.b_bytes = L.b_left = 0;
           L.K = 0;
         }
         ld_ks = 0;
