@@ -167,14 +167,24 @@ class PrefillHarness:
                 v = v.view(B, S, nkv, D).transpose(1, 2)
             with timer.section("mrope"):
                 if self.fuse:
-                    q, k = ops.multimodal_rope_from_positions(q, k, pos, self.inv_freq, list(wl.MROPE_SECTION))
+                    # rotated q / k stay token-major ([B, S, H, D] memory behind the [B, H, S, D] view the kernel
+                    # writes through strides), so attention's output comes back token-major as well and the
+                    # o projection reads it without a transposing copy
+                    qr = torch.empty(B, S, nq, D, dtype=q.dtype, device=self.dev).transpose(1, 2)
+                    kr = torch.empty(B, S, nkv, D, dtype=k.dtype, device=self.dev).transpose(1, 2)
+                    native.rope_from_positions(q, k, pos, self.inv_freq, qr, kr, [2 * s for s in wl.MROPE_SECTION])
+                    q, k = qr, kr
                 else:
                     q, k = ops.multimodal_rope(q, k, cos, sin, list(wl.MROPE_SECTION))
             with timer.section("sdpa_torch"):
                 a = F.scaled_dot_product_attention(q, k, v, attn_mask=attn_mask, is_causal=attn_mask is None,
                                                    enable_gqa=True)
             with timer.section("o_proj_torch"):
-                h = h + F.linear(a.transpose(1, 2).reshape(B, S, nq * D), layer["wo"])
+                a2d = a.transpose(1, 2).reshape(B * S, nq * D)  # a view when attention kept the token-major layout
+                if self.fuse:
+                    h = torch.addmm(h.view(B * S, H), a2d, layer["wo"].t()).view(B, S, H)  # residual in the GEMM
+                else:
+                    h = h + F.linear(a2d, layer["wo"]).view(B, S, H)
             h = self._ffn(h.view(B * S, H), layer["ln2"], routing, layer["packed"], timer).view(B, S, H)
         with timer.section("lm_head_torch"):
             last = rms_norm(h[:, -1], self.final_ln, self.eps)
