@@ -182,8 +182,15 @@ def main():
         _lib.call("wx_unpermute_rows_add", y_sorted.data_ptr(), x.data_ptr(), y.data_ptr(), row_id_map.data_ptr(), T, H,
                   stream)
 
+    normed = torch.empty_like(y)
+
+    def unpermute_add_norm():
+        _lib.call("wx_unpermute_rows_add_rmsnorm", y_sorted.data_ptr(), x.data_ptr(), y.data_ptr(), normed.data_ptr(),
+                  norm_w.data_ptr(), 1e-6, row_id_map.data_ptr(), T, H, stream)
+
     t_np, _ = event_ms(norm_permute, iters, batch=10)
     t_ua, _ = event_ms(unpermute_add, iters, batch=10)
+    t_uan, _ = event_ms(unpermute_add_norm, iters, batch=10)
     permute()  # x_tiled back to the plain permute's contents for anything that runs after this
     gate_up_tflops = gate_up_flops / (t_gate_up_avg * 1e-3) / 1e12
 
@@ -199,6 +206,8 @@ def main():
         "rmsnorm_permute_ms": round(t_np, 4), "rmsnorm_permute_GBps": round(row_bytes / t_np / 1e6, 1),
         "unpermute_residual_ms": round(t_ua, 4),
         "unpermute_residual_GBps": round((row_bytes + 2.0 * T * H) / t_ua / 1e6, 1),  # one more [T, H] read
+        "unpermute_residual_rmsnorm_ms": round(t_uan, 4),  # ... and one more [T, H] write (the next reader's norm)
+        "unpermute_residual_rmsnorm_GBps": round((row_bytes + 4.0 * T * H) / t_uan / 1e6, 1),
     }
 
     if not args.ops_only:

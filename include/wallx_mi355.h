@@ -241,6 +241,13 @@ int wx_rmsnorm_permute_rows_tiled(const void* x, const void* weight, float eps, 
                                   int64_t num_tokens, int64_t num_cols, wx_stream_t stream);
 int wx_unpermute_rows_add(const void* y, const void* residual, void* out, const int32_t* row_id_map,
                           int64_t num_tokens, int64_t num_cols, wx_stream_t stream);
+/* wx_unpermute_rows_add with the RMSNorm that consumes its result next folded in: out = residual + unpermuted y
+ * (the residual stream after the layer, act.py:265) and normed = weight * rmsnorm(out, eps), i.e. the following
+ * layer's input_layernorm (act.py:240) or the model's final norm (act.py:506), computed from the bf16-rounded
+ * sum as the separate module would.  num_cols: a multiple of 8, at most 4096. */
+int wx_unpermute_rows_add_rmsnorm(const void* y, const void* residual, void* out, void* normed,
+                                  const void* weight, float eps, const int32_t* row_id_map,
+                                  int64_t num_tokens, int64_t num_cols, wx_stream_t stream);
 
 /* dst [cols, rows] = transpose of src [rows, cols], both row-major and contiguous, 2-byte elements (bf16 / fp16),
  * rows and cols multiples of 8.  A utility without a counterpart in the reference; wx_dual_gemm does not need it

@@ -66,6 +66,30 @@ def test_unpermute_add(dev, T, H):
     assert torch.equal(got.cpu(), ref)
 
 
+@pytest.mark.parametrize("T,H", [(300, 256), (912, 2048), (7, 8), (33, 1000), (20, 4096)])
+def test_unpermute_add_rmsnorm(dev, T, H):
+    """The closing residual add of a layer with the next reader's RMSNorm in the same pass: the sum is bit-equal to
+    the eager add; the norm equals the oracle's RMSNorm of that (bf16) sum except where the fp32 sum of squares,
+    accumulated in another order, moves the normalised value across a rounding boundary: one bf16 step there, which
+    the rounded product with the weight can turn into two."""
+    g = torch.Generator().manual_seed(T * H + 1)
+    y, resid = _bf((T, H), g, 2.0), _bf((T, H), g, 2.0)
+    w = (1.0 + 0.1 * torch.randn(H, generator=g)).to(torch.bfloat16)
+    types = torch.rand(T, generator=g) < 0.2
+    _, rmap_ref, _ = oracle.permute_ref(y, types)
+    rmap, _, _, _ = native.partition(types.to(dev), 2, 0, None, want_sorted=False)
+    out, normed = native.unpermute_add_rmsnorm(y.to(dev), resid.to(dev), rmap, w.to(dev), 1e-6)
+    ref_sum = resid + oracle.unpermute_ref(y, rmap_ref)
+    assert torch.equal(out.cpu(), ref_sum)
+    ref_norm = oracle.rms_norm_ref(ref_sum, w, 1e-6).float()
+    got = normed.cpu().float()
+    bad = (got - ref_norm).abs() > 2.0 ** -6 * ref_norm.abs() + 1e-6
+    assert not bad.any(), f"{int(bad.sum())} of {bad.numel()} differ by more than two bf16 steps"
+    one = (got - ref_norm).abs() > 2.0 ** -7 * ref_norm.abs() + 1e-6
+    assert float(one.float().mean()) < 1e-4  # more than one step: a handful per million
+    assert float((got != ref_norm).float().mean()) < 0.02
+
+
 def test_moe_block_with_both_fusions(dev):
     """h + block(RMSNorm(h)) through the module's fused path against the same module fed by separate PyTorch ops."""
     from types import SimpleNamespace

@@ -1,7 +1,9 @@
 // The row movers fused with their neighbours in the decoder layer (act.py:256-265):
 //   rmsnorm_permute_tiled   post-attention RMSNorm + permute into the K-tiled activation matrix of the FFN
 //   unpermute_add           unpermute + residual add
-// Each replaces two passes over [T, H] by one.  bf16 only (the FFN kernels' type).
+//   unpermute_add_rmsnorm   the same, and the RMSNorm that reads the sum next (the following layer's
+//                           input_layernorm, act.py:240, or the final norm, act.py:506) as a second output
+// Each replaces two (three) passes over [T, H] by one.  bf16 only (the FFN kernels' type).
 //
 // RMSNorm follows the reference module op by op: x in fp32, variance = mean(x^2), x * rsqrt(variance + eps),
 // rounded to bf16, times the bf16 weight, rounded to bf16 (Qwen2RMSNorm as used at act.py:190-193).  The sum of
@@ -108,6 +110,63 @@ __global__ __launch_bounds__(256) void unpermute_add_kernel(const u32x4* __restr
   }
 }
 
+// out[t] = resid[t] + y[row_id_map[t]], normed[t] = weight * rmsnorm(out[t]); one wavefront per row, the row held
+// in registers (NV 16-byte chunks per lane).  The norm reads the bf16-rounded sum, as a separate kernel would.
+template <int NV>
+__global__ __launch_bounds__(256) void unpermute_add_rmsnorm_kernel(
+    const u32x4* __restrict__ y, const u32x4* __restrict__ resid, u32x4* __restrict__ out, u32x4* __restrict__ normed,
+    const u32x4* __restrict__ weight, float eps, const int32_t* __restrict__ row_id_map, int64_t num_tokens,
+    int vec_per_row) {
+  const int lane = threadIdx.x & 63;
+  const int64_t wave = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
+  const int64_t n_waves = static_cast<int64_t>(gridDim.x) * 4;
+  for (int64_t t = wave; t < num_tokens; t += n_waves) {
+    const int32_t src_row = row_id_map[t];
+    const u32x4* src = y + static_cast<int64_t>(src_row < 0 ? 0 : src_row) * vec_per_row;
+    const u32x4* res = resid + t * vec_per_row;
+    u32x4 a[NV], b[NV];
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+      const int cc = lane + u * 64;
+      if (cc < vec_per_row) {
+        a[u] = ld16(res + cc);
+        b[u] = src_row < 0 ? u32x4{0, 0, 0, 0} : ld16(src + cc);
+      }
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+      if (lane + u * 64 < vec_per_row) {
+        float fa[8], fb[8];
+        unpack16<WX_BF16>(a[u], fa);
+        unpack16<WX_BF16>(b[u], fb);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) fa[e] += fb[e];
+        a[u] = pack16<WX_BF16>(fa);  // the residual stream as stored
+        st16(out + t * vec_per_row + lane + u * 64, a[u]);
+        unpack16<WX_BF16>(a[u], fa);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) ss += fa[e] * fa[e];
+      }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) ss += __shfl_xor(ss, off);
+    const float inv = __frsqrt_rn(ss / static_cast<float>(vec_per_row * 8) + eps);
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+      const int cc = lane + u * 64;
+      if (cc < vec_per_row) {
+        float f[8], w[8];
+        unpack16<WX_BF16>(a[u], f);
+        unpack16<WX_BF16>(weight[cc], w);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) f[e] = w[e] * round_bf16(f[e] * inv);  // pack16 rounds the product
+        st16(normed + t * vec_per_row + cc, pack16<WX_BF16>(f));
+      }
+    }
+  }
+}
+
 }  // namespace
 }  // namespace wx
 
@@ -166,4 +225,39 @@ extern "C" int wx_unpermute_rows_add(const void* y, const void* residual, void* 
                      as_stream(stream), static_cast<const u32x4*>(y), static_cast<const u32x4*>(residual),
                      static_cast<u32x4*>(out), row_id_map, num_tokens, num_cols / 8);
   return check_launch("unpermute_add_kernel");
+}
+
+extern "C" int wx_unpermute_rows_add_rmsnorm(const void* y, const void* residual, void* out, void* normed,
+                                             const void* weight, float eps, const int32_t* row_id_map,
+                                             int64_t num_tokens, int64_t num_cols, wx_stream_t stream) {
+  const char* who = "wx_unpermute_rows_add_rmsnorm";
+  if (num_tokens < 0 || num_cols <= 0) return fail(WX_ERR_INVALID_ARGUMENT, "%s: bad sizes", who);
+  if (num_cols % 8 != 0 || num_cols > 4096)
+    return fail(WX_ERR_UNSUPPORTED, "%s: num_cols (%lld) must be a multiple of 8 and at most 4096", who,
+                static_cast<long long>(num_cols));
+  if (!(eps >= 0.f)) return fail(WX_ERR_INVALID_ARGUMENT, "%s: eps must be non-negative", who);
+  if (num_tokens == 0) return WX_OK;
+  if (num_tokens > INT32_MAX) return fail(WX_ERR_UNSUPPORTED, "%s: more than 2^31-1 rows", who);
+  if (!y || !residual || !out || !normed || !weight || !row_id_map)
+    return fail(WX_ERR_INVALID_ARGUMENT, "%s: null pointer", who);
+  if ((reinterpret_cast<uintptr_t>(y) | reinterpret_cast<uintptr_t>(residual) | reinterpret_cast<uintptr_t>(out) |
+       reinterpret_cast<uintptr_t>(normed) | reinterpret_cast<uintptr_t>(weight)) & 15)
+    return fail(WX_ERR_INVALID_ARGUMENT, "%s: buffers must be 16-byte aligned", who);
+  const int vec = static_cast<int>(num_cols / 8);
+  const int64_t want = (num_tokens + 3) / 4;
+  const int64_t cap = static_cast<int64_t>(device_cu_count()) * 8;
+  const dim3 grid(static_cast<unsigned>(want < cap ? want : cap)), block(256);
+  hipStream_t s = as_stream(stream);
+#define WX_CASE(N)                                                                                                   \
+  case N:                                                                                                            \
+    hipLaunchKernelGGL(unpermute_add_rmsnorm_kernel<N>, grid, block, 0, s, static_cast<const u32x4*>(y),             \
+                       static_cast<const u32x4*>(residual), static_cast<u32x4*>(out), static_cast<u32x4*>(normed),   \
+                       static_cast<const u32x4*>(weight), eps, row_id_map, num_tokens, vec);                         \
+    break;
+  switch ((vec + 63) / 64) {
+    WX_CASE(1) WX_CASE(2) WX_CASE(3) WX_CASE(4) WX_CASE(5) WX_CASE(6) WX_CASE(7) WX_CASE(8)
+    default: return fail(WX_ERR_UNSUPPORTED, "%s: num_cols too large", who);
+  }
+#undef WX_CASE
+  return check_launch("unpermute_add_rmsnorm_kernel");
 }

@@ -10,9 +10,11 @@ batch of full sequences (prefill).  What it states explicitly:
   * attention mask: plain causal by default (`mask="causal"`); `mask="action_block"` adds the reference's
     bidirectional block among action tokens (act.py:616-637) through a dense boolean mask,
   * rotary base 1e6, mrope_section [16, 24, 24], cos/sin built in fp32 and cast to bf16 (vl.py:679-712),
-  * `fuse=True` (default) runs the post-attention RMSNorm inside the permute and the residual add inside the
-    unpermute (one pass over [T, H] each instead of two), and M-RoPE evaluates cos/sin from the position ids in
-    the kernel (no [3, B, S, D] tables); `fuse=False` keeps them as separate PyTorch ops.
+  * `fuse=True` (default) runs the post-attention RMSNorm inside the permute, the residual add AND the next
+    reader's RMSNorm (the following layer's input_layernorm, or the final norm) inside the unpermute, M-RoPE
+    evaluates cos/sin from the position ids in the kernel (no [3, B, S, D] tables) and leaves q / k token-major,
+    and the attention residual is added by the o-projection GEMM; `fuse=False` keeps all of these as separate
+    PyTorch ops.
 """
 
 from contextlib import contextmanager
@@ -92,8 +94,10 @@ class PrefillHarness:
         self._ws = None
 
     # ------------------------------------------------------------------------------------------------
-    def _ffn(self, h: torch.Tensor, ln_weight: torch.Tensor, routing: moe.Routing, packed, timer: OpTimer) -> torch.Tensor:
-        """h [T, H] (the residual stream after attention) -> h + FFN(RMSNorm(h))."""
+    def _ffn(self, h: torch.Tensor, ln_weight: torch.Tensor, routing: moe.Routing, packed, timer: OpTimer,
+             next_norm: Optional[torch.Tensor] = None):
+        """h [T, H] (the residual stream after attention) -> (h + FFN(RMSNorm(h)), RMSNorm of that with `next_norm`
+        when fused, else None)."""
         from . import _lib
 
         T, H = h.shape
@@ -122,12 +126,12 @@ class PrefillHarness:
             _lib.call("wx_dual_down_proj", self._hmid.data_ptr(), y_sorted.data_ptr(), routing.expert_offsets.data_ptr(),
                       d0.data_ptr(), d1.data_ptr(), T, H, I0, I1, None, stream)
         if self.fuse:
-            with timer.section("unpermute+residual"):
-                return native.unpermute_add(y_sorted, h, routing.row_id_map)
+            with timer.section("unpermute+residual+rmsnorm"):
+                return native.unpermute_add_rmsnorm(y_sorted, h, routing.row_id_map, next_norm, self.eps)
         with timer.section("unpermute"):
             y = native.unpermute(y_sorted, routing.row_id_map, torch.tensor([]), T, 1)
         with timer.section("residual_torch"):
-            return h + y
+            return h + y, None
 
     @torch.no_grad()
     def forward(self, input_ids: torch.Tensor, image_grid_thw: torch.Tensor, moe_token_types: torch.Tensor,
@@ -156,9 +160,11 @@ class PrefillHarness:
             attn_mask = causal[None, None] | act
         with timer.section("embed_torch"):
             h = self.embed[input_ids]
-        for layer in self.layers:
-            with timer.section("rmsnorm_torch"):
-                x = rms_norm(h, layer["ln1"], self.eps)
+        x = None  # RMSNorm of h for the next reader, when the previous layer's closing kernel already made it
+        for li, layer in enumerate(self.layers):
+            if x is None:
+                with timer.section("rmsnorm_torch"):
+                    x = rms_norm(h, layer["ln1"], self.eps)
             with timer.section("qkv_proj_torch"):
                 qkv = F.linear(x, layer["wqkv"], layer["bqkv"])
                 q, k, v = qkv.split([nq * D, nkv * D, nkv * D], dim=-1)
@@ -185,9 +191,12 @@ class PrefillHarness:
                     h = torch.addmm(h.view(B * S, H), a2d, layer["wo"].t()).view(B, S, H)  # residual in the GEMM
                 else:
                     h = h + F.linear(a2d, layer["wo"]).view(B, S, H)
-            h = self._ffn(h.view(B * S, H), layer["ln2"], routing, layer["packed"], timer).view(B, S, H)
+            nxt = self.layers[li + 1]["ln1"] if li + 1 < len(self.layers) else self.final_ln
+            h, x = self._ffn(h.view(B * S, H), layer["ln2"], routing, layer["packed"], timer, nxt)
+            h = h.view(B, S, H)
+            x = x.view(B, S, H) if x is not None else None
         with timer.section("lm_head_torch"):
-            last = rms_norm(h[:, -1], self.final_ln, self.eps)
+            last = x[:, -1] if x is not None else rms_norm(h[:, -1], self.final_ln, self.eps)
             logits = F.linear(last, self.embed)
         return logits
 

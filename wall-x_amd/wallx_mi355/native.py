@@ -479,6 +479,24 @@ def unpermute_add(y_sorted: torch.Tensor, residual: torch.Tensor, row_id_map: to
     return out
 
 
+def unpermute_add_rmsnorm(y_sorted: torch.Tensor, residual: torch.Tensor, row_id_map: torch.Tensor,
+                          weight: torch.Tensor, eps: float):
+    """(residual + y_sorted[row_id_map], rmsnorm of that sum with `weight`) in one pass (topK 1, bf16): the layer's
+    closing residual add (act.py:265) and the next layer's input_layernorm (act.py:240) or the final norm."""
+    _need_cuda("y_sorted", y_sorted)
+    if y_sorted.dtype != torch.bfloat16 or residual.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
+        raise RuntimeError("All tensors must be BFloat16 for this kernel")
+    y_sorted, residual, weight = y_sorted.contiguous(), residual.contiguous(), weight.contiguous()
+    T, H = residual.shape
+    if y_sorted.shape[1] != H or row_id_map.numel() < T or weight.numel() != H:
+        raise RuntimeError("shape mismatch between residual, sorted rows, weight and row_id_map")
+    out, normed = torch.empty_like(residual), torch.empty_like(residual)
+    with _DeviceGuard(residual):
+        _lib.call("wx_unpermute_rows_add_rmsnorm", _ptr(y_sorted), _ptr(residual), _ptr(out), _ptr(normed),
+                  _ptr(weight), float(eps), _ptr(row_id_map), T, H, _stream(residual))
+    return out, normed
+
+
 def dual_swiglu_ffn(x_tiled: torch.Tensor, num_rows: int, expert_offsets: torch.Tensor, weights,
                     hmid: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
                     host_rows=None) -> torch.Tensor:
