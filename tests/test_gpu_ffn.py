@@ -167,6 +167,30 @@ def test_fused_ffn_small(dev, T, n_act, hidden, inters):
     _close(y, ref32, atol=2 * ATOL, rtol=2 * RTOL, what="moe layer vs fp32 math")
 
 
+@pytest.mark.parametrize("T,n_act,hidden,inters", [
+    (8600, 300, 2048, (1056, 256)),   # gate/up: 301 large tiles, 45 left over, among them a ragged last column
+    (8600, 8300, 2048, (256, 1056)),  # the action expert is the long one
+    (8600, 300, 2176, (512, 128)),    # down: 315 large tiles with a ragged last column; the short expert rides along
+])
+def test_fused_ffn_ragged_last_round(dev, T, n_act, hidden, inters):
+    """More 256 x 256 tiles than CUs with a few left over: the whole rounds run as large tiles and the leftover as
+    tiles of half the width in a second launch.  Whole output against the oracle, with the row split known only on
+    the device and with it handed over from the host (right and wrong)."""
+    g = torch.Generator().manual_seed(T + n_act + hidden)
+    x = _bf((T, hidden), g)
+    types = torch.zeros(T, dtype=torch.bool)
+    types[torch.randperm(T, generator=g)[:n_act]] = True
+    ws = _moe_weights(hidden, inters, g, 0.03)
+    ref = oracle.sparse_moe_block_ref(x[None], types[None], [w.as_tuple() for w in ws])[0]
+    wd = [w.to(dev).as_tuple() for w in ws]
+    y, routing = moe.moe_layer_forward(x.to(dev), types.to(dev), wd)
+    assert routing.expert_offsets.cpu().tolist() == [0, T - n_act, T]
+    _close(y, ref, what="device-side split")
+    for hint in ((T - n_act, n_act), (n_act, T - n_act), (T, 0)):
+        yh, _ = moe.moe_layer_forward(x.to(dev), types.to(dev), wd, routing=routing, host_rows=hint)
+        assert int((yh != y).sum()) == 0, f"host row counts {hint} changed the result"
+
+
 def test_moe_block_module_is_a_drop_in(dev):
     class Cfg:
         experts = [{"hidden_size": 256, "intermediate_size": 512, "hidden_act": "silu"},

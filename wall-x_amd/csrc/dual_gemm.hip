@@ -10,7 +10,9 @@
 // 32x32x16 accumulator blocks (256 accumulator registers per lane), one workgroup per CU; the gate/up launch runs
 // the same tile with eight wavefronts (2 x 4, wave tile 128 x 64).  Problems whose 256 x 256
 // tiles would leave most CUs idle (a denoise step of a few thousand action tokens) run the same kernel with a
-// 128 x 128 tile, two workgroups per CU.  Operands are K-contiguous, so both MFMA fragments are 16-byte LDS reads.
+// 128 x 128 tile, two workgroups per CU.  A ragged last round of the fused FFN launches (tiles left over after the
+// whole rounds of one tile per CU) runs as 256 x 128 tiles in a second launch when those fit the chip in one go.
+// Operands are K-contiguous, so both MFMA fragments are 16-byte LDS reads.
 // Global -> LDS uses buffer loads that write LDS directly (no register staging) into a ring of four K-step slots
 // per operand; the load stream runs four K steps ahead of the MFMAs and crosses tile boundaries, with one
 // workgroup barrier per K step.  LDS rows are 64 bytes; chunk c of row r sits in slot c ^ ((r >> 2) & 3), which
@@ -75,6 +77,8 @@ using BigTile8 = TileShape<256, 256, 2, 4>;
 using SmallTile = TileShape<128, 128, 2, 2>;  // two workgroups per CU; for problems with too few big tiles to fill the chip
 template <int MODE>
 using BigTileFor = std::conditional_t<MODE == 1 /* kGateUp */, BigTile8, BigTile>;
+// half as wide as BigTile: for the ragged last round of a launch (see tail_split_point)
+using HalfTile = TileShape<256, 128, 2, 2>;
 
 constexpr int kXcds = 8;
 constexpr int kGroupM = 8;                     // tile rows per patch in the tile order
@@ -99,6 +103,10 @@ struct Params {
   // number of 256 x 256 tiles is on its side of `gate_tiles`.  0 = always run, 1 = run if at most gate_tiles,
   // 2 = run if more.
   int gate, gate_tiles;
+  // Tail split (see tail_split_point): 0 = off; 1 = this launch does the whole rounds of 256 x 256 tiles and leaves
+  // the ragged last round to a second launch; 2 = this is that second launch, with tiles of half the width.
+  // split_cus = workgroups of the first launch (one per CU).
+  int split, split_cus;
 };
 
 #define LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
@@ -125,10 +133,7 @@ struct TileCoord {
 // contiguous range of "virtual" ids; virtual ids then sweep patches of kGroupM tile rows column by column.
 // Integer division runs on the vector ALU even for uniform operands, so the results are handed back through
 // readfirstlane to keep everything derived from them (descriptors, branches) scalar.
-__device__ __forceinline__ bool map_tile(int t, int total, const int* tiles_m, const int* tiles_n, TileCoord& tc) {
-  const int per = (total + kXcds - 1) / kXcds;
-  int v = (t % kXcds) * per + t / kXcds;
-  if (v >= total) return false;
+__device__ __forceinline__ void tile_coords(int v, const int* tiles_m, const int* tiles_n, TileCoord& tc) {
   int g = 0;
   const int c0 = tiles_m[0] * tiles_n[0];
   if (v >= c0) { g = 1; v -= c0; }
@@ -141,7 +146,30 @@ __device__ __forceinline__ bool map_tile(int t, int total, const int* tiles_m, c
   tc.group = g;
   tc.tm = first_m + (in_patch - q * rows);
   tc.tn = q;
+}
+__device__ __forceinline__ bool map_tile(int t, int total, const int* tiles_m, const int* tiles_n, TileCoord& tc) {
+  const int per = (total + kXcds - 1) / kXcds;
+  const int v = (t % kXcds) * per + t / kXcds;
+  if (v >= total) return false;
+  tile_coords(v, tiles_m, tiles_n, tc);
   return true;
+}
+
+// The ragged last round.  `total` 256 x 256 tiles on `cus` workgroups take ceil(total / cus) rounds however few
+// tiles the last round holds.  When the tiles left over after the whole rounds (in virtual-id order: the last tile
+// rows of expert 0, then expert 1) fit the chip as tiles of half the width -- one per workgroup, each taking about
+// 0.6 of a full tile's time -- the first launch stops at the whole rounds and a second launch runs the rest as
+// half tiles.  Tiles of an expert whose contraction is at most half as long as the other's are cheap enough to
+// ride along as second half tiles and are not counted.  Returns the number of tiles of the first launch
+// (== total: no split).  Evaluated identically by the host (when it knows the row counts) and by both launches.
+__host__ __device__ inline int tail_split_point(int tiles0, int tiles1, int k0, int k1, int cus) {
+  const int total = tiles0 + tiles1;
+  if (cus <= 0 || total <= cus) return total;
+  const int full = total / cus * cus, tail = total - full;
+  if (tail == 0) return total;
+  const int tail1 = tail < tiles1 ? tail : tiles1, tail0 = tail - tail1;
+  const int counted = (tiles1 > 0 && tiles0 > 0 && 2ll * k1 <= k0) ? tail0 : tail;
+  return 2 * counted <= cus ? full : total;
 }
 
 // Workgroup barrier without the fences of __syncthreads().  Those fences make the compiler wait for EVERY
@@ -236,7 +264,28 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
     const bool few = big(g0.m, g0.n) + big(g1.m, g1.n) <= p.gate_tiles;
     if (few != (p.gate == 1)) return;  // uniform: the other tile shape's launch does this problem
   }
-  const int total = tiles_m[0] * tiles_n[0] + tiles_m[1] * tiles_n[1];  // the host bounds this below 2^31
+  int total = tiles_m[0] * tiles_n[0] + tiles_m[1] * tiles_n[1];  // the host bounds this below 2^31
+  // tail split: the first launch (256 x 256 tiles) stops at `split_at`; the second (this shape: half as wide)
+  // takes virtual tiles [split_at, all) of the 256 x 256 tiling, two halves each
+  constexpr bool kIsHalf = std::is_same_v<TS, HalfTile>, kIsBig = std::is_same_v<TS, BigTileFor<MODE>>;
+  int big_m[2], big_n[2], split_at = 0, halves = 0;
+  if ((kIsBig && p.split == 1) || (kIsHalf && p.split == 2)) {
+    constexpr int kBigN = SWIGLU ? BigTile::BN / 2 : BigTile::BN;
+    big_m[0] = (g0.m + BigTile::BM - 1) / BigTile::BM;
+    big_n[0] = (g0.n + kBigN - 1) / kBigN;
+    if (g0.m <= 0 || g0.n <= 0) big_m[0] = big_n[0] = 0;
+    big_m[1] = (g1.m + BigTile::BM - 1) / BigTile::BM;
+    big_n[1] = (g1.n + kBigN - 1) / kBigN;
+    if (g1.m <= 0 || g1.n <= 0) big_m[1] = big_n[1] = 0;
+    const int all = big_m[0] * big_n[0] + big_m[1] * big_n[1];
+    split_at = tail_split_point(big_m[0] * big_n[0], big_m[1] * big_n[1], g0.k, g1.k, p.split_cus);
+    if constexpr (kIsBig) {
+      total = split_at;  // a multiple of 8 when smaller than `all`
+    } else {
+      if (split_at == all) return;  // no split: the first launch did everything
+      halves = 2 * (all - split_at);
+    }
+  }
   const int padded = (total + kXcds - 1) / kXcds * kXcds;
 
   // ---- per-lane constants -----------------------------------------------------------------------
@@ -657,6 +706,14 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
   int next_t = blockIdx.x;
   auto next_tile = [&](TileCoord& tc) {
     bool have = false;
+    if (kIsHalf && p.split == 2) {
+      for (; next_t < halves && !have; next_t += gridDim.x) {
+        tile_coords(split_at + (next_t >> 1), big_m, big_n, tc);
+        tc.tn = 2 * tc.tn + (next_t & 1);
+        have = tc.tn < (tc.group ? tiles_n[1] : tiles_n[0]);  // the second half of a ragged last column may be empty
+      }
+      return have;
+    }
     for (; next_t < padded && !have; next_t += gridDim.x) have = map_tile(next_t, total, tiles_m, tiles_n, tc);
     return have;
   };
@@ -786,12 +843,19 @@ int check_dims(const char* who, int64_t m, int64_t n, int64_t k, bool k_in_rows 
 // When they would occupy at most half of the CUs, the 128 x 128 tile gives four times as many workgroups to spread
 // over the chip.  If the bounds fall on both sides of that threshold the choice is made on the device: both
 // shapes are launched and the one on the wrong side returns immediately.
+// tiles_by_expert: the host's exact 256 x 256 tile counts per expert, or null when only the device knows the row
+// split.  The fused FFN launches use the tail split: a second launch with half-width tiles takes the ragged last
+// round when that pays; when the host cannot tell, both launches are made and the device decides (the second
+// returns at once if there is nothing to split).
 template <int MODE, bool KA = false, bool KB = false>
-int launch_mfma(Params p, int64_t tiles_lo, int64_t tiles_hi, hipStream_t s, const char* who) {
+int launch_mfma(Params p, int64_t tiles_lo, int64_t tiles_hi, hipStream_t s, const char* who,
+                const int64_t* tiles_by_expert = nullptr) {
   const int cus = device_cu_count();
   const int threshold = cus / 2;
   const bool small = tiles_lo <= threshold, big = tiles_hi > threshold;
   p.gate_tiles = threshold;
+  p.split = 0;
+  p.split_cus = cus;
   if (small) {
     p.gate = big ? 1 : 0;
     hipLaunchKernelGGL((dual_gemm_kernel<MODE, SmallTile, KA, KB>), dim3(cus * SmallTile::kWgPerCu),
@@ -800,7 +864,21 @@ int launch_mfma(Params p, int64_t tiles_lo, int64_t tiles_hi, hipStream_t s, con
   if (big) {
     p.gate = small ? 2 : 0;
     using Big = BigTileFor<MODE>;
-    hipLaunchKernelGGL((dual_gemm_kernel<MODE, Big, KA, KB>), dim3(cus * Big::kWgPerCu), dim3(Big::kThreads), 0, s, p);
+    static_assert(Big::kWgPerCu == 1 && HalfTile::kWgPerCu == 1, "the split counts one workgroup per CU");
+    bool split = MODE != kGeneric && tiles_hi > cus;
+    if (split && tiles_by_expert != nullptr) {
+      const int64_t all = tiles_by_expert[0] + tiles_by_expert[1];
+      split = all < INT32_MAX && tail_split_point(static_cast<int>(tiles_by_expert[0]), static_cast<int>(tiles_by_expert[1]),
+                                                  p.g[0].k, p.g[1].k, cus) != all;
+    }
+    p.split = split ? 1 : 0;
+    hipLaunchKernelGGL((dual_gemm_kernel<MODE, Big, KA, KB>), dim3(cus), dim3(Big::kThreads), 0, s, p);
+    if constexpr (MODE != kGeneric) {
+      if (split) {
+        p.split = 2;
+        hipLaunchKernelGGL((dual_gemm_kernel<MODE, HalfTile, KA, KB>), dim3(cus), dim3(HalfTile::kThreads), 0, s, p);
+      }
+    }
   }
   return check_launch(who);
 }
@@ -938,8 +1016,9 @@ int launch_gate_up(const FfnArgs& a, hipStream_t s) {
   p.offsets = a.offsets;
   const int64_t t0 = ceil_div(a.inter[0], BigTile::BN / 2), t1 = ceil_div(a.inter[1], BigTile::BN / 2);
   if (a.host_rows != nullptr) {  // the caller knows the split: one launch of the right tile shape
-    const int64_t tiles = ceil_div(a.host_rows[0], BigTile::BM) * t0 + ceil_div(a.host_rows[1], BigTile::BM) * t1;
-    return launch_mfma<kGateUp>(p, tiles, tiles, s, "dual_gemm_kernel<gate_up>");
+    const int64_t by_expert[2] = {ceil_div(a.host_rows[0], BigTile::BM) * t0, ceil_div(a.host_rows[1], BigTile::BM) * t1};
+    const int64_t tiles = by_expert[0] + by_expert[1];
+    return launch_mfma<kGateUp>(p, tiles, tiles, s, "dual_gemm_kernel<gate_up>", by_expert);
   }
   // the split of the rows between the experts is only known on the device: bound the tile count from the total
   const int64_t row_tiles = ceil_div(a.rows, BigTile::BM);
@@ -965,8 +1044,9 @@ int launch_down(const FfnArgs& a, hipStream_t s) {
   p.offsets = a.offsets;
   const int64_t col_tiles = ceil_div(a.hidden, BigTile::BN);
   if (a.host_rows != nullptr) {
-    const int64_t tiles = (ceil_div(a.host_rows[0], BigTile::BM) + ceil_div(a.host_rows[1], BigTile::BM)) * col_tiles;
-    return launch_mfma<kDown>(p, tiles, tiles, s, "dual_gemm_kernel<down>");
+    const int64_t by_expert[2] = {ceil_div(a.host_rows[0], BigTile::BM) * col_tiles, ceil_div(a.host_rows[1], BigTile::BM) * col_tiles};
+    const int64_t tiles = by_expert[0] + by_expert[1];
+    return launch_mfma<kDown>(p, tiles, tiles, s, "dual_gemm_kernel<down>", by_expert);
   }
   const int64_t row_tiles = ceil_div(a.rows, BigTile::BM);
   return launch_mfma<kDown>(p, row_tiles * col_tiles, (row_tiles + 1) * col_tiles, s, "dual_gemm_kernel<down>");
