@@ -216,6 +216,7 @@ def main():
         extra["cold_hbm"] = cold_measurements(dev, x, row_id_map, T, H, row_bytes, iters)
         extra["config4"] = config4_measurement(dev, weights)
         extra["asym_dual_gmm_op"] = backward_measurement(dev, x, weights, m0)
+        extra["block_training_step"] = training_step_measurement(dev, x, types, weights)
         extra["ceilings"] = ceiling_measurements(dev, x, weights, m0)
     if not args.ops_only and not args.no_prefill:
         del x_tiled, hmid, x_sorted, y_sorted, y
@@ -444,6 +445,50 @@ def backward_measurement(dev, x, weights, m0):
     return {"forward_nt_ms": round(t_fw, 3), "forward_nt_tflops": round(flops / t_fw / 1e9, 1),
             "dx_ms": round(t_dx, 3), "dx_tflops": round(flops / t_dx / 1e9, 1),
             "dw_ms": round(t_dw, 3), "dw_tflops": round(flops / t_dw / 1e9, 1)}
+
+
+def training_step_measurement(dev, x, token_types, weights):
+    """Forward + backward of the drop-in SparseMoeBlock (wallx_mi355/moe.py) on the config 3 batch: the fused forward,
+    then the block's own backward (gate / up recomputed, SwiGLU derivative in one elementwise kernel, dX and dW of
+    all three projections of both experts as dual GEMMs in their K-major layouts).  FLOPs counted as 3 x forward
+    (the recompute, one third more, is not counted)."""
+    import torch
+    from types import SimpleNamespace
+    from wallx_mi355 import moe
+
+    H = x.shape[1]
+    inters = [w[0].shape[0] for w in weights]
+    cfg = SimpleNamespace(experts=[dict(hidden_size=H, intermediate_size=i, hidden_act="silu") for i in inters])
+    block = moe.SparseMoeBlock(cfg, 2).to(dev).to(torch.bfloat16)
+    with torch.no_grad():
+        for e, (gw, uw, dw) in enumerate(weights):
+            block.experts[e].gate_proj.weight.copy_(gw)
+            block.experts[e].up_proj.weight.copy_(uw)
+            block.experts[e].down_proj.weight.copy_(dw)
+    xb = x.detach().clone().view(1, -1, H).requires_grad_(True)
+    tb = token_types.view(1, -1)
+    dy = torch.randn(xb.shape, device=dev).to(torch.bfloat16)
+    routing = block.route(tb)
+
+    def fwd():
+        with torch.no_grad():
+            block(xb, tb, routing=routing)
+
+    def step():
+        for prm in block.parameters():
+            prm.grad = None
+        xb.grad = None
+        block(xb, tb, routing=routing).backward(dy)
+
+    t_f, _ = event_ms(fwd, 5, warm=2)
+    t_s, _ = event_ms(step, 5, warm=2)
+    m1 = int(token_types.sum())
+    flops = 6.0 * H * ((x.shape[0] - m1) * inters[0] + m1 * inters[1])
+    out = {"forward_ms": round(t_f, 3), "forward_backward_ms": round(t_s, 3),
+           "tflops_counting_3x_forward": round(3 * flops / t_s / 1e9, 1)}
+    del block, xb, dy
+    torch.cuda.empty_cache()
+    return out
 
 
 def ceiling_measurements(dev, x, weights, m0):

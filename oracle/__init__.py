@@ -32,6 +32,8 @@ How each function is pinned (tests/test_oracle_*.py):
                                    brute force over small grids
   window_index_ref                 permutation / window-size invariants, brute
                                    force enumeration of windows on small grids
+  swiglu_bwd_ref                   central differences of silu(g) * u in float64,
+                                   the closed form of silu' at 0 and far from 0
   rms_norm_ref                     torch.nn.functional.rms_norm in fp32, the
                                    closed form for constant rows, transformers'
                                    Qwen2RMSNorm where it is importable
@@ -48,7 +50,7 @@ from .permute import (  # noqa: F401
     unpermute_bwd_ref,
     expert_offsets_ref,
 )
-from .ffn import dual_gemm_ref, swiglu_ffn_ref, sparse_moe_block_ref  # noqa: F401
+from .ffn import dual_gemm_ref, swiglu_ffn_ref, swiglu_bwd_ref, sparse_moe_block_ref  # noqa: F401
 from .mrope import (  # noqa: F401
     rotate_half_ref,
     mrope_axis_map,

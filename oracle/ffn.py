@@ -53,6 +53,22 @@ def swiglu_ffn_ref(x, gate_w, up_w, down_w, eager_rounding: bool = True):
     return y.to(dt)
 
 
+def swiglu_bwd_ref(gate, up, dh):
+    """(hmid, dgate, dup) for h = silu(gate) * up (act.py:79-82) and the gradient dh w.r.t. h.
+
+    The reference leaves this to autograd; so does this restatement (torch.autograd on the fp32 expression), with
+    hmid carrying the forward's eager rounding (silu rounded to the activation dtype before the product) and each
+    result rounded once.
+    """
+    dt = gate.dtype
+    g = gate.to(torch.float32).clone().requires_grad_(True)
+    u = up.to(torch.float32).clone().requires_grad_(True)
+    h = F.silu(g) * u
+    dg, du = torch.autograd.grad(h, (g, u), dh.to(torch.float32))
+    hm = (F.silu(g.detach()).to(dt).to(torch.float32) * u.detach()).to(dt)
+    return hm, dg.to(dt), du.to(dt)
+
+
 def sparse_moe_block_ref(hidden, experts_indices, weights, eager_rounding: bool = True):
     """SparseMoeBlock.forward (act.py:105-162).
 

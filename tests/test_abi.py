@@ -73,6 +73,9 @@ def test_argument_errors_without_a_gpu():
     assert lib.wx_unpermute_rows_add_rmsnorm(None, None, None, None, None, 1e-6, None, 4, 8192, None) == -2  # cols > 4096
     assert lib.wx_unpermute_rows_add_rmsnorm(None, None, None, None, None, 1e-6, None, 4, 2048, None) == -1
     assert lib.wx_unpermute_rows_add_rmsnorm(None, None, None, None, None, 1e-6, None, 0, 2048, None) == 0
+    assert lib.wx_swiglu_bwd(None, None, None, None, None, None, 12, None) == -2  # count % 8
+    assert lib.wx_swiglu_bwd(None, None, None, None, None, None, 16, None) == -1
+    assert lib.wx_swiglu_bwd(None, None, None, None, None, None, 0, None) == 0
     assert lib.wx_transpose_2d(None, None, 12, 16, 2, None) == -2  # rows % 8
     assert lib.wx_transpose_2d(None, None, 16, 16, 4, None) == -2  # element size
     assert lib.wx_transpose_2d(None, None, 16, 16, 2, None) == -1

@@ -289,6 +289,20 @@ def test_config4_skewed_and_empty_groups(dev):
         _close(y[rows.to(dev)], ref, what=f"prefill + {n_act} action")
 
 
+@pytest.mark.parametrize("shape", [(1, 8), (37, 264), (300, 1056), (0, 64)])
+def test_swiglu_bwd_kernel(dev, shape):
+    g = torch.Generator().manual_seed(shape[0] + shape[1])
+    gate, up, dh = _bf(shape, g, 2.0), _bf(shape, g), _bf(shape, g)
+    hm, dg, du = native.swiglu_bwd(gate.to(dev), up.to(dev), dh.to(dev))
+    rh, rg, ru = oracle.swiglu_bwd_ref(gate, up, dh)
+    # fp32 math with the device's exp against the host's: a bf16 step where a result sits on a rounding boundary
+    for got, ref, what in ((hm, rh, "hmid"), (dg, rg, "dgate"), (du, ru, "dup")):
+        got, ref = got.float().cpu(), ref.float()
+        bad = (got - ref).abs() > 2.0 ** -7 * ref.abs() + 1e-30
+        assert not bad.any(), f"{what}: {int(bad.sum())} of {bad.numel()} differ by more than a bf16 step"
+        assert got.numel() == 0 or float((got != ref).float().mean()) < 0.02, what
+
+
 @pytest.mark.parametrize("fused_extras", [False, True])
 def test_moe_block_backward_matches_autograd_of_the_plain_forward(dev, fused_extras):
     """Gradients of the block (inputs and all six weights) against torch autograd through the oracle's fp32

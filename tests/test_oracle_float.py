@@ -68,6 +68,36 @@ def test_swiglu_eager_rounding_close_to_fp32_math_in_bf16():
     assert torch.all((a - b).abs() <= 2e-2 + 1e-2 * b.abs())
 
 
+def test_swiglu_bwd_against_central_differences_and_closed_forms():
+    """dgate and dup of h = silu(g) * u: central differences of the float64 expression written out with exp (no
+    library silu), silu'(0) = 1/2, silu'(x) -> 1 and silu(x) -> x for large x, -> 0 for very negative x."""
+    g = torch.Generator().manual_seed(8)
+    gate = torch.randn(64, 40, generator=g) * 2
+    up = torch.randn(64, 40, generator=g)
+    dh = torch.randn(64, 40, generator=g)
+    hm, dg, du = oracle.swiglu_bwd_ref(gate, up, dh)
+    G, U, D = gate.double().numpy(), up.double().numpy(), dh.double().numpy()
+    h = lambda a, b: a / (1.0 + np.exp(-a)) * b
+    eps = 1e-6
+    num_dg = (h(G + eps, U) - h(G - eps, U)) / (2 * eps) * D
+    num_du = (h(G, U + eps) - h(G, U - eps)) / (2 * eps) * D
+    assert np.allclose(dg.double().numpy(), num_dg, rtol=1e-5, atol=1e-6)
+    assert np.allclose(du.double().numpy(), num_du, rtol=1e-5, atol=1e-6)
+    assert np.allclose(hm.double().numpy(), h(G, U), rtol=1e-5, atol=1e-6)
+    one = torch.ones(4)
+    _, dg0, du0 = oracle.swiglu_bwd_ref(torch.zeros(4), 3 * one, one)
+    assert torch.allclose(dg0, 1.5 * one) and torch.all(du0 == 0)       # silu'(0) = 1/2, silu(0) = 0
+    _, dgp, dup = oracle.swiglu_bwd_ref(30 * one, 2 * one, one)
+    assert torch.allclose(dgp, 2 * one, atol=1e-6) and torch.allclose(dup, 30 * one, atol=1e-4)
+    _, dgn, dun = oracle.swiglu_bwd_ref(-30 * one, 2 * one, one)
+    assert torch.allclose(dgn, 0 * one, atol=1e-6) and torch.allclose(dun, 0 * one, atol=1e-6)
+    # bf16: hmid carries the forward's rounding of silu before the product
+    gb, ub = gate.to(torch.bfloat16), up.to(torch.bfloat16)
+    hb, _, _ = oracle.swiglu_bwd_ref(gb, ub, dh.to(torch.bfloat16))
+    want = (torch.nn.functional.silu(gb.float()).to(torch.bfloat16).float() * ub.float()).to(torch.bfloat16)
+    assert torch.equal(hb, want)
+
+
 def test_moe_block_matches_per_token_evaluation():
     """The block equals applying each token's own expert to that token alone."""
     g = torch.Generator().manual_seed(9)

@@ -19,7 +19,7 @@ OUT_DIR = os.path.join(os.path.dirname(HERE), "wallx_mi355")
 LIB = os.path.join(OUT_DIR, "libwallx_mi355.so")
 OBJ_DIR = os.path.join(HERE, "build")
 
-SOURCES = ["common.hip", "partition.hip", "dual_gemm.hip", "mrope.hip", "rope_index.hip", "vision_index.hip", "transpose.hip", "fused_movers.hip", "probe.hip"]
+SOURCES = ["common.hip", "partition.hip", "dual_gemm.hip", "mrope.hip", "rope_index.hip", "vision_index.hip", "transpose.hip", "fused_movers.hip", "swiglu_bwd.hip", "probe.hip"]
 HEADERS = ["common.h", "grid_prefix.h", os.path.join(INCLUDE, "wallx_mi355.h")]
 
 FLAGS = [

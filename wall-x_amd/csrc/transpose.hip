@@ -1,6 +1,5 @@
-// bf16 / fp16 matrix transpose for the backward GEMMs: the MFMA kernel reads both operands with the contraction
-// index contiguous (A [m, k], B [n, k]); dX = dY @ W and dW = dY^T @ X have one or both operands the other way
-// round, and a transposed copy (one pass over HBM) is far cheaper than a GEMM that reads LDS column-wise.
+// bf16 / fp16 matrix transpose: a utility for callers that want a transposed copy (the dual GEMM itself reads every
+// operand layout in place).
 //
 // 64 x 64 element tiles through LDS: 16-byte global reads along the source rows, 2-byte LDS writes into the
 // transposed position, 16-byte reads of the transposed rows, 16-byte global stores.

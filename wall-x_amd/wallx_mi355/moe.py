@@ -74,7 +74,7 @@ class _MoeBlockFunction(torch.autograd.Function):
 
     Forward is the fused path.  Backward recomputes gate and up (they are not kept by the fused kernels) and runs
     every contraction of both experts as one dual GEMM: dHm = dY Wd, dWd = dY^T Hm, dX = dG Wg + dU Wu,
-    dWg = dG^T X, dWu = dU^T X, with the SwiGLU derivative elementwise in fp32.  The per-expert row counts are
+    dWg = dG^T X, dWu = dU^T X, with the SwiGLU derivative in one fused elementwise kernel (fp32 math).  The per-expert row counts are
     read back from the device once per backward (the forward never synchronises)."""
 
     @staticmethod
@@ -102,17 +102,8 @@ class _MoeBlockFunction(torch.autograd.Function):
         up0, up1 = _dual(x0, x1, u0, u1, I0, I1, False, True)
         dh0, dh1 = _dual(dy0, dy1, d0, d1, I0, I1, False, False)
 
-        def swiglu_grads(ga, up, dh):
-            g, u, d = ga.float(), up.float(), dh.float()
-            sig = torch.sigmoid(g)
-            silu = g * sig
-            hm = (silu.to(torch.bfloat16).float() * u).to(torch.bfloat16)  # what the forward fed to the down GEMM
-            dg = (d * u * sig * (1.0 + g * (1.0 - sig))).to(torch.bfloat16)
-            du = (d * silu).to(torch.bfloat16)
-            return hm, dg, du
-
-        hm0, dg0, du0 = swiglu_grads(ga0, up0, dh0)
-        hm1, dg1, du1 = swiglu_grads(ga1, up1, dh1)
+        hm0, dg0, du0 = native.swiglu_bwd(ga0, up0, dh0)
+        hm1, dg1, du1 = native.swiglu_bwd(ga1, up1, dh1)
         need = ctx.needs_input_grad
         grads = [None] * 6
         if need[5] or need[8]:  # gate weights
@@ -125,7 +116,9 @@ class _MoeBlockFunction(torch.autograd.Function):
         if need[0]:
             a0, a1 = _dual(dg0, dg1, g0, g1, H, H, False, False)
             b0, b1 = _dual(du0, du1, u0, u1, H, H, False, False)
-            dxs = torch.cat((a0.float() + b0.float(), a1.float() + b1.float())).to(torch.bfloat16)
+            dxs = torch.empty(T, H, dtype=torch.bfloat16, device=x.device)
+            torch.add(a0, b0, out=dxs[:m0])
+            torch.add(a1, b1, out=dxs[m0:m0 + m1])
             dx = native.unpermute(dxs, row_id_map, torch.tensor([]), T, 1)
         return (dx, None, None, None, None, *grads)
 

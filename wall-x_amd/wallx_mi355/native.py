@@ -106,6 +106,22 @@ def asym_dual_gmm(input_expert0, input_expert1, weight_expert0, weight_expert1, 
                   _stream(a0))
 
 
+def swiglu_bwd(gate: torch.Tensor, up: torch.Tensor, dh: torch.Tensor):
+    """(hmid, dgate, dup) of h = silu(gate) * up for the gradient dh, in one pass (bf16, same shapes)."""
+    for name, t in (("gate", gate), ("up", up), ("dh", dh)):
+        _need_cuda(name, t)
+        if t.dtype != torch.bfloat16:
+            raise RuntimeError("All tensors must be BFloat16 for this kernel")
+    if gate.shape != up.shape or gate.shape != dh.shape:
+        raise RuntimeError("gate, up and dh must have one shape")
+    gate, up, dh = gate.contiguous(), up.contiguous(), dh.contiguous()
+    hm, dg, du = torch.empty_like(gate), torch.empty_like(gate), torch.empty_like(gate)
+    with _DeviceGuard(gate):
+        _lib.call("wx_swiglu_bwd", _ptr(gate), _ptr(up), _ptr(dh), _ptr(hm), _ptr(dg), _ptr(du), gate.numel(),
+                  _stream(gate))
+    return hm, dg, du
+
+
 def transpose_2d(t: torch.Tensor) -> torch.Tensor:
     """Contiguous transposed copy of a contiguous 2-D bf16 / fp16 tensor whose sizes are multiples of 8."""
     _need_cuda("tensor", t)
