@@ -210,17 +210,28 @@ def main():
         "unpermute_residual_rmsnorm_GBps": round((row_bytes + 4.0 * T * H) / t_uan / 1e6, 1),
     }
 
+    # Side measurements: none of them enters `value`.  One that fails (out of memory on a smaller card, say) is
+    # reported in its place and must not cost the line its contract fields.
+    def side(name, fn, *fargs):
+        try:
+            out = fn(*fargs)
+        except Exception as exc:  # noqa: BLE001 - the message goes into the report
+            out = {"error": f"{type(exc).__name__}: {exc}"[:300]}
+        if name is None:
+            extra.update(out)
+        else:
+            extra[name] = out
+
     if not args.ops_only:
-        extra.update(side_measurements(dev, iters))
-    if not args.ops_only:
-        extra["cold_hbm"] = cold_measurements(dev, x, row_id_map, T, H, row_bytes, iters)
-        extra["config4"] = config4_measurement(dev, weights)
-        extra["asym_dual_gmm_op"] = backward_measurement(dev, x, weights, m0)
-        extra["block_training_step"] = training_step_measurement(dev, x, types, weights)
-        extra["ceilings"] = ceiling_measurements(dev, x, weights, m0)
+        side(None, side_measurements, dev, iters)
+        side("cold_hbm", cold_measurements, dev, x, row_id_map, T, H, row_bytes, iters)
+        side("config4", config4_measurement, dev, weights)
+        side("asym_dual_gmm_op", backward_measurement, dev, x, weights, m0)
+        side("block_training_step", training_step_measurement, dev, x, types, weights)
+        side("ceilings", ceiling_measurements, dev, x, weights, m0)
     if not args.ops_only and not args.no_prefill:
         del x_tiled, hmid, x_sorted, y_sorted, y
-        extra["prefill"] = prefill_measurement(dev, args.prefill_mask)
+        side("prefill", prefill_measurement, dev, args.prefill_mask)
 
     result = {
         "metric": "dual_expert_ffn_tflops",
