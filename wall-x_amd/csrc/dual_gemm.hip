@@ -11,7 +11,8 @@
 // the same tile with eight wavefronts (2 x 4, wave tile 128 x 64).  Problems whose 256 x 256
 // tiles would leave most CUs idle (a denoise step of a few thousand action tokens) run the same kernel with a
 // 128 x 128 tile, two workgroups per CU.  A ragged last round of the fused FFN launches (tiles left over after the
-// whole rounds of one tile per CU) runs as 256 x 128 tiles in a second launch when those fit the chip in one go.
+// whole rounds of one tile per CU) runs in that small shape too, in a second launch, when it then fits the chip in
+// one go.
 // Operands are K-contiguous, so both MFMA fragments are 16-byte LDS reads.
 // Global -> LDS uses buffer loads that write LDS directly (no register staging) into a ring of four K-step slots
 // per operand; the load stream runs four K steps ahead of the MFMAs and crosses tile boundaries, with one
@@ -77,8 +78,9 @@ using BigTile8 = TileShape<256, 256, 2, 4>;
 using SmallTile = TileShape<128, 128, 2, 2>;  // two workgroups per CU; for problems with too few big tiles to fill the chip
 template <int MODE>
 using BigTileFor = std::conditional_t<MODE == 1 /* kGateUp */, BigTile8, BigTile>;
-// half as wide as BigTile: for the ragged last round of a launch (see tail_split_point)
-using HalfTile = TileShape<256, 128, 2, 2>;
+// the shape that runs the ragged last round of a launch (see tail_split_point): BigTile cut in four.  (Cut in two,
+// 256 x 128 with one workgroup per CU, measures the same.)
+using TailTile = SmallTile;
 
 constexpr int kXcds = 8;
 constexpr int kGroupM = 8;                     // tile rows per patch in the tile order
@@ -104,7 +106,7 @@ struct Params {
   // 2 = run if more.
   int gate, gate_tiles;
   // Tail split (see tail_split_point): 0 = off; 1 = this launch does the whole rounds of 256 x 256 tiles and leaves
-  // the ragged last round to a second launch; 2 = this is that second launch, with tiles of half the width.
+  // the ragged last round to a second launch; 2 = this is that second launch, with 128 x 128 tiles.
   // split_cus = workgroups of the first launch (one per CU).
   int split, split_cus;
 };
@@ -157,10 +159,10 @@ __device__ __forceinline__ bool map_tile(int t, int total, const int* tiles_m, c
 
 // The ragged last round.  `total` 256 x 256 tiles on `cus` workgroups take ceil(total / cus) rounds however few
 // tiles the last round holds.  When the tiles left over after the whole rounds (in virtual-id order: the last tile
-// rows of expert 0, then expert 1) fit the chip as tiles of half the width -- one per workgroup, each taking about
-// 0.6 of a full tile's time -- the first launch stops at the whole rounds and a second launch runs the rest as
-// half tiles.  Tiles of an expert whose contraction is at most half as long as the other's are cheap enough to
-// ride along as second half tiles and are not counted.  Returns the number of tiles of the first launch
+// rows of expert 0, then expert 1) fit the chip as 128 x 128 tiles in one go -- four per large tile, two workgroups
+// per CU -- the first launch stops at the whole rounds and a second launch runs the rest in the small shape.
+// Tiles of an expert whose contraction is at most half as long as the other's are cheap enough to ride along
+// as a second helping and are not counted.  Returns the number of tiles of the first launch
 // (== total: no split).  Evaluated identically by the host (when it knows the row counts) and by both launches.
 __host__ __device__ inline int tail_split_point(int tiles0, int tiles1, int k0, int k1, int cus) {
   const int total = tiles0 + tiles1;
@@ -265,11 +267,12 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
     if (few != (p.gate == 1)) return;  // uniform: the other tile shape's launch does this problem
   }
   int total = tiles_m[0] * tiles_n[0] + tiles_m[1] * tiles_n[1];  // the host bounds this below 2^31
-  // tail split: the first launch (256 x 256 tiles) stops at `split_at`; the second (this shape: half as wide)
-  // takes virtual tiles [split_at, all) of the 256 x 256 tiling, two halves each
-  constexpr bool kIsHalf = std::is_same_v<TS, HalfTile>, kIsBig = std::is_same_v<TS, BigTileFor<MODE>>;
-  int big_m[2], big_n[2], split_at = 0, halves = 0;
-  if ((kIsBig && p.split == 1) || (kIsHalf && p.split == 2)) {
+  // tail split: the first launch (256 x 256 tiles) stops at `split_at`; the second (this shape: 128 x 128)
+  // takes virtual tiles [split_at, all) of the 256 x 256 tiling, kSubM x kSubN pieces each
+  constexpr bool kIsTail = std::is_same_v<TS, TailTile>, kIsBig = std::is_same_v<TS, BigTileFor<MODE>>;
+  constexpr int kSubM = BigTile::BM / BM, kSubN = BigTile::BN / BN;
+  int big_m[2], big_n[2], split_at = 0, pieces = 0;
+  if ((kIsBig && p.split == 1) || (kIsTail && p.split == 2)) {
     constexpr int kBigN = SWIGLU ? BigTile::BN / 2 : BigTile::BN;
     big_m[0] = (g0.m + BigTile::BM - 1) / BigTile::BM;
     big_n[0] = (g0.n + kBigN - 1) / kBigN;
@@ -283,7 +286,7 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
       total = split_at;  // a multiple of 8 when smaller than `all`
     } else {
       if (split_at == all) return;  // no split: the first launch did everything
-      halves = 2 * (all - split_at);
+      pieces = kSubM * kSubN * (all - split_at);
     }
   }
   const int padded = (total + kXcds - 1) / kXcds * kXcds;
@@ -706,11 +709,14 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
   int next_t = blockIdx.x;
   auto next_tile = [&](TileCoord& tc) {
     bool have = false;
-    if (kIsHalf && p.split == 2) {
-      for (; next_t < halves && !have; next_t += gridDim.x) {
-        tile_coords(split_at + (next_t >> 1), big_m, big_n, tc);
-        tc.tn = 2 * tc.tn + (next_t & 1);
-        have = tc.tn < (tc.group ? tiles_n[1] : tiles_n[0]);  // the second half of a ragged last column may be empty
+    if (kIsTail && p.split == 2) {
+      for (; next_t < pieces && !have; next_t += gridDim.x) {
+        const int piece = next_t % (kSubM * kSubN);
+        tile_coords(split_at + next_t / (kSubM * kSubN), big_m, big_n, tc);
+        tc.tm = kSubM * tc.tm + piece / kSubN;
+        tc.tn = kSubN * tc.tn + piece % kSubN;
+        // pieces past a ragged last row / column of tiles are empty
+        have = tc.tm < (tc.group ? tiles_m[1] : tiles_m[0]) && tc.tn < (tc.group ? tiles_n[1] : tiles_n[0]);
       }
       return have;
     }
@@ -844,7 +850,7 @@ int check_dims(const char* who, int64_t m, int64_t n, int64_t k, bool k_in_rows 
 // over the chip.  If the bounds fall on both sides of that threshold the choice is made on the device: both
 // shapes are launched and the one on the wrong side returns immediately.
 // tiles_by_expert: the host's exact 256 x 256 tile counts per expert, or null when only the device knows the row
-// split.  The fused FFN launches use the tail split: a second launch with half-width tiles takes the ragged last
+// split.  The fused FFN launches use the tail split: a second launch with 128 x 128 tiles takes the ragged last
 // round when that pays; when the host cannot tell, both launches are made and the device decides (the second
 // returns at once if there is nothing to split).
 template <int MODE, bool KA = false, bool KB = false>
@@ -864,7 +870,7 @@ int launch_mfma(Params p, int64_t tiles_lo, int64_t tiles_hi, hipStream_t s, con
   if (big) {
     p.gate = small ? 2 : 0;
     using Big = BigTileFor<MODE>;
-    static_assert(Big::kWgPerCu == 1 && HalfTile::kWgPerCu == 1, "the split counts one workgroup per CU");
+    static_assert(Big::kWgPerCu == 1, "the split counts one large tile per CU and round");
     bool split = MODE != kGeneric && tiles_hi > cus;
     if (split && tiles_by_expert != nullptr) {
       const int64_t all = tiles_by_expert[0] + tiles_by_expert[1];
@@ -876,7 +882,8 @@ int launch_mfma(Params p, int64_t tiles_lo, int64_t tiles_hi, hipStream_t s, con
     if constexpr (MODE != kGeneric) {
       if (split) {
         p.split = 2;
-        hipLaunchKernelGGL((dual_gemm_kernel<MODE, HalfTile, KA, KB>), dim3(cus), dim3(HalfTile::kThreads), 0, s, p);
+        hipLaunchKernelGGL((dual_gemm_kernel<MODE, TailTile, KA, KB>), dim3(cus * TailTile::kWgPerCu),
+                           dim3(TailTile::kThreads), 0, s, p);
       }
     }
   }
