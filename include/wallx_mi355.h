@@ -201,8 +201,10 @@ int wx_mrope_apply_positions(const void* q, const void* k, const int64_t* positi
  * (act.py:1123-1149).  position_ids [3, B, S] int64, deltas [B] int64.
  * status (may be NULL): device word set to 1 when a row is malformed in a way that makes the PyTorch
  * path raise (a vision item without its tokens, more items than grids, a fully masked row).
- * workspace: wx_rope_index_workspace_bytes(B) bytes. */
-size_t wx_rope_index_workspace_bytes(int64_t batch);
+ * workspace: wx_rope_index_workspace_bytes(B, S) bytes (a few bytes per row; rows longer than 30720 tokens also
+ * keep their compacted form there, 5 bytes per token, instead of in LDS).  No cap on S or on images per row (the
+ * reference kernel stops at 64 segments per row, csrc/rope_index.cu). */
+size_t wx_rope_index_workspace_bytes(int64_t batch, int64_t seq);
 int wx_rope_index(const int64_t* input_ids, const int64_t* attention_mask,
                   const int64_t* image_grid_thw, int64_t n_image, const int64_t* video_grid_thw,
                   int64_t n_video, const float* second_per_grid_ts, int64_t batch, int64_t seq,

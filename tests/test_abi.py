@@ -34,7 +34,8 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(lib, name), f"{name} is declared in the header but missing from the library"
     assert lib.wx_abi_version() == 1
     assert lib.wx_partition_workspace_bytes(29184) >= 29184 // 512 * 1024
-    assert lib.wx_rope_index_workspace_bytes(16) >= 128
+    assert lib.wx_rope_index_workspace_bytes(16, 896) >= 128
+    assert lib.wx_rope_index_workspace_bytes(2, 65536) >= 2 * 5 * 65536  # long rows are compacted in the workspace
 
 
 def test_ctypes_table_matches_header():

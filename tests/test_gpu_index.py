@@ -93,6 +93,26 @@ def test_rope_index_many_images_per_row(dev):
     _rope_both(dev, ids, ig=grid)
 
 
+@pytest.mark.parametrize("S", [20000, 30720, 30721, 65536])
+def test_rope_index_long_rows(dev, S):
+    """Long rows (thousands of images between short text runs, a masked tail on one row): up to 30 720 tokens the
+    compacted row stays in LDS (above 48 KiB of it with a raised limit), beyond that in the workspace."""
+    g = torch.Generator().manual_seed(5)
+    rows, masks, n_images = [], [], 0
+    for b in range(2):
+        valid = S - 40 * b  # the second row ends in 40 masked positions
+        row = []
+        while len(row) + 13 <= valid - 5:
+            row += [TX] * int(torch.randint(0, 4, (1,), generator=g)) + [S0] + [I] * 8 + [E0]
+            n_images += 1
+        row += [TX] * (valid - len(row))
+        rows.append(row + [TX] * (S - valid))
+        masks.append([1] * valid + [0] * (S - valid))
+    ids = torch.tensor(rows)
+    grid = torch.tensor([[1, 4, 8]] * n_images)
+    _rope_both(dev, ids, ig=grid, mask=torch.tensor(masks))
+
+
 def test_rope_index_malformed_row_sets_status(dev):
     ids = torch.tensor([[TX, S0, I, I, TX]], device=dev)
     # the grid claims 4 merged tokens but the row ends after 3: the PyTorch path builds 6 positions for 5 tokens

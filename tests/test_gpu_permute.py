@@ -100,6 +100,29 @@ def test_config3_full_size_properties(dev):
     assert torch.equal(p[:n_vl], xf[(~ids).to(dev)]) and torch.equal(p[n_vl:], xf[ids.to(dev)])
 
 
+def test_one_million_tokens_round_trip(dev):
+    """2^20 tokens x 1024 bf16 columns (2 GiB each way), eight experts, everything checked on the device through the
+    properties the partition guarantees: the map is a permutation, rows of an expert are contiguous and in source
+    order, offsets are the cumulative counts, and unpermute undoes permute bit for bit."""
+    T, H, E = 1 << 20, 1024, 8
+    g = torch.Generator(device=dev).manual_seed(1)
+    x = torch.randint(-32768, 32767, (T, H), device=dev, generator=g, dtype=torch.int16).view(torch.bfloat16)
+    ids = torch.randint(0, E, (T,), device=dev, generator=g, dtype=torch.int32)
+    rmap, off, inv, _ = native.partition(ids, E, 0, None, want_sorted=True)
+    counts = torch.bincount(ids.long(), minlength=E)
+    assert torch.equal(off.long(), torch.cat([counts.new_zeros(1), counts.cumsum(0)]))
+    assert torch.equal(torch.sort(rmap.long()).values, torch.arange(T, device=dev))
+    assert torch.equal(inv.long()[rmap.long()], torch.arange(T, device=dev))          # inverse map
+    sorted_ids = ids[inv.long()]
+    assert bool((sorted_ids[1:] >= sorted_ids[:-1]).all())                             # experts contiguous, ascending
+    same = sorted_ids[1:] == sorted_ids[:-1]
+    assert bool((inv[1:][same] > inv[:-1][same]).all())                                # stable inside an expert
+    p = native.permute_rows(x, rmap, 1, T)
+    assert torch.equal(p.view(torch.int16), x.view(torch.int16)[inv.long()])
+    back = native.unpermute(p, rmap, torch.tensor([]), T, 1)
+    assert torch.equal(back.view(torch.int16), x.view(torch.int16))
+
+
 def test_config4_skewed_groups(dev):
     g = torch.Generator().manual_seed(0)
     x = torch.randn(2048, 256, generator=g).to(torch.bfloat16).to(dev)

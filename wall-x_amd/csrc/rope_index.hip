@@ -21,7 +21,13 @@ namespace {
 constexpr int kThreads = 256;
 constexpr int kWaves = kThreads / kWave;
 constexpr int kMaxSeg = 128;
-constexpr int kMaxSeq = 11264;  // cidx (4 B) + flag (1 B) per token plus the item table stay under 64 KiB of LDS
+// The compacted row -- cidx (4 B) and flag (1 B) per token -- lives in LDS up to this many tokens (with the item
+// table that stays under the 160 KiB a workgroup can have); longer rows keep it in the caller's workspace.
+constexpr int kMaxSeqLds = 30720;
+constexpr size_t kRowBytesAlign = 256;
+__host__ __device__ inline size_t row_bytes(int64_t seq) {
+  return (static_cast<size_t>(seq) * 5 + 16 + kRowBytesAlign - 1) / kRowBytesAlign * kRowBytesAlign;
+}
 constexpr uint8_t kImg = 1, kVid = 2, kStart = 4;
 
 struct Segment {
@@ -107,15 +113,17 @@ __device__ __forceinline__ RowLayout carve(unsigned char* smem, int64_t seq) {
 }
 
 // counts[b] = (#image items, #video items) of row b (act.py:995-1000)
+// ROW_IN_GLOBAL: the compacted row is kept in `row_ws` (row_bytes(seq) per row) instead of LDS.
+template <bool ROW_IN_GLOBAL>
 __global__ __launch_bounds__(kThreads) void rope_index_count(const int64_t* __restrict__ input_ids,
                                                              const int64_t* __restrict__ attention_mask,
                                                              int64_t seq, int64_t image_id, int64_t video_id,
                                                              int64_t start_id, int32_t* __restrict__ counts,
-                                                             int32_t* status) {
+                                                             int32_t* status, unsigned char* row_ws) {
   extern __shared__ __align__(16) unsigned char smem[];
   __shared__ int32_t s_wave[kWaves];
   const int64_t b = blockIdx.x;
-  RowLayout lay = carve(smem, seq);
+  RowLayout lay = carve(ROW_IN_GLOBAL ? row_ws + b * row_bytes(seq) : smem, seq);
   const int64_t* mask = attention_mask ? attention_mask + b * seq : nullptr;
   const int32_t L = compact_row(input_ids + b * seq, mask, seq, image_id, video_id, start_id, lay, s_wave);
   int32_t n_img = 0, n_vid = 0;
@@ -155,12 +163,14 @@ __device__ __forceinline__ int64_t temporal_id(int32_t t, const Segment& sg, flo
   return static_cast<int64_t>(f);
 }
 
+template <bool ROW_IN_GLOBAL>
 __global__ __launch_bounds__(kThreads) void rope_index_fill(
     const int64_t* __restrict__ input_ids, const int64_t* __restrict__ attention_mask,
     const int64_t* __restrict__ image_grid, int64_t n_image, const int64_t* __restrict__ video_grid,
     int64_t n_video, const float* __restrict__ sec_per_grid, int64_t seq, int merge, int64_t image_id,
     int64_t video_id, int64_t start_id, float tps, const int32_t* __restrict__ counts,
-    int64_t* __restrict__ position_ids, int64_t* __restrict__ deltas, int64_t batch, int32_t* status) {
+    int64_t* __restrict__ position_ids, int64_t* __restrict__ deltas, int64_t batch, int32_t* status,
+    unsigned char* row_ws) {
   extern __shared__ __align__(16) unsigned char smem[];
   __shared__ int32_t s_wave[kWaves];
   __shared__ int64_t s_wave64[kWaves];
@@ -170,7 +180,7 @@ __global__ __launch_bounds__(kThreads) void rope_index_fill(
 
   const int64_t b = blockIdx.x;
   const int tid = threadIdx.x, lane = lane_id();
-  RowLayout lay = carve(smem, seq);
+  RowLayout lay = carve(ROW_IN_GLOBAL ? row_ws + b * row_bytes(seq) : smem, seq);
   const int64_t* ids = input_ids + b * seq;
   const int64_t* mask = attention_mask ? attention_mask + b * seq : nullptr;
   const int32_t L = compact_row(ids, mask, seq, image_id, video_id, start_id, lay, s_wave);
@@ -359,8 +369,10 @@ __global__ __launch_bounds__(kThreads) void rope_index_text_only(const int64_t* 
 
 using namespace wx;
 
-extern "C" size_t wx_rope_index_workspace_bytes(int64_t batch) {
-  return static_cast<size_t>((batch > 0 ? batch : 1) * 2 * sizeof(int32_t) + 255) / 256 * 256;
+extern "C" size_t wx_rope_index_workspace_bytes(int64_t batch, int64_t seq) {
+  const size_t counts = static_cast<size_t>((batch > 0 ? batch : 1) * 2 * sizeof(int32_t) + 255) / 256 * 256;
+  const size_t rows = seq > kMaxSeqLds ? static_cast<size_t>(batch > 0 ? batch : 1) * row_bytes(seq) : 0;
+  return counts + rows;
 }
 
 extern "C" int wx_rope_index(const int64_t* input_ids, const int64_t* attention_mask, const int64_t* image_grid_thw,
@@ -383,17 +395,39 @@ extern "C" int wx_rope_index(const int64_t* input_ids, const int64_t* attention_
   }
   if (!input_ids) return fail(WX_ERR_INVALID_ARGUMENT, "wx_rope_index: null input_ids");
   if (spatial_merge_size <= 0) return fail(WX_ERR_INVALID_ARGUMENT, "wx_rope_index: spatial_merge_size must be positive");
-  if (seq > kMaxSeq) return fail(WX_ERR_UNSUPPORTED, "wx_rope_index: seq %lld > %d", static_cast<long long>(seq), kMaxSeq);
-  if (!workspace || workspace_bytes < wx_rope_index_workspace_bytes(batch))
+  if (seq > INT32_MAX / 8) return fail(WX_ERR_UNSUPPORTED, "wx_rope_index: seq %lld too long", static_cast<long long>(seq));
+  if (!workspace || workspace_bytes < wx_rope_index_workspace_bytes(batch, seq))
     return fail(WX_ERR_WORKSPACE, "wx_rope_index: workspace too small");
   int32_t* counts = static_cast<int32_t*>(workspace);
+  const dim3 grid(static_cast<unsigned>(batch)), block(kThreads);
+  if (seq > kMaxSeqLds) {
+    unsigned char* rows = static_cast<unsigned char*>(workspace) + wx_rope_index_workspace_bytes(batch, 0);
+    hipLaunchKernelGGL(rope_index_count<true>, grid, block, 0, s, input_ids, attention_mask, seq, image_token_id,
+                       video_token_id, vision_start_token_id, counts, status, rows);
+    if (int rc = check_launch("rope_index_count")) return rc;
+    hipLaunchKernelGGL(rope_index_fill<true>, grid, block, 0, s, input_ids, attention_mask, image_grid_thw, n_image,
+                       video_grid_thw, n_video, second_per_grid_ts, seq, spatial_merge_size, image_token_id,
+                       video_token_id, vision_start_token_id, tokens_per_second, counts, position_ids, deltas, batch,
+                       status, rows);
+    return check_launch("rope_index_fill");
+  }
   const size_t lds = static_cast<size_t>(seq) * 5 + 16;
-  hipLaunchKernelGGL(rope_index_count, dim3(static_cast<unsigned>(batch)), dim3(kThreads), lds, s, input_ids,
-                     attention_mask, seq, image_token_id, video_token_id, vision_start_token_id, counts, status);
+  if (lds > 48 * 1024) {  // above the default cap on dynamic LDS the kernels have to be told
+    const int want = static_cast<int>(row_bytes(kMaxSeqLds));
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(rope_index_count<false>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, want) != hipSuccess ||
+        hipFuncSetAttribute(reinterpret_cast<const void*>(rope_index_fill<false>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, want) != hipSuccess) {
+      (void)hipGetLastError();
+      return fail(WX_ERR_LAUNCH, "wx_rope_index: cannot raise the dynamic LDS limit");
+    }
+  }
+  hipLaunchKernelGGL(rope_index_count<false>, grid, block, lds, s, input_ids, attention_mask, seq, image_token_id,
+                     video_token_id, vision_start_token_id, counts, status, nullptr);
   if (int rc = check_launch("rope_index_count")) return rc;
-  hipLaunchKernelGGL(rope_index_fill, dim3(static_cast<unsigned>(batch)), dim3(kThreads), lds, s, input_ids,
-                     attention_mask, image_grid_thw, n_image, video_grid_thw, n_video, second_per_grid_ts, seq,
-                     spatial_merge_size, image_token_id, video_token_id, vision_start_token_id, tokens_per_second,
-                     counts, position_ids, deltas, batch, status);
+  hipLaunchKernelGGL(rope_index_fill<false>, grid, block, lds, s, input_ids, attention_mask, image_grid_thw, n_image,
+                     video_grid_thw, n_video, second_per_grid_ts, seq, spatial_merge_size, image_token_id,
+                     video_token_id, vision_start_token_id, tokens_per_second, counts, position_ids, deltas, batch,
+                     status, nullptr);
   return check_launch("rope_index_fill");
 }

@@ -331,7 +331,7 @@ def rope_index(input_ids, image_grid_thw, video_grid_thw, second_per_grid_ts, at
     pos = torch.empty((3, B, S), dtype=torch.int64, device=dev)
     deltas = torch.empty((B, 1), dtype=torch.int64, device=dev)
     status = torch.zeros(1, dtype=torch.int32, device=dev)
-    ws_bytes = _lib.load().wx_rope_index_workspace_bytes(B)
+    ws_bytes = _lib.load().wx_rope_index_workspace_bytes(B, S)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     with _DeviceGuard(ids):
         _lib.call("wx_rope_index", _ptr(ids), _ptr(mask), None if ig is None else ig.data_ptr(),
