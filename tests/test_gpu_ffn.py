@@ -191,6 +191,28 @@ def test_fused_ffn_ragged_last_round(dev, T, n_act, hidden, inters):
         assert int((yh != y).sum()) == 0, f"host row counts {hint} changed the result"
 
 
+def test_fused_ffn_intermediate_beyond_2_gib(dev):
+    """131 072 tokens at the BASELINE widths: the VL expert's intermediate is 2.9 GB, past what a buffer descriptor's
+    32-bit byte count holds, so the loads run with clamped counts.  Rows sampled across the whole range (first and
+    last tiles of both experts included) against the oracle; every output finite."""
+    T, n_act, H, inters = 131072, 4096, wl.HIDDEN, (wl.INTER_VL, wl.INTER_ACT)
+    g = torch.Generator(device=dev).manual_seed(9)
+    x = torch.randn(T, H, device=dev, generator=g).to(torch.bfloat16)
+    types = torch.zeros(T, dtype=torch.bool, device=dev)
+    types[torch.randperm(T, device=dev, generator=g)[:n_act]] = True
+    gc = torch.Generator().manual_seed(9)
+    ws = _moe_weights(H, inters, gc, 0.02)
+    y, routing = moe.moe_layer_forward(x, types, [w.to(dev).as_tuple() for w in ws])
+    assert routing.expert_offsets.cpu().tolist() == [0, T - n_act, T]
+    assert bool(torch.isfinite(y.float()).all())
+    inv = routing.sorted_row_id.long()
+    picks = torch.cat([torch.arange(0, 8), torch.arange(T - n_act - 8, T - n_act + 8), torch.arange(T - 8, T),
+                       torch.randint(0, T, (40,), generator=gc)]).to(dev)
+    rows = inv[picks]  # tokens at chosen sorted positions
+    ref = oracle.sparse_moe_block_ref(x[rows].cpu()[None], types[rows].cpu()[None], [w.as_tuple() for w in ws])[0]
+    _close(y[rows], ref, what="sampled rows")
+
+
 def test_moe_block_module_is_a_drop_in(dev):
     class Cfg:
         experts = [{"hidden_size": 256, "intermediate_size": 512, "hidden_act": "silu"},
