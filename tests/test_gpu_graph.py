@@ -69,3 +69,42 @@ def test_layer_graph_replays_match_eager(dev, n_vl, n_act):
         torch.cuda.synchronize()
         assert routing.expert_offsets.cpu().tolist() == [0, n_vl, T]
         assert int((got != h).sum()) == 0, f"replay {it} differs from the eager run"
+
+
+def test_prefill_forward_graph_replays_match_eager(dev):
+    """The whole harness forward (position builder, partition, per-layer projections / M-RoPE / attention on
+    PyTorch-ROCm, fused movers and both FFN launches) recorded once and replayed on fresh inputs: every replay equals
+    the eager forward on the same inputs, with eager work and synchronisations between the replays."""
+    from wallx_mi355 import harness, workloads as wl
+
+    h = harness.PrefillHarness(n_layers=2, hidden=256, n_q=4, n_kv=2, head_dim=128, inter=(512, 256), vocab=151936,
+                               device=dev, seed=5)
+    row = wl.vla_row_tokens(n_images=1, image_tokens=16, lead_text=5, tail_text=9, n_action=8)
+    ids_static = torch.tensor([row, row], dtype=torch.int64, device=dev)
+    grid = torch.tensor([[1, 8, 8]] * 2, dtype=torch.int64, device=dev)
+    types_static = ids_static == wl.ACTION_TOKEN_ID
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        h.forward(ids_static, grid, types_static)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out_static = h.forward(ids_static, grid, types_static)
+
+    g = torch.Generator().manual_seed(0)
+    for it in range(3):
+        # same layout, other text tokens: the embedding rows (hence every activation) change
+        ids = ids_static.clone().cpu()
+        is_text = ids == wl.TEXT_TOKEN_ID
+        ids[is_text] = torch.randint(1000, 2000, (int(is_text.sum()),), generator=g)
+        ids = ids.to(dev)
+        ids_static.copy_(ids)
+        graph.replay()
+        got = out_static.clone()
+        torch.cuda.synchronize()
+        want = h.forward(ids, grid, ids == wl.ACTION_TOKEN_ID)
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), f"replay {it} differs from the eager forward"
