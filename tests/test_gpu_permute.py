@@ -100,6 +100,40 @@ def test_config3_full_size_properties(dev):
     assert torch.equal(p[:n_vl], xf[(~ids).to(dev)]) and torch.equal(p[n_vl:], xf[ids.to(dev)])
 
 
+@pytest.mark.parametrize("T,H,n_act", [(300, 96, 37), (912, 2048, 32), (1000, 64, 1000), (70, 4096, 0), (515, 160, 200)])
+def test_permute_rows_tiled_layout(dev, T, H, n_act):
+    """The K-tiled activation matrix the FFN reads, decoded block by block on the host (16 x 32 blocks ordered
+    [column block][row block], 16-byte chunk c of row r in slot c ^ ((r >> 2) & 3), each expert's rows starting at a
+    multiple of 256, padding rows zero), against the rows in sorted order.  Both forms of the kernel (gather through
+    the inverse map, with an odd and an even number of column blocks; scatter through row_id_map) bit for bit."""
+    g = torch.Generator().manual_seed(T + H)
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    types = torch.zeros(T, dtype=torch.bool)
+    types[torch.randperm(T, generator=g)[:n_act]] = True
+    rmap, off, inv, _ = native.partition(types.to(dev), 2, 0, None, want_sorted=True)
+    rows_pad = native.padded_sorted_rows(T)
+    n0 = T - n_act
+    pad0 = (n0 + 255) // 256 * 256
+    want = torch.zeros(rows_pad, H, dtype=torch.bfloat16)
+    order = inv.cpu().long()
+    want[:n0] = x[order[:n0]]
+    want[pad0:pad0 + n_act] = x[order[n0:]]
+    for form, tiled in (("gather", native.permute_rows_tiled(x.to(dev), rmap, off, None, inv)),
+                        ("scatter", native.permute_rows_tiled(x.to(dev), rmap, off, None, None))):
+        rb, kb = rows_pad // 16, H // 32
+        t = tiled.cpu()[: rows_pad * H].view(kb, rb, 16, 4, 8)
+        got = torch.empty(rows_pad, H, dtype=torch.bfloat16)
+        for r in range(16):
+            for c in range(4):
+                got.view(rb, 16, kb, 4, 8)[:, r, :, c, :] = t[:, :, r, c ^ ((r >> 2) & 3), :].transpose(0, 1)
+        live = torch.zeros(rows_pad, dtype=torch.bool)
+        live[:n0] = True
+        live[pad0:pad0 + n_act] = True
+        assert torch.equal(got[live].view(torch.int16), want[live].view(torch.int16)), form
+        if form == "gather":  # the gather form also zero-fills the padding rows
+            assert torch.equal(got.view(torch.int16), want.view(torch.int16)), form
+
+
 def test_one_million_tokens_round_trip(dev):
     """2^20 tokens x 1024 bf16 columns (2 GiB each way), eight experts, everything checked on the device through the
     properties the partition guarantees: the map is a permutation, rows of an expert are contiguous and in source

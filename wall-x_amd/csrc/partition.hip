@@ -261,6 +261,62 @@ __global__ __launch_bounds__(kMoverWaves* kWave) void permute_rows_tiled_gather_
     st16(reinterpret_cast<u32x4*>(dst + ((kb * row_blocks) << 10)), src_tok < 0 ? zero : ld16(src + kb * 4));
 }
 
+// The same gather with 128-byte reads: a lane takes chunk (lane & 7) of the 128 bytes that span a PAIR of column
+// blocks, for rows (lane >> 3) and (lane >> 3) + 8 of the row block, so a load instruction touches 8 rows x one whole
+// cache line instead of 16 rows x half a line, and a store instruction writes two 512-byte runs (the upper or lower
+// 8 rows of the two blocks).  Needs an even number of column blocks.
+__global__ __launch_bounds__(kMoverWaves* kWave) void permute_rows_tiled_gather128_kernel(
+    const u32x4* __restrict__ x, unsigned char* __restrict__ out, const int32_t* __restrict__ sorted_row_id,
+    const int32_t* __restrict__ expert_offsets, int64_t num_tokens, int64_t col_blocks, int64_t row_blocks) {
+  const int lane = lane_id();
+  const int64_t wave = static_cast<int64_t>(blockIdx.x) * kMoverWaves + threadIdx.x / kWave;
+  const int64_t rb = wave / kGatherSplit;
+  const int part = static_cast<int>(wave % kGatherSplit);
+  if (rb >= row_blocks) return;
+  const int32_t o0 = expert_offsets[0], o1 = expert_offsets[1], o2 = expert_offsets[2];
+  const int64_t pad0 = round_up_256(o1 - o0);
+  const int r8 = lane >> 3, c8 = lane & 7;
+  const int64_t chunks_per_row = col_blocks * 4;
+  const u32x4* src[2];
+  bool live[2];
+  int dst_off[2];
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int r = 8 * h + r8;
+    const int64_t prow = rb * kBlkRows + r;
+    int64_t pos = -1;
+    if (prow < pad0) { if (prow < o1 - o0) pos = o0 + prow; }
+    else if (prow - pad0 < o2 - o1) pos = o1 + (prow - pad0);
+    const int64_t tok = (pos >= 0 && pos < num_tokens) ? sorted_row_id[pos] : -1;
+    live[h] = tok >= 0;
+    src[h] = x + (tok < 0 ? 0 : tok) * chunks_per_row + c8;
+    // inside its block the chunk (c8 & 3) of row r sits in slot (c8 & 3) ^ ((r >> 2) & 3)
+    dst_off[h] = r * 64 + (((c8 & 3) ^ ((r >> 2) & 3)) << 4);
+  }
+  const int64_t pairs = col_blocks / 2;
+  const int64_t per = (pairs + kGatherSplit - 1) / kGatherSplit;
+  const int64_t p0 = part * per, p1 = p0 + per < pairs ? p0 + per : pairs;
+  unsigned char* base = out + (rb << 10) + (((c8 >> 2) * row_blocks) << 10);  // block kb or kb + 1 of the pair
+  const u32x4 zero = {0, 0, 0, 0};
+  int64_t pr = p0;
+  for (; pr + 1 < p1; pr += 2) {
+    u32x4 v[2][2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int h = 0; h < 2; ++h) v[u][h] = live[h] ? ld16(src[h] + (pr + u) * 8) : zero;
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+        st16(reinterpret_cast<u32x4*>(base + (((pr + u) * 2 * row_blocks) << 10) + dst_off[h]), v[u][h]);
+  }
+  for (; pr < p1; ++pr)
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+      st16(reinterpret_cast<u32x4*>(base + ((pr * 2 * row_blocks) << 10) + dst_off[h]), live[h] ? ld16(src[h] + pr * 8) : zero);
+}
+
 // out[t] = y[row_id_map[t]] (zeros when the map entry is -1); one wavefront per destination row.
 __global__ __launch_bounds__(kMoverWaves* kWave) void gather_rows_kernel(
     const u32x4* __restrict__ y, u32x4* __restrict__ out, const int32_t* __restrict__ row_id_map,
@@ -466,8 +522,17 @@ extern "C" int wx_permute_rows_tiled(const void* x, void* out_tiled, const int32
   const int64_t row_blocks = padded_sorted_rows(num_tokens) / kBlkRows;
   if (sorted_row_id != nullptr) {
     const int64_t waves = row_blocks * kGatherSplit;
-    hipLaunchKernelGGL(permute_rows_tiled_gather_kernel, dim3(static_cast<unsigned>((waves + kMoverWaves - 1) / kMoverWaves)),
-                       dim3(kMoverWaves * kWave), 0, as_stream(stream), static_cast<const u32x4*>(x),
+    const dim3 grid(static_cast<unsigned>((waves + kMoverWaves - 1) / kMoverWaves)), block(kMoverWaves * kWave);
+#ifndef WX_GATHER128
+#define WX_GATHER128 1
+#endif
+    if (WX_GATHER128 && (num_cols / kBlkCols) % 2 == 0) {
+      hipLaunchKernelGGL(permute_rows_tiled_gather128_kernel, grid, block, 0, as_stream(stream),
+                         static_cast<const u32x4*>(x), static_cast<unsigned char*>(out_tiled), sorted_row_id,
+                         expert_offsets, num_tokens, num_cols / kBlkCols, row_blocks);
+      return check_launch("permute_rows_tiled_gather128_kernel");
+    }
+    hipLaunchKernelGGL(permute_rows_tiled_gather_kernel, grid, block, 0, as_stream(stream), static_cast<const u32x4*>(x),
                        static_cast<unsigned char*>(out_tiled), sorted_row_id, expert_offsets, num_tokens,
                        num_cols / kBlkCols, row_blocks);
     return check_launch("permute_rows_tiled_gather_kernel");
