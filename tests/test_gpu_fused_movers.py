@@ -34,8 +34,8 @@ def test_rmsnorm_permute_tiled(dev, T, H, n_act):
     types[torch.randperm(T, generator=g)[:n_act]] = True
     rmap, off, inv, _ = native.partition(types.to(dev), 2, 0, None, want_sorted=True)
     fused = native.rmsnorm_permute_rows_tiled(x.to(dev), w.to(dev), 1e-6, off, inv)
-    # the same layout from the unfused pair, fed with the oracle's norm: equal up to one bf16 step where the
-    # fp32 sum of squares (accumulated in a different order) moves a value across a rounding boundary
+    # the same layout from the unfused pair, fed with the oracle's norm: equal except where the fp32 sum of squares
+    # (accumulated in a different order) moves a value across a rounding boundary
     normed = oracle.rms_norm_ref(x, w, 1e-6)
     plain = native.permute_rows_tiled(normed.to(dev), rmap, off, None, inv)
     rows_pad = native.padded_sorted_rows(T)
@@ -48,9 +48,11 @@ def test_rmsnorm_permute_tiled(dev, T, H, n_act):
     live[pad0: pad0 + (o[2] - o[1])] = True
     a, b = a[live], b[live]
     assert a.shape[0] == T
-    tol = 2.0 ** -7 * b.abs() + 1e-6  # one bf16 step
-    bad = (a - b).abs() > tol
-    assert not bad.any(), f"{int(bad.sum())} of {bad.numel()} differ by more than a bf16 step"
+    # one bf16 step in the normalised value, which its rounded product with the weight can turn into two
+    bad = (a - b).abs() > 2.0 ** -6 * b.abs() + 1e-6
+    assert not bad.any(), f"{int(bad.sum())} of {bad.numel()} differ by more than two bf16 steps"
+    one = (a - b).abs() > 2.0 ** -7 * b.abs() + 1e-6
+    assert float(one.float().mean()) < 1e-4  # more than one step: a handful per million
     assert float((a != b).float().mean()) < 0.02  # and almost all values are identical
 
 

@@ -72,6 +72,78 @@ __global__ __launch_bounds__(kSplit * 64) void rmsnorm_permute_tiled_kernel(
   }
 }
 
+// The same with 128-byte reads: a lane takes chunk (lane & 7) of the 128 bytes spanning a PAIR of column blocks, for
+// rows (lane >> 3) and (lane >> 3) + 8 of the row block (a load instruction touches 8 rows x a whole cache line
+// instead of 16 rows x half a line; a store instruction writes two 512-byte runs).  NP = pairs of column blocks per
+// wavefront.
+template <int NP>
+__global__ __launch_bounds__(kSplit * 64) void rmsnorm_permute_tiled128_kernel(
+    const u32x4* __restrict__ x, const u32x4* __restrict__ weight, float eps, unsigned char* __restrict__ out,
+    const int32_t* __restrict__ sorted_row_id, const int32_t* __restrict__ expert_offsets, int64_t num_tokens,
+    int64_t row_blocks) {
+  __shared__ float s_part[kSplit][kBlkRows];
+  const int lane = threadIdx.x & 63, part = threadIdx.x >> 6;
+  const int64_t rb = blockIdx.x;
+  const int32_t o0 = expert_offsets[0], o1 = expert_offsets[1], o2 = expert_offsets[2];
+  const int64_t pad0 = round_up_256(o1 - o0);
+  const int r8 = lane >> 3, c8 = lane & 7;
+  constexpr int64_t kChunksPerRow = static_cast<int64_t>(NP) * 2 * kSplit * 4;
+  const int pair0 = part * NP;  // first pair of column blocks of this wavefront
+  u32x4 v[NP][2];
+  bool live[2];
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int64_t prow = rb * kBlkRows + 8 * h + r8;
+    int64_t pos = -1;
+    if (prow < pad0) { if (prow < o1 - o0) pos = o0 + prow; }
+    else if (prow - pad0 < o2 - o1) pos = o1 + (prow - pad0);
+    const int64_t tok = (pos >= 0 && pos < num_tokens) ? sorted_row_id[pos] : -1;
+    live[h] = tok >= 0;
+    const u32x4* src = x + (tok < 0 ? 0 : tok) * kChunksPerRow + pair0 * 8 + c8;
+#pragma unroll
+    for (int u = 0; u < NP; ++u) v[u][h] = live[h] ? ld16(src + u * 8) : u32x4{0, 0, 0, 0};
+  }
+  float inv[2];
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    float ss = 0.f;
+#pragma unroll
+    for (int u = 0; u < NP; ++u) {
+      float f[8];
+      unpack16<WX_BF16>(v[u][h], f);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ss += f[e] * f[e];
+    }
+    ss += __shfl_xor(ss, 1);
+    ss += __shfl_xor(ss, 2);
+    ss += __shfl_xor(ss, 4);  // the 8 lanes of a row
+    if (c8 == 0) s_part[part][8 * h + r8] = ss;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int r = 8 * h + r8;
+    const float total = s_part[0][r] + s_part[1][r] + s_part[2][r] + s_part[3][r];
+    inv[h] = __frsqrt_rn(total / static_cast<float>(kChunksPerRow * 8) + eps);
+  }
+  unsigned char* base = out + (rb << 10) + (((c8 >> 2) * row_blocks) << 10);  // first or second block of the pair
+#pragma unroll
+  for (int u = 0; u < NP; ++u) {
+    float w[8];
+    unpack16<WX_BF16>(weight[(pair0 + u) * 8 + c8], w);
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int r = 8 * h + r8;
+      float f[8];
+      unpack16<WX_BF16>(v[u][h], f);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) f[e] = w[e] * round_bf16(f[e] * inv[h]);  // pack16 rounds the product
+      const int off = r * 64 + (((c8 & 3) ^ ((r >> 2) & 3)) << 4);
+      st16(reinterpret_cast<u32x4*>(base + ((static_cast<int64_t>(pair0 + u) * 2 * row_blocks) << 10) + off), pack16<WX_BF16>(f));
+    }
+  }
+}
+
 // out[t] = resid[t] + y[row_id_map[t]] (resid[t] alone when the map entry is -1); one wavefront per destination row.
 __global__ __launch_bounds__(256) void unpermute_add_kernel(const u32x4* __restrict__ y, const u32x4* __restrict__ resid,
                                                             u32x4* __restrict__ out, const int32_t* __restrict__ row_id_map,
@@ -197,6 +269,18 @@ extern "C" int wx_rmsnorm_permute_rows_tiled(const void* x, const void* weight, 
                        static_cast<const u32x4*>(weight), eps, static_cast<unsigned char*>(out_tiled), sorted_row_id, \
                        expert_offsets, num_tokens, row_blocks);                                                     \
     break;
+#define WX_CASE128(N)                                                                                               \
+  case 2 * N:                                                                                                       \
+    hipLaunchKernelGGL(rmsnorm_permute_tiled128_kernel<N>, grid, block, 0, s, static_cast<const u32x4*>(x),         \
+                       static_cast<const u32x4*>(weight), eps, static_cast<unsigned char*>(out_tiled), sorted_row_id, \
+                       expert_offsets, num_tokens, row_blocks);                                                     \
+    return check_launch("rmsnorm_permute_tiled128_kernel");
+  switch (nch) {  // an even number of column blocks per wavefront: the form with whole-line reads
+    WX_CASE128(1) WX_CASE128(2) WX_CASE128(3) WX_CASE128(4) WX_CASE128(5) WX_CASE128(6) WX_CASE128(7) WX_CASE128(8)
+    WX_CASE128(10) WX_CASE128(12) WX_CASE128(14) WX_CASE128(16)
+    default: break;
+  }
+#undef WX_CASE128
   switch (nch) {
     WX_CASE(1) WX_CASE(2) WX_CASE(3) WX_CASE(4) WX_CASE(5) WX_CASE(6) WX_CASE(7) WX_CASE(8)
     WX_CASE(9) WX_CASE(10) WX_CASE(11) WX_CASE(12) WX_CASE(13) WX_CASE(14) WX_CASE(15) WX_CASE(16)
