@@ -40,7 +40,7 @@ def parse():
     ap.add_argument("--prefill-mask", default="causal", choices=["causal", "action_block"])
     ap.add_argument("--cpu-seqs", type=int, default=16, help="sequences of the batch the CPU baseline runs")
     ap.add_argument("--kernel-loop", default=None,
-                    choices=["gate_up", "down", "permute", "permute_plain", "unpermute", "partition", "copy"],
+                    choices=["gate_up", "down", "down_unpermute", "permute", "permute_plain", "unpermute", "partition", "copy"],
                     help="profiling aid: run only this kernel --steps times (no JSON line); 'copy' is a plain "
                          "device-to-device copy of the [T, H] activations, the known-size yardstick for HBM counters")
     return ap.parse_args()
@@ -126,24 +126,28 @@ def main():
         _lib.call("wx_dual_swiglu_gate_up", x_tiled.data_ptr(), hmid.data_ptr(), offsets.data_ptr(), pg0.data_ptr(),
                   pu0.data_ptr(), pg1.data_ptr(), pu1.data_ptr(), T, H, I0, I1, None, stream)
 
-    def down():
+    def down():  # on its own: rows come out in sorted order
         _lib.call("wx_dual_down_proj", hmid.data_ptr(), y_sorted.data_ptr(), offsets.data_ptr(), pd0.data_ptr(),
-                  pd1.data_ptr(), T, H, I0, I1, None, stream)
+                  pd1.data_ptr(), T, H, I0, I1, None, None, stream)
+
+    def down_unpermute():  # the layer's form: every row is stored at its token's position, no separate unpermute
+        _lib.call("wx_dual_down_proj", hmid.data_ptr(), y.data_ptr(), offsets.data_ptr(), pd0.data_ptr(),
+                  pd1.data_ptr(), T, H, I0, I1, None, inverse.data_ptr(), stream)
 
     def unpermute():
         _lib.call("wx_unpermute_rows", y_sorted.data_ptr(), y.data_ptr(), row_id_map.data_ptr(), None, T, 1, H,
                   _lib.WX_BF16, stream)
 
-    def step():
+    def step():  # partition -> permute -> gate/up + SwiGLU -> down with the unpermute in its stores
         partition()
         permute()
         gate_up()
-        down()
-        unpermute()
+        down_unpermute()
 
     if args.kernel_loop:
         permute(); gate_up(); down()
-        fn = {"gate_up": gate_up, "down": down, "permute": permute, "permute_plain": permute_plain,
+        fn = {"gate_up": gate_up, "down": down, "down_unpermute": down_unpermute, "permute": permute,
+              "permute_plain": permute_plain,
               "unpermute": unpermute, "partition": partition,
               "copy": lambda: x_sorted.copy_(x)}[args.kernel_loop]
         for _ in range(args.steps):
@@ -167,6 +171,7 @@ def main():
     iters = max(10, args.steps)
     t_gate_up, t_gate_up_avg = event_ms(gate_up, iters)
     t_down, _ = event_ms(down, iters)
+    t_down_unp, _ = event_ms(down_unpermute, iters)
     t_perm, _ = event_ms(permute, iters, batch=10)
     t_perm_plain, _ = event_ms(permute_plain, iters, batch=10)
     t_unperm, _ = event_ms(unpermute, iters, batch=10)
@@ -197,6 +202,7 @@ def main():
     extra = {
         "gate_up_swiglu_ms": round(t_gate_up, 4), "gate_up_tflops": round(gate_up_flops / t_gate_up / 1e9, 1),
         "down_ms": round(t_down, 4), "down_tflops": round(down_flops / t_down / 1e9, 1),
+        "down_with_unpermute_ms": round(t_down_unp, 4),  # what the step runs: rows stored at their token positions
         "ffn_kernels_tflops": round(ffn_flops / (t_gate_up + t_down) / 1e9, 1),
         "permute_ms": round(t_perm, 4), "permute_GBps": round(row_bytes / t_perm / 1e6, 1),
         "permute_rowmajor_ms": round(t_perm_plain, 4), "permute_rowmajor_GBps": round(row_bytes / t_perm_plain / 1e6, 1),

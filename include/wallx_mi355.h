@@ -132,7 +132,7 @@ int wx_dual_swiglu_ffn(const void* x_tiled, void* out, const int32_t* expert_off
                        const void* up0, const void* down0, const void* gate1, const void* up1,
                        const void* down1, void* hmid, int64_t num_rows, int64_t hidden,
                        int64_t inter0, int64_t inter1, const int64_t* host_rows_per_expert,
-                       wx_stream_t stream);
+                       const int32_t* out_row_id, wx_stream_t stream);
 
 /* The two launches of wx_dual_swiglu_ffn on their own, for callers that put work between them (and for
  * timing each kernel): hmid = silu(x @ gate^T) * (x @ up^T), then out = hmid @ down^T, per expert.
@@ -143,7 +143,12 @@ int wx_dual_swiglu_gate_up(const void* x_tiled, void* hmid, const int32_t* exper
                            const int64_t* host_rows_per_expert, wx_stream_t stream);
 int wx_dual_down_proj(const void* hmid, void* out, const int32_t* expert_offsets, const void* down0,
                       const void* down1, int64_t num_rows, int64_t hidden, int64_t inter0,
-                      int64_t inter1, const int64_t* host_rows_per_expert, wx_stream_t stream);
+                      int64_t inter1, const int64_t* host_rows_per_expert, const int32_t* out_row_id,
+                      wx_stream_t stream);
+/* out_row_id (optional, may be NULL): DEVICE int32[num_rows], the partition's sorted_row_id (sorted position ->
+ * token).  When given, the down launch stores sorted row r of the result at row out_row_id[r] of `out`, i.e. `out`
+ * comes back in token order and the separate unpermute (ops.unpermute at topK 1, act.py:157-161) is not needed:
+ * its row-granular stores are the same 256-byte runs either way. */
 /* host_rows_per_expert (optional, may be NULL): HOST int64[2], the rows of each expert when the caller already
  * has them on the host (the reference computes them there, act.py:1274-1283).  They only steer the choice between
  * the two tile shapes: without them, a call whose bounds on the tile count straddle the threshold launches both

@@ -59,10 +59,10 @@ def test_argument_errors_without_a_gpu():
     assert lib.wx_partition_build(None, 0, 4, 200, 2, 0, None, None, None, None, None, 0, None) == -2
     assert b"num_topK cannot exceed 128" in lib.wx_last_error_string()
     # a zero-width expert is refused (the MFMA kernels advance their tile loop from inside the K loop)
-    assert lib.wx_dual_swiglu_ffn(*([None] * 10), 4, 64, 64, 0, None, None) == -2
+    assert lib.wx_dual_swiglu_ffn(*([None] * 10), 4, 64, 64, 0, None, None, None) == -2
     assert b"must be positive" in lib.wx_last_error_string()
     # host row counts that do not add up to the token count are refused
-    assert lib.wx_dual_swiglu_ffn(*([None] * 10), 4, 64, 64, 64, _lib.i64x2((1, 2)), None) == -1
+    assert lib.wx_dual_swiglu_ffn(*([None] * 10), 4, 64, 64, 64, _lib.i64x2((1, 2)), None, None) == -1
     assert b"sum to num_rows" in lib.wx_last_error_string()
     # the fused movers, the transpose and the probe check their arguments the same way
     assert lib.wx_rmsnorm_permute_rows_tiled(None, None, 1e-6, None, None, None, 4, 100, None) == -2  # cols % 128

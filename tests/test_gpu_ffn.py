@@ -191,6 +191,32 @@ def test_fused_ffn_ragged_last_round(dev, T, n_act, hidden, inters):
         assert int((yh != y).sum()) == 0, f"host row counts {hint} changed the result"
 
 
+@pytest.mark.parametrize("T,n_act,hidden,inters", [
+    (700, 33, 512, (1056, 160)),      # small tiles
+    (5000, 300, 2048, (512, 256)),    # large tiles, ragged rows
+    (8600, 300, 2176, (512, 128)),    # large tiles + a ragged last round on the small-tile kernel, ragged columns
+    (300, 300, 256, (256, 128)),      # one expert empty
+])
+def test_down_launch_stores_rows_at_their_token_positions(dev, T, n_act, hidden, inters):
+    """wx_dual_swiglu_ffn with out_row_id (the partition's inverse map): the result in token order must equal the
+    sorted-order result put through the stand-alone unpermute, bit for bit."""
+    g = torch.Generator(device=dev).manual_seed(T + hidden)
+    x = torch.randn(T, hidden, device=dev, generator=g).to(torch.bfloat16)
+    types = torch.zeros(T, dtype=torch.bool, device=dev)
+    types[torch.randperm(T, device=dev, generator=g)[:n_act]] = True
+    ws = [w.to(dev).as_tuple() for w in _moe_weights(hidden, inters, torch.Generator().manual_seed(1), 0.03)]
+    rmap, off, inv, _ = native.partition(types, 2, 0, None, want_sorted=True)
+    x_tiled = native.permute_rows_tiled(x, rmap, off, None, inv)
+    y_sorted = native.dual_swiglu_ffn(x_tiled, T, off, ws)
+    want = native.unpermute(y_sorted, rmap, torch.tensor([]), T, 1)
+    got = torch.full((T, hidden), float("nan"), dtype=torch.bfloat16, device=dev)
+    native.dual_swiglu_ffn(x_tiled, T, off, ws, out=got, out_row_id=inv)
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+    for hint in ((T - n_act, n_act), (n_act, T - n_act)):
+        got2 = native.dual_swiglu_ffn(x_tiled, T, off, ws, host_rows=hint, out_row_id=inv)
+        assert torch.equal(got2.view(torch.int16), want.view(torch.int16))
+
+
 def test_fused_ffn_intermediate_beyond_2_gib(dev):
     """131 072 tokens at the BASELINE widths: the VL expert's intermediate is 2.9 GB, past what a buffer descriptor's
     32-bit byte count holds, so the loads run with clamped counts.  Rows sampled across the whole range (first and

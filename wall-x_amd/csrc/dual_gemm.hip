@@ -27,7 +27,8 @@
 //   gate/up  (wx_dual_swiglu_gate_up)  A = K-tiled activations, B = K-tiled gate and up weights (the B tile is 128
 //                                      gate rows + 128 up rows of the same output columns, so gate and up of an
 //                                      output element meet in one lane), C = K-tiled intermediate, SwiGLU epilogue.
-//   down     (wx_dual_down_proj)       A = K-tiled intermediate, B = K-tiled down weights, C row-major.
+//   down     (wx_dual_down_proj)       A = K-tiled intermediate, B = K-tiled down weights, C row-major; with a row
+//                                      id list the rows go straight to their token positions (the unpermute).
 // With K-tiled operands every load instruction moves one contiguous KiB (tiled_layout.h).
 // Results leave through a per-wave LDS staging area so that global stores are full 16-byte lanes on contiguous
 // runs (whole 1 KiB blocks for the tiled intermediate, 256-byte row segments for row-major outputs).
@@ -109,6 +110,9 @@ struct Params {
   // the ragged last round to a second launch; 2 = this is that second launch, with 128 x 128 tiles.
   // split_cus = workgroups of the first launch (one per CU).
   int split, split_cus;
+  // kDown only: when set (the partition's sorted_row_id), row r of the sorted result is stored to row scatter[r] of
+  // the output instead of row r -- the unpermute folded into the store.
+  const int32_t* scatter;
 };
 
 #define LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
@@ -228,6 +232,7 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
   // ---- problem table (uniform) ------------------------------------------------------------------
   // (kept as two named structs, selected per tile, so everything stays in scalar registers)
   Group g0 = p.g[0], g1 = p.g[1];
+  int sorted_first[2] = {0, 0};  // kDown: sorted position of each expert's first row
   if constexpr (MODE != kGeneric) {
     const int o0 = p.offsets[0], o1 = p.offsets[1], o2 = p.offsets[2];
     g0.m = o1 - o0;
@@ -248,8 +253,12 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
       g0.lda = pad0 / kBlkRows;
       g1.lda = pad1 / kBlkRows;
       g1.a = g0.a + static_cast<int64_t>(pad0) * g0.k;
-      g0.c += static_cast<int64_t>(o0) * g0.ldc;
-      g1.c += static_cast<int64_t>(o1) * g1.ldc;
+      if (p.scatter == nullptr) {
+        g0.c += static_cast<int64_t>(o0) * g0.ldc;
+        g1.c += static_cast<int64_t>(o1) * g1.ldc;
+      }
+      sorted_first[0] = o0;
+      sorted_first[1] = o1;
     }
   }
   constexpr int kTileN = SWIGLU ? BN / 2 : BN;  // output columns per tile
@@ -336,6 +345,7 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
   };
   struct Store {    // where the finished tile goes
     __bf16* c_base;
+    const int32_t* row_id;  // kDown with scatter: output row of each of the tile's rows (c_base is then row 0)
     int rows, cols_left, ldc, nk;
   };
 
@@ -350,6 +360,13 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
       S.c_base = G.c + ((static_cast<int64_t>(col0 / kBlkCols) * G.ldc + row0 / kBlkRows) << 9);
     } else {
       S.c_base = G.c + static_cast<int64_t>(row0) * G.ldc + col0;
+    }
+    S.row_id = nullptr;
+    if constexpr (MODE == kDown) {
+      if (p.scatter != nullptr) {
+        S.c_base = G.c + col0;
+        S.row_id = p.scatter + sorted_first[tc.group] + row0;
+      }
     }
     S.rows = G.m - row0 < BM ? G.m - row0 : BM;
     S.cols_left = G.n - col0;
@@ -685,14 +702,25 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
           __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, 0));
           // a row is kPitch bytes = kLanesPerRow lanes; one store instruction writes kRowsPerStore rows
           const int rl = lane_e / kLanesPerRow, cc = (lane_e % kLanesPerRow) * 8;
+          constexpr int kStores = kRound / kRowsPerStore;
+          int out_row[kStores];
 #pragma unroll
-          for (int q = 0; q < kRound / kRowsPerStore; ++q) {
+          for (int q = 0; q < kStores; ++q) {
+            const int row = wm * (FM * 32) + i * 32 + part * kRound + q * kRowsPerStore + rl;
+            out_row[q] = row;
+            if constexpr (MODE == kDown) {
+              // scatter: the row ids of the round are fetched together, ahead of the staging reads
+              if (S.row_id != nullptr && row < S.rows) out_row[q] = S.row_id[row];
+            }
+          }
+#pragma unroll
+          for (int q = 0; q < kStores; ++q) {
             const int srow = q * kRowsPerStore + rl;
             const u32x4 v = *reinterpret_cast<const u32x4*>(stage + srow * kPitch + cc * 2);
             const int row = wm * (FM * 32) + i * 32 + part * kRound + srow;
             const int col = wn * kOutCols + cc;
             if (row < S.rows && col < S.cols_left)
-              *reinterpret_cast<u32x4*>(S.c_base + static_cast<int64_t>(row) * S.ldc + col) = v;
+              *reinterpret_cast<u32x4*>(S.c_base + static_cast<int64_t>(out_row[q]) * S.ldc + col) = v;
           }
           __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, 0));
         }
@@ -980,6 +1008,7 @@ struct FfnArgs {
   const int64_t* host_rows;  // optional: rows of each expert as the caller knows them on the host
   const int32_t* offsets;
   int64_t rows, hidden, inter[2];
+  const int32_t* out_row_id = nullptr;  // optional: sorted row r of the result goes to row out_row_id[r] of `out`
 };
 
 int check_ffn(const char* who, const FfnArgs& a, bool need_gate_up, bool need_down) {
@@ -1049,6 +1078,7 @@ int launch_down(const FfnArgs& a, hipStream_t s) {
     g.a_row0 = 0;
   }
   p.offsets = a.offsets;
+  p.scatter = a.out_row_id;
   const int64_t col_tiles = ceil_div(a.hidden, BigTile::BN);
   if (a.host_rows != nullptr) {
     const int64_t by_expert[2] = {ceil_div(a.host_rows[0], BigTile::BM) * col_tiles, ceil_div(a.host_rows[1], BigTile::BM) * col_tiles};
@@ -1074,9 +1104,10 @@ extern "C" int wx_dual_swiglu_gate_up(const void* x_tiled, void* hmid, const int
 
 extern "C" int wx_dual_down_proj(const void* hmid, void* out, const int32_t* expert_offsets, const void* down0,
                                  const void* down1, int64_t num_rows, int64_t hidden, int64_t inter0,
-                                 int64_t inter1, const int64_t* host_rows_per_expert, wx_stream_t stream) {
+                                 int64_t inter1, const int64_t* host_rows_per_expert, const int32_t* out_row_id,
+                                 wx_stream_t stream) {
   const FfnArgs a{nullptr, {nullptr, nullptr}, {nullptr, nullptr}, {down0, down1}, out, const_cast<void*>(hmid),
-                  host_rows_per_expert, expert_offsets, num_rows, hidden, {inter0, inter1}};
+                  host_rows_per_expert, expert_offsets, num_rows, hidden, {inter0, inter1}, out_row_id};
   if (int rc = check_ffn("wx_dual_down_proj", a, false, true)) return rc;
   if (num_rows == 0) return WX_OK;
   return launch_down(a, as_stream(stream));
@@ -1085,9 +1116,10 @@ extern "C" int wx_dual_down_proj(const void* hmid, void* out, const int32_t* exp
 extern "C" int wx_dual_swiglu_ffn(const void* x_tiled, void* out, const int32_t* expert_offsets, const void* gate0,
                                   const void* up0, const void* down0, const void* gate1, const void* up1,
                                   const void* down1, void* hmid, int64_t num_rows, int64_t hidden, int64_t inter0,
-                                  int64_t inter1, const int64_t* host_rows_per_expert, wx_stream_t stream) {
+                                  int64_t inter1, const int64_t* host_rows_per_expert, const int32_t* out_row_id,
+                                  wx_stream_t stream) {
   const FfnArgs a{x_tiled, {gate0, gate1}, {up0, up1}, {down0, down1}, out, hmid, host_rows_per_expert, expert_offsets,
-                  num_rows, hidden, {inter0, inter1}};
+                  num_rows, hidden, {inter0, inter1}, out_row_id};
   if (int rc = check_ffn("wx_dual_swiglu_ffn", a, true, true)) return rc;
   if (num_rows == 0) return WX_OK;
   if (int rc = launch_gate_up(a, as_stream(stream))) return rc;

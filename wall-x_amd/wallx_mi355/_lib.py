@@ -33,9 +33,9 @@ PROTOTYPES = {
     "wx_padded_sorted_rows": (_i64, [_i64]),
     "wx_pack_tiled": (_i32, [_vp, _vp, _i64, _i64, _vp]),
     "wx_permute_rows_tiled": (_i32, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _vp]),
-    "wx_dual_swiglu_ffn": (_i32, [_vp] * 10 + [_i64] * 4 + [_vp, _vp]),
+    "wx_dual_swiglu_ffn": (_i32, [_vp] * 10 + [_i64] * 4 + [_vp, _vp, _vp]),
     "wx_dual_swiglu_gate_up": (_i32, [_vp] * 7 + [_i64] * 4 + [_vp, _vp]),
-    "wx_dual_down_proj": (_i32, [_vp] * 5 + [_i64] * 4 + [_vp, _vp]),
+    "wx_dual_down_proj": (_i32, [_vp] * 5 + [_i64] * 4 + [_vp, _vp, _vp]),
     "wx_mrope_apply": (_i32, [_vp] * 6 + [_i64, _i64, _i32, _i32, _i32] + [_c.POINTER(_i64)] * 4
                        + [_c.POINTER(_i32), _i32, _i32, _vp]),
     "wx_mrope_apply_bwd": (_i32, [_vp] * 6 + [_i64, _i64, _i32, _i32, _i32] + [_c.POINTER(_i64)] * 4

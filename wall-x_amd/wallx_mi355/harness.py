@@ -124,7 +124,7 @@ class PrefillHarness:
                       T, H, I0, I1, None, stream)
         with timer.section("ffn_down"):
             _lib.call("wx_dual_down_proj", self._hmid.data_ptr(), y_sorted.data_ptr(), routing.expert_offsets.data_ptr(),
-                      d0.data_ptr(), d1.data_ptr(), T, H, I0, I1, None, stream)
+                      d0.data_ptr(), d1.data_ptr(), T, H, I0, I1, None, None, stream)
         if self.fuse:
             with timer.section("unpermute+residual+rmsnorm"):
                 return native.unpermute_add_rmsnorm(y_sorted, h, routing.row_id_map, next_norm, self.eps)

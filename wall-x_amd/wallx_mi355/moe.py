@@ -48,12 +48,14 @@ class Routing:
 
 
 class _DualExpertFFN(torch.autograd.Function):
-    """The fused forward (tiled activations in, sorted rows out); used when nothing needs a gradient."""
+    """The fused forward (tiled activations in; rows out in sorted order, or in token order when out_row_id is
+    given); used when nothing needs a gradient."""
 
     @staticmethod
-    def forward(ctx, x_tiled, num_rows, expert_offsets, hmid, host_rows, *weights):
+    def forward(ctx, x_tiled, num_rows, expert_offsets, hmid, host_rows, out_row_id, *weights):
         w = ((weights[0], weights[1], weights[2]), (weights[3], weights[4], weights[5]))
-        return native.dual_swiglu_ffn(x_tiled, num_rows, expert_offsets, w, hmid=hmid, host_rows=host_rows)
+        return native.dual_swiglu_ffn(x_tiled, num_rows, expert_offsets, w, hmid=hmid, host_rows=host_rows,
+                                      out_row_id=out_row_id)
 
     @staticmethod
     def backward(ctx, grad):
@@ -83,8 +85,11 @@ class _MoeBlockFunction(torch.autograd.Function):
         scratch["x_tiled"] = native.permute_rows_tiled(x, row_id_map, expert_offsets, scratch.get("x_tiled"),
                                                        sorted_row_id)
         w = ((weights[0], weights[1], weights[2]), (weights[3], weights[4], weights[5]))
-        y_sorted = native.dual_swiglu_ffn(scratch["x_tiled"], T, expert_offsets, w, hmid=scratch.get("hmid"))
         ctx.save_for_backward(x, row_id_map, expert_offsets, *weights)
+        if sorted_row_id is not None:
+            return native.dual_swiglu_ffn(scratch["x_tiled"], T, expert_offsets, w, hmid=scratch.get("hmid"),
+                                          out_row_id=sorted_row_id)
+        y_sorted = native.dual_swiglu_ffn(scratch["x_tiled"], T, expert_offsets, w, hmid=scratch.get("hmid"))
         return native.unpermute(y_sorted, row_id_map, torch.tensor([]), T, 1)
 
     @staticmethod
@@ -195,11 +200,13 @@ class SparseMoeBlock(nn.Module):
         else:
             self._x_tiled = native.permute_rows_tiled(x, routing.row_id_map, routing.expert_offsets, self._x_tiled,
                                                       routing.sorted_row_id)
-        y_sorted = _DualExpertFFN.apply(self._x_tiled, x.size(0), routing.expert_offsets, self._hmid, host_rows, *flat)
         if residual:
+            y_sorted = _DualExpertFFN.apply(self._x_tiled, x.size(0), routing.expert_offsets, self._hmid, host_rows,
+                                            None, *flat)
             y = native.unpermute_add(y_sorted, x, routing.row_id_map)
-        else:
-            y = native.unpermute(y_sorted, routing.row_id_map, torch.tensor([]), x.size(0), 1)
+        else:  # the down launch stores every row at its token's position: no separate unpermute
+            y = _DualExpertFFN.apply(self._x_tiled, x.size(0), routing.expert_offsets, self._hmid, host_rows,
+                                     routing.sorted_row_id, *flat)
         return y.view(batch, seq, hidden)
 
 
@@ -213,6 +220,10 @@ def moe_layer_forward(x: torch.Tensor, token_types: torch.Tensor, weights, routi
         row_id_map, offsets, inverse, _ = native.partition(token_types.reshape(-1), 2, 0, workspace, want_sorted=True)
         routing = Routing(row_id_map, offsets, x.size(0), inverse)
     x_tiled = native.permute_rows_tiled(x, routing.row_id_map, routing.expert_offsets, None, routing.sorted_row_id)
+    if routing.sorted_row_id is not None:  # the down launch stores every row at its token's position
+        y = native.dual_swiglu_ffn(x_tiled, x.size(0), routing.expert_offsets, weights, hmid=hmid,
+                                   host_rows=host_rows, out_row_id=routing.sorted_row_id)
+        return y, routing
     y_sorted = native.dual_swiglu_ffn(x_tiled, x.size(0), routing.expert_offsets, weights, hmid=hmid,
                                       host_rows=host_rows)
     y = native.unpermute(y_sorted, routing.row_id_map, torch.tensor([]), x.size(0), 1)

@@ -515,14 +515,16 @@ def unpermute_add_rmsnorm(y_sorted: torch.Tensor, residual: torch.Tensor, row_id
 
 def dual_swiglu_ffn(x_tiled: torch.Tensor, num_rows: int, expert_offsets: torch.Tensor, weights,
                     hmid: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
-                    host_rows=None) -> torch.Tensor:
+                    host_rows=None, out_row_id: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Both experts' SwiGLU FFN over expert-sorted rows in two launches (act.py:79-82, 142-154).
 
     x_tiled: result of permute_rows_tiled for num_rows tokens; expert_offsets int32 [3] ON THE DEVICE (from
     partition()); weights = ((gate0, up0, down0), (gate1, up1, down1)) in nn.Linear layout (packed and cached
     here).  host_rows: optional (rows of expert 0, rows of expert 1) as host integers, when the caller has them
     anyway; they only spare the library a second, empty launch when it cannot tell which tile shape fits.
-    Returns out [num_rows, hidden] bf16 in sorted order.
+    out_row_id: optional int32 [num_rows] CUDA tensor, the partition's sorted_row_id; with it the result comes back
+    in token order (the unpermute happens in the down launch's stores).
+    Returns out [num_rows, hidden] bf16, in sorted order unless out_row_id is given.
     """
     _need_cuda("x_tiled", x_tiled)
     (g0, u0, d0), (g1, u1, d1) = weights
@@ -533,6 +535,9 @@ def dual_swiglu_ffn(x_tiled: torch.Tensor, num_rows: int, expert_offsets: torch.
         raise RuntimeError("expert weight shapes are inconsistent with hidden size")
     if expert_offsets.dtype != torch.int32 or expert_offsets.numel() < 3 or not expert_offsets.is_cuda:
         raise RuntimeError("expert_offsets must be an int32 CUDA tensor with 3 entries")
+    if out_row_id is not None and (out_row_id.dtype != torch.int32 or not out_row_id.is_cuda or
+                                   out_row_id.numel() < num_rows):
+        raise RuntimeError("out_row_id must be an int32 CUDA tensor with one entry per row")
     packed = [pack_weight(w) for w in (g0, u0, d0, g1, u1, d1)]
     dev = x_tiled.device
     need = padded_sorted_rows(num_rows) * max(I0, I1)
@@ -543,5 +548,6 @@ def dual_swiglu_ffn(x_tiled: torch.Tensor, num_rows: int, expert_offsets: torch.
     with _DeviceGuard(x_tiled):
         _lib.call("wx_dual_swiglu_ffn", x_tiled.data_ptr(), _ptr(out), expert_offsets.data_ptr(), _ptr(packed[0]),
                   _ptr(packed[1]), _ptr(packed[2]), _ptr(packed[3]), _ptr(packed[4]), _ptr(packed[5]),
-                  hmid.data_ptr(), int(num_rows), H, I0, I1, _lib.i64x2(host_rows), _stream(x_tiled))
+                  hmid.data_ptr(), int(num_rows), H, I0, I1, _lib.i64x2(host_rows), _ptr(out_row_id),
+                  _stream(x_tiled))
     return out
