@@ -37,7 +37,10 @@ def parse():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--ops-only", action="store_true", help="skip the side measurements (M-RoPE, index builders)")
     ap.add_argument("--no-prefill", action="store_true", help="skip the config 5 prefill measurement (36-layer decoder)")
-    ap.add_argument("--prefill-mask", default="causal", choices=["causal", "action_block"])
+    ap.add_argument("--prefill-mask", default="action_block", choices=["action_block", "action_block_dense", "causal"],
+                    help="config 5 attention mask: the reference's causal + bidirectional action block (as two "
+                         "maskless attention calls, the action tokens being the last 32 of every row; or through a "
+                         "dense mask), or plain causal")
     ap.add_argument("--cpu-seqs", type=int, default=16, help="sequences of the batch the CPU baseline runs")
     ap.add_argument("--kernel-loop", default=None,
                     choices=["gate_up", "down", "down_unpermute", "permute", "permute_plain", "unpermute", "partition", "copy"],
@@ -556,24 +559,28 @@ def prefill_measurement(dev, mask):
     import torch
     from wallx_mi355 import harness
 
-    model = harness.PrefillHarness(device=dev, mask=mask)
+    model = harness.PrefillHarness(device=dev, mask="causal" if mask == "causal" else "action_block")
     ids, grid, types = harness.config5_inputs(16, dev)
+    suffix = 32 if mask == "action_block" else None  # config 5: the 32 action tokens close every row
     for _ in range(2):
-        model.forward(ids, grid, types)
+        model.forward(ids, grid, types, action_suffix=suffix)
     torch.cuda.synchronize()
     reps = 5
     t0 = time.perf_counter()
     for _ in range(reps):
-        model.forward(ids, grid, types)
+        model.forward(ids, grid, types, action_suffix=suffix)
     torch.cuda.synchronize()
     dt = (time.perf_counter() - t0) / reps
     timer = harness.OpTimer()
-    model.forward(ids, grid, types, timer)
+    model.forward(ids, grid, types, timer, action_suffix=suffix)
     split = timer.report_ms()
     total = sum(split.values())
     return {
         "workload": "config 5 (BASELINE.json configs[4]): 36 layers, hidden 2048, 16 q / 2 kv heads x 128, experts "
-                    "11008 / 1024, 16 x 912 tokens (32 action each), bf16, random init, rms eps 1e-6, mask " + mask,
+                    "11008 / 1024, 16 x 912 tokens (32 action each), bf16, random init, rms eps 1e-6, mask " +
+                    {"action_block": "causal + bidirectional action block (act.py:616-637) as two maskless attention calls",
+                     "action_block_dense": "causal + bidirectional action block through a dense mask",
+                     "causal": "plain causal"}[mask],
         "tokens_per_s": round(ids.numel() / dt, 1),
         "ms_per_forward": round(dt * 1e3, 3),
         "op_split_ms": {k: round(v, 3) for k, v in sorted(split.items(), key=lambda kv: -kv[1])},

@@ -46,8 +46,9 @@ def _ref_forward(h, ids, grid, types, mask_mode):
     return norm(x[:, -1], h.final_ln) @ f(h.embed).T
 
 
-@pytest.mark.parametrize("mask_mode,fuse", [("causal", True), ("action_block", True), ("causal", False)])
-def test_prefill_harness_matches_plain_forward(dev, mask_mode, fuse):
+@pytest.mark.parametrize("mask_mode,fuse,suffix", [("causal", True, None), ("action_block", True, None),
+                                                  ("action_block", True, 8), ("causal", False, None)])
+def test_prefill_harness_matches_plain_forward(dev, mask_mode, fuse, suffix):
     from wallx_mi355 import harness
 
     h = harness.PrefillHarness(n_layers=2, hidden=256, n_q=4, n_kv=2, head_dim=128, inter=(512, 256), vocab=151936,
@@ -57,7 +58,7 @@ def test_prefill_harness_matches_plain_forward(dev, mask_mode, fuse):
     grid = torch.tensor([[1, 8, 8]] * 3, dtype=torch.int64, device=dev)
     types = ids == wl.ACTION_TOKEN_ID
     timer = harness.OpTimer()
-    got = h.forward(ids, grid, types, timer).float().cpu()
+    got = h.forward(ids, grid, types, timer, action_suffix=suffix).float().cpu()
     split = timer.report_ms()
     movers = {"rmsnorm+permute", "unpermute+residual+rmsnorm"} if fuse else {"permute", "unpermute"}
     assert movers | {"ffn_gate_up_swiglu", "ffn_down", "mrope", "rope_index", "sdpa_torch"} <= set(split)

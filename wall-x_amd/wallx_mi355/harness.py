@@ -8,7 +8,9 @@ batch of full sequences (prefill).  What it states explicitly:
   * RMSNorm eps 1e-6 (the Qwen2.5-VL-3B value; the reference's config default is 1e-5, cfg.py:179),
   * q/k/v projections with bias, o projection without (vl.py:821-832),
   * attention mask: plain causal by default (`mask="causal"`); `mask="action_block"` adds the reference's
-    bidirectional block among action tokens (act.py:616-637) through a dense boolean mask,
+    bidirectional block among action tokens (act.py:616-637): through a dense boolean mask in general, or, when the
+    caller states that the action tokens are the last n positions of every row, as two maskless attention calls
+    (causal over the prefix; the n action queries over all keys), which is the same function,
   * rotary base 1e6, mrope_section [16, 24, 24], cos/sin built in fp32 and cast to bf16 (vl.py:679-712),
   * `fuse=True` (default) runs the post-attention RMSNorm inside the permute, the residual add AND the next
     reader's RMSNorm (the following layer's input_layernorm, or the final norm) inside the unpermute, M-RoPE
@@ -135,9 +137,11 @@ class PrefillHarness:
 
     @torch.no_grad()
     def forward(self, input_ids: torch.Tensor, image_grid_thw: torch.Tensor, moe_token_types: torch.Tensor,
-                timer: Optional[OpTimer] = None) -> torch.Tensor:
+                timer: Optional[OpTimer] = None, action_suffix: Optional[int] = None) -> torch.Tensor:
         """input_ids [B, S] int64, image_grid_thw [n_img, 3], moe_token_types [B, S] bool -> logits of the last
-        position [B, vocab]."""
+        position [B, vocab].  action_suffix: with mask="action_block", the caller's statement that the action
+        tokens are exactly the last `action_suffix` positions of every row (the data pipeline's layout,
+        wall_x/data/utils.py:453-503), which lets the mask be expressed without a dense tensor."""
         timer = timer or OpTimer(False)
         B, S = input_ids.shape
         H, D, nq, nkv = self.hidden, self.head_dim, self.n_q, self.n_kv
@@ -153,11 +157,17 @@ class PrefillHarness:
             ids = moe_token_types.reshape(-1)
             rmap, off, inv, self._ws = native.partition(ids, 2, 0, self._ws, want_sorted=True)
             routing = moe.Routing(rmap, off, ids.numel(), inv)
-        attn_mask = None
+        attn_mask, n_tail = None, 0
         if self.mask_mode == "action_block":
-            causal = torch.ones(S, S, dtype=torch.bool, device=self.dev).tril()
-            act = moe_token_types[:, None, :, None] & moe_token_types[:, None, None, :]
-            attn_mask = causal[None, None] | act
+            if action_suffix is not None:
+                # the action tokens are the last `action_suffix` positions of every row: an action query then sees
+                # every key of its row (all earlier tokens causally, all action tokens through the block), the other
+                # queries stay causal among themselves -- two maskless attention calls instead of a dense mask
+                n_tail = int(action_suffix)
+            else:
+                causal = torch.ones(S, S, dtype=torch.bool, device=self.dev).tril()
+                act = moe_token_types[:, None, :, None] & moe_token_types[:, None, None, :]
+                attn_mask = causal[None, None] | act
         with timer.section("embed_torch"):
             h = self.embed[input_ids]
         x = None  # RMSNorm of h for the next reader, when the previous layer's closing kernel already made it
@@ -183,8 +193,15 @@ class PrefillHarness:
                 else:
                     q, k = ops.multimodal_rope(q, k, cos, sin, list(wl.MROPE_SECTION))
             with timer.section("sdpa_torch"):
-                a = F.scaled_dot_product_attention(q, k, v, attn_mask=attn_mask, is_causal=attn_mask is None,
-                                                   enable_gqa=True)
+                if n_tail:
+                    head = S - n_tail
+                    a = torch.empty_like(q)
+                    a[:, :, :head] = F.scaled_dot_product_attention(q[:, :, :head], k[:, :, :head], v[:, :, :head],
+                                                                    is_causal=True, enable_gqa=True)
+                    a[:, :, head:] = F.scaled_dot_product_attention(q[:, :, head:], k, v, enable_gqa=True)
+                else:
+                    a = F.scaled_dot_product_attention(q, k, v, attn_mask=attn_mask, is_causal=attn_mask is None,
+                                                       enable_gqa=True)
             with timer.section("o_proj_torch"):
                 a2d = a.transpose(1, 2).reshape(B * S, nq * D)  # a view when attention kept the token-major layout
                 if self.fuse:
