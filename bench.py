@@ -562,6 +562,8 @@ def prefill_measurement(dev, mask):
     model = harness.PrefillHarness(device=dev, mask="causal" if mask == "causal" else "action_block")
     ids, grid, types = harness.config5_inputs(16, dev)
     suffix = 32 if mask == "action_block" else None  # config 5: the 32 action tokens close every row
+    if suffix is not None and not (bool(types[:, -suffix:].all()) and not bool(types[:, :-suffix].any())):
+        raise RuntimeError("config 5 layout changed: the action tokens are not the last 32 of every row")
     for _ in range(2):
         model.forward(ids, grid, types, action_suffix=suffix)
     torch.cuda.synchronize()
