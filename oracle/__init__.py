@@ -38,10 +38,21 @@ How each function is pinned (tests/test_oracle_*.py):
                                    closed form for constant rows, transformers'
                                    Qwen2RMSNorm where it is importable
 
-  unpermute_ref with topK > 1 and probs, unpermute_bwd_ref, mrope_apply_ref in
-  its "csrc" channel layout and rope_index_ref's "csrc" padding mode follow
-  the reference's CUDA sources, which cannot be run anywhere in this build:
-  parity unpinned for those (they are specified from source reading only).
+  unpermute_ref with topK > 1      the fp32 weighted sum x * sum_k p; in bf16 the
+                                   exactly representable cases and a bound of one
+                                   rounding per operation
+  unpermute_bwd_ref                torch autograd of the scalar-loop expression
+                                   out[t] = sum_k p[t,k] y[map[k*T+t]] on tiny
+                                   inputs (with dropped rows), the adjoint identity
+  mrope_apply_ref(layout="csrc")   per-channel closed form with distinct t / h / w
+                                   positions and the plane thresholds written out
+                                   from csrc/rope.cu:104-117
+
+  One aspect no CPU fact can fix: WHERE the reference's CUDA kernels round to
+  bf16 inside a topK > 1 combine (csrc/permute.cu:69-154 rounds every product and
+  every partial sum).  The oracle follows that source; the tests above bound the
+  effect (one rounding per operation) and wall-x itself only ever runs topK == 1,
+  where the ops are bit copies.
 """
 
 from .permute import (  # noqa: F401

@@ -185,6 +185,37 @@ def test_mrope_hf_layout_is_a_rotation_per_pair_with_per_axis_angles():
         assert torch.allclose(qo[0, 0, :, d].double(), ref, atol=1e-5)
 
 
+def test_mrope_csrc_layout_per_channel_closed_form_with_distinct_axes():
+    """The CUDA kernel's channel map (csrc/rope.cu:104-117: d < 32 -> t, d < 80 -> h, else w, thresholds from
+    the elementwise-doubled sections [32, 48, 48]) with DIFFERENT t / h / w positions, channel by channel:
+    out[d] = x[d] cos(p[axis(d)] f[d % 64]) -/+ x[d +/- 64] sin(p[axis(d)] f[d % 64]).  The two halves of a rotation
+    pair take different planes here, so the hf layout, a swapped pair of planes or a shifted threshold all fail."""
+    g = torch.Generator().manual_seed(18)
+    B, S = 2, 5
+    q = torch.randn(B, 3, S, 128, generator=g, dtype=torch.float64)
+    k = torch.randn(B, 1, S, 128, generator=g, dtype=torch.float64)
+    pos = torch.stack([torch.randint(0, 40, (B, S), generator=g), torch.randint(100, 140, (B, S), generator=g),
+                       torch.randint(300, 340, (B, S), generator=g)])
+    cos, sin = oracle.rotary_cos_sin_ref(pos, wl.text_inv_freq(), torch.float64)
+    qo, ko = oracle.mrope_apply_ref(q, k, cos, sin, list(wl.MROPE_SECTION), "csrc")
+    inv = wl.text_inv_freq().double()
+    plane_of = lambda d: 0 if d < 32 else (1 if d < 80 else 2)  # noqa: E731  (written out from csrc/rope.cu:104-117)
+    for x, xo in ((q, qo), (k, ko)):
+        for d in range(128):
+            ang = pos[plane_of(d)].double() * inv[d % 64]  # [B, S]
+            if d < 64:
+                ref = x[..., d] * torch.cos(ang)[:, None] - x[..., d + 64] * torch.sin(ang)[:, None]
+            else:
+                ref = x[..., d] * torch.cos(ang)[:, None] + x[..., d - 64] * torch.sin(ang)[:, None]
+            assert torch.allclose(xo[..., d], ref, atol=2e-4), d  # the table builder forms the angle in fp32
+    # and it is NOT the hf layout on these positions: the 80 channels whose plane differs all change
+    qh, _ = oracle.mrope_apply_ref(q, k, cos, sin, list(wl.MROPE_SECTION), "hf")
+    differs = [(qo[..., d] - qh[..., d]).abs().max() > 1e-7 for d in range(128)]
+    hf_plane = [0] * 16 + [1] * 24 + [2] * 24
+    assert [bool(v) for v in differs] == [plane_of(d) != hf_plane[d % 64] for d in range(128)]
+    assert sum(bool(v) for v in differs) == 80
+
+
 def test_mrope_against_transformers():
     try:
         from transformers.models.qwen2_5_vl.modeling_qwen2_5_vl import apply_multimodal_rotary_pos_emb as hf_apply

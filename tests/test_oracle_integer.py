@@ -80,6 +80,85 @@ def test_unpermute_topk2_weighted_sum_fp32():
     assert torch.equal(oracle.unpermute_ref(p1, m1, torch.rand(T, 1, generator=g)), x)
 
 
+def _scalar_unpermute(y, rmap, probs, T, K):
+    """out[t] = sum_k p[t, k] * y[map[k*T + t]] written as scalar loops over differentiable tensors."""
+    rows = []
+    for t in range(T):
+        acc = torch.zeros(y.shape[1], dtype=y.dtype)
+        for k in range(K):
+            r = int(rmap[k * T + t])
+            if r >= 0:
+                acc = acc + (probs[t, k] * y[r] if K > 1 else y[r])
+        rows.append(acc)
+    return torch.stack(rows)
+
+
+@pytest.mark.parametrize("T,E,K,drop", [(1, 1, 1, 0), (8, 2, 1, 0), (8, 2, 1, 3), (7, 3, 2, 0), (6, 4, 3, 5), (5, 2, 2, 4)])
+def test_unpermute_bwd_is_the_autograd_gradient(T, E, K, drop):
+    """unpermute_bwd_ref against torch autograd of the fp32 expression it is the backward of, on tiny inputs
+    (with and without rows dropped by num_out_tokens).  A transposed map index, a missing probability factor on
+    act_grad, or a prob_grad taken against the wrong row each fail this."""
+    g = torch.Generator().manual_seed(1000 * T + 100 * E + 10 * K + drop)
+    H = 5
+    ids = torch.randint(0, E, (T, K), generator=g, dtype=torch.int32)
+    n_out = T * K - drop
+    x = torch.randn(T, H, generator=g)
+    permuted, rmap, _ = oracle.permute_ref(x, ids if K > 1 else ids[:, 0], num_out_tokens=n_out if drop else 0)
+    y = torch.randn(permuted.shape[0], H, generator=g).requires_grad_(True)  # any sorted-space activations
+    probs = torch.rand(T, K, generator=g).requires_grad_(True)
+    out = _scalar_unpermute(y, rmap, probs, T, K)
+    # the forward oracle is the same function
+    assert torch.allclose(oracle.unpermute_ref(y.detach(), rmap, probs.detach(), T, K), out.detach(), atol=1e-6)
+    grad_out = torch.randn(T, H, generator=g)
+    (out * grad_out).sum().backward()
+    act_grad, prob_grad, written = oracle.unpermute_bwd_ref(grad_out, y.detach(), rmap, probs.detach())
+    assert torch.allclose(act_grad, y.grad, atol=1e-6)
+    # rows no token maps to: the oracle reports them as unwritten (their gradient is zero)
+    mapped = torch.zeros(permuted.shape[0], dtype=torch.bool)
+    mapped[rmap[rmap >= 0].long()] = True
+    assert torch.equal(written, mapped) and bool((y.grad[~mapped] == 0).all())
+    if K > 1:
+        assert torch.allclose(prob_grad, probs.grad, atol=1e-5)
+    else:
+        assert float(prob_grad.abs().max()) == 0.0  # csrc/permute.cu:405-415: probabilities play no part at K == 1
+
+
+def test_unpermute_bwd_is_the_adjoint_of_unpermute():
+    """<unpermute(y), g> == <y, unpermute_bwd(g)> for fixed probabilities (fp64-exact inputs in fp32)."""
+    g = torch.Generator().manual_seed(77)
+    T, K, H = 11, 2, 6
+    ids = torch.randint(0, 3, (T, K), generator=g, dtype=torch.int32)
+    _, rmap, _ = oracle.permute_ref(torch.zeros(T, H), ids)
+    y = torch.randint(-8, 8, (T * K, H), generator=g).float()
+    go = torch.randint(-8, 8, (T, H), generator=g).float()
+    probs = torch.randint(0, 4, (T, K), generator=g).float() / 4  # exact in every dtype
+    lhs = (oracle.unpermute_ref(y, rmap, probs) * go).sum()
+    act_grad, _, _ = oracle.unpermute_bwd_ref(go, y, rmap, probs)
+    assert float(lhs) == float((y * act_grad).sum())
+
+
+def test_unpermute_topk_bf16_exact_cases_and_rounding_bound():
+    """bf16 at topK > 1.  Where every product and partial sum is representable the result is the exact one,
+    whatever the rounding order; in general it stays within K roundings of the fp32 value."""
+    g = torch.Generator().manual_seed(12)
+    T, K, H = 16, 3, 8
+    ids = torch.stack([torch.randperm(4, generator=g)[:K] for _ in range(T)]).to(torch.int32)
+    x = torch.randint(-16, 16, (T, H), generator=g).to(torch.bfloat16)        # small integers
+    probs = (2.0 ** -torch.randint(0, 3, (T, K), generator=g).float())          # powers of two
+    p, rmap, _ = oracle.permute_ref(x, ids)
+    got = oracle.unpermute_ref(p, rmap, probs)
+    assert got.dtype == torch.bfloat16
+    assert torch.equal(got.double(), x.double() * probs.double().sum(1, keepdim=True))
+    # general values: each of the K products and K - 1 sums rounds once (relative 2^-9 each)
+    xr = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    pr = torch.rand(T, K, generator=g)
+    p, rmap, _ = oracle.permute_ref(xr, ids)
+    got = oracle.unpermute_ref(p, rmap, pr).double()
+    exact = xr.double() * pr.to(torch.bfloat16).double().sum(1, keepdim=True)
+    bound = (2 * K) * 2.0 ** -9 * (xr.double().abs() * pr.double().sum(1, keepdim=True)) + 1e-30
+    assert bool(((got - exact).abs() <= bound).all())
+
+
 # ----------------------------------------------------------------------------- rope_index
 def test_rope_index_reference_docstring_vector():
     """vl.py:1744-1760: a 3x2x2 (after merge) video at 2 temporal patches per second with
