@@ -41,11 +41,14 @@ def parse():
                     help="config 5 attention mask: the reference's causal + bidirectional action block (as two "
                          "maskless attention calls, the action tokens being the last 32 of every row; or through a "
                          "dense mask), or plain causal")
-    ap.add_argument("--cpu-seqs", type=int, default=16, help="sequences of the batch the CPU baseline runs")
+    ap.add_argument("--cpu-seqs", type=int, default=32, help="sequences of the batch the CPU baseline runs (32 = all)")
     ap.add_argument("--kernel-loop", default=None,
                     choices=["gate_up", "down", "down_unpermute", "permute", "permute_plain", "unpermute", "partition", "copy"],
                     help="profiling aid: run only this kernel --steps times (no JSON line); 'copy' is a plain "
                          "device-to-device copy of the [T, H] activations, the known-size yardstick for HBM counters")
+    ap.add_argument("--kernel-shape", default="config3", choices=["config3", "denoise"],
+                    help="with --kernel-loop: the batch the kernel runs on -- config 3 (29184 tokens, 28160 VL + 1024 "
+                         "action) or config 4's denoise step (2048 action tokens, VL group empty)")
     return ap.parse_args()
 
 
@@ -89,6 +92,10 @@ def main():
 
     # ---- synthetic inputs, resident in HBM ----------------------------------------------------------
     x_cpu, types_cpu, w_cpu = wl.config3()
+    if args.kernel_loop and args.kernel_shape == "denoise":
+        T = 2048
+        x_cpu = wl.randn((1, T, H), 1.0, torch.bfloat16, torch.Generator().manual_seed(4))
+        types_cpu = torch.ones(1, T, dtype=torch.bool)
     x = x_cpu.view(T, H).to(dev)
     types = types_cpu.view(T).to(dev)
     weights = [w.to(dev).as_tuple() for w in w_cpu]
@@ -242,6 +249,7 @@ def main():
         del x_tiled, hmid, x_sorted, y_sorted, y
         side("prefill", prefill_measurement, dev, args.prefill_mask)
 
+    traffic, traffic_source = measured_traffic("gate_up")
     result = {
         "metric": "dual_expert_ffn_tflops",
         "value": round(tflops, 2),
@@ -272,7 +280,8 @@ def main():
             "frac": round(gate_up_tflops / PEAK_BF16_TFLOPS, 4),
             "flops_per_launch": gate_up_flops,
             "avg_launch_ms": round(t_gate_up_avg, 4),
-            "traffic": measured_traffic("gate_up"),
+            "traffic": traffic,
+            "traffic_source": traffic_source,
         },
         "extra": extra,
     }
@@ -281,17 +290,33 @@ def main():
     print(json.dumps(result), flush=True)
 
 
+def _sha256(path):
+    import hashlib
+
+    with open(path, "rb") as f:
+        return hashlib.sha256(f.read()).hexdigest()
+
+
 def measured_traffic(kernel):
-    """HBM-side bytes per launch of `kernel` from the committed rocprofv3 --pmc summary (FETCH_SIZE + WRITE_SIZE,
-    each scaled by what the same counter reads for a plain copy of known size); None when the summary is absent.
-    Counters need their own profiler runs, so this figure is read, not measured, by a bench.py run."""
-    path = os.path.join(ROOT, "profiles", "config3_hbm_traffic.json")
+    """(bytes, source) -- HBM-side bytes per launch of `kernel` from the committed rocprofv3 --pmc summary
+    (FETCH_SIZE + WRITE_SIZE, each scaled by what the same counter reads for a plain copy of known size).  Counters
+    need profiler runs of their own, so a bench.py run READS this figure; `source` says from where, and the figure is
+    withheld (None) when the kernel source has changed since the counters were taken."""
+    rel = os.path.join("profiles", "config3_hbm_traffic.json")
     try:
-        with open(path) as f:
-            k = json.load(f)["kernels"][kernel]
-        return round(k["read_bytes"] + k["write_bytes"])
+        with open(os.path.join(ROOT, rel)) as f:
+            doc = json.load(f)
+        k = doc["kernels"][kernel]
     except (OSError, KeyError, ValueError):
-        return None
+        return None, f"{rel} absent: not measured"
+    want = doc.get("kernel_source_sha256")
+    have = _sha256(os.path.join(ROOT, "wall-x_amd", "csrc", "dual_gemm.hip"))
+    if want != have:
+        return None, (f"{rel} was taken on another version of wall-x_amd/csrc/dual_gemm.hip (recorded sha256 "
+                      f"{str(want)[:12]}, current {have[:12]}): stale, withheld")
+    return round(k["read_bytes"] + k["write_bytes"]), (
+        f"read from {rel} (rocprofv3 --pmc runs of bench.py --kernel-loop {kernel}, taken at commit "
+        f"{doc.get('commit', 'unknown')} on dual_gemm.hip sha256 {have[:12]}); not measured in this run")
 
 
 def side_measurements(dev, iters):
@@ -520,11 +545,14 @@ def ceiling_measurements(dev, x, weights, m0):
     own tensors, without the SwiGLU epilogue or the second expert."""
     import ctypes
     import torch
-    from wallx_mi355 import _lib
 
     out = {}
-    lib = _lib.load()
-    n = lib.wx_probe_mfma_operand_bytes() // 2
+    # the probe is a benchmark-only library of its own (wall-x_amd/csrc/probe.hip), not part of the product ABI
+    probe = ctypes.CDLL(os.path.join(ROOT, "wall-x_amd", "wallx_mi355", "libwallx_probe.so"))
+    probe.wxprobe_mfma_operand_bytes.restype = ctypes.c_size_t
+    probe.wxprobe_mfma_rate.restype = ctypes.c_int
+    probe.wxprobe_mfma_rate.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
+    n = probe.wxprobe_mfma_operand_bytes() // 2
     sink = torch.zeros(1, dtype=torch.float32, device=dev)
     flops = ctypes.c_double(0.0)
     stream = torch.cuda.current_stream().cuda_stream
@@ -533,7 +561,8 @@ def ceiling_measurements(dev, x, weights, m0):
     data[n // 2:] *= 0.02  # half the fragments look like activations N(0, 1), half like weights N(0, 0.02)
     for name, ops in (("zeros", torch.zeros(n, dtype=torch.bfloat16, device=dev)), ("normal", data.to(torch.bfloat16))):
         def run():
-            _lib.call("wx_probe_mfma_rate", ops.data_ptr(), 4000, sink.data_ptr(), ctypes.byref(flops), stream)
+            if probe.wxprobe_mfma_rate(ops.data_ptr(), 4000, sink.data_ptr(), ctypes.byref(flops), stream) != 0:
+                raise RuntimeError("wxprobe_mfma_rate failed")
         t, _ = event_ms(run, 5, warm=2)
         out[f"mfma_only_{name}_operands_tflops"] = round(flops.value / t / 1e9, 1)
     (g0, u0, d0) = weights[0]
@@ -591,36 +620,67 @@ def prefill_measurement(dev, mask):
     }
 
 
+def physical_cores():
+    """Physical cores of the host from /proc/cpuinfo (distinct (physical id, core id) pairs); None if unreadable."""
+    try:
+        pairs, cur = set(), {}
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if ":" in line:
+                    key, val = (t.strip() for t in line.split(":", 1))
+                    cur[key] = val
+                elif cur:
+                    pairs.add((cur.get("physical id", "0"), cur.get("core id", cur.get("processor"))))
+                    cur = {}
+        if cur:
+            pairs.add((cur.get("physical id", "0"), cur.get("core id", cur.get("processor"))))
+        return len(pairs) or None
+    except OSError:
+        return None
+
+
 def cpu_baseline(x_cpu, types_cpu, w_cpu, n_seq, H, I0, I1):
-    """The CPU oracle on the first n_seq sequences of the same batch (bf16 inputs upcast to fp32 inside)."""
+    """The CPU oracle (a restatement of the reference's PyTorch path) on the first n_seq sequences of the same batch,
+    fp32 math on the bf16-valued inputs: median of 5 runs after 2 warm-ups on the threads torch uses on this box,
+    and the single-thread figure on one sequence for scale."""
     import torch
     import oracle
 
-    xs, ts = x_cpu[:n_seq], types_cpu[:n_seq]
     weights = [w.as_tuple() for w in w_cpu]
-    m1 = int(ts.sum())
-    m0 = ts.numel() - m1
-    flops = 6.0 * H * (m0 * I0 + m1 * I1)
     w32 = [tuple(t.float() for t in w) for w in weights]  # upcast once, outside the timed region
-    x32 = xs.float()
 
-    def run():
-        return oracle.sparse_moe_block_ref(x32, ts, w32, eager_rounding=False)
+    def timed(n, warm, runs):
+        xs, ts = x_cpu[:n].float(), types_cpu[:n]
+        m1 = int(ts.sum())
+        flops = 6.0 * H * ((ts.numel() - m1) * I0 + m1 * I1)
+        for _ in range(warm):
+            oracle.sparse_moe_block_ref(xs, ts, w32, eager_rounding=False)
+        times = []
+        for _ in range(runs):
+            t0 = time.perf_counter()
+            oracle.sparse_moe_block_ref(xs, ts, w32, eager_rounding=False)
+            times.append(time.perf_counter() - t0)
+        return flops, statistics.median(times), ts.numel()
 
-    run()
-    times = []
-    for _ in range(3):
-        t0 = time.perf_counter()
-        run()
-        times.append(time.perf_counter() - t0)
-    best = statistics.median(times)
+    threads = torch.get_num_threads()
+    flops, best, tokens = timed(n_seq, 2, 5)
+    torch.set_num_threads(1)
+    try:
+        flops1, best1, tokens1 = timed(1, 1, 3)
+    finally:
+        torch.set_num_threads(threads)
     return {
         "value": round(flops / best / 1e12, 4),
         "unit": "TFLOP/s",
-        "cores": torch.get_num_threads(),
+        "cores": threads,
+        "physical_cores_of_host": physical_cores(),
+        "logical_cpus_of_host": os.cpu_count(),
+        "single_thread_value": round(flops1 / best1 / 1e12, 4),
         "kind": "port",
-        "sample": f"first {n_seq} of 32 sequences of the same batch ({ts.numel()} tokens, {flops / 1e12:.3f} TFLOP), "
-                  f"fp32 math on bf16-valued inputs, median of 3 runs after 1 warm-up, {best * 1e3:.0f} ms per run",
+        "sample": f"first {n_seq} of 32 sequences of the same batch ({tokens} tokens, {flops / 1e12:.3f} TFLOP), "
+                  f"fp32 math on bf16-valued inputs, {threads} threads (the CPU share torch is given on this box), "
+                  f"median of 5 runs after 2 warm-ups, {best * 1e3:.0f} ms per run; single_thread_value: first "
+                  f"sequence ({tokens1} tokens), 1 thread, median of 3 runs after 1 warm-up, {best1 * 1e3:.0f} ms per run",
     }
 
 

@@ -263,21 +263,6 @@ int wx_unpermute_rows_add_rmsnorm(const void* y, const void* residual, void* out
 int wx_swiglu_bwd(const void* gate, const void* up, const void* dh, void* hmid, void* dgate, void* dup,
                   int64_t num_elems, wx_stream_t stream);
 
-/* dst [cols, rows] = transpose of src [rows, cols], both row-major and contiguous, 2-byte elements (bf16 / fp16),
- * rows and cols multiples of 8.  A utility without a counterpart in the reference; wx_dual_gemm does not need it
- * (it reads every layout of ops.py:78-144 in place). */
-int wx_transpose_2d(const void* src, void* dst, int64_t rows, int64_t cols, int elem_bytes, wx_stream_t stream);
-
-/* ---- measurement probe (no counterpart in the reference; used by bench.py) --------------------------------
- * Runs bf16 32x32x16 MFMA instructions back to back on every CU, operands taken from `operands`
- * (wx_probe_mfma_operand_bytes() bytes of bf16 values, device memory, 16-byte aligned) and held in registers:
- * no LDS or memory traffic inside the loop.  The sustained MFMA rate depends on the operand VALUES (switching
- * activity moves the clock the chip can hold), so timing this on the same kind of data as a GEMM gives the
- * ceiling an MFMA-bound kernel can reach on that data.  *flops_per_launch receives the flops one launch performs
- * (host pointer, may be NULL); sink is one float of device memory that is practically never written. */
-size_t wx_probe_mfma_operand_bytes(void);
-int wx_probe_mfma_rate(const void* operands, int iters, float* sink, double* flops_per_launch, wx_stream_t stream);
-
 #ifdef __cplusplus
 }
 #endif

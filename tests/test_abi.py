@@ -64,7 +64,7 @@ def test_argument_errors_without_a_gpu():
     # host row counts that do not add up to the token count are refused
     assert lib.wx_dual_swiglu_ffn(*([None] * 10), 4, 64, 64, 64, _lib.i64x2((1, 2)), None, None) == -1
     assert b"sum to num_rows" in lib.wx_last_error_string()
-    # the fused movers, the transpose and the probe check their arguments the same way
+    # the fused movers check their arguments the same way
     assert lib.wx_rmsnorm_permute_rows_tiled(None, None, 1e-6, None, None, None, 4, 100, None) == -2  # cols % 128
     assert lib.wx_rmsnorm_permute_rows_tiled(None, None, 1e-6, None, None, None, 4, 8192, None) == -2  # cols > 4096
     assert lib.wx_rmsnorm_permute_rows_tiled(None, None, 1e-6, None, None, None, 4, 2048, None) == -1  # null pointers
@@ -77,10 +77,6 @@ def test_argument_errors_without_a_gpu():
     assert lib.wx_swiglu_bwd(None, None, None, None, None, None, 12, None) == -2  # count % 8
     assert lib.wx_swiglu_bwd(None, None, None, None, None, None, 16, None) == -1
     assert lib.wx_swiglu_bwd(None, None, None, None, None, None, 0, None) == 0
-    assert lib.wx_transpose_2d(None, None, 12, 16, 2, None) == -2  # rows % 8
-    assert lib.wx_transpose_2d(None, None, 16, 16, 4, None) == -2  # element size
-    assert lib.wx_transpose_2d(None, None, 16, 16, 2, None) == -1
-    assert lib.wx_probe_mfma_rate(None, 10, None, None, None) == -1
     # M-RoPE from positions: shapes the row kernel cannot take are refused, not routed elsewhere
     st = _lib.i64x3((128 * 4, 128, 128 * 4))
     assert lib.wx_mrope_apply_positions(None, None, None, None, None, None, 1, 4, 2, 1, 128, st, st, st, st,
@@ -90,7 +86,6 @@ def test_argument_errors_without_a_gpu():
     assert lib.wx_mrope_apply_positions(p_, p_, p_, p_, p_, p_, 1, 4, 2, 1, 128, st, st, st, st,
                                         _lib.i32x3((10, 27, 27)), 0, _lib.WX_BF16, 0, None) == -2
     assert b"chunk boundaries" in lib.wx_last_error_string()
-    assert lib.wx_probe_mfma_operand_bytes() == 4 * 8 * 64 * 16
 
 
 def test_op_layer_validation_matches_reference_behaviour():

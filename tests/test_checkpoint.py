@@ -82,3 +82,14 @@ def test_errors():
         checkpoint.load_expert_weights(short, blocks)
     with pytest.raises(FileNotFoundError):
         checkpoint.load_expert_weights("/nonexistent/dir", blocks)
+
+
+def test_strict_moe_checkpoint_must_hold_both_experts_and_params_must_be_bf16():
+    sd = _state(1)
+    only0 = {k: v for k, v in sd.items() if "experts.1." not in k}  # MoE key names, expert 1 absent altogether
+    with pytest.raises(KeyError, match="expert 1"):
+        checkpoint.load_expert_weights(only0, _blocks(1))
+    assert checkpoint.load_expert_weights(only0, _blocks(1), strict=False) == {0: 3}
+    fp32_block = {0: moe.SparseMoeBlock(_Cfg(), 2)}
+    with pytest.raises(TypeError, match="bfloat16"):
+        checkpoint.load_expert_weights(sd, fp32_block)

@@ -67,3 +67,58 @@ def test_prefill_harness_matches_plain_forward(dev, mask_mode, fuse, suffix):
     scale = float(ref.abs().max())
     err = float((got - ref).abs().max())
     assert err <= 0.04 * scale, f"max |diff| {err} vs logits scale {scale}"
+
+
+def test_config5_full_shape_piece_by_piece(dev):
+    """Config 5 at its stated shape (36 layers, hidden 2048, 16 query / 2 KV heads of 128, experts 11008 / 1024,
+    16 sequences x 912 tokens, bf16 N(0, 0.02)).  A CPU forward of the whole model is out of reach, so the forward
+    is checked piece by piece on what the kernels actually read and wrote inside it: the position ids exactly, and
+    for layers 0 / 17 / 35 the M-RoPE output and the layer's closing half (RMSNorm -> permute -> both experts' FFN
+    -> unpermute -> residual -> next RMSNorm) on sampled tokens, each against the oracle on the captured input."""
+    from wallx_mi355 import harness
+
+    layers = (0, 17, 35)
+    h = harness.PrefillHarness(device=dev, seed=0, mask="action_block", keep_dense=layers)
+    assert (h.n_layers, h.hidden, h.n_q, h.n_kv, h.head_dim, tuple(h.inter)) == (36, 2048, 16, 2, 128, (11008, 1024))
+    ids, grid, types = harness.config5_inputs(16, dev)
+    assert ids.shape == (16, 912) and int(types.sum()) == 16 * 32
+    cap = {"layers": layers}
+    logits = h.forward(ids, grid, types, action_suffix=32, capture=cap)
+    assert logits.shape == (16, 151936) and bool(torch.isfinite(logits.float()).all())
+    # position ids: bit-exact
+    rpos, _ = oracle.rope_index_ref(ids.cpu(), 2, wl.IMAGE_TOKEN_ID, wl.VIDEO_TOKEN_ID, wl.VISION_START_TOKEN_ID, 2,
+                                    image_grid_thw=grid.cpu())
+    assert torch.equal(cap["pos"].cpu(), rpos)
+    cos, sin = oracle.rotary_cos_sin_ref(rpos, wl.text_inv_freq(128), torch.bfloat16)
+    tf = types.view(-1).cpu()
+    g = torch.Generator().manual_seed(5)
+    T = tf.numel()
+    act, vl = torch.nonzero(tf).flatten(), torch.nonzero(~tf).flatten()
+    pick = torch.cat([vl[torch.randperm(vl.numel(), generator=g)[:40]], vl[:2], vl[-2:],
+                      act[torch.randperm(act.numel(), generator=g)[:12]], act[:2], act[-2:]])
+    for li in layers:
+        c = cap[li]
+        # M-RoPE inside the forward (cos / sin evaluated in the kernel from the position ids): two batch rows in full
+        for b in (0, 15):
+            rq, rk = oracle.mrope_apply_ref(c["q_in"][b:b + 1].cpu(), c["k_in"][b:b + 1].cpu(), cos[:, b:b + 1],
+                                            sin[:, b:b + 1], list(wl.MROPE_SECTION))
+            for got, ref, what in ((c["q_out"][b:b + 1], rq, "q"), (c["k_out"][b:b + 1], rk, "k")):
+                err = (got.float().cpu() - ref.float()).abs()
+                assert bool((err <= 2e-2 + 1e-2 * ref.float().abs()).all()), f"layer {li} M-RoPE {what}: {float(err.max())}"
+                # the device's sincosf against the CPU table builder's: a bf16 step on a small share of the entries
+                assert float((got.cpu() != ref).float().mean()) < 5e-3
+        # closing half of the layer on sampled tokens
+        layer = h.layers[li]
+        hin = c["ffn_in"][pick.to(dev)].cpu()
+        ws = [tuple(w.cpu() for w in e) for e in layer["experts"]]
+        xn = oracle.rms_norm_ref(hin, layer["ln2"].cpu(), h.eps)
+        y = oracle.sparse_moe_block_ref(xn[None], tf[pick][None], ws)[0]
+        ref_out = (hin.float() + y.float()).to(torch.bfloat16)
+        got_out = c["ffn_out"].view(T, -1)[pick.to(dev)].cpu()
+        err = (got_out.float() - ref_out.float()).abs()
+        assert bool((err <= 2e-2 + 1e-2 * ref_out.float().abs()).all()), f"layer {li} FFN + residual: {float(err.max())}"
+        nxt = h.layers[li + 1]["ln1"] if li + 1 < h.n_layers else h.final_ln
+        ref_n = oracle.rms_norm_ref(got_out, nxt.cpu(), h.eps)  # the norm of what the kernel itself stored
+        got_n = c["next_normed"].view(T, -1)[pick.to(dev)].cpu()
+        err = (got_n.float() - ref_n.float()).abs()
+        assert bool((err <= 2e-2 + 1e-2 * ref_n.float().abs()).all()), f"layer {li} next RMSNorm: {float(err.max())}"

@@ -39,11 +39,7 @@ def test_mrope_matches_eager_bit_for_bit(dev, dtype, layout):
     q, k, cos, sin = _inputs(2, 37, dtype, 5)
     qt, kt = q.transpose(1, 2), k.transpose(1, 2)  # [B, H, S, D] views of token-major memory
     rq, rk = oracle.mrope_apply_ref(qt, kt, cos, sin, list(wl.MROPE_SECTION), layout, eager_rounding=True)
-    native.set_mrope_layout(layout)
-    try:
-        gq, gk = ops.multimodal_rope(qt.to(dev), kt.to(dev), cos.to(dev), sin.to(dev), list(wl.MROPE_SECTION))
-    finally:
-        native.set_mrope_layout("hf")
+    gq, gk = ops.multimodal_rope(qt.to(dev), kt.to(dev), cos.to(dev), sin.to(dev), list(wl.MROPE_SECTION), layout)
     assert gq.shape == rq.shape and gq.is_contiguous() and gk.is_contiguous()
     _close(gq, rq)
     _close(gk, rk)
@@ -103,14 +99,10 @@ def test_mrope_backward(dev, layout):
     q, k, cos, sin = _inputs(2, 11, torch.float32, 13)
     qd = q.transpose(1, 2).to(dev).requires_grad_(True)
     kd = k.transpose(1, 2).to(dev).requires_grad_(True)
-    native.set_mrope_layout(layout)
-    try:
-        oq, ok = ops.multimodal_rope(qd, kd, cos.to(dev), sin.to(dev), list(wl.MROPE_SECTION))
-        g = torch.Generator().manual_seed(3)
-        gq, gk = torch.randn(oq.shape, generator=g), torch.randn(ok.shape, generator=g)
-        torch.autograd.backward([oq, ok], [gq.to(dev), gk.to(dev)])
-    finally:
-        native.set_mrope_layout("hf")
+    oq, ok = ops.multimodal_rope(qd, kd, cos.to(dev), sin.to(dev), list(wl.MROPE_SECTION), layout)
+    g = torch.Generator().manual_seed(3)
+    gq, gk = torch.randn(oq.shape, generator=g), torch.randn(ok.shape, generator=g)
+    torch.autograd.backward([oq, ok], [gq.to(dev), gk.to(dev)])
     rq, rk = oracle.mrope_apply_bwd_ref(gq, gk, cos, sin, list(wl.MROPE_SECTION), layout)
     assert torch.allclose(qd.grad.cpu(), rq, rtol=1e-5, atol=1e-5)
     assert torch.allclose(kd.grad.cpu(), rk, rtol=1e-5, atol=1e-5)
@@ -137,12 +129,8 @@ def test_mrope_from_positions_matches_the_table_path(dev, dtype, layout):
     cos, sin = oracle.rotary_cos_sin_ref(pos, inv_freq, dtype)
     qt, kt = q.transpose(1, 2), k.transpose(1, 2)
     rq, rk = oracle.mrope_apply_ref(qt, kt, cos, sin, list(wl.MROPE_SECTION), layout, eager_rounding=True)
-    native.set_mrope_layout(layout)
-    try:
-        gq, gk = ops.multimodal_rope_from_positions(qt.to(dev), kt.to(dev), pos.to(dev), inv_freq.to(dev),
-                                                    list(wl.MROPE_SECTION))
-    finally:
-        native.set_mrope_layout("hf")
+    gq, gk = ops.multimodal_rope_from_positions(qt.to(dev), kt.to(dev), pos.to(dev), inv_freq.to(dev),
+                                                list(wl.MROPE_SECTION), layout)
     assert gq.is_contiguous() and gk.is_contiguous()
     if dtype == torch.float32:
         # fp32 tables keep the full last-place difference; angles reach 2000 rad, where one ulp of the angle is 1e-4
@@ -204,3 +192,27 @@ def test_mrope_from_positions_refuses_what_it_cannot_do(dev):
     with pytest.raises(RuntimeError, match="position_ids"):
         ops.multimodal_rope_from_positions(q.transpose(1, 2).to(dev), k.transpose(1, 2).to(dev),
                                            pos[:, :, :5].to(dev), inv_freq, [16, 24, 24])
+
+
+def test_extension_level_rope_uses_the_cuda_kernels_layout(dev):
+    """wallx_csrc.rope / rope_bwd stand in for the reference's extension (csrc/ops.cu:11-21), whose kernel maps
+    channels d < 32 -> t, d < 80 -> h, else w (csrc/rope.cu:104-117): called the way the reference's own ops.py
+    calls them (ops.py:451-456, no layout argument) they must give that layout, not the PyTorch path's."""
+    import wallx_csrc
+
+    q, k, cos, sin = _inputs(2, 19, torch.bfloat16, 31)
+    qt, kt = q.transpose(1, 2).contiguous(), k.transpose(1, 2).contiguous()
+    doubled = [2 * s for s in wl.MROPE_SECTION]
+    qo, ko = torch.empty_like(qt, device=dev), torch.empty_like(kt, device=dev)
+    wallx_csrc.rope(qt.to(dev), kt.to(dev), cos.to(dev), sin.to(dev), qo, ko, doubled)
+    rq, rk = oracle.mrope_apply_ref(qt, kt, cos, sin, list(wl.MROPE_SECTION), "csrc", eager_rounding=True)
+    assert _n_diff(qo, rq) == 0 and _n_diff(ko, rk) == 0
+    hq, _ = oracle.mrope_apply_ref(qt, kt, cos, sin, list(wl.MROPE_SECTION), "hf", eager_rounding=True)
+    assert _n_diff(qo, hq) > 0
+    g = torch.Generator().manual_seed(2)
+    gq, gk = torch.randn(qt.shape, generator=g).to(torch.bfloat16), torch.randn(kt.shape, generator=g).to(torch.bfloat16)
+    dq, dk = torch.empty_like(qo), torch.empty_like(ko)
+    wallx_csrc.rope_bwd(gq.to(dev), gk.to(dev), qt.to(dev), kt.to(dev), cos.to(dev), sin.to(dev), dq, dk, doubled)
+    bq, bk = oracle.mrope_apply_bwd_ref(gq, gk, cos, sin, list(wl.MROPE_SECTION), "csrc")
+    _close(dq, bq)
+    _close(dk, bk)

@@ -1,9 +1,10 @@
 """Builds libwallx_mi355.so (the C-ABI library) for gfx950 with hipcc.
 
-    python wall-x_amd/csrc/build.py [--force]
+    python wall-x_amd/csrc/build.py [--force] [--no-probe]
 
 Sources are compiled one by one (objects under csrc/build/) and linked into
-wall-x_amd/wallx_mi355/libwallx_mi355.so, next to the Python package that loads it.
+wall-x_amd/wallx_mi355/libwallx_mi355.so, next to the Python package that loads it.  The benchmark's MFMA rate
+probe (probe.hip) goes into a library of its own, libwallx_probe.so, beside it.
 """
 
 import os
@@ -19,8 +20,12 @@ OUT_DIR = os.path.join(os.path.dirname(HERE), "wallx_mi355")
 LIB = os.path.join(OUT_DIR, "libwallx_mi355.so")
 OBJ_DIR = os.path.join(HERE, "build")
 
-SOURCES = ["common.hip", "partition.hip", "dual_gemm.hip", "mrope.hip", "rope_index.hip", "vision_index.hip", "transpose.hip", "fused_movers.hip", "swiglu_bwd.hip", "probe.hip"]
-HEADERS = ["common.h", "grid_prefix.h", os.path.join(INCLUDE, "wallx_mi355.h")]
+SOURCES = ["common.hip", "partition.hip", "dual_gemm.hip", "mrope.hip", "rope_index.hip", "vision_index.hip",
+           "fused_movers.hip", "swiglu_bwd.hip"]
+HEADERS = ["common.h", "grid_prefix.h", "tiled_layout.h", os.path.join(INCLUDE, "wallx_mi355.h")]
+# benchmark-only MFMA rate probe: its own library, not part of the product library or its ABI
+PROBE_SOURCE = "probe.hip"
+PROBE_LIB = os.path.join(OUT_DIR, "libwallx_probe.so")
 
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
@@ -81,7 +86,17 @@ def _run(cmd):
         sys.stderr.write(err + "\n")
 
 
-def build(force: bool = False, verbose: bool = True) -> str:
+def build_probe(force: bool = False, verbose: bool = True) -> str:
+    hipcc = _hipcc()
+    path = os.path.join(HERE, PROBE_SOURCE)
+    if force or not _newer(PROBE_LIB, [path]):
+        _run([hipcc] + FLAGS + ["-shared", path, "-o", PROBE_LIB])
+        if verbose:
+            print(f"[wallx_mi355] built {PROBE_LIB}", flush=True)
+    return PROBE_LIB
+
+
+def build(force: bool = False, verbose: bool = True, probe: bool = True) -> str:
     hipcc = _hipcc()
     os.makedirs(OBJ_DIR, exist_ok=True)
     headers = [h if os.path.isabs(h) else os.path.join(HERE, h) for h in HEADERS]
@@ -102,8 +117,10 @@ def build(force: bool = False, verbose: bool = True) -> str:
         _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs)
         if verbose:
             print(f"[wallx_mi355] linked {LIB}", flush=True)
+    if probe:
+        build_probe(force, verbose)
     return LIB
 
 
 if __name__ == "__main__":
-    build(force="--force" in sys.argv)
+    build(force="--force" in sys.argv, probe="--no-probe" not in sys.argv)

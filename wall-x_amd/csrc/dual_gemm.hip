@@ -803,7 +803,7 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
 }
 
 // ---- plain FMA tiles: any transpose combination, any k --------------------------------------------------------
-// Used for what the MFMA kernel does not take: an empty contraction, K-major operands of 4 GiB or more.
+// Used for what the MFMA kernel does not take: K-major operands of 4 GiB or more.
 __global__ __launch_bounds__(256) void dual_gemm_reference_layout_kernel(Params p, int trans_a, int trans_b) {
   __shared__ float s_a[32][33];
   __shared__ float s_b[32][33];
@@ -856,6 +856,14 @@ __global__ __launch_bounds__(256) void pack_tiled_kernel(const u32x4* __restrict
     const u32x4 v = row < rows ? src[i] : u32x4{0, 0, 0, 0};
     *reinterpret_cast<u32x4*>(dst + tiled_chunk_offset(row, c * 8, row_blocks)) = v;
   }
+}
+
+// Zeros for the output of an empty contraction (k == 0): a fill kernel rather than a memset node, so that the call
+// stays capturable in a HIP graph like every other launch here.  n16 = number of 16-byte chunks.
+__global__ __launch_bounds__(256) void zero_fill_kernel(u32x4* __restrict__ dst, int64_t n16) {
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n16;
+       i += static_cast<int64_t>(gridDim.x) * blockDim.x)
+    dst[i] = u32x4{0, 0, 0, 0};
 }
 
 // k_in_rows: both operands are stored with K as the slow dimension, so K needs no alignment
@@ -956,17 +964,29 @@ extern "C" int wx_dual_gemm(const void* in0, const void* in1, const void* w0, co
   p.offsets = nullptr;
   if ((m0 == 0 || n0 == 0) && (m1 == 0 || n1 == 0)) return WX_OK;
   hipStream_t s = as_stream(stream);
-  // an empty contraction (k == 0) has zeros as its result: the plain kernel below writes them (it also takes
-  // K-major operands too large for the MFMA kernel's 32-bit byte counts)
-  const bool empty_k = (k0 == 0 && m0 > 0 && n0 > 0) || (k1 == 0 && m1 > 0 && n1 > 0);
+  // an empty contraction (k == 0) has zeros as its result: a fill launch writes them and the group leaves the
+  // problem, so the other expert still runs on the MFMA kernel (a training batch without action tokens has k == 0
+  // in the action expert's weight gradients next to the VL expert's full-size ones)
+  for (int e = 0; e < 2; ++e) {
+    const int64_t m = dims[e][0], n = dims[e][1];
+    if (dims[e][2] != 0 || m <= 0 || n <= 0) continue;
+    const int64_t n16 = m * n / 8;  // n is a multiple of 8 and the buffer 16-byte aligned
+    const int64_t want = (n16 + 255) / 256, cap = static_cast<int64_t>(device_cu_count()) * 8;
+    hipLaunchKernelGGL(zero_fill_kernel, dim3(static_cast<unsigned>(want < cap ? want : cap)), dim3(256), 0, s,
+                       static_cast<u32x4*>(const_cast<void*>(ptrs[e][2])), n16);
+    if (int rc = check_launch("zero_fill_kernel")) return rc;
+    p.g[e].m = 0;
+  }
+  if ((p.g[0].m == 0 || n0 == 0) && (p.g[1].m == 0 || n1 == 0)) return WX_OK;
+  const int64_t mm0 = p.g[0].m, mm1 = p.g[1].m;  // row counts left after the empty contractions are done
   // K-major operands (A stored [k, m], B stored [k, n]) advance by whole rows of K through a 32-bit byte count
   bool fits = true;
   for (int e = 0; e < 2; ++e) {
     if (trans_a && dims[e][2] * dims[e][0] * 2 >= (1ll << 32)) fits = false;
     if (!trans_b && dims[e][2] * dims[e][1] * 2 >= (1ll << 32)) fits = false;
   }
-  if (!empty_k && fits) {
-    const int64_t tiles = ceil_div(m0, BigTile::BM) * ceil_div(n0, BigTile::BN) + ceil_div(m1, BigTile::BM) * ceil_div(n1, BigTile::BN);
+  if (fits) {
+    const int64_t tiles = ceil_div(mm0, BigTile::BM) * ceil_div(n0, BigTile::BN) + ceil_div(mm1, BigTile::BM) * ceil_div(n1, BigTile::BN);
     const char* who = "dual_gemm_kernel<generic>";
     if (!trans_a && trans_b) return launch_mfma<kGeneric, false, false>(p, tiles, tiles, s, who);
     if (!trans_a && !trans_b) return launch_mfma<kGeneric, false, true>(p, tiles, tiles, s, who);

@@ -2,10 +2,16 @@
 // values, with no LDS or memory traffic in the loop.  The rate depends on the values (switching activity moves
 // the sustained clock), so benchmarks time this on the same kind of data as the GEMM they are judging: it is the
 // ceiling an MFMA-bound kernel can reach on that data, below the nominal peak.
-#include "common.h"
+//
+// Benchmark-only: built into its own library (libwallx_probe.so) next to the product library, never linked into it
+// and not part of its C ABI.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
 
 namespace wx {
 namespace {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
@@ -47,18 +53,21 @@ __global__ __launch_bounds__(256, 1) void mfma_rate_kernel(const u32x4* __restri
 
 using namespace wx;
 
-extern "C" size_t wx_probe_mfma_operand_bytes(void) { return static_cast<size_t>(4) * kProbeFrags * 64 * 16; }
+extern "C" size_t wxprobe_mfma_operand_bytes(void) { return static_cast<size_t>(4) * kProbeFrags * 64 * 16; }
 
-extern "C" int wx_probe_mfma_rate(const void* operands, int iters, float* sink, double* flops_per_launch,
-                                  wx_stream_t stream) {
-  if (!operands || !sink) return fail(WX_ERR_INVALID_ARGUMENT, "wx_probe_mfma_rate: null pointer");
-  if (reinterpret_cast<uintptr_t>(operands) & 15)
-    return fail(WX_ERR_INVALID_ARGUMENT, "wx_probe_mfma_rate: operands must be 16-byte aligned");
-  if (iters < 1 || iters > (1 << 24)) return fail(WX_ERR_INVALID_ARGUMENT, "wx_probe_mfma_rate: iters out of range");
-  const int cus = device_cu_count();
+// Runs `iters` x 32 MFMAs per wave on every CU, operands (wxprobe_mfma_operand_bytes() bytes of bf16 values, device
+// memory, 16-byte aligned) held in registers.  *flops_per_launch (host pointer, may be NULL) receives the flops one
+// launch performs; sink is one float of device memory that is practically never written.  Returns 0, -1 for bad
+// arguments, -4 when the launch failed.
+extern "C" int wxprobe_mfma_rate(const void* operands, int iters, float* sink, double* flops_per_launch, void* stream) {
+  if (!operands || !sink || (reinterpret_cast<uintptr_t>(operands) & 15) || iters < 1 || iters > (1 << 24)) return -1;
+  int dev = 0, cus = 0;
+  if (hipGetDevice(&dev) != hipSuccess ||
+      hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+    return -4;
   if (flops_per_launch)
     *flops_per_launch = 2.0 * 32 * 32 * 16 * kProbeMfmaPerIter * static_cast<double>(iters) * 4 * cus;
-  hipLaunchKernelGGL(mfma_rate_kernel, dim3(cus), dim3(256), 0, as_stream(stream),
+  hipLaunchKernelGGL(mfma_rate_kernel, dim3(cus), dim3(256), 0, reinterpret_cast<hipStream_t>(stream),
                      static_cast<const u32x4*>(operands), iters, sink);
-  return check_launch("mfma_rate_kernel");
+  return hipGetLastError() == hipSuccess ? 0 : -4;
 }

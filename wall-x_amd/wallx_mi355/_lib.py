@@ -51,9 +51,6 @@ PROTOTYPES = {
     "wx_unpermute_rows_add": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _vp]),
     "wx_unpermute_rows_add_rmsnorm": (_i32, [_vp, _vp, _vp, _vp, _vp, _f32, _vp, _i64, _i64, _vp]),
     "wx_swiglu_bwd": (_i32, [_vp] * 6 + [_i64, _vp]),
-    "wx_transpose_2d": (_i32, [_vp, _vp, _i64, _i64, _i32, _vp]),
-    "wx_probe_mfma_operand_bytes": (_sz, []),
-    "wx_probe_mfma_rate": (_i32, [_vp, _i32, _vp, _vp, _vp]),
 }
 
 _lock = threading.Lock()

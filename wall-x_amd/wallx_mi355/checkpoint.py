@@ -51,35 +51,56 @@ def iter_safetensors(path: str) -> Iterable:
 
 
 def load_expert_weights(source, blocks: Mapping[int, torch.nn.Module], dense_as_expert0: bool = True,
-                        strict: bool = True) -> Dict[int, int]:
+                        strict: bool = True, pack_only: bool = False) -> Dict[int, int]:
     """Copies expert projection weights into `blocks` (decoder layer index -> SparseMoeBlock).
 
     source: a checkpoint directory / safetensors file, or an already loaded state dict.
-    Returns {layer: number of tensors loaded}.  With strict=True every block must receive all six tensors unless
-    the checkpoint is a dense one (then expert 0's three).  Shapes and the bf16 requirement of the kernels are
-    checked; the packed copies the kernels read are rebuilt lazily because the parameters are modified in place.
+    Returns {layer: number of tensors loaded}.  With strict=True a layer for which the checkpoint holds any
+    ``moe.experts.*`` key must receive all six tensors; a layer that only has dense ``mlp.*`` keys must receive
+    expert 0's three (the action expert then keeps its initialisation, as in the trainer).  Shapes are checked, and
+    so is the dtype of the block's parameters: the kernels are bf16 only.  Cached K-tiled copies of the touched
+    parameters are dropped, so the next forward packs the new values.
+    pack_only=True finishes with `block.pack_for_inference()` on every block: the weights are packed into the
+    K-tiled layout and the nn.Linear copies released (forward-only blocks, half the expert memory).
     """
+    from . import native
+
     items = source.items() if isinstance(source, Mapping) else iter_safetensors(source)
     loaded: Dict[int, set] = {layer: set() for layer in blocks}
+    moe_format: Dict[int, bool] = {layer: False for layer in blocks}
+    for layer, block in blocks.items():
+        for e in block.experts:
+            for w in e.weights():
+                if w.dtype != torch.bfloat16:
+                    raise TypeError(f"layer {layer}: expert parameters are {w.dtype}; the kernels need torch.bfloat16 "
+                                    "(call block.to(torch.bfloat16) before loading)")
     for key, tensor in items:
         hit = classify_key(key, dense_as_expert0)
         if hit is None:
             continue
         layer, expert, proj = hit
         block = blocks.get(layer)
-        if block is None or expert >= len(block.experts):
+        if block is None:
+            continue
+        if _EXPERT_KEY.search(key):
+            moe_format[layer] = True
+        if expert >= len(block.experts):
             continue
         param = getattr(block.experts[expert], f"{proj}_proj").weight
         if tuple(param.shape) != tuple(tensor.shape):
             raise ValueError(f"{key}: checkpoint shape {tuple(tensor.shape)} != module shape {tuple(param.shape)}")
         with torch.no_grad():
             param.copy_(tensor.to(device=param.device, dtype=param.dtype))
+        native.invalidate_packed(param)
         loaded[layer].add((expert, proj))
     if strict:
         for layer, got in loaded.items():
-            experts_seen = {e for e, _ in got}
-            for e in experts_seen or {0}:
+            must = range(len(blocks[layer].experts)) if moe_format[layer] else (0,)
+            for e in must:
                 missing = {"gate", "up", "down"} - {p for ee, p in got if ee == e}
                 if missing:
                     raise KeyError(f"layer {layer}, expert {e}: missing {sorted(missing)} projection weights")
+    if pack_only:
+        for block in blocks.values():
+            block.pack_for_inference(free_dense=True)
     return {layer: len(got) for layer, got in loaded.items()}

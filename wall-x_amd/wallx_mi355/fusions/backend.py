@@ -50,19 +50,22 @@ def unpermute_bwd(input_bwd, input_fwd, row_id_map, prob):
     return native.unpermute_bwd(input_bwd, input_fwd, row_id_map, prob)
 
 
-def rope(q, k, cos, sin, q_out, k_out, mrope_section_doubled) -> None:
-    """backend.py:233-262."""
-    return native.rope(q, k, cos, sin, q_out, k_out, mrope_section_doubled)
+def rope(q, k, cos, sin, q_out, k_out, mrope_section_doubled, layout: str = "csrc") -> None:
+    """backend.py:233-262.  layout: "csrc" = the channel map of the reference's kernel, "hf" = its PyTorch path."""
+    return native.rope(q, k, cos, sin, q_out, k_out, mrope_section_doubled, layout)
 
 
-def rope_bwd(grad_q_out, grad_k_out, q, k, cos, sin, grad_q, grad_k, mrope_section_doubled) -> None:
+def rope_bwd(grad_q_out, grad_k_out, q, k, cos, sin, grad_q, grad_k, mrope_section_doubled,
+             layout: str = "csrc") -> None:
     """backend.py:265-299."""
-    return native.rope_bwd(grad_q_out, grad_k_out, q, k, cos, sin, grad_q, grad_k, mrope_section_doubled)
+    return native.rope_bwd(grad_q_out, grad_k_out, q, k, cos, sin, grad_q, grad_k, mrope_section_doubled, layout)
 
 
-def rope_from_positions(q, k, position_ids, inv_freq, q_out, k_out, mrope_section_doubled, backward=False) -> None:
+def rope_from_positions(q, k, position_ids, inv_freq, q_out, k_out, mrope_section_doubled, backward=False,
+                        layout: str = "hf") -> None:
     """No counterpart in backend.py: the rope op with the cos/sin builder (vl.py:679-712) folded in."""
-    return native.rope_from_positions(q, k, position_ids, inv_freq, q_out, k_out, mrope_section_doubled, backward)
+    return native.rope_from_positions(q, k, position_ids, inv_freq, q_out, k_out, mrope_section_doubled, backward,
+                                      layout)
 
 
 def get_rope_index(input_ids, image_grid_thw, video_grid_thw, second_per_grid_ts, attention_mask,

@@ -5,8 +5,10 @@ exceptions, running on the MI355X kernels.
     (ops.py:147, 386, 391, 496, 507, 589, 685)
 
 Differences a caller can observe, all deliberate:
-  * multimodal_rope follows the PyTorch path's channel layout (vl.py:763-769) by default; call
-    wallx_mi355.native.set_mrope_layout("csrc") for the layout of the reference's CUDA kernel.
+  * multimodal_rope takes a per-call layout= argument.  Its default, "hf", is the channel layout of the model's
+    PyTorch path (apply_multimodal_rotary_pos_emb, vl.py:763-769), which is what this build is checked against;
+    layout="csrc" gives the layout of the reference's CUDA kernel (csrc/rope.cu:104-117).  The extension-level
+    names wallx_csrc.rope / rope_bwd default to "csrc", like the extension they stand in for.
   * bool / int64 expert ids are consumed as they are (no cast kernel); the reference's dtype warning is kept.
   * rot_pos_emb / get_window_index accept grid_thw_host= to skip the device->host read of grid_thw.
 """
@@ -196,7 +198,7 @@ class MultimodalRoPE(torch.autograd.Function):
     """
 
     @staticmethod
-    def forward(ctx, q, k, cos, sin, mrope_section):
+    def forward(ctx, q, k, cos, sin, mrope_section, layout="hf"):
         for name, t in (("q", q), ("k", k), ("cos", cos), ("sin", sin)):
             if t.is_cpu:
                 raise RuntimeError(f"[Error] The input `{name}` of multimodal_rope op is on the device: CPU!")
@@ -217,9 +219,10 @@ class MultimodalRoPE(torch.autograd.Function):
         doubled = [2 * int(v) for v in mrope_section]
         q_out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
         k_out = torch.empty(k.shape, dtype=k.dtype, device=k.device)
-        backend.rope(q, k, cos, sin, q_out, k_out, doubled)
+        backend.rope(q, k, cos, sin, q_out, k_out, doubled, layout)
         ctx.save_for_backward(q, k, cos, sin)
         ctx.mrope_section_doubled = doubled
+        ctx.layout = layout
         return q_out, k_out
 
     @staticmethod
@@ -227,19 +230,21 @@ class MultimodalRoPE(torch.autograd.Function):
         q, k, cos, sin = ctx.saved_tensors
         want_q, want_k = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
         if not (want_q or want_k):
-            return None, None, None, None, None
+            return None, None, None, None, None, None
         gq = torch.empty(q.shape, dtype=q.dtype, device=q.device)
         gk = torch.empty(k.shape, dtype=k.dtype, device=k.device)
         if grad_q_out.stride(-1) != 1:
             grad_q_out = grad_q_out.contiguous()
         if grad_k_out.stride(-1) != 1:
             grad_k_out = grad_k_out.contiguous()
-        backend.rope_bwd(grad_q_out, grad_k_out, q, k, cos, sin, gq, gk, ctx.mrope_section_doubled)
-        return (gq if want_q else None), (gk if want_k else None), None, None, None
+        backend.rope_bwd(grad_q_out, grad_k_out, q, k, cos, sin, gq, gk, ctx.mrope_section_doubled, ctx.layout)
+        return (gq if want_q else None), (gk if want_k else None), None, None, None, None
 
 
-def multimodal_rope(q, k, cos, sin, mrope_section):
-    return MultimodalRoPE.apply(q, k, cos, sin, mrope_section)
+def multimodal_rope(q, k, cos, sin, mrope_section, layout="hf"):
+    """(q', k') = M-RoPE of q and k (ops.py:496-497).  layout="hf": the channel -> plane map of the model's PyTorch
+    path (vl.py:763-769); layout="csrc": that of the reference's CUDA kernel (csrc/rope.cu:104-117)."""
+    return MultimodalRoPE.apply(q, k, cos, sin, mrope_section, layout)
 
 
 class MultimodalRoPEFromPositions(torch.autograd.Function):
@@ -249,7 +254,7 @@ class MultimodalRoPEFromPositions(torch.autograd.Function):
     through their strides, contiguous outputs, gradients for q and k only."""
 
     @staticmethod
-    def forward(ctx, q, k, position_ids, inv_freq, mrope_section):
+    def forward(ctx, q, k, position_ids, inv_freq, mrope_section, layout="hf"):
         for name, t in (("q", q), ("k", k), ("position_ids", position_ids), ("inv_freq", inv_freq)):
             if t.is_cpu:
                 raise RuntimeError(f"[Error] The input `{name}` of multimodal_rope op is on the device: CPU!")
@@ -265,9 +270,10 @@ class MultimodalRoPEFromPositions(torch.autograd.Function):
         inv_freq = inv_freq.to(torch.float32)
         q_out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
         k_out = torch.empty(k.shape, dtype=k.dtype, device=k.device)
-        backend.rope_from_positions(q, k, position_ids, inv_freq, q_out, k_out, doubled)
+        backend.rope_from_positions(q, k, position_ids, inv_freq, q_out, k_out, doubled, layout=layout)
         ctx.save_for_backward(position_ids, inv_freq)
         ctx.mrope_section_doubled = doubled
+        ctx.layout = layout
         return q_out, k_out
 
     @staticmethod
@@ -275,7 +281,7 @@ class MultimodalRoPEFromPositions(torch.autograd.Function):
         position_ids, inv_freq = ctx.saved_tensors
         want_q, want_k = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
         if not (want_q or want_k):
-            return None, None, None, None, None
+            return None, None, None, None, None, None
         if grad_q_out.stride(-1) != 1:
             grad_q_out = grad_q_out.contiguous()
         if grad_k_out.stride(-1) != 1:
@@ -283,12 +289,12 @@ class MultimodalRoPEFromPositions(torch.autograd.Function):
         gq = torch.empty(grad_q_out.shape, dtype=grad_q_out.dtype, device=grad_q_out.device)
         gk = torch.empty(grad_k_out.shape, dtype=grad_k_out.dtype, device=grad_k_out.device)
         backend.rope_from_positions(grad_q_out, grad_k_out, position_ids, inv_freq, gq, gk,
-                                    ctx.mrope_section_doubled, backward=True)
-        return (gq if want_q else None), (gk if want_k else None), None, None, None
+                                    ctx.mrope_section_doubled, backward=True, layout=ctx.layout)
+        return (gq if want_q else None), (gk if want_k else None), None, None, None, None
 
 
-def multimodal_rope_from_positions(q, k, position_ids, inv_freq, mrope_section):
-    return MultimodalRoPEFromPositions.apply(q, k, position_ids, inv_freq, mrope_section)
+def multimodal_rope_from_positions(q, k, position_ids, inv_freq, mrope_section, layout="hf"):
+    return MultimodalRoPEFromPositions.apply(q, k, position_ids, inv_freq, mrope_section, layout)
 
 
 # ----------------------------------------------------------------------------- index builders

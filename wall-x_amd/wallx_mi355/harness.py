@@ -86,7 +86,10 @@ class PrefillHarness:
             }
             # the FFN kernels read K-tiled weights; pack now (static weights) and drop the nn.Linear copies
             layer["packed"] = [tuple(native.pack_weight(t, cache=False) for t in e) for e in layer["experts"]]
-            if not keep_dense:  # tests keep the nn.Linear-layout copies to run a plain PyTorch forward beside this one
+            # tests keep the nn.Linear-layout copies (of every layer, or of the listed ones) to evaluate the same
+            # weights on the CPU beside this forward
+            keep = keep_dense if isinstance(keep_dense, bool) else len(self.layers) in tuple(keep_dense)
+            if not keep:
                 layer["experts"] = None
             self.layers.append(layer)
         self.final_ln = torch.ones(hidden, dtype=torch.bfloat16, device=self.dev)
@@ -137,11 +140,15 @@ class PrefillHarness:
 
     @torch.no_grad()
     def forward(self, input_ids: torch.Tensor, image_grid_thw: torch.Tensor, moe_token_types: torch.Tensor,
-                timer: Optional[OpTimer] = None, action_suffix: Optional[int] = None) -> torch.Tensor:
+                timer: Optional[OpTimer] = None, action_suffix: Optional[int] = None,
+                capture: Optional[dict] = None) -> torch.Tensor:
         """input_ids [B, S] int64, image_grid_thw [n_img, 3], moe_token_types [B, S] bool -> logits of the last
         position [B, vocab].  action_suffix: with mask="action_block", the caller's statement that the action
         tokens are exactly the last `action_suffix` positions of every row (the data pipeline's layout,
-        wall_x/data/utils.py:453-503), which lets the mask be expressed without a dense tensor."""
+        wall_x/data/utils.py:453-503), which lets the mask be expressed without a dense tensor.
+        capture: optional dict with a "layers" entry (layer indices); the forward then leaves in it the position ids
+        ("pos") and, per listed layer, what the M-RoPE and FFN kernels read and wrote (q / k before and after the
+        rotation, the residual stream before and after the FFN), for checking a full-size forward piece by piece."""
         timer = timer or OpTimer(False)
         B, S = input_ids.shape
         H, D, nq, nkv = self.hidden, self.head_dim, self.n_q, self.n_kv
@@ -157,6 +164,8 @@ class PrefillHarness:
             ids = moe_token_types.reshape(-1)
             rmap, off, inv, self._ws = native.partition(ids, 2, 0, self._ws, want_sorted=True)
             routing = moe.Routing(rmap, off, ids.numel(), inv)
+        if capture is not None:
+            capture["pos"] = pos
         attn_mask, n_tail = None, 0
         if self.mask_mode == "action_block":
             if action_suffix is not None:
@@ -189,9 +198,11 @@ class PrefillHarness:
                     qr = torch.empty(B, S, nq, D, dtype=q.dtype, device=self.dev).transpose(1, 2)
                     kr = torch.empty(B, S, nkv, D, dtype=k.dtype, device=self.dev).transpose(1, 2)
                     native.rope_from_positions(q, k, pos, self.inv_freq, qr, kr, [2 * s for s in wl.MROPE_SECTION])
-                    q, k = qr, kr
                 else:
-                    q, k = ops.multimodal_rope(q, k, cos, sin, list(wl.MROPE_SECTION))
+                    qr, kr = ops.multimodal_rope(q, k, cos, sin, list(wl.MROPE_SECTION))
+                if capture is not None and li in capture.get("layers", ()):
+                    capture[li] = {"q_in": q, "k_in": k, "q_out": qr, "k_out": kr}
+                q, k = qr, kr
             with timer.section("sdpa_torch"):
                 if n_tail:
                     head = S - n_tail
@@ -209,7 +220,10 @@ class PrefillHarness:
                 else:
                     h = h + F.linear(a2d, layer["wo"]).view(B, S, H)
             nxt = self.layers[li + 1]["ln1"] if li + 1 < len(self.layers) else self.final_ln
-            h, x = self._ffn(h.view(B * S, H), layer["ln2"], routing, layer["packed"], timer, nxt)
+            ffn_in = h.view(B * S, H)
+            h, x = self._ffn(ffn_in, layer["ln2"], routing, layer["packed"], timer, nxt)
+            if capture is not None and li in capture.get("layers", ()):
+                capture[li].update(ffn_in=ffn_in, ffn_out=h, next_normed=x)
             h = h.view(B, S, H)
             x = x.view(B, S, H) if x is not None else None
         with timer.section("lm_head_torch"):

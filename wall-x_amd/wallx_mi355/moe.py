@@ -10,6 +10,8 @@ stay on the device (expert_offsets from the partition), so nothing synchronises 
 Parameter names match the reference (``experts.{e}.{gate,up,down}_proj.weight``), so its checkpoints load.
 """
 
+import threading
+import weakref
 from dataclasses import dataclass
 from typing import List, Optional
 
@@ -45,6 +47,38 @@ class Routing:
     expert_offsets: torch.Tensor  # int32 [E + 1] on the device
     num_tokens: int
     sorted_row_id: Optional[torch.Tensor] = None  # int32 [T]: token at each sorted position (inverse map)
+
+
+class _RoutingCache(threading.local):
+    """The partition of the token types last seen on this thread, shared by every block of a model.
+
+    The reference's decoder hands the SAME `moe_token_types` tensor to all of its layers (act.py:257-261, 486), and
+    each layer's block would partition it again.  The cache answers with the previous result when the caller passes
+    the very same tensor object (so its memory cannot have been recycled for other data), unmodified (same version
+    counter), on the same stream and for the same expert count: one partition per forward without any change to
+    the reference's model code.  The partition's scratch buffers are kept here too, per device."""
+
+    def __init__(self):
+        self.ref = None
+        self.key = None
+        self.routing = None
+        self.workspace = {}  # device -> [histograms, status word]
+
+    def lookup(self, ids: torch.Tensor, num_experts: int):
+        key = (ids._version, tuple(ids.shape), ids.dtype, ids.device, num_experts,
+               torch.cuda.current_stream(ids.device).cuda_stream)
+        if self.ref is not None and self.ref() is ids and self.key == key:
+            return self.routing
+        flat = ids.reshape(-1)
+        row_id_map, offsets, inverse, ws = native.partition(flat, num_experts, 0, self.workspace.get(ids.device),
+                                                            want_sorted=True)
+        self.workspace[ids.device] = ws
+        self.ref, self.key = weakref.ref(ids), key
+        self.routing = Routing(row_id_map, offsets, flat.numel(), inverse)
+        return self.routing
+
+
+_routing_cache = _RoutingCache()
 
 
 class _DualExpertFFN(torch.autograd.Function):
@@ -86,10 +120,13 @@ class _MoeBlockFunction(torch.autograd.Function):
                                                        sorted_row_id)
         w = ((weights[0], weights[1], weights[2]), (weights[3], weights[4], weights[5]))
         ctx.save_for_backward(x, row_id_map, expert_offsets, *weights)
+        # weights that train are repacked on every forward: writes through `.data` (master-weight or EMA copies) do
+        # not move the version counter a cached copy would be checked against
         if sorted_row_id is not None:
             return native.dual_swiglu_ffn(scratch["x_tiled"], T, expert_offsets, w, hmid=scratch.get("hmid"),
-                                          out_row_id=sorted_row_id)
-        y_sorted = native.dual_swiglu_ffn(scratch["x_tiled"], T, expert_offsets, w, hmid=scratch.get("hmid"))
+                                          out_row_id=sorted_row_id, cache_packed=False)
+        y_sorted = native.dual_swiglu_ffn(scratch["x_tiled"], T, expert_offsets, w, hmid=scratch.get("hmid"),
+                                          cache_packed=False)
         return native.unpermute(y_sorted, row_id_map, torch.tensor([]), T, 1)
 
     @staticmethod
@@ -137,16 +174,31 @@ class SparseMoeBlock(nn.Module):
             raise ValueError("the dual-expert kernel runs exactly two experts (VL and action)")
         self.num_experts = num_experts
         self.experts = nn.ModuleList([ExpertMLP(config.experts[i]) for i in range(num_experts)])
-        self._partition_ws: Optional[List[torch.Tensor]] = None
         self._hmid: Optional[torch.Tensor] = None
         self._x_tiled: Optional[torch.Tensor] = None
+        self._packed: Optional[List[torch.Tensor]] = None  # set by pack_for_inference()
 
     def route(self, experts_indices: torch.Tensor) -> Routing:
-        """Stable partition of the flattened token types; reuse the result for all layers of a forward."""
-        ids = experts_indices.reshape(-1)
-        row_id_map, offsets, inverse, self._partition_ws = native.partition(ids, self.num_experts, 0,
-                                                                            self._partition_ws, want_sorted=True)
-        return Routing(row_id_map, offsets, ids.numel(), inverse)
+        """Stable partition of the flattened token types.  The result is valid for all layers of a forward; it is
+        remembered (per thread) for as long as the caller keeps passing the same, unmodified tensor object, which is
+        what the reference's decoder does for its 36 layers (act.py:257-261)."""
+        return _routing_cache.lookup(experts_indices, self.num_experts)
+
+    def pack_for_inference(self, free_dense: bool = True) -> "SparseMoeBlock":
+        """Packs the six projection weights into the K-tiled layout the kernels read and, with free_dense, releases
+        the nn.Linear copies (the parameters stay registered, emptied, so the module tree keeps its shape): half the
+        expert memory of a block that holds both.  The block is forward-only afterwards; load weights first."""
+        flat = [w for e in self.experts for w in e.weights()]
+        if any(w.numel() == 0 for w in flat):
+            raise RuntimeError("pack_for_inference: the nn.Linear weights were already released")
+        self._packed = [native.pack_weight(w.detach(), cache=False) for w in flat]
+        if free_dense:
+            for e in self.experts:
+                for proj in (e.gate_proj, e.up_proj, e.down_proj):
+                    native.invalidate_packed(proj.weight)
+                    proj.weight = nn.Parameter(torch.empty(0, dtype=proj.weight.dtype, device=proj.weight.device),
+                                               requires_grad=False)
+        return self
 
     def forward(self, hidden_states: torch.Tensor, experts_indices: torch.Tensor,
                 start_indices: Optional[torch.Tensor] = None, end_indices: Optional[torch.Tensor] = None,
@@ -179,6 +231,10 @@ class SparseMoeBlock(nn.Module):
         need = native.padded_sorted_rows(x.size(0)) * max(e.intermediate_size for e in self.experts)
         if self._hmid is None or self._hmid.numel() < need or self._hmid.device != x.device:
             self._hmid = torch.empty(need, dtype=torch.bfloat16, device=x.device)
+        if self._packed is not None:
+            if torch.is_grad_enabled() and x.requires_grad:
+                raise RuntimeError("a block packed for inference has no backward")
+            return self._forward_packed(x, routing, host_rows, pre_norm, residual).view(batch, seq, hidden)
         if torch.is_grad_enabled() and (x.requires_grad or any(w.requires_grad for w in flat)):
             # training: norm and residual stay PyTorch ops (autograd differentiates them), the block itself has
             # its own backward
@@ -208,6 +264,23 @@ class SparseMoeBlock(nn.Module):
             y = _DualExpertFFN.apply(self._x_tiled, x.size(0), routing.expert_offsets, self._hmid, host_rows,
                                      routing.sorted_row_id, *flat)
         return y.view(batch, seq, hidden)
+
+
+    def _forward_packed(self, x, routing, host_rows, pre_norm, residual):
+        dims = (self.experts[0].hidden_size, self.experts[0].intermediate_size, self.experts[1].intermediate_size)
+        if pre_norm is not None:
+            norm_weight, eps = pre_norm
+            self._x_tiled = native.rmsnorm_permute_rows_tiled(x, norm_weight, eps, routing.expert_offsets,
+                                                              routing.sorted_row_id, self._x_tiled)
+        else:
+            self._x_tiled = native.permute_rows_tiled(x, routing.row_id_map, routing.expert_offsets, self._x_tiled,
+                                                      routing.sorted_row_id)
+        if residual:
+            y_sorted = native.dual_swiglu_ffn_packed(self._x_tiled, x.size(0), routing.expert_offsets, self._packed,
+                                                     dims, hmid=self._hmid, host_rows=host_rows)
+            return native.unpermute_add(y_sorted, x, routing.row_id_map)
+        return native.dual_swiglu_ffn_packed(self._x_tiled, x.size(0), routing.expert_offsets, self._packed, dims,
+                                             hmid=self._hmid, host_rows=host_rows, out_row_id=routing.sorted_row_id)
 
 
 def moe_layer_forward(x: torch.Tensor, token_types: torch.Tensor, weights, routing: Optional[Routing] = None,

@@ -5,6 +5,8 @@ torch is used for allocation and stream lookup only; every computation is a HIP 
 Nothing here falls back to PyTorch math: without the library, or with CPU tensors, calls raise.
 """
 
+import os
+import warnings
 from typing import List, Optional, Tuple
 
 import torch
@@ -15,19 +17,35 @@ from ._lib import WX_BF16, WX_F16, WX_F32, WX_I32, WX_I64, WX_U8, WX_MROPE_CSRC,
 _DTYPES = {torch.float32: WX_F32, torch.float16: WX_F16, torch.bfloat16: WX_BF16}
 _ITYPES = {torch.int32: WX_I32, torch.int64: WX_I64, torch.bool: WX_U8, torch.uint8: WX_U8}
 
-# Channel layout used by rope()/rope_bwd().  "hf" follows the reference's PyTorch path
-# (vl.py:763-769); "csrc" follows its CUDA kernel (csrc/rope.cu:104-117).  They differ on 80 of 128
-# channels for mrope_section [16, 24, 24] and coincide only when the three position planes are equal.
-_mrope_layout = WX_MROPE_HF
+# Channel -> position-plane layouts of the M-RoPE kernels.  "csrc" is the reference's CUDA kernel
+# (csrc/rope.cu:104-117), "hf" its PyTorch path (vl.py:763-769).  They differ on 80 of 128 channels for
+# mrope_section [16, 24, 24] and coincide only when the three position planes are equal.  The layout is an argument
+# of every call (no process-wide switch): rope() / rope_bwd(), the two names of the reference's extension module,
+# default to the extension's own layout; the ops that follow the model's PyTorch path pass "hf".
+_LAYOUTS = {"hf": WX_MROPE_HF, "csrc": WX_MROPE_CSRC}
 
 
-def set_mrope_layout(name: str) -> None:
-    global _mrope_layout
-    _mrope_layout = {"hf": WX_MROPE_HF, "csrc": WX_MROPE_CSRC}[name]
+def _layout_code(layout: str) -> int:
+    try:
+        return _LAYOUTS[layout]
+    except KeyError:
+        raise RuntimeError(f"mrope layout must be 'hf' or 'csrc', got {layout!r}")
 
 
-def get_mrope_layout() -> str:
-    return "hf" if _mrope_layout == WX_MROPE_HF else "csrc"
+# Checked mode.  The kernels report malformed input (expert ids outside the bins, rows whose vision tokens and grids
+# do not add up) through a device status word instead of stopping; reading it costs a host synchronisation, which the
+# hot path never makes.  With WALLX_MI355_CHECKED=1 in the environment, or set_checked(True), every partition() and
+# rope_index() call reads its status word back and raises where the reference's Python path raises.
+_checked = os.environ.get("WALLX_MI355_CHECKED", "0") not in ("", "0")
+
+
+def set_checked(flag: bool) -> None:
+    global _checked
+    _checked = bool(flag)
+
+
+def is_checked() -> bool:
+    return _checked
 
 
 def _stream(t: torch.Tensor) -> int:
@@ -122,17 +140,6 @@ def swiglu_bwd(gate: torch.Tensor, up: torch.Tensor, dh: torch.Tensor):
     return hm, dg, du
 
 
-def transpose_2d(t: torch.Tensor) -> torch.Tensor:
-    """Contiguous transposed copy of a contiguous 2-D bf16 / fp16 tensor whose sizes are multiples of 8."""
-    _need_cuda("tensor", t)
-    if t.dim() != 2 or t.element_size() != 2 or not t.is_contiguous():
-        raise RuntimeError("transpose_2d takes a contiguous 2-D tensor of 2-byte elements")
-    out = torch.empty((t.size(1), t.size(0)), dtype=t.dtype, device=t.device)
-    with _DeviceGuard(t):
-        _lib.call("wx_transpose_2d", _ptr(t), _ptr(out), t.size(0), t.size(1), 2, _stream(t))
-    return out
-
-
 # ----------------------------------------------------------------------------- permute / unpermute
 def partition(indices: torch.Tensor, num_experts: int, num_out_tokens: int = 0,
               workspace: Optional[List[torch.Tensor]] = None, want_sorted: bool = False):
@@ -140,6 +147,9 @@ def partition(indices: torch.Tensor, num_experts: int, num_out_tokens: int = 0,
 
     Returns (row_id_map int32 [T*K], expert_offsets int32 [E+1], sorted_row_id or None, workspace).
     workspace = [hist scratch, status word]; pass the returned list back in to avoid reallocation.
+    Ids outside [0, num_experts) are clamped into range and flagged in the status word (workspace[1], a device
+    int32 that stays set until cleared); in checked mode (set_checked / WALLX_MI355_CHECKED=1) the word is cleared
+    before and read after every call and such ids raise.
     """
     _need_cuda("indices", indices)
     ids = indices if indices.is_contiguous() else indices.contiguous()
@@ -153,6 +163,8 @@ def partition(indices: torch.Tensor, num_experts: int, num_out_tokens: int = 0,
     if not workspace or workspace[0].numel() < need or workspace[0].device != dev:
         workspace = [torch.empty(need, dtype=torch.uint8, device=dev),
                      torch.zeros(1, dtype=torch.int32, device=dev)]
+    elif _checked:
+        workspace[1].zero_()  # the status word only ever gets set by the kernels: start each checked call from 0
     row_id_map = torch.empty(n, dtype=torch.int32, device=dev)
     offsets = torch.empty(num_experts + 1, dtype=torch.int32, device=dev)
     sorted_row_id = torch.empty(n, dtype=torch.int32, device=dev) if want_sorted else None
@@ -160,6 +172,9 @@ def partition(indices: torch.Tensor, num_experts: int, num_out_tokens: int = 0,
         _lib.call("wx_partition_build", _ptr(ids), _ITYPES[ids.dtype], T, K, int(num_experts),
                   int(num_out_tokens), _ptr(row_id_map), _ptr(sorted_row_id), offsets.data_ptr(),
                   workspace[1].data_ptr(), workspace[0].data_ptr(), workspace[0].numel(), _stream(ids))
+    if _checked and n and int(workspace[1].item()):
+        raise RuntimeError(f"partition: expert ids outside [0, {int(num_experts)}) (they were clamped into range; "
+                           "the grouping does not follow the ids)")
     return row_id_map, offsets, sorted_row_id, workspace
 
 
@@ -246,7 +261,7 @@ def _bhsd_strides(t: torch.Tensor):
     return _lib.i64x3((t.stride(0), t.stride(1), t.stride(2)))
 
 
-def _rope_common(fn_name, q_in, k_in, cos, sin, q_out, k_out, mrope_section_doubled):
+def _rope_common(fn_name, q_in, k_in, cos, sin, q_out, k_out, mrope_section_doubled, layout):
     for name, t in (("q", q_in), ("k", k_in), ("cos", cos), ("sin", sin), ("q_out", q_out), ("k_out", k_out)):
         _need_cuda(name, t)
     if len(mrope_section_doubled) != 3:
@@ -266,20 +281,25 @@ def _rope_common(fn_name, q_in, k_in, cos, sin, q_out, k_out, mrope_section_doub
     with _DeviceGuard(q_in):
         _lib.call(fn_name, _ptr(q_in), _ptr(k_in), _ptr(cos), _ptr(sin), _ptr(q_out), _ptr(k_out), B, S, Hq, Hk,
                   D, _bhsd_strides(q_in), _bhsd_strides(k_in), _bhsd_strides(q_out), _bhsd_strides(k_out),
-                  section, _mrope_layout, _dtype_code(q_in), _stream(q_in))
+                  section, _layout_code(layout), _dtype_code(q_in), _stream(q_in))
 
 
-def rope(q, k, cos, sin, q_out, k_out, mrope_section_doubled) -> None:
-    """csrc/rope.cu:453-509.  q [B,Hq,S,D], k [B,Hkv,S,D] (any batch/head/seq strides), cos/sin [3,B,S,D]."""
-    _rope_common("wx_mrope_apply", q, k, cos, sin, q_out, k_out, mrope_section_doubled)
+def rope(q, k, cos, sin, q_out, k_out, mrope_section_doubled, layout: str = "csrc") -> None:
+    """csrc/rope.cu:453-509.  q [B,Hq,S,D], k [B,Hkv,S,D] (any batch/head/seq strides), cos/sin [3,B,S,D].
+    With the default layout channel d takes plane t for d < 2 s0, h for d < 2 s0 + 2 s1, else w, as the reference's
+    kernel does (csrc/rope.cu:104-117); layout="hf" gives apply_multimodal_rotary_pos_emb (vl.py:763-769)."""
+    _rope_common("wx_mrope_apply", q, k, cos, sin, q_out, k_out, mrope_section_doubled, layout)
 
 
-def rope_bwd(grad_q_out, grad_k_out, q, k, cos, sin, grad_q, grad_k, mrope_section_doubled) -> None:
+def rope_bwd(grad_q_out, grad_k_out, q, k, cos, sin, grad_q, grad_k, mrope_section_doubled,
+             layout: str = "csrc") -> None:
     """csrc/rope.cu:511-571.  q and k are accepted for signature parity; the adjoint does not need them."""
-    _rope_common("wx_mrope_apply_bwd", grad_q_out, grad_k_out, cos, sin, grad_q, grad_k, mrope_section_doubled)
+    _rope_common("wx_mrope_apply_bwd", grad_q_out, grad_k_out, cos, sin, grad_q, grad_k, mrope_section_doubled,
+                 layout)
 
 
-def rope_from_positions(q, k, position_ids, inv_freq, q_out, k_out, mrope_section_doubled, backward: bool = False) -> None:
+def rope_from_positions(q, k, position_ids, inv_freq, q_out, k_out, mrope_section_doubled, backward: bool = False,
+                        layout: str = "hf") -> None:
     """M-RoPE with cos/sin evaluated in the kernel (vl.py:679-712 folded into vl.py:731-773): position_ids
     [3, B, S] int64, inv_freq [D/2] fp32.  With backward=True, q/k carry the output gradients and q_out/k_out
     receive the input gradients."""
@@ -304,7 +324,7 @@ def rope_from_positions(q, k, position_ids, inv_freq, q_out, k_out, mrope_sectio
     with _DeviceGuard(q):
         _lib.call("wx_mrope_apply_positions", _ptr(q), _ptr(k), _ptr(position_ids), _ptr(inv_freq), _ptr(q_out),
                   _ptr(k_out), B, S, Hq, Hk, D, _bhsd_strides(q), _bhsd_strides(k), _bhsd_strides(q_out),
-                  _bhsd_strides(k_out), section, _mrope_layout, _dtype_code(q), int(bool(backward)), _stream(q))
+                  _bhsd_strides(k_out), section, _layout_code(layout), _dtype_code(q), int(bool(backward)), _stream(q))
 
 
 # ----------------------------------------------------------------------------- index builders
@@ -339,6 +359,10 @@ def rope_index(input_ids, image_grid_thw, video_grid_thw, second_per_grid_ts, at
                   0 if vg is None else vg.size(0), _ptr(spg), B, S, int(spatial_merge_size), int(image_token_id),
                   int(video_token_id), int(vision_start_token_id), float(tokens_per_second), _ptr(pos),
                   _ptr(deltas), status.data_ptr(), ws.data_ptr(), ws_bytes, _stream(ids))
+    if _checked and int(status.item()):
+        # the Python path raises on such rows (list.index / grid indexing, act.py:1013-1045)
+        raise ValueError("rope_index: a row's vision tokens, <vision_start> markers and grids do not add up "
+                         "(or a row is fully masked)")
     if return_status:
         return pos, deltas, status
     return pos, deltas
@@ -409,7 +433,7 @@ def get_window_index(grid_thw: torch.Tensor, spatial_merge_size: int, vit_merger
 # ----------------------------------------------------------------------------- fused dual-expert FFN
 import weakref
 
-_packed_cache = {}  # id(weight) -> (weakref to weight, version, packed tensor)
+_packed_cache = {}  # id(weight) -> (weakref to weight, (data_ptr, version, shape, device), packed tensor)
 
 
 def padded_sorted_rows(num_tokens: int) -> int:
@@ -417,18 +441,34 @@ def padded_sorted_rows(num_tokens: int) -> int:
     return int(_lib.load().wx_padded_sorted_rows(int(num_tokens)))
 
 
+def invalidate_packed(w: Optional[torch.Tensor] = None) -> None:
+    """Drops the cached K-tiled copy of `w` (of every weight when w is None).  Call it after writing a weight in a
+    way torch's version counter does not see -- `w.data.copy_(...)`, `w.data.normal_()`, a write through another
+    view of `.data` -- before the next forward that does not track gradients."""
+    if w is None:
+        _packed_cache.clear()
+    else:
+        _packed_cache.pop(id(w), None)
+
+
 def pack_weight(w: torch.Tensor, cache: bool = True) -> torch.Tensor:
     """nn.Linear weight [out, in] (bf16, CUDA) -> the K-tiled layout the MFMA kernels read (flat bf16 tensor).
 
-    Packed copies are cached per weight tensor and rebuilt when the tensor is modified in place.
-    """
+    Packed copies are cached per weight tensor, keyed on its storage address, shape and version counter, so an
+    in-place update through the tensor itself (an optimizer step, `copy_`, `load_state_dict`) or a re-assigned
+    `.data` repacks.  Writes through `.data` do not move the version counter: callers whose weights train pass
+    cache=False (the MoE block does, on its autograd path: tens of microseconds beside the GEMMs the weights feed
+    and their backward), and frozen weights written that way need invalidate_packed()."""
     _need_cuda("weight", w)
     if w.dtype != torch.bfloat16 or w.dim() != 2:
         raise RuntimeError("expert weights must be 2-D BFloat16 tensors")
     key = id(w)
+    if not cache:
+        _packed_cache.pop(key, None)
+    state = (w.data_ptr(), w._version, tuple(w.shape), w.device)
     if cache:
         hit = _packed_cache.get(key)
-        if hit is not None and hit[0]() is w and hit[1] == w._version and hit[2].device == w.device:
+        if hit is not None and hit[0]() is w and hit[1] == state:
             return hit[2]
     src = w.detach().contiguous()
     rows, cols = src.shape
@@ -437,7 +477,7 @@ def pack_weight(w: torch.Tensor, cache: bool = True) -> torch.Tensor:
     with _DeviceGuard(src):
         _lib.call("wx_pack_tiled", _ptr(src), packed.data_ptr(), rows, cols, _stream(src))
     if cache:
-        _packed_cache[key] = (weakref.ref(w, lambda _r, k=key: _packed_cache.pop(k, None)), w._version, packed)
+        _packed_cache[key] = (weakref.ref(w, lambda _r, k=key: _packed_cache.pop(k, None)), state, packed)
     return packed
 
 
@@ -513,32 +553,27 @@ def unpermute_add_rmsnorm(y_sorted: torch.Tensor, residual: torch.Tensor, row_id
     return out, normed
 
 
-def dual_swiglu_ffn(x_tiled: torch.Tensor, num_rows: int, expert_offsets: torch.Tensor, weights,
-                    hmid: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
-                    host_rows=None, out_row_id: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """Both experts' SwiGLU FFN over expert-sorted rows in two launches (act.py:79-82, 142-154).
-
-    x_tiled: result of permute_rows_tiled for num_rows tokens; expert_offsets int32 [3] ON THE DEVICE (from
-    partition()); weights = ((gate0, up0, down0), (gate1, up1, down1)) in nn.Linear layout (packed and cached
-    here).  host_rows: optional (rows of expert 0, rows of expert 1) as host integers, when the caller has them
-    anyway; they only spare the library a second, empty launch when it cannot tell which tile shape fits.
-    out_row_id: optional int32 [num_rows] CUDA tensor, the partition's sorted_row_id; with it the result comes back
-    in token order (the unpermute happens in the down launch's stores).
-    Returns out [num_rows, hidden] bf16, in sorted order unless out_row_id is given.
-    """
+def dual_swiglu_ffn_packed(x_tiled: torch.Tensor, num_rows: int, expert_offsets: torch.Tensor, packed, dims,
+                           hmid: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
+                           host_rows=None, out_row_id: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """dual_swiglu_ffn on weights that are already K-tiled: packed = (gate0, up0, down0, gate1, up1, down1) from
+    pack_weight, dims = (hidden, inter0, inter1)."""
     _need_cuda("x_tiled", x_tiled)
-    (g0, u0, d0), (g1, u1, d1) = weights
-    H = g0.size(1)
-    I0, I1 = g0.size(0), g1.size(0)
-    if tuple(g0.shape) != (I0, H) or tuple(u0.shape) != (I0, H) or tuple(d0.shape) != (H, I0) or \
-            tuple(g1.shape) != (I1, H) or tuple(u1.shape) != (I1, H) or tuple(d1.shape) != (H, I1):
-        raise RuntimeError("expert weight shapes are inconsistent with hidden size")
+    H, I0, I1 = (int(v) for v in dims)
+    lib = _lib.load()
+    want = [lib.wx_tiled_bytes(I0, H), lib.wx_tiled_bytes(I0, H), lib.wx_tiled_bytes(H, I0),
+            lib.wx_tiled_bytes(I1, H), lib.wx_tiled_bytes(I1, H), lib.wx_tiled_bytes(H, I1)]
+    if len(packed) != 6:
+        raise RuntimeError("packed must hold gate, up and down of both experts")
+    for t, nbytes in zip(packed, want):
+        _need_cuda("packed weight", t)
+        if t.dtype != torch.bfloat16 or t.numel() * 2 < nbytes or t.device != x_tiled.device:
+            raise RuntimeError("packed expert weights do not match (hidden, inter0, inter1)")
     if expert_offsets.dtype != torch.int32 or expert_offsets.numel() < 3 or not expert_offsets.is_cuda:
         raise RuntimeError("expert_offsets must be an int32 CUDA tensor with 3 entries")
     if out_row_id is not None and (out_row_id.dtype != torch.int32 or not out_row_id.is_cuda or
                                    out_row_id.numel() < num_rows):
         raise RuntimeError("out_row_id must be an int32 CUDA tensor with one entry per row")
-    packed = [pack_weight(w) for w in (g0, u0, d0, g1, u1, d1)]
     dev = x_tiled.device
     need = padded_sorted_rows(num_rows) * max(I0, I1)
     if hmid is None or hmid.numel() < need or hmid.dtype != torch.bfloat16:
@@ -551,3 +586,29 @@ def dual_swiglu_ffn(x_tiled: torch.Tensor, num_rows: int, expert_offsets: torch.
                   hmid.data_ptr(), int(num_rows), H, I0, I1, _lib.i64x2(host_rows), _ptr(out_row_id),
                   _stream(x_tiled))
     return out
+
+
+def dual_swiglu_ffn(x_tiled: torch.Tensor, num_rows: int, expert_offsets: torch.Tensor, weights,
+                    hmid: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
+                    host_rows=None, out_row_id: Optional[torch.Tensor] = None,
+                    cache_packed: bool = True) -> torch.Tensor:
+    """Both experts' SwiGLU FFN over expert-sorted rows in two launches (act.py:79-82, 142-154).
+
+    x_tiled: result of permute_rows_tiled for num_rows tokens; expert_offsets int32 [3] ON THE DEVICE (from
+    partition()); weights = ((gate0, up0, down0), (gate1, up1, down1)) in nn.Linear layout (packed here; the
+    packed copies are cached per tensor unless cache_packed is False).  host_rows: optional (rows of expert 0, rows
+    of expert 1) as host integers, when the caller has them
+    anyway; they only spare the library a second, empty launch when it cannot tell which tile shape fits.
+    out_row_id: optional int32 [num_rows] CUDA tensor, the partition's sorted_row_id; with it the result comes back
+    in token order (the unpermute happens in the down launch's stores).
+    Returns out [num_rows, hidden] bf16, in sorted order unless out_row_id is given.
+    """
+    (g0, u0, d0), (g1, u1, d1) = weights
+    H = g0.size(1)
+    I0, I1 = g0.size(0), g1.size(0)
+    if tuple(g0.shape) != (I0, H) or tuple(u0.shape) != (I0, H) or tuple(d0.shape) != (H, I0) or \
+            tuple(g1.shape) != (I1, H) or tuple(u1.shape) != (I1, H) or tuple(d1.shape) != (H, I1):
+        raise RuntimeError("expert weight shapes are inconsistent with hidden size")
+    packed = [pack_weight(w, cache=cache_packed) for w in (g0, u0, d0, g1, u1, d1)]
+    return dual_swiglu_ffn_packed(x_tiled, num_rows, expert_offsets, packed, (H, I0, I1), hmid, out, host_rows,
+                                  out_row_id)
