@@ -57,6 +57,21 @@ int wx_partition_build(const void* ids, int id_type /* wx_itype */, int64_t num_
                        int32_t* sorted_row_id, int32_t* expert_offsets, int32_t* status,
                        void* workspace, size_t workspace_bytes, wx_stream_t stream);
 
+/* wx_partition_build for callers that cannot allocate device memory or hand over a workspace (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference, whose
+ * permute op allocates its sort workspace with torch (csrc/permute.cu:462-482).  Same arguments, outputs and
+ * status codes as wx_partition_build minus the workspace pair: the per-segment histograms go to a 1 MiB device
+ * array built into the library (one copy per GPU, held until the process ends), which covers every size the
+ * partition takes (up to 2^31 - 1 expanded tokens; larger counts are refused with WX_ERR_UNSUPPORTED, a count whose
+ * histograms would not fit with WX_ERR_WORKSPACE).  The call allocates nothing and does not synchronise.  The first
+ * call on a device looks up the array's address (hipGetSymbolAddress); make that call outside graph capture.
+ * All calls on one GPU share the array: calls that overlap there (different streams or threads) race -- order them
+ * on one stream.  Nothing in the array needs clearing between calls (every word read is written first). */
+int wx_partition_build_noalloc(const void* ids, int id_type /* wx_itype */, int64_t num_tokens, int num_topk,
+                               int num_experts, int64_t num_out_tokens, int32_t* row_id_map,
+                               int32_t* sorted_row_id, int32_t* expert_offsets, int32_t* status,
+                               wx_stream_t stream);
+
 /* Row scatter of the permute op: out[row_id_map[k*T + t], :] = x[t, :] for every k with a map entry
  * != -1.  Replaces moe_permute_topK_kernel, forward branch (csrc/permute.cu:156-262, 294-305).
  * num_cols * sizeof(dtype) must be a multiple of 16 and rows 16-byte aligned. */

@@ -7,6 +7,8 @@
 //   pass 1  partition_count    per-segment histogram  -> hist[segment][256]
 //   pass 2  partition_scatter  per-block prefix over hist (bins, then earlier segments), then ranks
 // The row movers are pure HBM streams: one wavefront per token row, 16-byte lanes, several rows in flight.
+#include <mutex>
+
 #include "common.h"
 #include "tiled_layout.h"
 
@@ -464,30 +466,31 @@ extern "C" size_t wx_partition_workspace_bytes(int64_t n) {
   return static_cast<size_t>(padded) * kBins * sizeof(int32_t);
 }
 
-extern "C" int wx_partition_build(const void* ids, int id_type, int64_t num_tokens, int num_topk, int num_experts,
-                                  int64_t num_out_tokens, int32_t* row_id_map, int32_t* sorted_row_id,
-                                  int32_t* expert_offsets, int32_t* status, void* workspace,
-                                  size_t workspace_bytes, wx_stream_t stream) {
-  if (num_tokens < 0 || num_topk < 1) return fail(WX_ERR_INVALID_ARGUMENT, "wx_partition_build: bad sizes");
-  if (num_topk > 128) return fail(WX_ERR_UNSUPPORTED, "wx_partition_build: num_topK cannot exceed 128.");
+namespace {
+
+// Argument checks and the two launches shared by the partition entry points; `hist` holds
+// wx_partition_workspace_bytes(n) bytes.  Every histogram word the second launch reads is written by the first, so
+// the buffer needs no clearing between calls.
+int partition_launch(const char* who, const void* ids, int id_type, int64_t num_tokens, int num_topk, int num_experts,
+                     int64_t num_out_tokens, int32_t* row_id_map, int32_t* sorted_row_id, int32_t* expert_offsets,
+                     int32_t* status, int32_t* hist, size_t hist_bytes, hipStream_t s) {
+  if (num_tokens < 0 || num_topk < 1) return fail(WX_ERR_INVALID_ARGUMENT, "%s: bad sizes", who);
+  if (num_topk > 128) return fail(WX_ERR_UNSUPPORTED, "%s: num_topK cannot exceed 128.", who);
   if (num_experts < 1 || num_experts > kBins)
-    return fail(WX_ERR_UNSUPPORTED, "wx_partition_build: num_experts %d outside [1, %d]", num_experts, kBins);
+    return fail(WX_ERR_UNSUPPORTED, "%s: num_experts %d outside [1, %d]", who, num_experts, kBins);
   if (id_type != WX_I32 && id_type != WX_I64 && id_type != WX_U8)
-    return fail(WX_ERR_INVALID_ARGUMENT, "wx_partition_build: bad id_type %d", id_type);
+    return fail(WX_ERR_INVALID_ARGUMENT, "%s: bad id_type %d", who, id_type);
   const int64_t n = num_tokens * num_topk;
-  if (n > INT32_MAX) return fail(WX_ERR_UNSUPPORTED, "wx_partition_build: more than 2^31-1 expanded tokens");
-  if (n > 0 && (ids == nullptr || row_id_map == nullptr || workspace == nullptr))
-    return fail(WX_ERR_INVALID_ARGUMENT, "wx_partition_build: null pointer");
-  if (workspace_bytes < wx_partition_workspace_bytes(n))
-    return fail(WX_ERR_WORKSPACE, "wx_partition_build: workspace %zu < %zu bytes", workspace_bytes,
-                wx_partition_workspace_bytes(n));
-  hipStream_t s = as_stream(stream);
+  if (n > INT32_MAX) return fail(WX_ERR_UNSUPPORTED, "%s: more than 2^31-1 expanded tokens", who);
+  if (n > 0 && (ids == nullptr || row_id_map == nullptr || hist == nullptr))
+    return fail(WX_ERR_INVALID_ARGUMENT, "%s: null pointer", who);
+  if (hist_bytes < wx_partition_workspace_bytes(n))
+    return fail(WX_ERR_WORKSPACE, "%s: workspace %zu < %zu bytes", who, hist_bytes, wx_partition_workspace_bytes(n));
   const int64_t seg = segment_len(n > 0 ? n : 1);
   const int64_t num_seg = n > 0 ? (n + seg - 1) / seg : 0;
   // at least one block even for n == 0 so expert_offsets are written
   const int blocks = static_cast<int>(num_seg > 0 ? (num_seg + kWavesPerBlock - 1) / kWavesPerBlock : 1);
   const int64_t num_out = num_out_tokens > 0 ? num_out_tokens : n;
-  int32_t* hist = static_cast<int32_t*>(workspace);
   if (n > 0) {
     hipLaunchKernelGGL(partition_count, dim3(blocks), dim3(kBlock), 0, s, ids, id_type, n, num_experts, seg, hist,
                        status);
@@ -496,6 +499,72 @@ extern "C" int wx_partition_build(const void* ids, int id_type, int64_t num_toke
   hipLaunchKernelGGL(partition_scatter, dim3(blocks), dim3(kBlock), 0, s, ids, id_type, num_tokens, num_topk,
                      num_experts, num_out, seg, num_seg, hist, row_id_map, sorted_row_id, expert_offsets);
   return check_launch("partition_scatter");
+}
+
+}  // namespace
+
+extern "C" int wx_partition_build(const void* ids, int id_type, int64_t num_tokens, int num_topk, int num_experts,
+                                  int64_t num_out_tokens, int32_t* row_id_map, int32_t* sorted_row_id,
+                                  int32_t* expert_offsets, int32_t* status, void* workspace,
+                                  size_t workspace_bytes, wx_stream_t stream) {
+  return partition_launch("wx_partition_build", ids, id_type, num_tokens, num_topk, num_experts, num_out_tokens,
+                          row_id_map, sorted_row_id, expert_offsets, status, static_cast<int32_t*>(workspace),
+                          workspace_bytes, as_stream(stream));
+}
+
+// ---- the partition without a workspace argument ----------------------------------------------------------------
+// The per-segment histograms live in a device array that is part of the library's code object: each GPU the library
+// runs on holds its own 1 MiB copy from the moment the code object is loaded there until the process ends.
+// segment_len() never cuts the key stream into more than 1024 segments, so the array covers every size the
+// partition takes.  In host code the array's name is only a handle for hipGetSymbolAddress: the address kernels and
+// copies use is looked up once per device, with that device current, and kept.
+constexpr int kStaticSegments = 1024;
+static __device__ __align__(256) int32_t scratch[kStaticSegments * wx::kBins];
+
+namespace {
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+int32_t* g_scratch_ptr[kMaxDevices] = {};
+
+int static_scratch(int32_t** out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices)
+    return fail(WX_ERR_LAUNCH, "wx_partition_build_noalloc: no current device (or its index is %d or above)", kMaxDevices);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || p == nullptr)
+      return fail(WX_ERR_LAUNCH, "wx_partition_build_noalloc: hipGetSymbolAddress: %s", hipGetErrorString(e));
+    g_scratch_ptr[dev] = static_cast<int32_t*>(p);
+  }
+  *out = g_scratch_ptr[dev];
+  return WX_OK;
+}
+
+}  // namespace
+
+extern "C" int wx_partition_build_noalloc(const void* ids, int id_type, int64_t num_tokens, int num_topk,
+                                          int num_experts, int64_t num_out_tokens, int32_t* row_id_map,
+                                          int32_t* sorted_row_id, int32_t* expert_offsets, int32_t* status,
+                                          wx_stream_t stream) {
+  constexpr size_t kScratchBytes = sizeof(int32_t) * kStaticSegments * kBins;
+  // sizes the partition refuses anyway (negative, topK > 128, more than 2^31-1 expanded tokens) get their message
+  // from partition_launch; anything else must fit the array
+  const bool sane = num_tokens >= 0 && num_topk >= 1 && num_topk <= 128 && num_tokens <= INT32_MAX / num_topk;
+  if (!sane)
+    return partition_launch("wx_partition_build_noalloc", ids, id_type, num_tokens, num_topk, num_experts,
+                            num_out_tokens, row_id_map, sorted_row_id, expert_offsets, status, nullptr, 0,
+                            as_stream(stream));
+  if (wx_partition_workspace_bytes(num_tokens * num_topk) > kScratchBytes)
+    return fail(WX_ERR_WORKSPACE, "wx_partition_build_noalloc: %lld expanded tokens need %zu bytes of histograms, the built-in scratch has %zu",
+                static_cast<long long>(num_tokens * num_topk), wx_partition_workspace_bytes(num_tokens * num_topk), kScratchBytes);
+  int32_t* hist = nullptr;
+  if (int rc = static_scratch(&hist)) return rc;
+  return partition_launch("wx_partition_build_noalloc", ids, id_type, num_tokens, num_topk, num_experts,
+                          num_out_tokens, row_id_map, sorted_row_id, expert_offsets, status, hist, kScratchBytes,
+                          as_stream(stream));
 }
 
 extern "C" int wx_permute_rows(const void* x, void* out, const int32_t* row_id_map, int64_t num_tokens,

@@ -25,6 +25,7 @@ PROTOTYPES = {
     "wx_abi_version": (_i32, []),
     "wx_partition_workspace_bytes": (_sz, [_i64]),
     "wx_partition_build": (_i32, [_vp, _i32, _i64, _i32, _i32, _i64, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "wx_partition_build_noalloc": (_i32, [_vp, _i32, _i64, _i32, _i32, _i64, _vp, _vp, _vp, _vp, _vp]),
     "wx_permute_rows": (_i32, [_vp, _vp, _vp, _i64, _i32, _i64, _i32, _vp]),
     "wx_unpermute_rows": (_i32, [_vp, _vp, _vp, _vp, _i64, _i32, _i64, _i32, _vp]),
     "wx_unpermute_rows_bwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i32, _i64, _i32, _vp]),
