@@ -212,6 +212,26 @@ int wx_mrope_apply_positions(const void* q, const void* k, const int64_t* positi
                              const int mrope_section[3], int layout, int dtype, int backward,
                              wx_stream_t stream);
 
+/* The attention block's q / k / v projections with the rotary embedding in the GEMM's epilogue: replaces
+ * q_proj / k_proj / v_proj (nn.Linear with bias, vl.py:821-832, 955-957) followed by the rope op
+ * (vl.py:962-964, ops.py:402-497) -- one launch, and q / k are not written and read again for the rotation.
+ * wx_mrope_table builds what the epilogue reads: table[token][d], d < head_dim / 2, = bf16 cos | bf16 sin << 16 of
+ * position_ids[plane(d)][token] * inv_freq[d] (fp32 angle, fp32 cos / sin, rounded to bf16 as vl.py:679-712 does);
+ * position_ids [3, B, S] int64, inv_freq [head_dim / 2] fp32, table uint32 [B * S, head_dim / 2].  Channels d and
+ * d + head_dim / 2 must share a position plane: true for WX_MROPE_HF, refused (WX_ERR_UNSUPPORTED) for WX_MROPE_CSRC.
+ * wx_qkv_rope_proj: out [num_tokens, (n_q + 2 n_kv) * head_dim] = x [num_tokens, hidden] @ weight^T + bias, weight
+ * [(n_q + 2 n_kv) * head_dim, hidden] = the three nn.Linear weights stacked q, k, v (row-major, read in place), bias
+ * likewise or NULL; the q and k heads (the first (n_q + n_kv) * head_dim columns) come out rotated:
+ * head[d] * cos[d] + rotate_half(head)[d] * sin[d], evaluated like eager bf16 code (the projection rounded once, every
+ * product and the sum rounded).  bf16; head_dim must be 128 (a wavefront's 128 output columns are one head), hidden a
+ * multiple of 8.  Row t of the table belongs to row t of x. */
+int wx_mrope_table(const int64_t* position_ids, const float* inv_freq, int64_t batch, int64_t seq, int head_dim,
+                   const int mrope_section[3], int layout /* wx_mrope_layout */, uint32_t* table,
+                   wx_stream_t stream);
+int wx_qkv_rope_proj(const void* x, const void* weight, const void* bias, const uint32_t* rope_table, void* out,
+                     int64_t num_tokens, int64_t hidden, int n_q_heads, int n_kv_heads, int head_dim,
+                     wx_stream_t stream);
+
 /* ------------------------------------------------------------------------------------------------
  * 3D position ids.  Replaces get_rope_index (csrc/rope_index.cu:464-569) with the semantics of the
  * PyTorch path (act.py:929-1149), exact integer arithmetic.

@@ -46,13 +46,14 @@ def _ref_forward(h, ids, grid, types, mask_mode):
     return norm(x[:, -1], h.final_ln) @ f(h.embed).T
 
 
-@pytest.mark.parametrize("mask_mode,fuse,suffix", [("causal", True, None), ("action_block", True, None),
-                                                  ("action_block", True, 8), ("causal", False, None)])
-def test_prefill_harness_matches_plain_forward(dev, mask_mode, fuse, suffix):
+@pytest.mark.parametrize("mask_mode,fuse,suffix,qkv", [("causal", True, None, False), ("action_block", True, None, False),
+                                                      ("action_block", True, 8, False), ("causal", False, None, False),
+                                                      ("action_block", True, 8, True)])
+def test_prefill_harness_matches_plain_forward(dev, mask_mode, fuse, suffix, qkv):
     from wallx_mi355 import harness
 
     h = harness.PrefillHarness(n_layers=2, hidden=256, n_q=4, n_kv=2, head_dim=128, inter=(512, 256), vocab=151936,
-                               device=dev, seed=3, mask=mask_mode, keep_dense=True, fuse=fuse)
+                               device=dev, seed=3, mask=mask_mode, keep_dense=True, fuse=fuse, fuse_qkv_rope=qkv)
     row = wl.vla_row_tokens(n_images=1, image_tokens=16, lead_text=5, tail_text=9, n_action=8)
     ids = torch.tensor([row, row, row], dtype=torch.int64, device=dev)
     grid = torch.tensor([[1, 8, 8]] * 3, dtype=torch.int64, device=dev)
@@ -61,7 +62,7 @@ def test_prefill_harness_matches_plain_forward(dev, mask_mode, fuse, suffix):
     got = h.forward(ids, grid, types, timer, action_suffix=suffix).float().cpu()
     split = timer.report_ms()
     movers = {"rmsnorm+permute", "unpermute+residual+rmsnorm"} if fuse else {"permute", "unpermute"}
-    assert movers | {"ffn_gate_up_swiglu", "ffn_down", "mrope", "rope_index", "sdpa_torch"} <= set(split)
+    assert movers | {"ffn_gate_up_swiglu", "ffn_down", "qkv_proj+mrope" if qkv else "mrope", "rope_index", "sdpa_torch"} <= set(split)
     ref = _ref_forward(h, ids, grid, types, mask_mode)
     # bf16 storage of every intermediate over two layers against an fp32 forward: bound the error by the logits' scale
     scale = float(ref.abs().max())

@@ -86,7 +86,7 @@ using TailTile = SmallTile;
 constexpr int kXcds = 8;
 constexpr int kGroupM = 8;                     // tile rows per patch in the tile order
 
-enum Mode { kGeneric = 0, kGateUp = 1, kDown = 2 };
+enum Mode { kGeneric = 0, kGateUp = 1, kDown = 2, kQkvRope = 3 };
 
 struct Group {
   const __bf16* a;   // generic: [m, k] row-major (lda).  tiled: base of the K-tiled matrix
@@ -113,6 +113,12 @@ struct Params {
   // kDown only: when set (the partition's sorted_row_id), row r of the sorted result is stored to row scatter[r] of
   // the output instead of row r -- the unpermute folded into the store.
   const int32_t* scatter;
+  // kQkvRope only (group 0 is the projection, row-major operands): bias[n] (may be null), the packed rotary table
+  // [m, 64] (bf16 cos | bf16 sin << 16 per token and channel pair) and the number of leading output columns that are
+  // rotated (whole heads of 128: the q and k heads; the v heads behind them only take the bias).
+  const __bf16* bias;
+  const uint32_t* rope_table;
+  int rope_cols;
 };
 
 #define LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
@@ -205,7 +211,7 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
   constexpr int kLoadsPerStep = kLoadsA + kLoadsB;
   constexpr int kSlotBytesA = TS::kSlotBytesA, kSlotBytesB = TS::kSlotBytesB, kStageBytes = TS::kStageBytes;
   constexpr bool SWIGLU = MODE == kGateUp;
-  constexpr bool TILED_IN = MODE != kGeneric;   // A and B are K-tiled
+  constexpr bool TILED_IN = MODE == kGateUp || MODE == kDown;   // A and B are K-tiled
   constexpr bool TILED_OUT = MODE == kGateUp;   // C is K-tiled
   static_assert(MODE == kGeneric || (!KA && !KB), "K-major operands exist in the generic mode only");
   // kStages ring slots per operand, each one K step (256 rows x 32 bf16).  Separate arrays let the compiler
@@ -233,7 +239,7 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
   // (kept as two named structs, selected per tile, so everything stays in scalar registers)
   Group g0 = p.g[0], g1 = p.g[1];
   int sorted_first[2] = {0, 0};  // kDown: sorted position of each expert's first row
-  if constexpr (MODE != kGeneric) {
+  if constexpr (TILED_IN) {
     const int o0 = p.offsets[0], o1 = p.offsets[1], o2 = p.offsets[2];
     g0.m = o1 - o0;
     g1.m = o2 - o1;
@@ -347,6 +353,7 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
     __bf16* c_base;
     const int32_t* row_id;  // kDown with scatter: output row of each of the tile's rows (c_base is then row 0)
     int rows, cols_left, ldc, nk;
+    int row0, col0;         // first row / column of the tile inside its group's output
   };
 
   // K steps of a tile rounded up to whole ring rounds (padding steps read zeros).  The host never launches this
@@ -370,6 +377,8 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
     }
     S.rows = G.m - row0 < BM ? G.m - row0 : BM;
     S.cols_left = G.n - col0;
+    S.row0 = row0;
+    S.col0 = col0;
     S.ldc = G.ldc;
     S.nk = padded_steps(G.k);
   };
@@ -679,6 +688,51 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
         __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, 0));  // staging is rewritten by the next round
       }
     } else {
+      if constexpr (MODE == kQkvRope) {
+        // Bias and rotary embedding on the accumulators, before they are staged.  A wavefront's 128 columns are one
+        // head; channel d of the head sits in block d / 32 at lane d % 32, so its rotation partner d +/- 64 is two
+        // blocks away in the same lane.  Evaluated like eager bf16 code: the projection (with its bias) rounded once,
+        // then q * cos + rotate_half(q) * sin with each product and the sum rounded (vl.py:771-772).
+        static_assert(FN == 4 && FM * 32 == 128, "a wavefront covers whole heads of 128 channels");
+        const int col_w = S.col0 + wn * 128;  // first output column of this wavefront's head
+        const bool live = wn * 128 < S.cols_left;
+        float bias_v[4] = {0.f, 0.f, 0.f, 0.f};
+        if (p.bias != nullptr && live) {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) bias_v[j] = static_cast<float>(p.bias[col_w + j * 32 + el32]);
+        }
+        const bool rotate = live && col_w < p.rope_cols;  // wave-uniform: q and k heads rotate, v heads do not
+#pragma unroll
+        for (int i = 0; i < FM; ++i) {
+          uint32_t cs[16][2];
+          if (rotate) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+              const int row = wm * (FM * 32) + i * 32 + 8 * (r >> 2) + 4 * elhi + (r & 3);
+              const bool in = row < S.rows;
+              const uint32_t* t = p.rope_table + static_cast<int64_t>(S.row0 + (in ? row : 0)) * 64 + el32;
+              cs[r][0] = t[0];
+              cs[r][1] = t[32];
+            }
+          }
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+#pragma unroll
+            for (int jp = 0; jp < 2; ++jp) {
+              const float lo = round_bf16(acc[i][jp][r] + bias_v[jp]);
+              const float hi = round_bf16(acc[i][jp + 2][r] + bias_v[jp + 2]);
+              if (rotate) {
+                const float c = __uint_as_float(cs[r][jp] << 16), sn = __uint_as_float(cs[r][jp] & 0xffff0000u);
+                acc[i][jp][r] = round_bf16(lo * c) - round_bf16(hi * sn);
+                acc[i][jp + 2][r] = round_bf16(hi * c) + round_bf16(lo * sn);
+              } else {
+                acc[i][jp][r] = lo;
+                acc[i][jp + 2][r] = hi;
+              }
+            }
+          }
+        }
+      }
       // wave output: 128 rows x kOutCols columns row-major, staged kRound rows at a time
       constexpr int kOutCols = FN * 32;
       constexpr int kPitch = kOutCols * 2;
@@ -995,6 +1049,39 @@ extern "C" int wx_dual_gemm(const void* in0, const void* in1, const void* w0, co
   }
   hipLaunchKernelGGL(dual_gemm_reference_layout_kernel, dim3(device_cu_count() * 4), dim3(256), 0, s, p, trans_a, trans_b);
   return check_launch("dual_gemm_reference_layout_kernel");
+}
+
+extern "C" int wx_qkv_rope_proj(const void* x, const void* weight, const void* bias, const uint32_t* rope_table,
+                                void* out, int64_t num_tokens, int64_t hidden, int n_q_heads, int n_kv_heads,
+                                int head_dim, wx_stream_t stream) {
+  const char* who = "wx_qkv_rope_proj";
+  if (n_q_heads < 0 || n_kv_heads < 0) return fail(WX_ERR_INVALID_ARGUMENT, "%s: negative head count", who);
+  if (head_dim != 128)
+    return fail(WX_ERR_UNSUPPORTED, "%s: head_dim %d; the epilogue rotates heads of 128 channels", who, head_dim);
+  const int64_t n = static_cast<int64_t>(n_q_heads + 2 * n_kv_heads) * head_dim;
+  if (int rc = check_dims(who, num_tokens, n, hidden)) return rc;
+  if (num_tokens == 0 || n == 0) return WX_OK;
+  if (hidden == 0) return fail(WX_ERR_UNSUPPORTED, "%s: hidden must be positive", who);
+  if (!x || !weight || !out || !rope_table) return fail(WX_ERR_INVALID_ARGUMENT, "%s: null pointer", who);
+  if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(weight) | reinterpret_cast<uintptr_t>(out)) & 15)
+    return fail(WX_ERR_INVALID_ARGUMENT, "%s: buffers must be 16-byte aligned", who);
+  if ((reinterpret_cast<uintptr_t>(bias) & 1) || (reinterpret_cast<uintptr_t>(rope_table) & 3))
+    return fail(WX_ERR_INVALID_ARGUMENT, "%s: misaligned bias or table", who);
+  Params p{};
+  Group& g = p.g[0];
+  g.a = static_cast<const __bf16*>(x);
+  g.b0 = static_cast<const __bf16*>(weight);
+  g.c = static_cast<__bf16*>(out);
+  g.m = static_cast<int>(num_tokens); g.n = static_cast<int>(n); g.k = static_cast<int>(hidden);
+  g.lda = g.ldb = static_cast<int>(hidden);
+  g.ldc = static_cast<int>(n);
+  p.bias = static_cast<const __bf16*>(bias);
+  p.rope_table = rope_table;
+  p.rope_cols = (n_q_heads + n_kv_heads) * head_dim;
+  // the large tile only: its wavefronts cover whole heads (the small tile's 64 columns would split a rotation pair)
+  hipLaunchKernelGGL((dual_gemm_kernel<kQkvRope, BigTile, false, false>), dim3(device_cu_count()), dim3(BigTile::kThreads),
+                     0, as_stream(stream), p);
+  return check_launch("dual_gemm_kernel<qkv_rope>");
 }
 
 extern "C" size_t wx_tiled_bytes(int64_t rows, int64_t cols) {

@@ -375,6 +375,24 @@ int launch(const void* q, const void* k, const void* cos_t, const void* sin_t, v
   }
 }
 
+// Packed rotary table for the projection kernel that rotates q and k in its epilogue: entry [token][d], d <
+// head_dim / 2, holds cos (low half) and sin (high half) of position[plane(d)] * inv_freq[d], rounded to bf16 like
+// the table builder's output (vl.py:679-712).  Channels d and d + head_dim / 2 must take the same plane, which is the
+// case for the PyTorch path's layout (vl.py:763-769) and not for the CUDA kernel's (csrc/rope.cu:104-117).
+__global__ __launch_bounds__(256) void mrope_table_kernel(const int64_t* __restrict__ pos,
+                                                          const float* __restrict__ inv_freq,
+                                                          uint32_t* __restrict__ out, int64_t n_tokens, int half,
+                                                          AxisTable ax) {
+  const int64_t gid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (gid >= n_tokens * half) return;
+  const int64_t token = gid / half;
+  const int d = static_cast<int>(gid - token * half);
+  const float pf = static_cast<float>(pos[ax.axis[d] * n_tokens + token]);
+  float sv, cv;
+  sincosf(__fmul_rn(pf, inv_freq[d]), &sv, &cv);
+  out[gid] = f32_to_bf16_bits(cv) | (f32_to_bf16_bits(sv) << 16);
+}
+
 }  // namespace
 }  // namespace wx
 
@@ -409,4 +427,29 @@ extern "C" int wx_mrope_apply_positions(const void* q, const void* k, const int6
   return wx::launch<false, true>(q, k, position_ids, inv_freq, q_out, k_out, batch, seq, n_q_heads, n_kv_heads,
                                  head_dim, q_strides, k_strides, qo_strides, ko_strides, mrope_section, layout, dtype,
                                  stream);
+}
+
+extern "C" int wx_mrope_table(const int64_t* position_ids, const float* inv_freq, int64_t batch, int64_t seq,
+                              int head_dim, const int mrope_section[3], int layout, uint32_t* table,
+                              wx_stream_t stream) {
+  using namespace wx;
+  const char* who = "wx_mrope_table";
+  if (batch < 0 || seq < 0) return fail(WX_ERR_INVALID_ARGUMENT, "%s: negative size", who);
+  if (head_dim <= 0 || head_dim % 16 != 0 || head_dim > kMaxHeadDim)
+    return fail(WX_ERR_UNSUPPORTED, "%s: head_dim %d must be a multiple of 16 and <= %d", who, head_dim, kMaxHeadDim);
+  if (!mrope_section) return fail(WX_ERR_INVALID_ARGUMENT, "%s: null section", who);
+  AxisTable ax{};
+  if (int rc = build_axis_table(mrope_section, head_dim, layout, ax)) return rc;
+  const int half = head_dim / 2;
+  for (int d = 0; d < half; ++d)
+    if (ax.axis[d] != ax.axis[d + half])
+      return fail(WX_ERR_UNSUPPORTED, "%s: channels %d and %d take different position planes in this layout; the "
+                  "packed table (and the projection that rotates in its epilogue) needs them equal", who, d, d + half);
+  const int64_t n = batch * seq * half;
+  if (n == 0) return WX_OK;
+  if (!position_ids || !inv_freq || !table) return fail(WX_ERR_INVALID_ARGUMENT, "%s: null pointer", who);
+  if ((n + 255) / 256 > 0x7fffffffll) return fail(WX_ERR_UNSUPPORTED, "%s: too many tokens", who);
+  hipLaunchKernelGGL(mrope_table_kernel, dim3(static_cast<unsigned>((n + 255) / 256)), dim3(256), 0, as_stream(stream),
+                     position_ids, inv_freq, table, batch * seq, half, ax);
+  return check_launch(who);
 }

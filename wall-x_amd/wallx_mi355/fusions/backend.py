@@ -68,6 +68,16 @@ def rope_from_positions(q, k, position_ids, inv_freq, q_out, k_out, mrope_sectio
                                       layout)
 
 
+def mrope_table(position_ids, inv_freq, mrope_section, layout: str = "hf"):
+    """No counterpart in backend.py: the packed cos/sin table the projection below reads (vl.py:679-712)."""
+    return native.mrope_table(position_ids, inv_freq, mrope_section, layout)
+
+
+def qkv_rope_proj(x, weight, bias, table, n_q_heads, n_kv_heads, head_dim=128, out=None):
+    """No counterpart in backend.py: q / k / v projections with the rotary embedding in the epilogue (vl.py:955-964)."""
+    return native.qkv_rope_proj(x, weight, bias, table, n_q_heads, n_kv_heads, head_dim, out)
+
+
 def get_rope_index(input_ids, image_grid_thw, video_grid_thw, second_per_grid_ts, attention_mask,
                    spatial_merge_size, image_token_id, video_token_id, vision_start_token_id, tokens_per_second):
     """backend.py:302-352 (forwards to the native op named rope_index)."""

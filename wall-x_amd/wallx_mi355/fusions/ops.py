@@ -297,6 +297,41 @@ def multimodal_rope_from_positions(q, k, position_ids, inv_freq, mrope_section, 
     return MultimodalRoPEFromPositions.apply(q, k, position_ids, inv_freq, mrope_section, layout)
 
 
+def multimodal_rope_table(position_ids, inv_freq, mrope_section):
+    """The packed cos/sin table `qkv_projection_with_rope` reads: build it once per forward from the position ids
+    (it replaces the [3, B, S, D] tables of Qwen2_5_VLRotaryEmbedding.forward, vl.py:679-712) and hand it to every
+    layer.  PyTorch-path channel layout (vl.py:763-769)."""
+    if position_ids.is_cpu or inv_freq.is_cpu:
+        raise RuntimeError("[Error] The inputs of multimodal_rope_table are on the device: CPU!")
+    return backend.mrope_table(position_ids, inv_freq.to(torch.float32), list(mrope_section))
+
+
+def qkv_projection_with_rope(hidden_states, qkv_weight, qkv_bias, rope_table, num_heads, num_key_value_heads,
+                             head_dim=128):
+    """Not in the reference's op set: the first lines of the attention forward (vl.py:955-964) as one launch.
+
+        q = q_proj(h).view(B, S, Hq, D).transpose(1, 2); k, v likewise; q, k = multimodal_rope(q, k, cos, sin, sec)
+
+    hidden_states [B, S, hidden] bf16; qkv_weight / qkv_bias = the q, k and v projections' weights / biases stacked
+    along the output dimension (torch.cat((q_proj.weight, k_proj.weight, v_proj.weight)), once per module);
+    rope_table from multimodal_rope_table for the same tokens.  Returns (q [B, Hq, S, D], k [B, Hkv, S, D],
+    v [B, Hkv, S, D]) as views of one [B, S, (Hq + 2 Hkv) D] buffer (token-major memory, what attention kernels
+    take through strides), q and k rotated.  Forward only (inference / prefill)."""
+    if hidden_states.is_cpu:
+        raise RuntimeError("[Error] The input `hidden_states` of qkv_projection_with_rope op is on the device: CPU!")
+    if hidden_states.dim() != 3:
+        raise RuntimeError("[Error] hidden_states must be [batch, seq, hidden]")
+    if torch.is_grad_enabled() and (hidden_states.requires_grad or qkv_weight.requires_grad):
+        raise RuntimeError("qkv_projection_with_rope has no backward: use the separate projections and multimodal_rope "
+                           "under autograd")
+    B, S, _ = hidden_states.shape
+    D, nq, nkv = head_dim, num_heads, num_key_value_heads
+    out = backend.qkv_rope_proj(hidden_states, qkv_weight, qkv_bias, rope_table, nq, nkv, D)
+    q, k, v = out.split([nq * D, nkv * D, nkv * D], dim=-1)
+    return (q.view(B, S, nq, D).transpose(1, 2), k.view(B, S, nkv, D).transpose(1, 2),
+            v.view(B, S, nkv, D).transpose(1, 2))
+
+
 # ----------------------------------------------------------------------------- index builders
 def get_rope_index(input_ids, spatial_merge_size, image_token_id, video_token_id, vision_start_token_id,
                    tokens_per_second, image_grid_thw=None, video_grid_thw=None, second_per_grid_ts=None,

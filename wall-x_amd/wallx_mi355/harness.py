@@ -16,7 +16,9 @@ batch of full sequences (prefill).  What it states explicitly:
     reader's RMSNorm (the following layer's input_layernorm, or the final norm) inside the unpermute, M-RoPE
     evaluates cos/sin from the position ids in the kernel (no [3, B, S, D] tables) and leaves q / k token-major,
     and the attention residual is added by the o-projection GEMM; `fuse=False` keeps all of these as separate
-    PyTorch ops.
+    PyTorch ops,
+  * `fuse_qkv_rope=True` replaces the vendor GEMM of the q / k / v projection and the rope kernel by one launch of
+    this library's GEMM with bias and M-RoPE in its epilogue (vl.py:955-964).
 """
 
 from contextlib import contextmanager
@@ -64,8 +66,11 @@ class PrefillHarness:
     def __init__(self, n_layers: int = 36, hidden: int = wl.HIDDEN, n_q: int = wl.N_Q_HEADS, n_kv: int = wl.N_KV_HEADS,
                  head_dim: int = wl.HEAD_DIM, inter=(wl.INTER_VL, wl.INTER_ACT), vocab: int = 151936,
                  eps: float = 1e-6, device="cuda:0", seed: int = 0, mask: str = "causal", keep_dense: bool = False,
-                 fuse: bool = True):
+                 fuse: bool = True, fuse_qkv_rope: bool = False):
         self.dev = torch.device(device)
+        # the q / k / v projection with M-RoPE in its epilogue (one launch of this library's GEMM kernel) instead of
+        # the vendor GEMM followed by the rope kernel; needs fuse=True (token-major q / k) and head_dim 128
+        self.fuse_qkv_rope = fuse_qkv_rope and fuse and head_dim == 128
         self.n_layers, self.hidden, self.n_q, self.n_kv, self.head_dim = n_layers, hidden, n_q, n_kv, head_dim
         self.inter, self.eps, self.mask_mode, self.fuse = inter, eps, mask, fuse
         g = torch.Generator(device=self.dev).manual_seed(seed)
@@ -166,6 +171,10 @@ class PrefillHarness:
             routing = moe.Routing(rmap, off, ids.numel(), inv)
         if capture is not None:
             capture["pos"] = pos
+        rope_table = None
+        if self.fuse_qkv_rope:
+            with timer.section("mrope_table"):
+                rope_table = native.mrope_table(pos, self.inv_freq, wl.MROPE_SECTION)
         attn_mask, n_tail = None, 0
         if self.mask_mode == "action_block":
             if action_suffix is not None:
@@ -184,25 +193,35 @@ class PrefillHarness:
             if x is None:
                 with timer.section("rmsnorm_torch"):
                     x = rms_norm(h, layer["ln1"], self.eps)
-            with timer.section("qkv_proj_torch"):
-                qkv = F.linear(x, layer["wqkv"], layer["bqkv"])
-                q, k, v = qkv.split([nq * D, nkv * D, nkv * D], dim=-1)
-                q = q.view(B, S, nq, D).transpose(1, 2)
-                k = k.view(B, S, nkv, D).transpose(1, 2)
-                v = v.view(B, S, nkv, D).transpose(1, 2)
-            with timer.section("mrope"):
-                if self.fuse:
-                    # rotated q / k stay token-major ([B, S, H, D] memory behind the [B, H, S, D] view the kernel
-                    # writes through strides), so attention's output comes back token-major as well and the
-                    # o projection reads it without a transposing copy
-                    qr = torch.empty(B, S, nq, D, dtype=q.dtype, device=self.dev).transpose(1, 2)
-                    kr = torch.empty(B, S, nkv, D, dtype=k.dtype, device=self.dev).transpose(1, 2)
-                    native.rope_from_positions(q, k, pos, self.inv_freq, qr, kr, [2 * s for s in wl.MROPE_SECTION])
-                else:
-                    qr, kr = ops.multimodal_rope(q, k, cos, sin, list(wl.MROPE_SECTION))
+            if self.fuse_qkv_rope:
+                with timer.section("qkv_proj+mrope"):
+                    qkv = native.qkv_rope_proj(x, layer["wqkv"], layer["bqkv"], rope_table, nq, nkv, D)
+                    q, k, v = qkv.split([nq * D, nkv * D, nkv * D], dim=-1)
+                    q = q.view(B, S, nq, D).transpose(1, 2)
+                    k = k.view(B, S, nkv, D).transpose(1, 2)
+                    v = v.view(B, S, nkv, D).transpose(1, 2)
                 if capture is not None and li in capture.get("layers", ()):
-                    capture[li] = {"q_in": q, "k_in": k, "q_out": qr, "k_out": kr}
-                q, k = qr, kr
+                    capture[li] = {"x_in": x, "q_out": q, "k_out": k, "v_out": v}
+            else:
+                with timer.section("qkv_proj_torch"):
+                    qkv = F.linear(x, layer["wqkv"], layer["bqkv"])
+                    q, k, v = qkv.split([nq * D, nkv * D, nkv * D], dim=-1)
+                    q = q.view(B, S, nq, D).transpose(1, 2)
+                    k = k.view(B, S, nkv, D).transpose(1, 2)
+                    v = v.view(B, S, nkv, D).transpose(1, 2)
+                with timer.section("mrope"):
+                    if self.fuse:
+                        # rotated q / k stay token-major ([B, S, H, D] memory behind the [B, H, S, D] view the kernel
+                        # writes through strides), so attention's output comes back token-major as well and the
+                        # o projection reads it without a transposing copy
+                        qr = torch.empty(B, S, nq, D, dtype=q.dtype, device=self.dev).transpose(1, 2)
+                        kr = torch.empty(B, S, nkv, D, dtype=k.dtype, device=self.dev).transpose(1, 2)
+                        native.rope_from_positions(q, k, pos, self.inv_freq, qr, kr, [2 * s for s in wl.MROPE_SECTION])
+                    else:
+                        qr, kr = ops.multimodal_rope(q, k, cos, sin, list(wl.MROPE_SECTION))
+                    if capture is not None and li in capture.get("layers", ()):
+                        capture[li] = {"q_in": q, "k_in": k, "q_out": qr, "k_out": kr}
+                    q, k = qr, kr
             with timer.section("sdpa_torch"):
                 if n_tail:
                     head = S - n_tail

@@ -327,6 +327,62 @@ def rope_from_positions(q, k, position_ids, inv_freq, q_out, k_out, mrope_sectio
                   _bhsd_strides(k_out), section, _layout_code(layout), _dtype_code(q), int(bool(backward)), _stream(q))
 
 
+def mrope_table(position_ids: torch.Tensor, inv_freq: torch.Tensor, mrope_section, layout: str = "hf") -> torch.Tensor:
+    """Packed rotary table for qkv_rope_proj: int32 [B * S, D / 2], entry = bf16 cos | bf16 sin << 16 of
+    position_ids[plane(d)] * inv_freq[d] (vl.py:679-712 rounded to bf16).  position_ids [3, B, S] int64, inv_freq
+    [D / 2] fp32, mrope_section the three (un-doubled) section sizes.  Only layouts whose channels d and d + D / 2
+    share a position plane ("hf")."""
+    _need_cuda("position_ids", position_ids)
+    _need_cuda("inv_freq", inv_freq)
+    if position_ids.dim() != 3 or position_ids.size(0) != 3 or position_ids.dtype != torch.int64:
+        raise RuntimeError("position_ids must be int64 [3, B, S]")
+    if inv_freq.dim() != 1 or inv_freq.dtype != torch.float32:
+        raise RuntimeError("inv_freq must be fp32 [D / 2]")
+    if len(mrope_section) != 3:
+        raise RuntimeError("mrope_section must have 3 entries")
+    _, B, S = position_ids.shape
+    half = inv_freq.numel()
+    position_ids, inv_freq = position_ids.contiguous(), inv_freq.contiguous()
+    table = torch.empty((B * S, half), dtype=torch.int32, device=position_ids.device)
+    with _DeviceGuard(position_ids):
+        _lib.call("wx_mrope_table", _ptr(position_ids), _ptr(inv_freq), B, S, 2 * half,
+                  _lib.i32x3([int(v) for v in mrope_section]), _layout_code(layout), _ptr(table), _stream(position_ids))
+    return table
+
+
+def qkv_rope_proj(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], table: torch.Tensor,
+                  n_q_heads: int, n_kv_heads: int, head_dim: int = 128, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x [..., hidden] @ weight^T + bias with M-RoPE applied to the q and k heads in the GEMM's epilogue
+    (vl.py:955-964 in one launch).  weight [(n_q + 2 n_kv) * head_dim, hidden] = q, k, v weights stacked, bias likewise
+    or None, table from mrope_table (one row per row of x).  Returns [..., (n_q + 2 n_kv) * head_dim]: columns
+    [0, n_q D) are the rotated q heads, the next n_kv D the rotated k heads, the last n_kv D the v heads."""
+    for name, t in (("x", x), ("weight", weight), ("table", table)):
+        _need_cuda(name, t)
+    if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16 or (bias is not None and bias.dtype != torch.bfloat16):
+        raise RuntimeError("All tensors must be BFloat16 for this kernel")
+    hidden = x.shape[-1]
+    n = (n_q_heads + 2 * n_kv_heads) * head_dim
+    if weight.dim() != 2 or tuple(weight.shape) != (n, hidden):
+        raise RuntimeError(f"weight must be [{n}, {hidden}] (q, k and v projection weights stacked)")
+    if bias is not None and tuple(bias.shape) != (n,):
+        raise RuntimeError(f"bias must be [{n}]")
+    x2 = x.reshape(-1, hidden)
+    if not x2.is_contiguous():
+        x2 = x2.contiguous()
+    T = x2.size(0)
+    if table.dtype != torch.int32 or tuple(table.shape) != (T, head_dim // 2):
+        raise RuntimeError(f"table must be int32 [{T}, {head_dim // 2}] (mrope_table of the same tokens)")
+    weight = weight.contiguous()
+    table = table.contiguous()
+    bias = None if bias is None else bias.contiguous()
+    if out is None or out.dtype != torch.bfloat16 or out.numel() != T * n or not out.is_contiguous() or out.device != x.device:
+        out = torch.empty((T, n), dtype=torch.bfloat16, device=x.device)
+    with _DeviceGuard(x2):
+        _lib.call("wx_qkv_rope_proj", _ptr(x2), _ptr(weight), _ptr(bias), _ptr(table), _ptr(out), T, hidden,
+                  int(n_q_heads), int(n_kv_heads), int(head_dim), _stream(x2))
+    return out.view(*x.shape[:-1], n)
+
+
 # ----------------------------------------------------------------------------- index builders
 def rope_index(input_ids, image_grid_thw, video_grid_thw, second_per_grid_ts, attention_mask,
                spatial_merge_size: int, image_token_id: int, video_token_id: int, vision_start_token_id: int,
