@@ -6,9 +6,10 @@
 // XCD inside a compact patch of the output so they share operand slabs through that XCD's L2.  A skewed pair
 // (thousands of VL rows next to tens of action rows, or an empty group) is just a longer or shorter tile list.
 //
-// Workgroup tile 256 x 256, K step 32, four wavefronts (one per SIMD) as 2 x 2, wave tile 128 x 128 = 4 x 4 MFMA
-// 32x32x16 accumulator blocks (256 accumulator registers per lane), one workgroup per CU; the gate/up launch runs
-// the same tile with eight wavefronts (2 x 4, wave tile 128 x 64).  Problems whose 256 x 256
+// Workgroup tile 256 x 256, K step 32, one workgroup per CU: eight wavefronts (two per SIMD) as 2 x 4, wave tile
+// 128 x 64 = 4 x 2 MFMA 32x32x16 accumulator blocks (128 accumulator registers per lane), of which one per SIMD
+// issues the global -> LDS loads; the projection that rotates heads in its epilogue runs the same tile with four
+// wavefronts as 2 x 2 (wave tile 128 x 128, 256 accumulator registers).  Problems whose 256 x 256
 // tiles would leave most CUs idle (a denoise step of a few thousand action tokens) run the same kernel with a
 // 128 x 128 tile, two workgroups per CU.  A ragged last round of the fused FFN launches (tiles left over after the
 // whole rounds of one tile per CU) runs in that small shape too, in a second launch, when it then fits the chip in
@@ -19,7 +20,7 @@
 // workgroup barrier per K step.  LDS rows are 64 bytes; chunk c of row r sits in slot c ^ ((r >> 2) & 3), which
 // makes the 16-byte fragment reads bank-conflict free.
 //
-// Three operand layouts:
+// Operand layouts:
 //   generic  (wx_dual_gemm)            A, B, C row-major; loads touch 16 rows x 64 bytes per instruction.  An
 //                                      operand stored with K as its slow dimension (A as [k, m], B as [k, n]: the
 //                                      backward GEMMs) is loaded as K rows of 256 columns and transposed by the LDS
@@ -29,6 +30,8 @@
 //                                      output element meet in one lane), C = K-tiled intermediate, SwiGLU epilogue.
 //   down     (wx_dual_down_proj)       A = K-tiled intermediate, B = K-tiled down weights, C row-major; with a row
 //                                      id list the rows go straight to their token positions (the unpermute).
+//   qkv+rope (wx_qkv_rope_proj)        A, B, C row-major like the generic mode, one group; bias and the rotary
+//                                      embedding of the q and k heads are applied to the accumulators.
 // With K-tiled operands every load instruction moves one contiguous KiB (tiled_layout.h).
 // Results leave through a per-wave LDS staging area so that global stores are full 16-byte lanes on contiguous
 // runs (whole 1 KiB blocks for the tiled intermediate, 256-byte row segments for row-major outputs).
@@ -50,16 +53,18 @@ constexpr int kRowBytes = BK * 2;              // 64 bytes of K per LDS row
 
 // Workgroup tile shapes.  Everything else (wave tile, loads per step, LDS footprint, resident workgroups per CU)
 // follows from the two numbers.
-template <int BM_, int BN_, int WM_, int WN_>
+// LW_: how many of the wavefronts (the first LW_) issue the global -> LDS loads; 0 = all of them.
+template <int BM_, int BN_, int WM_, int WN_, int LW_ = 0>
 struct TileShape {
   static constexpr int BM = BM_, BN = BN_;
   static constexpr int kWavesM = WM_, kWavesN = WN_;  // wavefront grid over the tile
   static constexpr int kWaves = kWavesM * kWavesN;
+  static constexpr int kLoadWaves = LW_ > 0 ? LW_ : kWaves;
   static constexpr int kThreads = kWaves * 64;
   static constexpr int FM = BM / kWavesM / 32;        // 32x32 accumulator blocks per wave along M
   static constexpr int FN = BN / kWavesN / 32;        // ... and along N
-  static constexpr int kLoadRowsA = BM / kWaves;      // LDS rows of A one wave loads per K step
-  static constexpr int kLoadRowsB = BN / kWaves;      // ... and of B
+  static constexpr int kLoadRowsA = BM / kLoadWaves;  // LDS rows of A one loading wave loads per K step
+  static constexpr int kLoadRowsB = BN / kLoadWaves;  // ... and of B
   static constexpr int kLoadsA = kLoadRowsA / 16;     // 16-row load instructions per wave per K step: A
   static constexpr int kLoadsB = kLoadRowsB / 16;     // ... and B
   static constexpr int kSlotBytesA = BM * kRowBytes;  // bytes of A per K step
@@ -72,13 +77,17 @@ struct TileShape {
 };
 // four wavefronts (one per SIMD) as 2 x 2: wave tile 128 x 128, 256 accumulator registers per lane
 using BigTile = TileShape<256, 256, 2, 2>;
-// eight wavefronts (two per SIMD) as 2 x 4: wave tile 128 x 64, 128 accumulator registers per lane.  Measures 2 %
-// faster than BigTile on the gate/up launch (the second wave fills part of the bubbles the loads and the SwiGLU
-// epilogue leave) and 1 % slower on the others (it reads 1.5 x the LDS bytes per MFMA).
-using BigTile8 = TileShape<256, 256, 2, 4>;
+// eight wavefronts (two per SIMD) as 2 x 4: wave tile 128 x 64, 128 accumulator registers per lane, and only the
+// first four (one per SIMD) issue the global -> LDS loads.  A wavefront that issues a load stalls while the CU's load
+// path takes the instruction in; here its partner on the same SIMD issues no loads and keeps the MFMA pipe fed
+// meanwhile.  Against BigTile, on the config 3 shapes: gate/up 4-7 % faster, down 3 %, the row-major op 2-6 %.
+// (With all eight loading on one schedule, both partners stall together: that form was 2 % ahead of BigTile on
+// gate/up and behind it elsewhere.)
+using BigTile8 = TileShape<256, 256, 2, 4, 4>;
 using SmallTile = TileShape<128, 128, 2, 2>;  // two workgroups per CU; for problems with too few big tiles to fill the chip
+// The large tile of a launch: BigTile8, except where the epilogue needs a wavefront to hold whole 128-column heads.
 template <int MODE>
-using BigTileFor = std::conditional_t<MODE == 1 /* kGateUp */, BigTile8, BigTile>;
+using BigTileFor = std::conditional_t<MODE == 3 /* kQkvRope */, BigTile, BigTile8>;
 // the shape that runs the ragged last round of a launch (see tail_split_point): BigTile cut in four.  (Cut in two,
 // 256 x 128 with one workgroup per CU, measures the same.)
 using TailTile = SmallTile;
@@ -234,6 +243,13 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keeps descriptors and LDS bases scalar
   const int wm = wave / kWavesN, wn = wave % kWavesN;
   const int l32 = lane & 31, lhi = lane >> 5;
+  // With more wavefronts than SIMDs only the first kLoadWaves (one per SIMD) issue the global -> LDS loads.  A
+  // wavefront that issues a load is held while the CU's load path takes the instruction in; its partner on the same
+  // SIMD, which issues none, keeps the MFMA pipe fed meanwhile.  When both partners load on the same schedule they
+  // stall together and the pipe idles.
+  constexpr int kLoadWaves = TS::kLoadWaves;
+  constexpr bool ASYM = kLoadWaves != kWaves;
+  const bool loads = !ASYM || wave < kLoadWaves;
 
   // ---- problem table (uniform) ------------------------------------------------------------------
   // (kept as two named structs, selected per tile, so everything stays in scalar registers)
@@ -387,7 +403,7 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
     const int row0 = tc.tm * BM, col0 = tc.tn * kTileN;
     L.K = G.k;
     L.nk = padded_steps(G.k);
-    constexpr int kHalfWaves = kWaves / 2;  // SwiGLU: the first half of the waves load gate rows, the rest up rows
+    constexpr int kHalfWaves = kLoadWaves / 2;  // SwiGLU: the first half of the loading waves load gate rows, the rest up rows
     const bool up_half = SWIGLU && wave >= kHalfWaves;
     const __bf16* b_src = up_half ? G.b1 : G.b0;
     const int b_wave = SWIGLU ? wave % kHalfWaves : wave;
@@ -557,29 +573,31 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
   // Scheduling hints.  Before the barrier: the LDS reads of the other fragment set and the B half of the previous
   // slot's refill go out among the first half of this group's MFMAs; the second half covers the read latency, so
   // the wait in front of the barrier finds the reads done.
-  auto schedule_before_barrier = [&]() {
+  auto schedule_before_barrier = [&](auto with_loads) {
+    constexpr int kB = decltype(with_loads)::value ? kLoadsB : 0;
     constexpr int kMfma = FM * FN, kReads = FM * (KA ? 2 : 1) + FN * (KB ? 2 : 1);
     constexpr int kCarry = kMfma / 2;                              // MFMAs that carry other instructions
     constexpr int kReadsPer = (kReads + kCarry - 1) / kCarry;      // LDS reads per carrying MFMA
-    constexpr int kLoadEvery = kCarry / kLoadsB > 0 ? kCarry / kLoadsB : 1;
+    constexpr int kLoadEvery = kB > 0 && kCarry / kB > 0 ? kCarry / kB : 1;
 #pragma unroll
     for (int m = 0; m < kCarry; ++m) {
       __builtin_amdgcn_sched_group_barrier(0x100, kReadsPer, 0);
-      if (m % kLoadEvery == 0 && m / kLoadEvery < kLoadsB) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+      if (m % kLoadEvery == 0 && m / kLoadEvery < kB) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
     }
     __builtin_amdgcn_sched_group_barrier(0x008, kMfma - kCarry, 0);
     __builtin_amdgcn_sched_barrier(0);
   };
   // After the barrier: the A half of the refill and the next slot's fragment reads are spread over the whole group.
-  auto schedule_after_barrier = [&]() {
+  auto schedule_after_barrier = [&](auto with_loads) {
+    constexpr int kA = decltype(with_loads)::value ? kLoadsA : 0;
     constexpr int kMfma = FM * FN, kReads = FM * (KA ? 2 : 1) + FN * (KB ? 2 : 1);
     constexpr int kReadEvery = kMfma / kReads > 0 ? kMfma / kReads : 1;
     constexpr int kReadsPer = kReads * kReadEvery > kMfma ? (kReads + kMfma - 1) / kMfma : 1;
-    constexpr int kLoadEvery = kMfma / kLoadsA > 0 ? kMfma / kLoadsA : 1;
+    constexpr int kLoadEvery = kA > 0 && kMfma / kA > 0 ? kMfma / kA : 1;
 #pragma unroll
     for (int m = 0; m < kMfma; ++m) {
-      if (m % kLoadEvery == 0 && m / kLoadEvery < kLoadsA) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+      if (m % kLoadEvery == 0 && m / kLoadEvery < kA) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
       if (m % kReadEvery == 0 && m / kReadEvery * kReadsPer < kReads) __builtin_amdgcn_sched_group_barrier(0x100, kReadsPer, 0);
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
     }
@@ -590,23 +608,25 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
   // fragment set 0 holds kk = 0 of this slot.  After the barrier every wave has finished reading this slot, so its
   // refill with the K step kStages ahead in the load stream (step `ld_ks` of tile `L`) starts at once: the A half
   // here, the B half in the next step's first group.  The next slot's data was issued kStages - 1 steps ago.
+  // A wavefront that does not load runs the same step without the load instructions (and its counted wait passes
+  // at once: it has no loads in flight).
   Pending pend;
-  auto k_step = [&](Loader& L, int ld_ks, unsigned char* sa, unsigned char* sb, unsigned char* sa_n,
-                    unsigned char* sb_n, unsigned char* sb_p) {
+  auto k_step_as = [&](auto with_loads, Loader& L, int ld_ks, unsigned char* sa, unsigned char* sb, unsigned char* sa_n,
+                       unsigned char* sb_n, unsigned char* sb_p) {
+    constexpr bool LD = decltype(with_loads)::value;
     read_frags(sa, sb, 1, 1);
-    issue_b(pend, sb_p);
+    if constexpr (LD) issue_b(pend, sb_p);
     mma(0);
-    schedule_before_barrier();
+    schedule_before_barrier(with_loads);
     // my LDS reads have returned; of my loads at most the kStages - 2 youngest K steps' worth are still in flight,
     // i.e. the next slot is complete
-    __builtin_amdgcn_s_waitcnt(waitcnt_imm((kStages - 2) * kLoadsPerStep, 0));
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(LD ? (kStages - 2) * kLoadsPerStep : 63, 0));
     barrier_no_fence();
-    issue_a(L, ld_ks, sa, pend);
+    if constexpr (LD) issue_a(L, ld_ks, sa, pend);
     read_frags(sa_n, sb_n, 0, 0);
     mma(1);
-    schedule_after_barrier();
+    schedule_after_barrier(with_loads);
   };
-
   // ---- epilogue ------------------------------------------------------------------------------------------
   // Accumulator register r of lane l holds row 8*(r/4) + 4*(l/32) + r%4, column l%32 of its 32x32 block.  Values
   // are rounded to bf16, paired with the neighbouring column through a lane swap (even lanes keep the even
@@ -808,50 +828,63 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
   TileCoord tc;
   bool have = next_tile(tc);
   if (!have) return;
-  Loader L;
-  Store S;
-  setup_loader(tc, L);
-  setup_store(tc, S);
+  // The whole tile loop exists in two forms, with and without the load instructions; a wavefront picks its form
+  // once (all of them the first, unless only some wavefronts load).
+  auto run = [&](auto with_loads) {
+    constexpr bool LD = decltype(with_loads)::value;
+    Loader L;
+    Store S;
+    if constexpr (LD) setup_loader(tc, L);
+    setup_store(tc, S);
+    if constexpr (LD) {
 #pragma unroll
-  for (int s = 0; s < kStages; ++s) {
-    issue_a(L, s, slot_a(s), pend);
-    if (s + 1 < kStages) issue_b(pend, slot_b(s));  // the last slot's B half goes out in the first K step
-  }
-  // slot 0 must be complete before its first fragments are read: the younger loads may remain in flight
-  __builtin_amdgcn_s_waitcnt(waitcnt_imm((kStages - 2) * kLoadsPerStep + kLoadsA, 15));
-  __syncthreads();
-  read_frags(s_a0, s_b0, 0, 0);
-
-  while (have) {
-#pragma unroll
-    for (int i = 0; i < FM; ++i)
-#pragma unroll
-      for (int j = 0; j < FN; ++j)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-
-    const Store done = S;
-    const int nk = S.nk;
-    for (int ks = 0; ks < nk; ks += kStages) {
-      int ld_ks = ks + kStages;
-      if (ld_ks == nk) {  // the loader moves on to the next tile (or to the empty descriptor)
-        have = next_tile(tc);
-        if (have) {
-          setup_loader(tc, L);
-          setup_store(tc, S);
-        } else {
-          L.a_bytes = L.a_left = 0;
-          L.b_bytes = L.b_left = 0;
-          L.K = 0;
-        }
-        ld_ks = 0;
+      for (int s = 0; s < kStages; ++s) {
+        issue_a(L, s, slot_a(s), pend);
+        if (s + 1 < kStages) issue_b(pend, slot_b(s));  // the last slot's B half goes out in the first K step
       }
-#pragma unroll
-      for (int s = 0; s < kStages; ++s)
-        k_step(L, ld_ks + s, slot_a(s), slot_b(s), slot_a((s + 1) % kStages), slot_b((s + 1) % kStages),
-               slot_b((s + kStages - 1) % kStages));
+      // slot 0 must be complete before its first fragments are read: the younger loads may remain in flight
+      __builtin_amdgcn_s_waitcnt(waitcnt_imm((kStages - 2) * kLoadsPerStep + kLoadsA, 15));
     }
-    epilogue(done);
+    __syncthreads();
+    read_frags(s_a0, s_b0, 0, 0);
+
+    while (have) {
+#pragma unroll
+      for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+      const Store done = S;
+      const int nk = S.nk;
+      for (int ks = 0; ks < nk; ks += kStages) {
+        int ld_ks = ks + kStages;
+        if (ld_ks == nk) {  // the loader moves on to the next tile (or to the empty descriptor)
+          have = next_tile(tc);
+          if (have) {
+            if constexpr (LD) setup_loader(tc, L);
+            setup_store(tc, S);
+          } else if constexpr (LD) {
+            L.a_bytes = L.a_left = 0;
+            L.b_bytes = L.b_left = 0;
+            L.K = 0;
+          }
+          ld_ks = 0;
+        }
+#pragma unroll
+        for (int s = 0; s < kStages; ++s)
+          k_step_as(with_loads, L, ld_ks + s, slot_a(s), slot_b(s), slot_a((s + 1) % kStages), slot_b((s + 1) % kStages),
+                    slot_b((s + kStages - 1) % kStages));
+      }
+      epilogue(done);
+    }
+  };
+  if constexpr (!ASYM) {
+    run(std::true_type{});
+  } else {
+    if (loads) run(std::true_type{});
+    else run(std::false_type{});
   }
 #endif
 }
