@@ -120,9 +120,9 @@ def main():
 
     row_id_map, offsets, inverse, ws = native.partition(types, 2, 0, ws, want_sorted=True)
 
-    def partition():
-        nonlocal row_id_map, offsets, inverse, ws
-        row_id_map, offsets, inverse, ws = native.partition(types, 2, 0, ws, want_sorted=True)
+    def partition():  # straight through the C ABI into the buffers above, like the other launches of a step
+        _lib.call("wx_partition_build", types.data_ptr(), _lib.WX_U8, T, 1, 2, 0, row_id_map.data_ptr(),
+                  inverse.data_ptr(), offsets.data_ptr(), ws[1].data_ptr(), ws[0].data_ptr(), ws[0].numel(), stream)
 
     def permute():  # the layer's permute: rows go straight into the K-tiled activation matrix
         _lib.call("wx_permute_rows_tiled", x.data_ptr(), x_tiled.data_ptr(), row_id_map.data_ptr(),
@@ -247,7 +247,9 @@ def main():
         side("ceilings", ceiling_measurements, dev, x, weights, m0)
     if not args.ops_only and not args.no_prefill:
         del x_tiled, hmid, x_sorted, y_sorted, y
-        side("prefill", prefill_measurement, dev, args.prefill_mask)
+        side("prefill", prefill_measurement, dev, args.prefill_mask, False)
+        # the same forward with the q / k / v projection and M-RoPE as one launch of this library's GEMM
+        side("prefill_qkv_rope_in_gemm_epilogue", prefill_measurement, dev, args.prefill_mask, True)
 
     traffic, traffic_source = measured_traffic("gate_up")
     result = {
@@ -426,6 +428,14 @@ def config4_measurement(dev, weights):
     I0, I1 = weights[0][0].shape[0], weights[1][0].shape[0]
     g = torch.Generator(device=dev).manual_seed(4)
     out = {}
+    from types import SimpleNamespace
+    cfg = SimpleNamespace(experts=[dict(hidden_size=H, intermediate_size=i, hidden_act="silu") for i in (I0, I1)])
+    block = moe.SparseMoeBlock(cfg, 2).to(dev).to(torch.bfloat16)
+    with torch.no_grad():
+        for e, ws in enumerate(weights):
+            for prm, w in zip(block.experts[e].weights(), ws):
+                prm.copy_(w)
+    block.pack_for_inference(free_dense=True)
     cases = [("denoise_2048_action", 0, 2048)] + [(f"prefill_4096_vl_plus_{n}_action", 4096, n) for n in (0, 1, 8, 32, 64)]
     for name, n_vl, n_act in cases:
         T = n_vl + n_act
@@ -437,6 +447,13 @@ def config4_measurement(dev, weights):
         flops = 6.0 * H * (n_vl * I0 + n_act * I1)
         out[name] = {"us": round(t * 1e3, 1), "tflops": round(flops / t / 1e9, 1),
                      "us_with_host_row_counts": round(th * 1e3, 1)}
+        # the drop-in module called the way the reference's decoder calls it: every layer gets the same token-type
+        # tensor and the CPU row ranges (act.py:257-261, 1274-1283), so the partition is shared between the layers
+        x3, types2 = x.view(1, T, H), types.view(1, T)
+        start, end = torch.tensor([0, n_vl]), torch.tensor([n_vl, T])
+        with torch.no_grad():
+            tb, _ = event_ms(lambda: block(x3, types2, start, end), 20, warm=5)
+        out[name]["us_drop_in_block_same_token_types"] = round(tb * 1e3, 1)
         if n_vl == 0:
             # the denoise loop repeats this shape 10 x 36 times per action chunk: record 36 layers once into a HIP
             # graph (the entry points neither allocate nor synchronise) and time its replays
@@ -582,13 +599,14 @@ def ceiling_measurements(dev, x, weights, m0):
     return out
 
 
-def prefill_measurement(dev, mask):
+def prefill_measurement(dev, mask, fuse_qkv_rope=False):
     """BASELINE config 5: one prefill of 16 x 912 tokens through a randomly initialised 36-layer decoder of the
     Qwen2.5-VL-3B shape with the dual-expert FFN in every layer; attention, projections and norms on PyTorch."""
     import torch
     from wallx_mi355 import harness
 
-    model = harness.PrefillHarness(device=dev, mask="causal" if mask == "causal" else "action_block")
+    model = harness.PrefillHarness(device=dev, mask="causal" if mask == "causal" else "action_block",
+                                   fuse_qkv_rope=fuse_qkv_rope)
     ids, grid, types = harness.config5_inputs(16, dev)
     suffix = 32 if mask == "action_block" else None  # config 5: the 32 action tokens close every row
     if suffix is not None and not (bool(types[:, -suffix:].all()) and not bool(types[:, :-suffix].any())):
@@ -606,7 +624,11 @@ def prefill_measurement(dev, mask):
     model.forward(ids, grid, types, timer, action_suffix=suffix)
     split = timer.report_ms()
     total = sum(split.values())
+    del model
+    torch.cuda.empty_cache()
     return {
+        "qkv_projection": "this library's GEMM with bias and M-RoPE in its epilogue (wx_qkv_rope_proj)" if fuse_qkv_rope
+                          else "vendor GEMM (F.linear), then the M-RoPE kernel",
         "workload": "config 5 (BASELINE.json configs[4]): 36 layers, hidden 2048, 16 q / 2 kv heads x 128, experts "
                     "11008 / 1024, 16 x 912 tokens (32 action each), bf16, random init, rms eps 1e-6, mask " +
                     {"action_block": "causal + bidirectional action block (act.py:616-637) as two maskless attention calls",

@@ -84,7 +84,11 @@ using BigTile = TileShape<256, 256, 2, 2>;
 // (With all eight loading on one schedule, both partners stall together: that form was 2 % ahead of BigTile on
 // gate/up and behind it elsewhere.)
 using BigTile8 = TileShape<256, 256, 2, 4, 4>;
-using SmallTile = TileShape<128, 128, 2, 2>;  // two workgroups per CU; for problems with too few big tiles to fill the chip
+// The small tile, for problems with too few large tiles to fill the chip: two workgroups per CU, each eight
+// wavefronts as 4 x 2 (wave tile 32 x 64), four of them loading, like the large tile.  (Four wavefronts of 64 x 64
+// measure 6 % slower on a denoise step; timestamps inside that kernel put 254 ns on a K step whose 8 MFMAs per
+// wavefront need 110, and 169 ns with the loads taken out.)
+using SmallTile = TileShape<128, 128, 4, 2, 4>;
 // The large tile of a launch: BigTile8, except where the epilogue needs a wavefront to hold whole 128-column heads.
 template <int MODE>
 using BigTileFor = std::conditional_t<MODE == 3 /* kQkvRope */, BigTile, BigTile8>;
