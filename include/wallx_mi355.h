@@ -160,6 +160,15 @@ int wx_dual_down_proj(const void* hmid, void* out, const int32_t* expert_offsets
                       const void* down1, int64_t num_rows, int64_t hidden, int64_t inter0,
                       int64_t inter1, const int64_t* host_rows_per_expert, const int32_t* out_row_id,
                       wx_stream_t stream);
+/* wx_dual_swiglu_gate_up for a forward pass whose backward will follow: besides hmid it stores the two projections
+ * themselves (rounded to bf16, before the SwiGLU) into gate_keep / up_keep, K-tiled buffers of hmid's size and
+ * geometry, so that the backward does not run the two projections again.  The reference keeps these activations
+ * through autograd (act.py:79-82 under torch.autograd saves gate, up, act_fn(gate) and the product). */
+int wx_dual_swiglu_gate_up_keep(const void* x_tiled, void* hmid, void* gate_keep, void* up_keep,
+                                const int32_t* expert_offsets, const void* gate0, const void* up0,
+                                const void* gate1, const void* up1, int64_t num_rows, int64_t hidden,
+                                int64_t inter0, int64_t inter1, const int64_t* host_rows_per_expert,
+                                wx_stream_t stream);
 /* out_row_id (optional, may be NULL): DEVICE int32[num_rows], the partition's sorted_row_id (sorted position ->
  * token).  When given, the down launch stores sorted row r of the result at row out_row_id[r] of `out`, i.e. `out`
  * comes back in token order and the separate unpermute (ops.unpermute at topK 1, act.py:157-161) is not needed:
@@ -297,6 +306,11 @@ int wx_unpermute_rows_add_rmsnorm(const void* y, const void* residual, void* out
  * with s = sigmoid(g), dup = dh * silu(g).  bf16 in and out, fp32 math; num_elems a multiple of 8. */
 int wx_swiglu_bwd(const void* gate, const void* up, const void* dh, void* hmid, void* dgate, void* dup,
                   int64_t num_elems, wx_stream_t stream);
+/* The same with gate and up of ONE expert read from the K-tiled buffers wx_dual_swiglu_gate_up_keep filled:
+ * gate_tiled / up_tiled point at that expert's tiled matrix of tiled_rows rows (its row count rounded up to 256) and
+ * cols columns; dh and the three outputs are row-major [rows, cols].  cols a multiple of 64. */
+int wx_swiglu_bwd_tiled(const void* gate_tiled, const void* up_tiled, int64_t tiled_rows, const void* dh, void* hmid,
+                        void* dgate, void* dup, int64_t rows, int64_t cols, wx_stream_t stream);
 
 #ifdef __cplusplus
 }

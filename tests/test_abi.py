@@ -77,6 +77,15 @@ def test_argument_errors_without_a_gpu():
     assert lib.wx_swiglu_bwd(None, None, None, None, None, None, 12, None) == -2  # count % 8
     assert lib.wx_swiglu_bwd(None, None, None, None, None, None, 16, None) == -1
     assert lib.wx_swiglu_bwd(None, None, None, None, None, None, 0, None) == 0
+    assert lib.wx_swiglu_bwd_tiled(None, None, 256, None, None, None, None, 16, 96, None) == -2  # cols % 64
+    assert lib.wx_swiglu_bwd_tiled(None, None, 8, None, None, None, None, 16, 64, None) == -1    # tiled_rows < rows
+    assert lib.wx_swiglu_bwd_tiled(None, None, 256, None, None, None, None, 16, 64, None) == -1  # null pointers
+    assert lib.wx_dual_swiglu_gate_up_keep(*([None] * 9), 4, 64, 64, 64, None, None) == -1
+    assert lib.wx_qkv_rope_proj(None, None, None, None, None, 4, 64, 1, 1, 96, None) == -2
+    assert b"head_dim" in lib.wx_last_error_string()
+    assert lib.wx_qkv_rope_proj(None, None, None, None, None, 4, 64, 1, 1, 128, None) == -1
+    assert lib.wx_mrope_table(None, None, 1, 4, 128, _lib.i32x3((16, 24, 24)), _lib.WX_MROPE_CSRC, None, None) == -2
+    assert b"different position planes" in lib.wx_last_error_string()
     # M-RoPE from positions: shapes the row kernel cannot take are refused, not routed elsewhere
     st = _lib.i64x3((128 * 4, 128, 128 * 4))
     assert lib.wx_mrope_apply_positions(None, None, None, None, None, None, 1, 4, 2, 1, 128, st, st, st, st,

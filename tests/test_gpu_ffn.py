@@ -503,21 +503,24 @@ def test_swiglu_bwd_kernel(dev, shape):
 
 
 @pytest.mark.parametrize("fused_extras", [False, True])
-def test_moe_block_backward_matches_autograd_of_the_plain_forward(dev, fused_extras):
+@pytest.mark.parametrize("n_tok,inters", [(203, (256, 64)), (700, (192, 96)), (700, (320, 128))])
+def test_moe_block_backward_matches_autograd_of_the_plain_forward(dev, fused_extras, n_tok, inters):
     """Gradients of the block (inputs and all six weights) against torch autograd through the oracle's fp32
-    forward; with fused_extras the layer's RMSNorm and residual ride along (PyTorch ops under autograd)."""
+    forward; with fused_extras the layer's RMSNorm and residual ride along (PyTorch ops under autograd).
+    Intermediate sizes that are multiples of 64 take the path that keeps the gate / up projections of the forward
+    (one and several 256-row tiles per expert); (192, 96) takes the one that recomputes them."""
     class Cfg:
-        experts = [{"hidden_size": 128, "intermediate_size": 256, "hidden_act": "silu"},
-                   {"hidden_size": 128, "intermediate_size": 64, "hidden_act": "silu"}]
+        experts = [{"hidden_size": 128, "intermediate_size": inters[0], "hidden_act": "silu"},
+                   {"hidden_size": 128, "intermediate_size": inters[1], "hidden_act": "silu"}]
 
     g = torch.Generator().manual_seed(12)
     block = moe.SparseMoeBlock(Cfg(), 2).to(torch.bfloat16)
     with torch.no_grad():
         for prm in block.parameters():
             prm.copy_(_bf(prm.shape, g, 0.08))
-    x = _bf((1, 203, 128), g)
-    types = torch.rand(1, 203, generator=g) > 0.7
-    dy = _bf((1, 203, 128), g)
+    x = _bf((1, n_tok, 128), g)
+    types = torch.rand(1, n_tok, generator=g) > 0.6
+    dy = _bf((1, n_tok, 128), g)
     nw = (1.0 + 0.1 * torch.randn(128, generator=g)).to(torch.bfloat16)
     # reference: fp32 leaves, oracle forward, torch autograd
     xr = x.float().requires_grad_(True)

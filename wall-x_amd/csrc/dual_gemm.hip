@@ -132,6 +132,10 @@ struct Params {
   const __bf16* bias;
   const uint32_t* rope_table;
   int rope_cols;
+  // kGateUp only (training): when set, the two projections themselves (rounded to bf16, before the SwiGLU) are
+  // stored as well, K-tiled with the geometry of the intermediate, so that a backward pass need not recompute them.
+  __bf16* keep_gate;
+  __bf16* keep_up;
 };
 
 #define LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
@@ -663,53 +667,63 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
       constexpr int kRound = kStageBytes / kPitch;  // rows per round (64 / 32)
       constexpr int kIPerRound = kRound / 32;       // 32-row accumulator blocks per round
       static_assert(kIPerRound >= 1 && FM % kIPerRound == 0, "staging holds whole accumulator blocks");
+      // what == 0: the intermediate h; 1 / 2: the gate / up projections themselves, when the caller keeps them
+      const int n_what = p.keep_gate != nullptr ? 3 : 1;
+      const int64_t keep_off[3] = {0, reinterpret_cast<unsigned char*>(p.keep_gate) - reinterpret_cast<unsigned char*>(p.g[0].c),
+                                   reinterpret_cast<unsigned char*>(p.keep_up) - reinterpret_cast<unsigned char*>(p.g[0].c)};
 #pragma unroll
       for (int round = 0; round < FM / kIPerRound; ++round) {
+        for (int what = 0; what < n_what; ++what) {
 #pragma unroll
-        for (int ii = 0; ii < kIPerRound; ++ii) {
-          const int i = round * kIPerRound + ii;
+          for (int ii = 0; ii < kIPerRound; ++ii) {
+            const int i = round * kIPerRound + ii;
 #pragma unroll
-          for (int j = 0; j < FN / 2; ++j) {
+            for (int j = 0; j < FN / 2; ++j) {
 #pragma unroll
-            for (int r = 0; r < 16; r += 2) {
-              float h[2];
+              for (int r = 0; r < 16; r += 2) {
+                float h[2];
 #pragma unroll
-              for (int q = 0; q < 2; ++q) {
-                // eager bf16 evaluation of act_fn(gate) * up (act.py:80-82): gate, up, silu(gate) and the
-                // product are each rounded to bf16
-                const uint32_t gu = pack_bf16x2(acc[i][j][r + q], acc[i][j + FN / 2][r + q]);  // one convert for both
-                const float g = __uint_as_float(gu << 16);
-                const float u = __uint_as_float(gu & 0xffff0000u);
-                const float sg = round_bf16(g * __builtin_amdgcn_rcpf(1.0f + __expf(-g)));
-                h[q] = sg * u;
+                for (int q = 0; q < 2; ++q) {
+                  // eager bf16 evaluation of act_fn(gate) * up (act.py:80-82): gate, up, silu(gate) and the
+                  // product are each rounded to bf16
+                  const uint32_t gu = pack_bf16x2(acc[i][j][r + q], acc[i][j + FN / 2][r + q]);  // one convert for both
+                  const float g = __uint_as_float(gu << 16);
+                  const float u = __uint_as_float(gu & 0xffff0000u);
+                  if (what == 0) {
+                    const float sg = round_bf16(g * __builtin_amdgcn_rcpf(1.0f + __expf(-g)));
+                    h[q] = sg * u;
+                  } else {
+                    h[q] = what == 1 ? g : u;
+                  }
+                }
+                const int srow = ii * 32 + 8 * (r >> 2) + 4 * elhi + (r & 3);
+                stage_pair(h[0], h[1], srow, j * 32 + el32, kPitch, odd);
               }
-              const int srow = ii * 32 + 8 * (r >> 2) + 4 * elhi + (r & 3);
-              stage_pair(h[0], h[1], srow, j * 32 + el32, kPitch, odd);
             }
           }
-        }
-        __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, 0));
-        // kRound rows x kOutCols columns = (kRound / 16) row blocks x (kOutCols / 32) column blocks of the tiled
-        // intermediate, 1 KiB each; one store instruction per block: lane -> (row lane/4, slot lane%4) holding
-        // chunk slot ^ ((row >> 2) & 3)
-        const int r16 = lane_e >> 2, slot = lane_e & 3, chunk = slot ^ ((r16 >> 2) & 3);
+          __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, 0));
+          // kRound rows x kOutCols columns = (kRound / 16) row blocks x (kOutCols / 32) column blocks of the tiled
+          // intermediate, 1 KiB each; one store instruction per block: lane -> (row lane/4, slot lane%4) holding
+          // chunk slot ^ ((row >> 2) & 3)
+          const int r16 = lane_e >> 2, slot = lane_e & 3, chunk = slot ^ ((r16 >> 2) & 3);
 #pragma unroll
-        for (int rbl = 0; rbl < kRound / 16; ++rbl) {
+          for (int rbl = 0; rbl < kRound / 16; ++rbl) {
 #pragma unroll
-          for (int kbl = 0; kbl < kOutCols / 32; ++kbl) {
-            const u32x4 v =
-                *reinterpret_cast<const u32x4*>(stage + (rbl * 16 + r16) * kPitch + (kbl * 32 + chunk * 8) * 2);
-            const int row = wm * (FM * 32) + round * kRound + rbl * 16;  // first row of the block inside the tile
-            const int col = wn * kOutCols + kbl * 32;                     // first column of the block inside the tile
-            // rows past the expert's last row are padding of the tiled matrix: harmless to write, never read
-            if (col < S.cols_left) {
-              unsigned char* dst = reinterpret_cast<unsigned char*>(S.c_base) +
-                                   ((static_cast<int64_t>(col / kBlkCols) * S.ldc + row / kBlkRows) << 10);
-              *reinterpret_cast<u32x4*>(dst + lane_e * 16) = v;
+            for (int kbl = 0; kbl < kOutCols / 32; ++kbl) {
+              const u32x4 v =
+                  *reinterpret_cast<const u32x4*>(stage + (rbl * 16 + r16) * kPitch + (kbl * 32 + chunk * 8) * 2);
+              const int row = wm * (FM * 32) + round * kRound + rbl * 16;  // first row of the block inside the tile
+              const int col = wn * kOutCols + kbl * 32;                     // first column of the block inside the tile
+              // rows past the expert's last row are padding of the tiled matrix: harmless to write, never read
+              if (col < S.cols_left) {
+                unsigned char* dst = reinterpret_cast<unsigned char*>(S.c_base) + keep_off[what] +
+                                     ((static_cast<int64_t>(col / kBlkCols) * S.ldc + row / kBlkRows) << 10);
+                *reinterpret_cast<u32x4*>(dst + lane_e * 16) = v;
+              }
             }
           }
+          __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, 0));  // staging is rewritten by the next round
         }
-        __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, 0));  // staging is rewritten by the next round
       }
     } else {
       if constexpr (MODE == kQkvRope) {
@@ -1153,6 +1167,7 @@ struct FfnArgs {
   const int32_t* offsets;
   int64_t rows, hidden, inter[2];
   const int32_t* out_row_id = nullptr;  // optional: sorted row r of the result goes to row out_row_id[r] of `out`
+  void *keep_gate = nullptr, *keep_up = nullptr;  // optional: the gate / up projections, K-tiled like hmid
 };
 
 int check_ffn(const char* who, const FfnArgs& a, bool need_gate_up, bool need_down) {
@@ -1194,6 +1209,8 @@ int launch_gate_up(const FfnArgs& a, hipStream_t s) {
     g.a_row0 = 0;
   }
   p.offsets = a.offsets;
+  p.keep_gate = static_cast<__bf16*>(a.keep_gate);
+  p.keep_up = static_cast<__bf16*>(a.keep_up);
   const int64_t t0 = ceil_div(a.inter[0], BigTile::BN / 2), t1 = ceil_div(a.inter[1], BigTile::BN / 2);
   if (a.host_rows != nullptr) {  // the caller knows the split: one launch of the right tile shape
     const int64_t by_expert[2] = {ceil_div(a.host_rows[0], BigTile::BM) * t0, ceil_div(a.host_rows[1], BigTile::BM) * t1};
@@ -1243,6 +1260,23 @@ extern "C" int wx_dual_swiglu_gate_up(const void* x_tiled, void* hmid, const int
                   num_rows, hidden, {inter0, inter1}};
   if (int rc = check_ffn("wx_dual_swiglu_gate_up", a, true, false)) return rc;
   if (num_rows == 0) return WX_OK;
+  return launch_gate_up(a, as_stream(stream));
+}
+
+extern "C" int wx_dual_swiglu_gate_up_keep(const void* x_tiled, void* hmid, void* gate_keep, void* up_keep,
+                                           const int32_t* expert_offsets, const void* gate0, const void* up0,
+                                           const void* gate1, const void* up1, int64_t num_rows, int64_t hidden,
+                                           int64_t inter0, int64_t inter1, const int64_t* host_rows_per_expert,
+                                           wx_stream_t stream) {
+  FfnArgs a{x_tiled, {gate0, gate1}, {up0, up1}, {nullptr, nullptr}, nullptr, hmid, host_rows_per_expert, expert_offsets,
+            num_rows, hidden, {inter0, inter1}};
+  if (int rc = check_ffn("wx_dual_swiglu_gate_up_keep", a, true, false)) return rc;
+  if (num_rows == 0) return WX_OK;
+  if (!gate_keep || !up_keep) return fail(WX_ERR_INVALID_ARGUMENT, "wx_dual_swiglu_gate_up_keep: null pointer");
+  if ((reinterpret_cast<uintptr_t>(gate_keep) | reinterpret_cast<uintptr_t>(up_keep)) & 15)
+    return fail(WX_ERR_INVALID_ARGUMENT, "wx_dual_swiglu_gate_up_keep: buffers must be 16-byte aligned");
+  a.keep_gate = gate_keep;
+  a.keep_up = up_keep;
   return launch_gate_up(a, as_stream(stream));
 }
 

@@ -36,6 +36,7 @@ PROTOTYPES = {
     "wx_permute_rows_tiled": (_i32, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _vp]),
     "wx_dual_swiglu_ffn": (_i32, [_vp] * 10 + [_i64] * 4 + [_vp, _vp, _vp]),
     "wx_dual_swiglu_gate_up": (_i32, [_vp] * 7 + [_i64] * 4 + [_vp, _vp]),
+    "wx_dual_swiglu_gate_up_keep": (_i32, [_vp] * 9 + [_i64] * 4 + [_vp, _vp]),
     "wx_dual_down_proj": (_i32, [_vp] * 5 + [_i64] * 4 + [_vp, _vp, _vp]),
     "wx_mrope_apply": (_i32, [_vp] * 6 + [_i64, _i64, _i32, _i32, _i32] + [_c.POINTER(_i64)] * 4
                        + [_c.POINTER(_i32), _i32, _i32, _vp]),
@@ -54,6 +55,7 @@ PROTOTYPES = {
     "wx_unpermute_rows_add": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _vp]),
     "wx_unpermute_rows_add_rmsnorm": (_i32, [_vp, _vp, _vp, _vp, _vp, _f32, _vp, _i64, _i64, _vp]),
     "wx_swiglu_bwd": (_i32, [_vp] * 6 + [_i64, _vp]),
+    "wx_swiglu_bwd_tiled": (_i32, [_vp, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _vp]),
 }
 
 _lock = threading.Lock()

@@ -108,10 +108,12 @@ def _dual(a0, a1, w0, w1, n0, n1, trans_a, trans_b):
 class _MoeBlockFunction(torch.autograd.Function):
     """permute -> both experts' SwiGLU FFN -> unpermute with a backward (act.py:105-162 under autograd).
 
-    Forward is the fused path.  Backward recomputes gate and up (they are not kept by the fused kernels) and runs
-    every contraction of both experts as one dual GEMM: dHm = dY Wd, dWd = dY^T Hm, dX = dG Wg + dU Wu,
-    dWg = dG^T X, dWu = dU^T X, with the SwiGLU derivative in one fused elementwise kernel (fp32 math).  The per-expert row counts are
-    read back from the device once per backward (the forward never synchronises)."""
+    Forward is the fused path; its gate / up launch also keeps the two projections (the reference's autograd keeps
+    them too, along with act_fn(gate) and the product, act.py:79-82).  Backward runs every remaining contraction of
+    both experts as one dual GEMM each: dHm = dY Wd, dWd = dY^T Hm, dX = dG Wg + dU Wu, dWg = dG^T X, dWu = dU^T X,
+    with the SwiGLU derivative (and Hm in row-major form) from one fused elementwise kernel per expert (fp32 math).
+    Intermediate sizes that are not multiples of 64 recompute the two projections instead.  The per-expert row
+    counts are read back from the device once per backward (the forward never synchronises)."""
 
     @staticmethod
     def forward(ctx, x, row_id_map, expert_offsets, sorted_row_id, scratch, *weights):
@@ -119,9 +121,18 @@ class _MoeBlockFunction(torch.autograd.Function):
         scratch["x_tiled"] = native.permute_rows_tiled(x, row_id_map, expert_offsets, scratch.get("x_tiled"),
                                                        sorted_row_id)
         w = ((weights[0], weights[1], weights[2]), (weights[3], weights[4], weights[5]))
-        ctx.save_for_backward(x, row_id_map, expert_offsets, *weights)
+        I0, I1 = weights[0].size(0), weights[3].size(0)
+        ctx.keep = I0 % 64 == 0 and I1 % 64 == 0
         # weights that train are repacked on every forward: writes through `.data` (master-weight or EMA copies) do
         # not move the version counter a cached copy would be checked against
+        if ctx.keep:
+            y, gate_keep, up_keep, scratch["hmid"] = native.dual_swiglu_ffn_keep(
+                scratch["x_tiled"], T, expert_offsets, w, hmid=scratch.get("hmid"), out_row_id=sorted_row_id)
+            if sorted_row_id is None:
+                y = native.unpermute(y, row_id_map, torch.tensor([]), T, 1)
+            ctx.save_for_backward(x, row_id_map, expert_offsets, gate_keep, up_keep, *weights)
+            return y
+        ctx.save_for_backward(x, row_id_map, expert_offsets, *weights)
         if sorted_row_id is not None:
             return native.dual_swiglu_ffn(scratch["x_tiled"], T, expert_offsets, w, hmid=scratch.get("hmid"),
                                           out_row_id=sorted_row_id, cache_packed=False)
@@ -131,7 +142,10 @@ class _MoeBlockFunction(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, dy):
-        x, row_id_map, expert_offsets, g0, u0, d0, g1, u1, d1 = ctx.saved_tensors
+        if ctx.keep:
+            x, row_id_map, expert_offsets, gate_keep, up_keep, g0, u0, d0, g1, u1, d1 = ctx.saved_tensors
+        else:
+            x, row_id_map, expert_offsets, g0, u0, d0, g1, u1, d1 = ctx.saved_tensors
         T, H = x.shape
         o = expert_offsets.cpu().tolist()
         m0, m1 = o[1] - o[0], o[2] - o[1]
@@ -140,12 +154,17 @@ class _MoeBlockFunction(torch.autograd.Function):
         x0, x1 = xs[:m0], xs[m0:m0 + m1]
         dy0, dy1 = dys[:m0], dys[m0:m0 + m1]
         I0, I1 = g0.size(0), g1.size(0)
-        ga0, ga1 = _dual(x0, x1, g0, g1, I0, I1, False, True)
-        up0, up1 = _dual(x0, x1, u0, u1, I0, I1, False, True)
         dh0, dh1 = _dual(dy0, dy1, d0, d1, I0, I1, False, False)
-
-        hm0, dg0, du0 = native.swiglu_bwd(ga0, up0, dh0)
-        hm1, dg1, du1 = native.swiglu_bwd(ga1, up1, dh1)
+        if ctx.keep:
+            pad0 = (m0 + 255) // 256 * 256
+            pad1 = (m1 + 255) // 256 * 256
+            hm0, dg0, du0 = native.swiglu_bwd_tiled(gate_keep, up_keep, 0, pad0, dh0)
+            hm1, dg1, du1 = native.swiglu_bwd_tiled(gate_keep, up_keep, pad0 * I0, pad1, dh1)
+        else:
+            ga0, ga1 = _dual(x0, x1, g0, g1, I0, I1, False, True)
+            up0, up1 = _dual(x0, x1, u0, u1, I0, I1, False, True)
+            hm0, dg0, du0 = native.swiglu_bwd(ga0, up0, dh0)
+            hm1, dg1, du1 = native.swiglu_bwd(ga1, up1, dh1)
         need = ctx.needs_input_grad
         grads = [None] * 6
         if need[5] or need[8]:  # gate weights

@@ -644,6 +644,53 @@ def dual_swiglu_ffn_packed(x_tiled: torch.Tensor, num_rows: int, expert_offsets:
     return out
 
 
+def dual_swiglu_ffn_keep(x_tiled: torch.Tensor, num_rows: int, expert_offsets: torch.Tensor, weights,
+                         hmid: Optional[torch.Tensor] = None, host_rows=None,
+                         out_row_id: Optional[torch.Tensor] = None):
+    """dual_swiglu_ffn for a forward pass whose backward follows: the gate / up launch also stores the two
+    projections (K-tiled, the intermediate's geometry) so the backward need not run them again.  The weights are
+    packed afresh (they train).  Returns (out, gate_keep, up_keep, hmid)."""
+    _need_cuda("x_tiled", x_tiled)
+    (g0, u0, d0), (g1, u1, d1) = weights
+    H, I0, I1 = g0.size(1), g0.size(0), g1.size(0)
+    packed = [pack_weight(w, cache=False) for w in (g0, u0, d0, g1, u1, d1)]
+    dev = x_tiled.device
+    need = padded_sorted_rows(num_rows) * max(I0, I1)
+    if hmid is None or hmid.numel() < need or hmid.dtype != torch.bfloat16:
+        hmid = torch.empty(need, dtype=torch.bfloat16, device=dev)
+    gate_keep = torch.empty(need, dtype=torch.bfloat16, device=dev)
+    up_keep = torch.empty(need, dtype=torch.bfloat16, device=dev)
+    out = torch.empty((num_rows, H), dtype=torch.bfloat16, device=dev)
+    if num_rows == 0:
+        return out, gate_keep, up_keep, hmid
+    with _DeviceGuard(x_tiled):
+        _lib.call("wx_dual_swiglu_gate_up_keep", x_tiled.data_ptr(), hmid.data_ptr(), gate_keep.data_ptr(),
+                  up_keep.data_ptr(), expert_offsets.data_ptr(), _ptr(packed[0]), _ptr(packed[1]), _ptr(packed[3]),
+                  _ptr(packed[4]), int(num_rows), H, I0, I1, _lib.i64x2(host_rows), _stream(x_tiled))
+        _lib.call("wx_dual_down_proj", hmid.data_ptr(), _ptr(out), expert_offsets.data_ptr(), _ptr(packed[2]),
+                  _ptr(packed[5]), int(num_rows), H, I0, I1, _lib.i64x2(host_rows), _ptr(out_row_id), _stream(x_tiled))
+    return out, gate_keep, up_keep, hmid
+
+
+def swiglu_bwd_tiled(gate_keep: torch.Tensor, up_keep: torch.Tensor, elem_offset: int, tiled_rows: int,
+                     dh: torch.Tensor):
+    """(hmid, dgate, dup), row-major like dh [rows, cols], of h = silu(gate) * up for one expert whose gate / up
+    projections sit K-tiled in the buffers dual_swiglu_ffn_keep returned, at element offset `elem_offset`, as a
+    matrix of `tiled_rows` rows (the expert's row count rounded up to 256)."""
+    _need_cuda("dh", dh)
+    if dh.dtype != torch.bfloat16 or gate_keep.dtype != torch.bfloat16 or up_keep.dtype != torch.bfloat16:
+        raise RuntimeError("All tensors must be BFloat16 for this kernel")
+    dh = dh.contiguous()
+    rows, cols = dh.shape
+    hm, dg, du = torch.empty_like(dh), torch.empty_like(dh), torch.empty_like(dh)
+    if rows == 0:
+        return hm, dg, du
+    with _DeviceGuard(dh):
+        _lib.call("wx_swiglu_bwd_tiled", gate_keep.data_ptr() + 2 * elem_offset, up_keep.data_ptr() + 2 * elem_offset,
+                  int(tiled_rows), _ptr(dh), _ptr(hm), _ptr(dg), _ptr(du), rows, cols, _stream(dh))
+    return hm, dg, du
+
+
 def dual_swiglu_ffn(x_tiled: torch.Tensor, num_rows: int, expert_offsets: torch.Tensor, weights,
                     hmid: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
                     host_rows=None, out_row_id: Optional[torch.Tensor] = None,
