@@ -13,12 +13,12 @@ Parameter names match the reference (``experts.{e}.{gate,up,down}_proj.weight``)
 import threading
 import weakref
 from dataclasses import dataclass
-from typing import List, Optional
+from typing import Optional
 
 import torch
 from torch import nn
 
-from . import native
+from . import _lib, native
 
 
 class ExpertMLP(nn.Module):
@@ -65,8 +65,8 @@ class _RoutingCache(threading.local):
         self.workspace = {}  # device -> [histograms, status word]
 
     def lookup(self, ids: torch.Tensor, num_experts: int):
-        key = (ids._version, tuple(ids.shape), ids.dtype, ids.device, num_experts,
-               torch.cuda.current_stream(ids.device).cuda_stream)
+        stream = torch.cuda.current_stream(ids.device).cuda_stream if ids.is_cuda else 0
+        key = (ids._version, ids.shape, ids.dtype, ids.device, num_experts, stream)
         if self.ref is not None and self.ref() is ids and self.key == key:
             return self.routing
         flat = ids.reshape(-1)
@@ -79,21 +79,6 @@ class _RoutingCache(threading.local):
 
 
 _routing_cache = _RoutingCache()
-
-
-class _DualExpertFFN(torch.autograd.Function):
-    """The fused forward (tiled activations in; rows out in sorted order, or in token order when out_row_id is
-    given); used when nothing needs a gradient."""
-
-    @staticmethod
-    def forward(ctx, x_tiled, num_rows, expert_offsets, hmid, host_rows, out_row_id, *weights):
-        w = ((weights[0], weights[1], weights[2]), (weights[3], weights[4], weights[5]))
-        return native.dual_swiglu_ffn(x_tiled, num_rows, expert_offsets, w, hmid=hmid, host_rows=host_rows,
-                                      out_row_id=out_row_id)
-
-    @staticmethod
-    def backward(ctx, grad):
-        raise NotImplementedError("wallx_mi355.moe: gradients go through _MoeBlockFunction, not the fused forward")
 
 
 def _dual(a0, a1, w0, w1, n0, n1, trans_a, trans_b):
@@ -193,9 +178,12 @@ class SparseMoeBlock(nn.Module):
             raise ValueError("the dual-expert kernel runs exactly two experts (VL and action)")
         self.num_experts = num_experts
         self.experts = nn.ModuleList([ExpertMLP(config.experts[i]) for i in range(num_experts)])
-        self._hmid: Optional[torch.Tensor] = None
+        self._dims = (self.experts[0].hidden_size, self.experts[0].intermediate_size,
+                      self.experts[1].intermediate_size)
+        self._hmid: Optional[torch.Tensor] = None      # training path only; inference shares buffers per stream
         self._x_tiled: Optional[torch.Tensor] = None
-        self._packed: Optional[List[torch.Tensor]] = None  # set by pack_for_inference()
+        self._packed: Optional[native.PackedExperts] = None  # set by pack_for_inference()
+        self._rows_seen = None
 
     def route(self, experts_indices: torch.Tensor) -> Routing:
         """Stable partition of the flattened token types.  The result is valid for all layers of a forward; it is
@@ -210,7 +198,7 @@ class SparseMoeBlock(nn.Module):
         flat = [w for e in self.experts for w in e.weights()]
         if any(w.numel() == 0 for w in flat):
             raise RuntimeError("pack_for_inference: the nn.Linear weights were already released")
-        self._packed = [native.pack_weight(w.detach(), cache=False) for w in flat]
+        self._packed = native.PackedExperts([native.pack_weight(w.detach(), cache=False) for w in flat], self._dims)
         if free_dense:
             for e in self.experts:
                 for proj in (e.gate_proj, e.up_proj, e.down_proj):
@@ -233,73 +221,76 @@ class SparseMoeBlock(nn.Module):
         residual=True returns hidden_states + block(...) with the add done inside the unpermute.  With both, the
         layer's `residual = h; h = norm(h); h = moe(h); h = residual + h` is `h = moe(h, ..., pre_norm, True)`.
         """
-        host_rows = None
-        if start_indices is not None and end_indices is not None and not start_indices.is_cuda:
-            counts = (end_indices - start_indices).tolist()
-            if len(counts) == 2 and min(counts) >= 0 and sum(counts) == hidden_states.numel() // hidden_states.shape[-1]:
-                host_rows = counts
         batch, seq, hidden = hidden_states.shape
         x = hidden_states.reshape(-1, hidden)
         if x.dtype != torch.bfloat16:
             raise RuntimeError("All tensors must be BFloat16 for this kernel")
+        T = x.size(0)
+        host_rows = self._host_rows(start_indices, end_indices, T)
         if routing is None:
-            routing = self.route(experts_indices)
-        if routing.num_tokens != x.size(0):
-            raise RuntimeError(f"routing was built for {routing.num_tokens} tokens, got {x.size(0)}")
-        flat = [w for e in self.experts for w in e.weights()]
-        need = native.padded_sorted_rows(x.size(0)) * max(e.intermediate_size for e in self.experts)
+            routing = _routing_cache.lookup(experts_indices, self.num_experts)
+        if routing.num_tokens != T:
+            raise RuntimeError(f"routing was built for {routing.num_tokens} tokens, got {T}")
+        grad = torch.is_grad_enabled()
+        if self._packed is not None:
+            if grad and x.requires_grad:
+                raise RuntimeError("a block packed for inference has no backward")
+            experts = self._packed
+        else:
+            flat = [w for e in self.experts for w in e.weights()]
+            if grad and (x.requires_grad or any(w.requires_grad for w in flat)):
+                return self._forward_training(x, routing, flat, pre_norm, residual).view(batch, seq, hidden)
+            # frozen nn.Linear weights: their packed copies are cached per tensor and checked on every call
+            experts = native.PackedExperts([native.pack_weight(w) for w in flat], self._dims)
+        if routing.sorted_row_id is None:
+            return self._forward_scatter(x, routing, experts, host_rows, pre_norm, residual).view(batch, seq, hidden)
+        return native.packed_block_forward(experts, x, routing.row_id_map, routing.sorted_row_id,
+                                           routing.expert_offsets, host_rows, pre_norm, residual
+                                           ).view(batch, seq, hidden)
+
+    def _host_rows(self, start_indices, end_indices, num_tokens):
+        """The per-expert row counts as a host int64[2] when the caller's CPU tensors give them, else None.  The
+        answer is kept for as long as the caller passes the same two unmodified tensor objects (the reference
+        builds them once per forward, act.py:1274-1283, and hands them to all 36 layers)."""
+        if start_indices is None or end_indices is None or start_indices.is_cuda or end_indices.is_cuda:
+            return None
+        hit = self._rows_seen
+        if hit is not None and hit[0] is start_indices and hit[1] is end_indices and \
+                hit[2] == (start_indices._version, end_indices._version, num_tokens):
+            return hit[3]
+        counts = (end_indices - start_indices).tolist()
+        rows = None
+        if len(counts) == 2 and min(counts) >= 0 and sum(counts) == num_tokens:
+            rows = _lib.i64x2(counts)
+        self._rows_seen = (start_indices, end_indices, (start_indices._version, end_indices._version, num_tokens),
+                           rows)
+        return rows
+
+    def _forward_training(self, x, routing, flat, pre_norm, residual):
+        # norm and residual stay PyTorch ops (autograd differentiates them), the block itself has its own backward
+        xin = x
+        if pre_norm is not None:
+            norm_weight, eps = pre_norm
+            xin = torch.nn.functional.rms_norm(x, (x.size(1),), norm_weight, eps)
+        need = native.padded_sorted_rows(x.size(0)) * max(self._dims[1:])
         if self._hmid is None or self._hmid.numel() < need or self._hmid.device != x.device:
             self._hmid = torch.empty(need, dtype=torch.bfloat16, device=x.device)
-        if self._packed is not None:
-            if torch.is_grad_enabled() and x.requires_grad:
-                raise RuntimeError("a block packed for inference has no backward")
-            return self._forward_packed(x, routing, host_rows, pre_norm, residual).view(batch, seq, hidden)
-        if torch.is_grad_enabled() and (x.requires_grad or any(w.requires_grad for w in flat)):
-            # training: norm and residual stay PyTorch ops (autograd differentiates them), the block itself has
-            # its own backward
-            xin = x
-            if pre_norm is not None:
-                norm_weight, eps = pre_norm
-                xin = torch.nn.functional.rms_norm(x, (hidden,), norm_weight, eps)
-            scratch = {"x_tiled": self._x_tiled, "hmid": self._hmid}
-            y = _MoeBlockFunction.apply(xin, routing.row_id_map, routing.expert_offsets, routing.sorted_row_id,
-                                        scratch, *flat)
-            self._x_tiled = scratch["x_tiled"]
-            if residual:
-                y = x + y
-            return y.view(batch, seq, hidden)
-        if pre_norm is not None:
-            norm_weight, eps = pre_norm
-            self._x_tiled = native.rmsnorm_permute_rows_tiled(x, norm_weight, eps, routing.expert_offsets,
-                                                              routing.sorted_row_id, self._x_tiled)
-        else:
-            self._x_tiled = native.permute_rows_tiled(x, routing.row_id_map, routing.expert_offsets, self._x_tiled,
-                                                      routing.sorted_row_id)
-        if residual:
-            y_sorted = _DualExpertFFN.apply(self._x_tiled, x.size(0), routing.expert_offsets, self._hmid, host_rows,
-                                            None, *flat)
-            y = native.unpermute_add(y_sorted, x, routing.row_id_map)
-        else:  # the down launch stores every row at its token's position: no separate unpermute
-            y = _DualExpertFFN.apply(self._x_tiled, x.size(0), routing.expert_offsets, self._hmid, host_rows,
-                                     routing.sorted_row_id, *flat)
-        return y.view(batch, seq, hidden)
+        scratch = {"x_tiled": self._x_tiled, "hmid": self._hmid}
+        y = _MoeBlockFunction.apply(xin, routing.row_id_map, routing.expert_offsets, routing.sorted_row_id,
+                                    scratch, *flat)
+        self._x_tiled = scratch["x_tiled"]
+        return x + y if residual else y
 
-
-    def _forward_packed(self, x, routing, host_rows, pre_norm, residual):
-        dims = (self.experts[0].hidden_size, self.experts[0].intermediate_size, self.experts[1].intermediate_size)
+    def _forward_scatter(self, x, routing, experts, host_rows, pre_norm, residual):
+        # a caller's Routing without the inverse map: scatter rows by row_id_map, separate unpermute
         if pre_norm is not None:
-            norm_weight, eps = pre_norm
-            self._x_tiled = native.rmsnorm_permute_rows_tiled(x, norm_weight, eps, routing.expert_offsets,
-                                                              routing.sorted_row_id, self._x_tiled)
-        else:
-            self._x_tiled = native.permute_rows_tiled(x, routing.row_id_map, routing.expert_offsets, self._x_tiled,
-                                                      routing.sorted_row_id)
+            raise RuntimeError("pre_norm needs a routing with sorted_row_id (partition(..., want_sorted=True))")
+        x_tiled = native.permute_rows_tiled(x, routing.row_id_map, routing.expert_offsets, None, None)
+        y_sorted = native.dual_swiglu_ffn_packed(x_tiled, x.size(0), routing.expert_offsets, experts.tensors,
+                                                 self._dims, host_rows=host_rows)
         if residual:
-            y_sorted = native.dual_swiglu_ffn_packed(self._x_tiled, x.size(0), routing.expert_offsets, self._packed,
-                                                     dims, hmid=self._hmid, host_rows=host_rows)
             return native.unpermute_add(y_sorted, x, routing.row_id_map)
-        return native.dual_swiglu_ffn_packed(self._x_tiled, x.size(0), routing.expert_offsets, self._packed, dims,
-                                             hmid=self._hmid, host_rows=host_rows, out_row_id=routing.sorted_row_id)
+        return native.unpermute(y_sorted, routing.row_id_map, torch.tensor([]), x.size(0), 1)
 
 
 def moe_layer_forward(x: torch.Tensor, token_types: torch.Tensor, weights, routing: Optional[Routing] = None,

@@ -644,6 +644,116 @@ def dual_swiglu_ffn_packed(x_tiled: torch.Tensor, num_rows: int, expert_offsets:
     return out
 
 
+_ffn_scratch = {}  # (device index, stream handle) -> (tiled activations, intermediate), grown on demand
+
+
+def _ffn_buffers(device: torch.device, stream: int, x_elems: int, h_elems: int):
+    """The tiled-activation and intermediate buffers of the block forward, one pair per device and stream: the
+    layers of a model run one after the other on a stream, so they can all work in the same two buffers (a pair per
+    block would hold 0.45 GB per layer at 29 184 tokens).  Calls that overlap on one stream's pair from two threads
+    race, like any two launches writing one buffer."""
+    key = (device.index, stream)
+    hit = _ffn_scratch.get(key)
+    if hit is None or hit[0].numel() < x_elems or hit[1].numel() < h_elems:
+        if hit is not None:
+            x_elems, h_elems = max(x_elems, hit[0].numel()), max(h_elems, hit[1].numel())
+        hit = (torch.empty(x_elems, dtype=torch.bfloat16, device=device),
+               torch.empty(h_elems, dtype=torch.bfloat16, device=device))
+        _ffn_scratch[key] = hit
+    return hit
+
+
+def release_ffn_buffers() -> None:
+    """Drops the buffers _ffn_buffers keeps (they come back, sized for the next call, when needed)."""
+    _ffn_scratch.clear()
+
+
+class PackedExperts:
+    """The six K-tiled projection weights of a two-expert block, checked once, with their addresses ready for the
+    launches: what packed_block_forward needs so that a call is two or three library calls and one allocation."""
+
+    __slots__ = ("tensors", "ptrs", "hidden", "inter0", "inter1", "device", "_sizes")
+
+    def __init__(self, packed, dims):
+        H, I0, I1 = (int(v) for v in dims)
+        lib = _lib.load()
+        want = [lib.wx_tiled_bytes(I0, H), lib.wx_tiled_bytes(I0, H), lib.wx_tiled_bytes(H, I0),
+                lib.wx_tiled_bytes(I1, H), lib.wx_tiled_bytes(I1, H), lib.wx_tiled_bytes(H, I1)]
+        packed = list(packed)
+        if len(packed) != 6:
+            raise RuntimeError("packed must hold gate, up and down of both experts")
+        for t, nbytes in zip(packed, want):
+            _need_cuda("packed weight", t)
+            if t.dtype != torch.bfloat16 or t.numel() * 2 < nbytes or t.device != packed[0].device or \
+                    not t.is_contiguous():
+                raise RuntimeError("packed expert weights do not match (hidden, inter0, inter1)")
+        self.tensors = packed
+        self.ptrs = tuple(_ptr(t) for t in packed)
+        self.hidden, self.inter0, self.inter1 = H, I0, I1
+        self.device = packed[0].device
+        self._sizes = {}
+
+    def sizes(self, num_rows: int):
+        """(elements of the tiled activation matrix, elements of the intermediate) for num_rows tokens."""
+        hit = self._sizes.get(num_rows)
+        if hit is None:
+            pad = padded_sorted_rows(num_rows)
+            hit = (_lib.load().wx_tiled_bytes(pad, self.hidden) // 2, pad * max(self.inter0, self.inter1))
+            if len(self._sizes) >= 64:
+                self._sizes.clear()
+            self._sizes[num_rows] = hit
+        return hit
+
+
+def packed_block_forward(experts: PackedExperts, x: torch.Tensor, row_id_map: torch.Tensor,
+                         sorted_row_id: torch.Tensor, expert_offsets: torch.Tensor, host_rows_c=None,
+                         pre_norm=None, residual: bool = False) -> torch.Tensor:
+    """One block forward on packed weights, in token order: [RMSNorm ->] permute -> gate/up + SwiGLU -> down with
+    the unpermute in its stores [-> + x].  x [T, hidden] bf16; the three routing tensors are the partition's
+    (int32, on x's device); host_rows_c is None or _lib.i64x2((rows of expert 0, rows of expert 1)).  The work
+    buffers are shared per stream (see _ffn_buffers); the result is a new tensor."""
+    dev = x.device
+    if dev != experts.device or x.dtype != torch.bfloat16 or x.dim() != 2 or x.shape[1] != experts.hidden:
+        raise RuntimeError("x must be a [tokens, hidden] BFloat16 tensor on the device of the packed weights")
+    if not x.is_contiguous():
+        x = x.contiguous()
+    T = x.shape[0]
+    for t in (row_id_map, sorted_row_id):
+        if t.dtype != torch.int32 or t.device != dev or t.numel() < T:
+            raise RuntimeError("row_id_map / sorted_row_id must be int32 tensors on x's device, one entry per token")
+    if expert_offsets.dtype != torch.int32 or expert_offsets.device != dev or expert_offsets.numel() < 3:
+        raise RuntimeError("expert_offsets must be an int32 CUDA tensor with 3 entries")
+    out = torch.empty_like(x)
+    if T == 0:
+        return out
+    lib = _lib.load()
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    x_elems, h_elems = experts.sizes(T)
+    x_tiled, hmid = _ffn_buffers(dev, stream, x_elems, h_elems)
+    H, I0, I1 = experts.hidden, experts.inter0, experts.inter1
+    xt, hm, off, srt = x_tiled.data_ptr(), hmid.data_ptr(), expert_offsets.data_ptr(), sorted_row_id.data_ptr()
+    with _DeviceGuard(x):
+        if pre_norm is not None:
+            weight, eps = pre_norm
+            if weight.dtype != torch.bfloat16 or weight.numel() != H or weight.device != dev or \
+                    not weight.is_contiguous():
+                raise RuntimeError("the norm weight must be a contiguous BFloat16 tensor of the hidden size")
+            _lib.check(lib.wx_rmsnorm_permute_rows_tiled(x.data_ptr(), weight.data_ptr(), float(eps), xt, srt, off,
+                                                         T, H, stream))
+        else:
+            _lib.check(lib.wx_permute_rows_tiled(x.data_ptr(), xt, row_id_map.data_ptr(), srt, off, T, H, stream))
+        if residual:
+            y_sorted = torch.empty_like(x)
+            _lib.check(lib.wx_dual_swiglu_ffn(xt, y_sorted.data_ptr(), off, *experts.ptrs, hm, T, H, I0, I1,
+                                              host_rows_c, None, stream))
+            _lib.check(lib.wx_unpermute_rows_add(y_sorted.data_ptr(), x.data_ptr(), out.data_ptr(),
+                                                 row_id_map.data_ptr(), T, H, stream))
+        else:
+            _lib.check(lib.wx_dual_swiglu_ffn(xt, out.data_ptr(), off, *experts.ptrs, hm, T, H, I0, I1,
+                                              host_rows_c, srt, stream))
+    return out
+
+
 def dual_swiglu_ffn_keep(x_tiled: torch.Tensor, num_rows: int, expert_offsets: torch.Tensor, weights,
                          hmid: Optional[torch.Tensor] = None, host_rows=None,
                          out_row_id: Optional[torch.Tensor] = None):
