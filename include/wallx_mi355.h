@@ -106,6 +106,15 @@ int wx_dual_gemm(const void* in0, const void* in1, const void* w0, const void* w
                  void* out1, int64_t m0, int64_t n0, int64_t k0, int64_t m1, int64_t n1, int64_t k1,
                  int trans_a, int trans_b, wx_stream_t stream);
 
+/* wx_dual_gemm with an addend per expert: out_e = op(in_e) @ op(w_e) + add_e, where add_e is [m_e, n_e] bf16
+ * row-major like out_e, may be out_e itself and may be NULL (plain product).  The product is rounded to bf16 and
+ * the sum formed in fp32 and rounded once, i.e. the result of two eager bf16 ops.  For sums of products over
+ * several weight matrices, as in the input gradient of a gated FFN, dX = dG @ Wg + dU @ Wu (the backward of
+ * act.py:79-82, ops.py:78-144): the second product accumulates onto the first instead of a separate add pass. */
+int wx_dual_gemm_add(const void* in0, const void* in1, const void* w0, const void* w1, void* out0,
+                     void* out1, const void* add0, const void* add1, int64_t m0, int64_t n0, int64_t k0,
+                     int64_t m1, int64_t n1, int64_t k1, int trans_a, int trans_b, wx_stream_t stream);
+
 /* ------------------------------------------------------------------------------------------------
  * K-tiled operands of the fused FFN.  The MFMA kernels read activations and weights from a block layout in
  * which every 16-row x 32-column block (1 KiB, bank-swizzled for LDS) is contiguous and the 256 x 32 slab a
@@ -160,6 +169,16 @@ int wx_dual_down_proj(const void* hmid, void* out, const int32_t* expert_offsets
                       const void* down1, int64_t num_rows, int64_t hidden, int64_t inter0,
                       int64_t inter1, const int64_t* host_rows_per_expert, const int32_t* out_row_id,
                       wx_stream_t stream);
+/* wx_dual_down_proj with the decoder layer's closing residual add (act.py:256-265: `hidden_states = residual +
+ * hidden_states` after the MoE block) in its epilogue: out[t, :] = residual[t, :] + y[t, :] in token order, where
+ * y is the block's bf16 result and the sum is formed in fp32 and rounded once, like the eager add.  residual is
+ * [num_rows, hidden] bf16 laid out like out and may be out itself; out_row_id (the partition's sorted_row_id) is
+ * required.  Replaces wx_dual_down_proj + wx_unpermute_rows_add: the sorted result is never written. */
+int wx_dual_down_proj_residual(const void* hmid, void* out, const void* residual,
+                               const int32_t* expert_offsets, const void* down0, const void* down1,
+                               int64_t num_rows, int64_t hidden, int64_t inter0, int64_t inter1,
+                               const int64_t* host_rows_per_expert, const int32_t* out_row_id,
+                               wx_stream_t stream);
 /* wx_dual_swiglu_gate_up for a forward pass whose backward will follow: besides hmid it stores the two projections
  * themselves (rounded to bf16, before the SwiGLU) into gate_keep / up_keep, K-tiled buffers of hmid's size and
  * geometry, so that the backward does not run the two projections again.  The reference keeps these activations

@@ -54,6 +54,7 @@ def test_argument_errors_without_a_gpu():
     lib = _lib.load()
     assert lib.wx_dual_gemm(None, None, None, None, None, None, 8, 12, 8, 0, 8, 8, 0, 1, None) == -2  # n % 8
     assert b"multiples of 8" in lib.wx_last_error_string()
+    assert lib.wx_dual_gemm_add(*([None] * 8), 8, 12, 8, 0, 8, 8, 0, 1, None) == -2  # n % 8
     assert lib.wx_permute_rows(None, None, None, 4, 1, 3, _lib.WX_BF16, None) == -2  # 6-byte rows
     assert lib.wx_partition_build(None, 0, 4, 1, 300, 0, None, None, None, None, None, 0, None) == -2
     assert lib.wx_partition_build(None, 0, 4, 200, 2, 0, None, None, None, None, None, 0, None) == -2
@@ -81,6 +82,8 @@ def test_argument_errors_without_a_gpu():
     assert lib.wx_swiglu_bwd_tiled(None, None, 8, None, None, None, None, 16, 64, None) == -1    # tiled_rows < rows
     assert lib.wx_swiglu_bwd_tiled(None, None, 256, None, None, None, None, 16, 64, None) == -1  # null pointers
     assert lib.wx_dual_swiglu_gate_up_keep(*([None] * 9), 4, 64, 64, 64, None, None) == -1
+    assert lib.wx_dual_down_proj_residual(*([None] * 6), 4, 64, 64, 64, None, None, None) == -1  # null pointers
+    assert lib.wx_dual_down_proj_residual(*([None] * 6), 0, 64, 64, 64, None, None, None) == 0   # nothing to do
     assert lib.wx_qkv_rope_proj(None, None, None, None, None, 4, 64, 1, 1, 96, None) == -2
     assert b"head_dim" in lib.wx_last_error_string()
     assert lib.wx_qkv_rope_proj(None, None, None, None, None, 4, 64, 1, 1, 128, None) == -1

@@ -125,6 +125,40 @@ def test_dual_gemm_k_major_layouts_through_the_c_abi(dev, shape):
         _close(o1, r1, what=f"C ABI ta={ta} tb={tb}")
 
 
+@pytest.mark.parametrize("trans_a,trans_b", [(False, False), (False, True), (True, False), (True, True)])
+def test_dual_gemm_add_accumulates_onto_an_addend(dev, trans_a, trans_b):
+    """wx_dual_gemm_add: out_e = op(a_e) @ op(w_e) + add_e, bit-equal to the plain product followed by an eager bf16
+    add, with the addend in a buffer of its own, in the output itself, missing for one expert, and next to an empty
+    contraction (whose result is the addend)."""
+    g = torch.Generator(device=dev).manual_seed(11 + 2 * trans_a + trans_b)
+    (m0, n0, k0), (m1, n1, k1) = (520, 264, 328), (72, 136, 96)
+
+    def operand(rows, cols, transposed):
+        t = torch.randn((cols, rows) if transposed else (rows, cols), device=dev, generator=g)
+        return (t * 0.1).to(torch.bfloat16)
+
+    a0, a1 = operand(m0, k0, trans_a), operand(m1, k1, trans_a)
+    w0, w1 = operand(k0, n0, trans_b), operand(k1, n1, trans_b)
+    c0, c1 = (torch.randn(m0, n0, device=dev, generator=g).to(torch.bfloat16),
+              torch.randn(m1, n1, device=dev, generator=g).to(torch.bfloat16))
+    p0, p1 = torch.empty_like(c0), torch.empty_like(c1)
+    native.asym_dual_gmm(a0, a1, w0, w1, p0, p1, trans_a, trans_b)
+    want0, want1 = p0 + c0, p1 + c1  # eager: fp32 sum of two bf16 values, rounded once
+    o0, o1 = torch.empty_like(c0), torch.empty_like(c1)
+    native.asym_dual_gmm(a0, a1, w0, w1, o0, o1, trans_a, trans_b, add_expert0=c0, add_expert1=c1)
+    assert torch.equal(o0, want0) and torch.equal(o1, want1)
+    i0, i1 = c0.clone(), c1.clone()
+    native.asym_dual_gmm(a0, a1, w0, w1, i0, i1, trans_a, trans_b, add_expert0=i0, add_expert1=i1)  # in place
+    assert torch.equal(i0, want0) and torch.equal(i1, want1)
+    native.asym_dual_gmm(a0, a1, w0, w1, o0, o1, trans_a, trans_b, add_expert1=c1)  # expert 0 without an addend
+    assert torch.equal(o0, p0) and torch.equal(o1, want1)
+    # an empty contraction next to a full one: 0 + addend
+    e_a = torch.empty((0, m1) if trans_a else (m1, 0), dtype=torch.bfloat16, device=dev)
+    e_w = torch.empty((n1, 0) if trans_b else (0, n1), dtype=torch.bfloat16, device=dev)
+    native.asym_dual_gmm(a0, e_a, w0, e_w, o0, o1, trans_a, trans_b, add_expert0=c0, add_expert1=c1)
+    assert torch.equal(o0, want0) and torch.equal(o1, c1)
+
+
 def test_empty_contraction_of_one_expert_keeps_the_other_on_the_mfma_kernel(dev):
     """A weight gradient dW = dY^T X has k = the expert's token count: a batch without action tokens gives k1 = 0
     next to the VL expert's full-size contraction.  The empty one must come out as zeros and the other must not be
@@ -233,6 +267,57 @@ def test_down_launch_stores_rows_at_their_token_positions(dev, T, n_act, hidden,
     for hint in ((T - n_act, n_act), (n_act, T - n_act)):
         got2 = native.dual_swiglu_ffn(x_tiled, T, off, ws, host_rows=hint, out_row_id=inv)
         assert torch.equal(got2.view(torch.int16), want.view(torch.int16))
+
+
+@pytest.mark.parametrize("T,n_act,hidden,inters", [
+    (700, 33, 512, (1056, 160)),      # small tiles
+    (5000, 300, 2048, (512, 256)),    # large tiles, ragged rows
+    (8600, 300, 2176, (512, 128)),    # large tiles + a ragged last round on the small-tile kernel, ragged columns
+    (300, 300, 256, (256, 128)),      # one expert empty
+])
+def test_down_launch_adds_the_residual_in_its_epilogue(dev, T, n_act, hidden, inters):
+    """wx_dual_down_proj_residual through the C ABI: residual + block output in token order, formed in the down
+    launch's stores.  It must equal the sorted-order result put through the stand-alone unpermute + add bit for bit
+    (both round bf16(y) + residual once), also when the result overwrites the residual, and the oracle's
+    `h + moe(h)` (act.py:256-265) within the stated tolerance."""
+    from wallx_mi355 import _lib
+
+    g = torch.Generator(device=dev).manual_seed(T + hidden + 1)
+    x = torch.randn(T, hidden, device=dev, generator=g).to(torch.bfloat16)
+    res = torch.randn(T, hidden, device=dev, generator=g).to(torch.bfloat16)
+    types = torch.zeros(T, dtype=torch.bool, device=dev)
+    types[torch.randperm(T, device=dev, generator=g)[:n_act]] = True
+    wsc = _moe_weights(hidden, inters, torch.Generator().manual_seed(2), 0.03)
+    ws = [w.to(dev).as_tuple() for w in wsc]
+    rmap, off, inv, _ = native.partition(types, 2, 0, None, want_sorted=True)
+    x_tiled = native.permute_rows_tiled(x, rmap, off, None, inv)
+    y_sorted = native.dual_swiglu_ffn(x_tiled, T, off, ws)
+    want = native.unpermute_add(y_sorted, res, rmap)
+    packed = [native.pack_weight(t, cache=False) for w in ws for t in w]
+    hmid = torch.empty(native.padded_sorted_rows(T) * max(inters), dtype=torch.bfloat16, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    _lib.call("wx_dual_swiglu_gate_up", x_tiled.data_ptr(), hmid.data_ptr(), off.data_ptr(), packed[0].data_ptr(),
+              packed[1].data_ptr(), packed[3].data_ptr(), packed[4].data_ptr(), T, hidden, inters[0], inters[1], None,
+              stream)
+    for hint in (None, (T - n_act, n_act)):
+        got = torch.full((T, hidden), float("nan"), dtype=torch.bfloat16, device=dev)
+        _lib.call("wx_dual_down_proj_residual", hmid.data_ptr(), got.data_ptr(), res.data_ptr(), off.data_ptr(),
+                  packed[2].data_ptr(), packed[5].data_ptr(), T, hidden, inters[0], inters[1], _lib.i64x2(hint),
+                  inv.data_ptr(), stream)
+        assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+    inplace = res.clone()
+    _lib.call("wx_dual_down_proj_residual", hmid.data_ptr(), inplace.data_ptr(), inplace.data_ptr(), off.data_ptr(),
+              packed[2].data_ptr(), packed[5].data_ptr(), T, hidden, inters[0], inters[1], None, inv.data_ptr(), stream)
+    assert torch.equal(inplace.view(torch.int16), want.view(torch.int16))
+    pick = torch.randperm(T, generator=torch.Generator().manual_seed(3))[:96]
+    y_ref = oracle.sparse_moe_block_ref(x.cpu()[pick][None], types.cpu()[pick][None], [w.as_tuple() for w in wsc])[0]
+    ref = (res.cpu()[pick].float() + y_ref.float()).to(torch.bfloat16)
+    _close(want[pick.to(dev)], ref, what="residual + block output")
+    # refused: no residual, no row ids
+    for bad_res, bad_inv in ((None, inv.data_ptr()), (res.data_ptr(), None)):
+        with pytest.raises(RuntimeError):
+            _lib.call("wx_dual_down_proj_residual", hmid.data_ptr(), got.data_ptr(), bad_res, off.data_ptr(),
+                      packed[2].data_ptr(), packed[5].data_ptr(), T, hidden, inters[0], inters[1], None, bad_inv, stream)
 
 
 def test_fused_ffn_intermediate_beyond_2_gib(dev):

@@ -109,6 +109,7 @@ struct Group {
   int m, n, k;
   int lda, ldb, ldc;  // row-major: leading dimension in elements.  tiled: number of 16-row blocks of the matrix
   int a_row0;         // tiled A: first row of this group inside the tiled matrix (a multiple of 256)
+  const __bf16* add;  // generic: optional [m, n] row-major (ldc) matrix added to the product (may be c itself)
 };
 
 struct Params {
@@ -126,6 +127,10 @@ struct Params {
   // kDown only: when set (the partition's sorted_row_id), row r of the sorted result is stored to row scatter[r] of
   // the output instead of row r -- the unpermute folded into the store.
   const int32_t* scatter;
+  // kDown with scatter only: when set, a [tokens, n] matrix laid out like the output whose rows are added to the
+  // result before the store (out[t] = residual[t] + y[t], each term bf16, one rounding) -- the decoder layer's
+  // closing residual add.  May be the output itself.
+  const __bf16* residual;
   // kQkvRope only (group 0 is the projection, row-major operands): bias[n] (may be null), the packed rotary table
   // [m, 64] (bf16 cos | bf16 sin << 16 per token and channel pair) and the number of leading output columns that are
   // rotated (whole heads of 128: the q and k heads; the v heads behind them only take the bias).
@@ -376,6 +381,8 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
   struct Store {    // where the finished tile goes
     __bf16* c_base;
     const int32_t* row_id;  // kDown with scatter: output row of each of the tile's rows (c_base is then row 0)
+    const __bf16* res;      // kDown with scatter and a residual: the residual's column col0 of row 0; generic with
+                            // an addend: its element under c_base; else null
     int rows, cols_left, ldc, nk;
     int row0, col0;         // first row / column of the tile inside its group's output
   };
@@ -393,11 +400,16 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
       S.c_base = G.c + static_cast<int64_t>(row0) * G.ldc + col0;
     }
     S.row_id = nullptr;
+    S.res = nullptr;
     if constexpr (MODE == kDown) {
       if (p.scatter != nullptr) {
         S.c_base = G.c + col0;
         S.row_id = p.scatter + sorted_first[tc.group] + row0;
+        if (p.residual != nullptr) S.res = p.residual + col0;
       }
+    }
+    if constexpr (MODE == kGeneric) {
+      if (G.add != nullptr) S.res = G.add + static_cast<int64_t>(row0) * G.ldc + col0;
     }
     S.rows = G.m - row0 < BM ? G.m - row0 : BM;
     S.cols_left = G.n - col0;
@@ -782,6 +794,33 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
       for (int i = 0; i < FM; ++i) {
 #pragma unroll
         for (int part = 0; part < kParts; ++part) {
+          // a row is kPitch bytes = kLanesPerRow lanes; one store instruction writes kRowsPerStore rows
+          const int rl = lane_e / kLanesPerRow, cc = (lane_e % kLanesPerRow) * 8;
+          const int col = wn * kOutCols + cc;
+          constexpr int kStores = kRound / kRowsPerStore;
+          int out_row[kStores];
+          u32x4 resv[kStores];
+#pragma unroll
+          for (int q = 0; q < kStores; ++q) {
+            const int row = wm * (FM * 32) + i * 32 + part * kRound + q * kRowsPerStore + rl;
+            out_row[q] = row;
+            if constexpr (MODE == kDown) {
+              // scatter: the row ids of the round (and the residual's chunks) are fetched together, ahead of the
+              // staging writes and reads
+              if (S.row_id != nullptr && row < S.rows) out_row[q] = S.row_id[row];
+            }
+          }
+          if constexpr (MODE == kDown || MODE == kGeneric) {
+            if (S.res != nullptr) {
+#pragma unroll
+              for (int q = 0; q < kStores; ++q) {
+                const int row = wm * (FM * 32) + i * 32 + part * kRound + q * kRowsPerStore + rl;
+                resv[q] = u32x4{0u, 0u, 0u, 0u};
+                if (row < S.rows && col < S.cols_left)
+                  resv[q] = *reinterpret_cast<const u32x4*>(S.res + static_cast<int64_t>(out_row[q]) * S.ldc + col);
+              }
+            }
+          }
 #pragma unroll
           for (int j = 0; j < FN; ++j) {
 #pragma unroll
@@ -792,25 +831,22 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
             }
           }
           __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, 0));
-          // a row is kPitch bytes = kLanesPerRow lanes; one store instruction writes kRowsPerStore rows
-          const int rl = lane_e / kLanesPerRow, cc = (lane_e % kLanesPerRow) * 8;
-          constexpr int kStores = kRound / kRowsPerStore;
-          int out_row[kStores];
-#pragma unroll
-          for (int q = 0; q < kStores; ++q) {
-            const int row = wm * (FM * 32) + i * 32 + part * kRound + q * kRowsPerStore + rl;
-            out_row[q] = row;
-            if constexpr (MODE == kDown) {
-              // scatter: the row ids of the round are fetched together, ahead of the staging reads
-              if (S.row_id != nullptr && row < S.rows) out_row[q] = S.row_id[row];
-            }
-          }
 #pragma unroll
           for (int q = 0; q < kStores; ++q) {
             const int srow = q * kRowsPerStore + rl;
-            const u32x4 v = *reinterpret_cast<const u32x4*>(stage + srow * kPitch + cc * 2);
+            u32x4 v = *reinterpret_cast<const u32x4*>(stage + srow * kPitch + cc * 2);
             const int row = wm * (FM * 32) + i * 32 + part * kRound + srow;
-            const int col = wn * kOutCols + cc;
+            if constexpr (MODE == kDown || MODE == kGeneric) {
+              if (S.res != nullptr) {  // bf16(y) + bf16(residual), summed in fp32 and rounded once, like the eager add
+#pragma unroll
+                for (int w = 0; w < 4; ++w) {
+                  const float lo = __builtin_bit_cast(float, v[w] << 16) + __builtin_bit_cast(float, resv[q][w] << 16);
+                  const float hi = __builtin_bit_cast(float, v[w] & 0xFFFF0000u) +
+                                   __builtin_bit_cast(float, resv[q][w] & 0xFFFF0000u);
+                  v[w] = pack_bf16x2(lo, hi);
+                }
+              }
+            }
             if (row < S.rows && col < S.cols_left)
               *reinterpret_cast<u32x4*>(S.c_base + static_cast<int64_t>(out_row[q]) * S.ldc + col) = v;
           }
@@ -943,7 +979,11 @@ __global__ __launch_bounds__(256) void dual_gemm_reference_layout_kernel(Params 
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         const int m = row0 + ty + 8 * q, n = col0 + tx;
-        if (m < G.m && n < G.n) G.c[static_cast<int64_t>(m) * G.ldc + n] = static_cast<__bf16>(acc[q]);
+        if (m < G.m && n < G.n) {
+          __bf16 v = static_cast<__bf16>(acc[q]);
+          if (G.add != nullptr) v = static_cast<__bf16>(static_cast<float>(v) + static_cast<float>(G.add[static_cast<int64_t>(m) * G.ldc + n]));
+          G.c[static_cast<int64_t>(m) * G.ldc + n] = v;
+        }
       }
     }
   }
@@ -1038,9 +1078,31 @@ int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
 using namespace wx;
 
+namespace {
+int dual_gemm_impl(const void* in0, const void* in1, const void* w0, const void* w1, void* out0, void* out1,
+                   const void* add0, const void* add1, int64_t m0, int64_t n0, int64_t k0, int64_t m1, int64_t n1,
+                   int64_t k1, int trans_a, int trans_b, wx_stream_t stream);
+}
+
 extern "C" int wx_dual_gemm(const void* in0, const void* in1, const void* w0, const void* w1, void* out0, void* out1,
                             int64_t m0, int64_t n0, int64_t k0, int64_t m1, int64_t n1, int64_t k1, int trans_a,
                             int trans_b, wx_stream_t stream) {
+  return dual_gemm_impl(in0, in1, w0, w1, out0, out1, nullptr, nullptr, m0, n0, k0, m1, n1, k1, trans_a, trans_b, stream);
+}
+
+extern "C" int wx_dual_gemm_add(const void* in0, const void* in1, const void* w0, const void* w1, void* out0,
+                                void* out1, const void* add0, const void* add1, int64_t m0, int64_t n0, int64_t k0,
+                                int64_t m1, int64_t n1, int64_t k1, int trans_a, int trans_b, wx_stream_t stream) {
+  if ((reinterpret_cast<uintptr_t>(add0) | reinterpret_cast<uintptr_t>(add1)) & 15)
+    return fail(WX_ERR_INVALID_ARGUMENT, "wx_dual_gemm_add: buffers must be 16-byte aligned");
+  return dual_gemm_impl(in0, in1, w0, w1, out0, out1, add0, add1, m0, n0, k0, m1, n1, k1, trans_a, trans_b, stream);
+}
+
+namespace {
+int dual_gemm_impl(const void* in0, const void* in1, const void* w0, const void* w1, void* out0, void* out1,
+                   const void* add0, const void* add1, int64_t m0, int64_t n0, int64_t k0, int64_t m1, int64_t n1,
+                   int64_t k1, int trans_a, int trans_b, wx_stream_t stream) {
+  const void* adds[2] = {add0, add1};
   const bool k_in_rows = trans_a && !trans_b;  // A [k, m] and B [k, n]
   if (int rc = check_dims("wx_dual_gemm", m0, n0, k0, k_in_rows)) return rc;
   if (int rc = check_dims("wx_dual_gemm", m1, n1, k1, k_in_rows)) return rc;
@@ -1065,6 +1127,7 @@ extern "C" int wx_dual_gemm(const void* in0, const void* in1, const void* w0, co
     g.ldb = static_cast<int>(trans_b ? k : n);
     g.ldc = static_cast<int>(n);
     g.a_row0 = 0;
+    g.add = static_cast<const __bf16*>(adds[e]);
   }
   p.offsets = nullptr;
   if ((m0 == 0 || n0 == 0) && (m1 == 0 || n1 == 0)) return WX_OK;
@@ -1075,6 +1138,13 @@ extern "C" int wx_dual_gemm(const void* in0, const void* in1, const void* w0, co
   for (int e = 0; e < 2; ++e) {
     const int64_t m = dims[e][0], n = dims[e][1];
     if (dims[e][2] != 0 || m <= 0 || n <= 0) continue;
+    if (adds[e] != nullptr) {  // 0 + addend
+      if (adds[e] != ptrs[e][2] &&
+          hipMemcpyAsync(const_cast<void*>(ptrs[e][2]), adds[e], static_cast<size_t>(m) * n * 2, hipMemcpyDeviceToDevice, s) != hipSuccess)
+        return fail(WX_ERR_LAUNCH, "wx_dual_gemm_add: copy of the addend failed");
+      p.g[e].m = 0;
+      continue;
+    }
     const int64_t n16 = m * n / 8;  // n is a multiple of 8 and the buffer 16-byte aligned
     const int64_t want = (n16 + 255) / 256, cap = static_cast<int64_t>(device_cu_count()) * 8;
     hipLaunchKernelGGL(zero_fill_kernel, dim3(static_cast<unsigned>(want < cap ? want : cap)), dim3(256), 0, s,
@@ -1101,6 +1171,7 @@ extern "C" int wx_dual_gemm(const void* in0, const void* in1, const void* w0, co
   hipLaunchKernelGGL(dual_gemm_reference_layout_kernel, dim3(device_cu_count() * 4), dim3(256), 0, s, p, trans_a, trans_b);
   return check_launch("dual_gemm_reference_layout_kernel");
 }
+}  // namespace
 
 extern "C" int wx_qkv_rope_proj(const void* x, const void* weight, const void* bias, const uint32_t* rope_table,
                                 void* out, int64_t num_tokens, int64_t hidden, int n_q_heads, int n_kv_heads,
@@ -1168,6 +1239,7 @@ struct FfnArgs {
   int64_t rows, hidden, inter[2];
   const int32_t* out_row_id = nullptr;  // optional: sorted row r of the result goes to row out_row_id[r] of `out`
   void *keep_gate = nullptr, *keep_up = nullptr;  // optional: the gate / up projections, K-tiled like hmid
+  const void* residual = nullptr;  // optional (with out_row_id): rows added to the result, laid out like `out`
 };
 
 int check_ffn(const char* who, const FfnArgs& a, bool need_gate_up, bool need_down) {
@@ -1240,6 +1312,7 @@ int launch_down(const FfnArgs& a, hipStream_t s) {
   }
   p.offsets = a.offsets;
   p.scatter = a.out_row_id;
+  p.residual = static_cast<const __bf16*>(a.residual);
   const int64_t col_tiles = ceil_div(a.hidden, BigTile::BN);
   if (a.host_rows != nullptr) {
     const int64_t by_expert[2] = {ceil_div(a.host_rows[0], BigTile::BM) * col_tiles, ceil_div(a.host_rows[1], BigTile::BM) * col_tiles};
@@ -1288,6 +1361,23 @@ extern "C" int wx_dual_down_proj(const void* hmid, void* out, const int32_t* exp
                   host_rows_per_expert, expert_offsets, num_rows, hidden, {inter0, inter1}, out_row_id};
   if (int rc = check_ffn("wx_dual_down_proj", a, false, true)) return rc;
   if (num_rows == 0) return WX_OK;
+  return launch_down(a, as_stream(stream));
+}
+
+extern "C" int wx_dual_down_proj_residual(const void* hmid, void* out, const void* residual,
+                                          const int32_t* expert_offsets, const void* down0, const void* down1,
+                                          int64_t num_rows, int64_t hidden, int64_t inter0, int64_t inter1,
+                                          const int64_t* host_rows_per_expert, const int32_t* out_row_id,
+                                          wx_stream_t stream) {
+  const char* who = "wx_dual_down_proj_residual";
+  FfnArgs a{nullptr, {nullptr, nullptr}, {nullptr, nullptr}, {down0, down1}, out, const_cast<void*>(hmid),
+            host_rows_per_expert, expert_offsets, num_rows, hidden, {inter0, inter1}, out_row_id};
+  if (int rc = check_ffn(who, a, false, true)) return rc;
+  if (num_rows == 0) return WX_OK;
+  if (!residual || !out_row_id)
+    return fail(WX_ERR_INVALID_ARGUMENT, "%s: residual and out_row_id are required (the sum is formed in token order)", who);
+  if (reinterpret_cast<uintptr_t>(residual) & 15) return fail(WX_ERR_INVALID_ARGUMENT, "%s: residual must be 16-byte aligned", who);
+  a.residual = residual;
   return launch_down(a, as_stream(stream));
 }
 

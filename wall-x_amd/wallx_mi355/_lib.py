@@ -30,6 +30,7 @@ PROTOTYPES = {
     "wx_unpermute_rows": (_i32, [_vp, _vp, _vp, _vp, _i64, _i32, _i64, _i32, _vp]),
     "wx_unpermute_rows_bwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i32, _i64, _i32, _vp]),
     "wx_dual_gemm": (_i32, [_vp] * 6 + [_i64] * 6 + [_i32, _i32, _vp]),
+    "wx_dual_gemm_add": (_i32, [_vp] * 8 + [_i64] * 6 + [_i32, _i32, _vp]),
     "wx_tiled_bytes": (_sz, [_i64, _i64]),
     "wx_padded_sorted_rows": (_i64, [_i64]),
     "wx_pack_tiled": (_i32, [_vp, _vp, _i64, _i64, _vp]),
@@ -38,6 +39,7 @@ PROTOTYPES = {
     "wx_dual_swiglu_gate_up": (_i32, [_vp] * 7 + [_i64] * 4 + [_vp, _vp]),
     "wx_dual_swiglu_gate_up_keep": (_i32, [_vp] * 9 + [_i64] * 4 + [_vp, _vp]),
     "wx_dual_down_proj": (_i32, [_vp] * 5 + [_i64] * 4 + [_vp, _vp, _vp]),
+    "wx_dual_down_proj_residual": (_i32, [_vp] * 6 + [_i64] * 4 + [_vp, _vp, _vp]),
     "wx_mrope_apply": (_i32, [_vp] * 6 + [_i64, _i64, _i32, _i32, _i32] + [_c.POINTER(_i64)] * 4
                        + [_c.POINTER(_i32), _i32, _i32, _vp]),
     "wx_mrope_apply_bwd": (_i32, [_vp] * 6 + [_i64, _i64, _i32, _i32, _i32] + [_c.POINTER(_i64)] * 4

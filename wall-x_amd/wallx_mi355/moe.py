@@ -95,7 +95,8 @@ class _MoeBlockFunction(torch.autograd.Function):
 
     Forward is the fused path; its gate / up launch also keeps the two projections (the reference's autograd keeps
     them too, along with act_fn(gate) and the product, act.py:79-82).  Backward runs every remaining contraction of
-    both experts as one dual GEMM each: dHm = dY Wd, dWd = dY^T Hm, dX = dG Wg + dU Wu, dWg = dG^T X, dWu = dU^T X,
+    both experts as one dual GEMM each: dHm = dY Wd, dWd = dY^T Hm, dX = dG Wg + dU Wu (the second product added onto
+    the first in its epilogue), dWg = dG^T X, dWu = dU^T X,
     with the SwiGLU derivative (and Hm in row-major form) from one fused elementwise kernel per expert (fp32 math).
     Intermediate sizes that are not multiples of 64 recompute the two projections instead.  The per-expert row
     counts are read back from the device once per backward (the forward never synchronises)."""
@@ -160,11 +161,12 @@ class _MoeBlockFunction(torch.autograd.Function):
             grads[2], grads[5] = _dual(dy0, dy1, hm0, hm1, I0, I1, True, False)
         dx = None
         if need[0]:
-            a0, a1 = _dual(dg0, dg1, g0, g1, H, H, False, False)
-            b0, b1 = _dual(du0, du1, u0, u1, H, H, False, False)
+            # dX = dG Wg + dU Wu: the second product accumulates onto the first in its epilogue (bf16 + bf16, rounded
+            # once -- what the two eager ops and their add give)
             dxs = torch.empty(T, H, dtype=torch.bfloat16, device=x.device)
-            torch.add(a0, b0, out=dxs[:m0])
-            torch.add(a1, b1, out=dxs[m0:m0 + m1])
+            d0_, d1_ = dxs[:m0], dxs[m0:m0 + m1]
+            native.asym_dual_gmm(dg0, dg1, g0, g1, d0_, d1_, False, False)
+            native.asym_dual_gmm(du0, du1, u0, u1, d0_, d1_, False, False, add_expert0=d0_, add_expert1=d1_)
             dx = native.unpermute(dxs, row_id_map, torch.tensor([]), T, 1)
         return (dx, None, None, None, None, *grads)
 

@@ -90,9 +90,16 @@ class _DeviceGuard:
 
 # ----------------------------------------------------------------------------- dual grouped GEMM
 def asym_dual_gmm(input_expert0, input_expert1, weight_expert0, weight_expert1, output_expert0,
-                  output_expert1, trans_a: bool, trans_b: bool) -> None:
-    """csrc/dual_asym_grouped_gemm.cu:308-366.  Writes into the caller's outputs."""
+                  output_expert1, trans_a: bool, trans_b: bool, add_expert0: Optional[torch.Tensor] = None,
+                  add_expert1: Optional[torch.Tensor] = None) -> None:
+    """csrc/dual_asym_grouped_gemm.cu:308-366.  Writes into the caller's outputs.  add_expert{0,1} (not in the
+    reference): contiguous tensors of the outputs' shapes added to the products (they may be the outputs)."""
     ts = (input_expert0, input_expert1, weight_expert0, weight_expert1, output_expert0, output_expert1)
+    adds = (add_expert0, add_expert1)
+    for add, out in zip(adds, (output_expert0, output_expert1)):
+        if add is not None and (add.shape != out.shape or add.dtype != out.dtype or add.device != out.device or
+                                not add.is_contiguous()):
+            raise RuntimeError("an addend must be a contiguous tensor of its output's shape, dtype and device")
     for t in ts:
         _need_cuda("All tensors", t)
         if t.device != ts[0].device:
@@ -119,9 +126,14 @@ def asym_dual_gmm(input_expert0, input_expert1, weight_expert0, weight_expert1, 
     # Every layout runs on the MFMA kernel: operands stored with K as the slow dimension (trans_a, or weights kept
     # [k, n]) are transposed between LDS and the registers, so no transposed copy is made.
     with _DeviceGuard(a0):
-        _lib.call("wx_dual_gemm", _ptr(a0), _ptr(a1), _ptr(w0), _ptr(w1), _ptr(output_expert0),
-                  _ptr(output_expert1), m0, n0, k0, m1, n1, k1, int(bool(trans_a)), int(bool(trans_b)),
-                  _stream(a0))
+        if add_expert0 is None and add_expert1 is None:
+            _lib.call("wx_dual_gemm", _ptr(a0), _ptr(a1), _ptr(w0), _ptr(w1), _ptr(output_expert0),
+                      _ptr(output_expert1), m0, n0, k0, m1, n1, k1, int(bool(trans_a)), int(bool(trans_b)),
+                      _stream(a0))
+        else:
+            _lib.call("wx_dual_gemm_add", _ptr(a0), _ptr(a1), _ptr(w0), _ptr(w1), _ptr(output_expert0),
+                      _ptr(output_expert1), _ptr(add_expert0), _ptr(add_expert1), m0, n0, k0, m1, n1, k1,
+                      int(bool(trans_a)), int(bool(trans_b)), _stream(a0))
 
 
 def swiglu_bwd(gate: torch.Tensor, up: torch.Tensor, dh: torch.Tensor):
@@ -709,7 +721,7 @@ def packed_block_forward(experts: PackedExperts, x: torch.Tensor, row_id_map: to
                          sorted_row_id: torch.Tensor, expert_offsets: torch.Tensor, host_rows_c=None,
                          pre_norm=None, residual: bool = False) -> torch.Tensor:
     """One block forward on packed weights, in token order: [RMSNorm ->] permute -> gate/up + SwiGLU -> down with
-    the unpermute in its stores [-> + x].  x [T, hidden] bf16; the three routing tensors are the partition's
+    the unpermute [and the residual add, + x] in its stores.  x [T, hidden] bf16; the three routing tensors are the partition's
     (int32, on x's device); host_rows_c is None or _lib.i64x2((rows of expert 0, rows of expert 1)).  The work
     buffers are shared per stream (see _ffn_buffers); the result is a new tensor."""
     dev = x.device
@@ -742,12 +754,11 @@ def packed_block_forward(experts: PackedExperts, x: torch.Tensor, row_id_map: to
                                                          T, H, stream))
         else:
             _lib.check(lib.wx_permute_rows_tiled(x.data_ptr(), xt, row_id_map.data_ptr(), srt, off, T, H, stream))
-        if residual:
-            y_sorted = torch.empty_like(x)
-            _lib.check(lib.wx_dual_swiglu_ffn(xt, y_sorted.data_ptr(), off, *experts.ptrs, hm, T, H, I0, I1,
-                                              host_rows_c, None, stream))
-            _lib.check(lib.wx_unpermute_rows_add(y_sorted.data_ptr(), x.data_ptr(), out.data_ptr(),
-                                                 row_id_map.data_ptr(), T, H, stream))
+        if residual:  # the add happens in the down launch's epilogue: the sorted result is never written
+            g0, u0, d0, g1, u1, d1 = experts.ptrs
+            _lib.check(lib.wx_dual_swiglu_gate_up(xt, hm, off, g0, u0, g1, u1, T, H, I0, I1, host_rows_c, stream))
+            _lib.check(lib.wx_dual_down_proj_residual(hm, out.data_ptr(), x.data_ptr(), off, d0, d1, T, H, I0, I1,
+                                                      host_rows_c, srt, stream))
         else:
             _lib.check(lib.wx_dual_swiglu_ffn(xt, out.data_ptr(), off, *experts.ptrs, hm, T, H, I0, I1,
                                               host_rows_c, srt, stream))
