@@ -52,7 +52,7 @@ def parse():
     return ap.parse_args()
 
 
-def event_ms(fn, iters, warm=3, batch=1):
+def event_ms(fn, iters, warm=10, batch=1):
     """(median, mean) duration of one fn() in ms from HIP events on the current stream.  batch > 1 times that many
     back-to-back calls per event pair, which keeps launch gaps out of the figure for kernels of a few tens of us."""
     import torch
@@ -182,7 +182,7 @@ def main():
     tflops = ffn_flops / (elapsed / args.steps) / 1e12
 
     # ---- per-kernel timings (HIP events on the launch stream) ------------------------------------------
-    iters = max(10, args.steps)
+    iters = max(50, args.steps)  # >= 50 timed launches after 10 warm-ups, median (and mean for the roofline)
     t_gate_up, t_gate_up_avg = event_ms(gate_up, iters)
     t_down, _ = event_ms(down, iters)
     t_down_unp, _ = event_ms(down_unpermute, iters)
@@ -459,7 +459,9 @@ def config4_measurement(dev, weights):
         start, end = torch.tensor([0, n_vl]), torch.tensor([n_vl, T])
         with torch.no_grad():
             tb, _ = event_ms(lambda: block(x3, types2, start, end), 20, warm=5)
-        out[name]["us_drop_in_block_same_token_types"] = round(tb * 1e3, 1)
+            tbb, _ = event_ms(lambda: block(x3, types2, start, end), 20, warm=5, batch=36)
+        out[name]["us_drop_in_block_same_token_types"] = round(tb * 1e3, 1)            # one call, GPU idle before it
+        out[name]["us_per_layer_drop_in_block_36_calls_back_to_back"] = round(tbb * 1e3, 1)  # as a decoder issues them
         if n_vl == 0:
             # the denoise loop repeats this shape 10 x 36 times per action chunk: record 36 layers once into a HIP
             # graph (the entry points neither allocate nor synchronise) and time its replays
@@ -507,9 +509,9 @@ def backward_measurement(dev, x, weights, m0):
     dw0, dw1 = torch.empty_like(g0), torch.empty_like(g1)
     flops = 2.0 * H * (m0 * I0 + m1 * I1)
     y0, y1 = torch.empty_like(dy0), torch.empty_like(dy1)
-    t_fw, _ = event_ms(lambda: native.asym_dual_gmm(x0, x1, g0, g1, y0, y1, False, True), 5, warm=2)
-    t_dx, _ = event_ms(lambda: native.asym_dual_gmm(dy0, dy1, g0, g1, dx0, dx1, False, False), 5, warm=2)
-    t_dw, _ = event_ms(lambda: native.asym_dual_gmm(dy0, dy1, x0, x1, dw0, dw1, True, False), 5, warm=2)
+    t_fw, _ = event_ms(lambda: native.asym_dual_gmm(x0, x1, g0, g1, y0, y1, False, True), 20, warm=5)
+    t_dx, _ = event_ms(lambda: native.asym_dual_gmm(dy0, dy1, g0, g1, dx0, dx1, False, False), 20, warm=5)
+    t_dw, _ = event_ms(lambda: native.asym_dual_gmm(dy0, dy1, x0, x1, dw0, dw1, True, False), 20, warm=5)
     return {"forward_nt_ms": round(t_fw, 3), "forward_nt_tflops": round(flops / t_fw / 1e9, 1),
             "dx_ms": round(t_dx, 3), "dx_tflops": round(flops / t_dx / 1e9, 1),
             "dw_ms": round(t_dw, 3), "dw_tflops": round(flops / t_dw / 1e9, 1)}

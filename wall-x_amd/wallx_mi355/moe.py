@@ -295,21 +295,54 @@ class SparseMoeBlock(nn.Module):
         return native.unpermute(y_sorted, routing.row_id_map, torch.tensor([]), x.size(0), 1)
 
 
+_functional_experts = {}  # ids of the six weight tensors -> (their storage / version state, weak references, PackedExperts)
+
+
+def _experts_for(weights) -> "native.PackedExperts":
+    """PackedExperts for weights given as ((gate0, up0, down0), (gate1, up1, down1)) in nn.Linear layout: packed
+    once per set of tensors and reused while those tensor objects keep their storage and version counters."""
+    flat = (*weights[0], *weights[1])
+    key = tuple(map(id, flat))
+    state = tuple((w.data_ptr(), w._version) for w in flat)
+    hit = _functional_experts.get(key)
+    if hit is not None and hit[0] == state and all(r() is w for r, w in zip(hit[1], flat)):
+        return hit[2]
+    g0, u0, d0, g1, u1, d1 = flat
+    H, I0, I1 = g0.size(1), g0.size(0), g1.size(0)
+    if tuple(u0.shape) != (I0, H) or tuple(d0.shape) != (H, I0) or tuple(g1.shape) != (I1, H) or \
+            tuple(u1.shape) != (I1, H) or tuple(d1.shape) != (H, I1):
+        raise RuntimeError("expert weight shapes are inconsistent with hidden size")
+    experts = native.PackedExperts([native.pack_weight(w) for w in flat], (H, I0, I1))
+    if len(_functional_experts) >= 64:
+        _functional_experts.clear()
+    _functional_experts[key] = (state, [weakref.ref(w) for w in flat], experts)
+    return experts
+
+
 def moe_layer_forward(x: torch.Tensor, token_types: torch.Tensor, weights, routing: Optional[Routing] = None,
                       hmid: Optional[torch.Tensor] = None, workspace=None, host_rows=None):
     """Functional form of one layer: permute -> dual-expert SwiGLU FFN -> unpermute.
 
     x [T, H] bf16, token_types [T] (bool / int), weights ((g0,u0,d0),(g1,u1,d1)).  Returns (y [T, H], routing).
+    Without `routing` the token types are partitioned on every call (pass the returned routing to the following
+    layers).  Frozen weights are packed once (see native.pack_weight for what invalidates the packed copies); the
+    work buffers are the per-stream pair every block shares, so `hmid` is accepted for compatibility and not used.
     """
     if routing is None:
-        row_id_map, offsets, inverse, _ = native.partition(token_types.reshape(-1), 2, 0, workspace, want_sorted=True)
+        dev = token_types.device
+        ws = workspace if workspace is not None else _routing_cache.workspace.get(dev)
+        row_id_map, offsets, inverse, ws = native.partition(token_types.reshape(-1), 2, 0, ws, want_sorted=True)
+        if workspace is None:
+            _routing_cache.workspace[dev] = ws
         routing = Routing(row_id_map, offsets, x.size(0), inverse)
-    x_tiled = native.permute_rows_tiled(x, routing.row_id_map, routing.expert_offsets, None, routing.sorted_row_id)
+    experts = _experts_for(weights)
+    rows = None if host_rows is None else _lib.i64x2(host_rows)
     if routing.sorted_row_id is not None:  # the down launch stores every row at its token's position
-        y = native.dual_swiglu_ffn(x_tiled, x.size(0), routing.expert_offsets, weights, hmid=hmid,
-                                   host_rows=host_rows, out_row_id=routing.sorted_row_id)
+        y = native.packed_block_forward(experts, x, routing.row_id_map, routing.sorted_row_id,
+                                        routing.expert_offsets, rows)
         return y, routing
-    y_sorted = native.dual_swiglu_ffn(x_tiled, x.size(0), routing.expert_offsets, weights, hmid=hmid,
-                                      host_rows=host_rows)
+    x_tiled = native.permute_rows_tiled(x, routing.row_id_map, routing.expert_offsets, None, None)
+    y_sorted = native.dual_swiglu_ffn_packed(x_tiled, x.size(0), routing.expert_offsets, experts.tensors,
+                                             (experts.hidden, experts.inter0, experts.inter1), host_rows=host_rows)
     y = native.unpermute(y_sorted, routing.row_id_map, torch.tensor([]), x.size(0), 1)
     return y, routing
