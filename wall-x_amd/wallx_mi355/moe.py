@@ -242,8 +242,8 @@ class SparseMoeBlock(nn.Module):
             flat = [w for e in self.experts for w in e.weights()]
             if grad and (x.requires_grad or any(w.requires_grad for w in flat)):
                 return self._forward_training(x, routing, flat, pre_norm, residual).view(batch, seq, hidden)
-            # frozen nn.Linear weights: their packed copies are cached per tensor and checked on every call
-            experts = native.PackedExperts([native.pack_weight(w) for w in flat], self._dims)
+            # frozen nn.Linear weights: packed once, the copies checked against storage and version on every call
+            experts = _experts_for((flat[:3], flat[3:]))
         if routing.sorted_row_id is None:
             return self._forward_scatter(x, routing, experts, host_rows, pre_norm, residual).view(batch, seq, hidden)
         return native.packed_block_forward(experts, x, routing.row_id_map, routing.sorted_row_id,
@@ -298,6 +298,9 @@ class SparseMoeBlock(nn.Module):
 _functional_experts = {}  # ids of the six weight tensors -> (their storage / version state, weak references, PackedExperts)
 
 
+native._invalidate_hooks.append(lambda _w: _functional_experts.clear())
+
+
 def _experts_for(weights) -> "native.PackedExperts":
     """PackedExperts for weights given as ((gate0, up0, down0), (gate1, up1, down1)) in nn.Linear layout: packed
     once per set of tensors and reused while those tensor objects keep their storage and version counters."""
@@ -315,7 +318,9 @@ def _experts_for(weights) -> "native.PackedExperts":
     experts = native.PackedExperts([native.pack_weight(w) for w in flat], (H, I0, I1))
     if len(_functional_experts) >= 64:
         _functional_experts.clear()
-    _functional_experts[key] = (state, [weakref.ref(w) for w in flat], experts)
+    # the entry (and with it the packed copies) goes when any of the six tensors does
+    refs = [weakref.ref(w, lambda _r, k=key: _functional_experts.pop(k, None)) for w in flat]
+    _functional_experts[key] = (state, refs, experts)
     return experts
 
 

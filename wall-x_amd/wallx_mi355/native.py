@@ -517,6 +517,11 @@ def invalidate_packed(w: Optional[torch.Tensor] = None) -> None:
         _packed_cache.clear()
     else:
         _packed_cache.pop(id(w), None)
+    for hook in _invalidate_hooks:  # holders of objects built from packed copies (moe's per-weight-set cache)
+        hook(w)
+
+
+_invalidate_hooks = []
 
 
 def pack_weight(w: torch.Tensor, cache: bool = True) -> torch.Tensor:
