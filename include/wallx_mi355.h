@@ -39,6 +39,11 @@ typedef enum { WX_MROPE_HF = 0, WX_MROPE_CSRC = 1 } wx_mrope_layout;
 
 const char* wx_last_error_string(void);
 int wx_abi_version(void);
+/* 1 and *id = the capture's id when `stream` is being captured into a HIP graph, 0 and *id = 0 when it is not
+ * (negative on error).  No counterpart in the reference; for hosts that keep results between calls (a cached token
+ * partition, work buffers) and must not carry them from inside a capture, where nothing has executed yet, to
+ * outside it. */
+int wx_stream_capture_id(wx_stream_t stream, unsigned long long* id);
 
 /* ------------------------------------------------------------------------------------------------
  * Token partition.  Replaces cub::DeviceRadixSort::SortPairs + moe_permute_topK_row_map

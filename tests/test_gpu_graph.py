@@ -71,6 +71,78 @@ def test_layer_graph_replays_match_eager(dev, n_vl, n_act):
         assert int((got != h).sum()) == 0, f"replay {it} differs from the eager run"
 
 
+def test_drop_in_blocks_under_graph_capture(dev):
+    """Four drop-in blocks called the way the reference's decoder calls them (same token-type tensor and CPU row
+    ranges for every layer) recorded into a HIP graph: the first block's partition is recorded, the others reuse it
+    within the capture, and every replay equals the eager result on the same inputs.  What the blocks keep between
+    calls (the cached partition, the shared work buffers) must not leak out of the capture, where nothing has executed
+    yet: an eager call right after the capture, on the capture's inputs, is checked as well."""
+    from types import SimpleNamespace
+
+    g = torch.Generator(device=dev).manual_seed(21)
+    hidden, inters, n_vl, n_act = 512, (768, 256), 300, 212
+    T = n_vl + n_act
+    cfg = SimpleNamespace(experts=[dict(hidden_size=hidden, intermediate_size=i, hidden_act="silu") for i in inters])
+    blocks = []
+    for _ in range(4):
+        b = moe.SparseMoeBlock(cfg, 2).to(dev).to(torch.bfloat16)
+        with torch.no_grad():
+            for prm in b.parameters():
+                prm.copy_((torch.randn(prm.shape, device=dev, generator=g) * 0.03).to(torch.bfloat16))
+        blocks.append(b.pack_for_inference())
+    x_static = torch.zeros(1, T, hidden, dtype=torch.bfloat16, device=dev)
+    types_static = torch.zeros(1, T, dtype=torch.bool, device=dev)
+    start, end = torch.tensor([0, n_vl]), torch.tensor([n_vl, T])
+
+    def run(x, types):
+        h = x
+        with torch.no_grad():
+            for b in blocks:
+                h = b(h, types, start, end, residual=True)
+        return h
+
+    def fill(it):
+        gi = torch.Generator(device=dev).manual_seed(100 + it)
+        x = torch.randn(1, T, hidden, device=dev, generator=gi).to(torch.bfloat16)
+        types = torch.zeros(T, dtype=torch.bool, device=dev)
+        types[torch.randperm(T, device=dev, generator=gi)[:n_act]] = True
+        return x, types.view(1, T)
+
+    x0, t0 = fill(0)
+    x_static.copy_(x0)
+    types_static.copy_(t0)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        run(x_static, types_static)  # warm-up outside the capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    want0 = run(x0, t0)
+    torch.cuda.synchronize()
+
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        out_static = run(x_static, types_static)
+    # nothing of the capture has executed: an eager call on the same tensor objects AND the capture's stream must
+    # partition for itself
+    with torch.cuda.stream(side):
+        eager_after = run(x_static, types_static)
+    side.synchronize()
+    assert torch.equal(eager_after, want0), "an eager call after the capture used state recorded inside it"
+    torch.cuda.current_stream().wait_stream(side)
+
+    for it in range(1, 4):
+        x, types = fill(it)
+        x_static.copy_(x)
+        types_static.copy_(types)
+        graph.replay()
+        got = out_static.clone()
+        torch.cuda.synchronize()
+        want = run(x, types)  # eager work between the replays, on the same inputs
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), f"replay {it} differs from the eager run"
+
+
 def test_prefill_forward_graph_replays_match_eager(dev):
     """The whole harness forward (position builder, partition, per-layer projections / M-RoPE / attention on
     PyTorch-ROCm, fused movers and both FFN launches) recorded once and replayed on fresh inputs: every replay equals

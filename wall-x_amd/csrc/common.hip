@@ -40,3 +40,15 @@ int device_cu_count() {
 
 extern "C" const char* wx_last_error_string(void) { return wx::g_error; }
 extern "C" int wx_abi_version(void) { return 1; }
+
+extern "C" int wx_stream_capture_id(wx_stream_t stream, unsigned long long* id) {
+  hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+  unsigned long long cap = 0;
+  if (hipStreamGetCaptureInfo(reinterpret_cast<hipStream_t>(stream), &status, &cap) != hipSuccess) {
+    (void)hipGetLastError();
+    return wx::fail(WX_ERR_LAUNCH, "wx_stream_capture_id: hipStreamGetCaptureInfo failed");
+  }
+  if (status != hipStreamCaptureStatusActive) cap = 0;
+  if (id != nullptr) *id = cap;
+  return status == hipStreamCaptureStatusActive ? 1 : 0;
+}

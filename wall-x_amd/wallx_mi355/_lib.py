@@ -23,6 +23,7 @@ _vp, _i64, _i32, _sz, _f32 = _c.c_void_p, _c.c_int64, _c.c_int, _c.c_size_t, _c.
 PROTOTYPES = {
     "wx_last_error_string": (_c.c_char_p, []),
     "wx_abi_version": (_i32, []),
+    "wx_stream_capture_id": (_i32, [_vp, ctypes.POINTER(ctypes.c_ulonglong)]),
     "wx_partition_workspace_bytes": (_sz, [_i64]),
     "wx_partition_build": (_i32, [_vp, _i32, _i64, _i32, _i32, _i64, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     "wx_partition_build_noalloc": (_i32, [_vp, _i32, _i64, _i32, _i32, _i64, _vp, _vp, _vp, _vp, _vp]),

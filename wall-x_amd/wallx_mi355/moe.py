@@ -62,17 +62,24 @@ class _RoutingCache(threading.local):
         self.ref = None
         self.key = None
         self.routing = None
-        self.workspace = {}  # device -> [histograms, status word]
+        self.workspace = {}  # (device, capture id) -> [histograms, status word]
 
     def lookup(self, ids: torch.Tensor, num_experts: int):
         stream = torch.cuda.current_stream(ids.device).cuda_stream if ids.is_cuda else 0
-        key = (ids._version, ids.shape, ids.dtype, ids.device, num_experts, stream)
+        # a partition recorded during a HIP graph capture has not run when the capture ends: it answers lookups of
+        # that capture only (its id is part of the key; 0 outside captures)
+        key = (ids._version, ids.shape, ids.dtype, ids.device, num_experts, stream, native.capture_id(stream))
         if self.ref is not None and self.ref() is ids and self.key == key:
             return self.routing
         flat = ids.reshape(-1)
-        row_id_map, offsets, inverse, ws = native.partition(flat, num_experts, 0, self.workspace.get(ids.device),
+        # the scratch pair of a capture stays with its graph (a fresh one per capture); eager calls share one per device
+        ws_key = (ids.device, key[-1])
+        row_id_map, offsets, inverse, ws = native.partition(flat, num_experts, 0, self.workspace.get(ws_key),
                                                             want_sorted=True)
-        self.workspace[ids.device] = ws
+        if key[-1] != 0:
+            for k in [k for k in self.workspace if k[1] not in (0, key[-1])]:
+                del self.workspace[k]
+        self.workspace[ws_key] = ws
         self.ref, self.key = weakref.ref(ids), key
         self.routing = Routing(row_id_map, offsets, flat.numel(), inverse)
         return self.routing
@@ -334,11 +341,11 @@ def moe_layer_forward(x: torch.Tensor, token_types: torch.Tensor, weights, routi
     work buffers are the per-stream pair every block shares, so `hmid` is accepted for compatibility and not used.
     """
     if routing is None:
-        dev = token_types.device
-        ws = workspace if workspace is not None else _routing_cache.workspace.get(dev)
+        ws_key = (token_types.device, native.capture_id(torch.cuda.current_stream(token_types.device).cuda_stream))
+        ws = workspace if workspace is not None else _routing_cache.workspace.get(ws_key)
         row_id_map, offsets, inverse, ws = native.partition(token_types.reshape(-1), 2, 0, ws, want_sorted=True)
         if workspace is None:
-            _routing_cache.workspace[dev] = ws
+            _routing_cache.workspace[ws_key] = ws
         routing = Routing(row_id_map, offsets, x.size(0), inverse)
     experts = _experts_for(weights)
     rows = None if host_rows is None else _lib.i64x2(host_rows)

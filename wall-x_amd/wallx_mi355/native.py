@@ -52,6 +52,24 @@ def _stream(t: torch.Tensor) -> int:
     return torch.cuda.current_stream(t.device).cuda_stream
 
 
+_capture_id_out = None
+
+
+def capture_id(stream: int) -> int:
+    """Id of the HIP graph capture `stream` is in, 0 when it is not being captured.  State kept between calls (the
+    cached token partition, the shared work buffers) is keyed on it: what is recorded during a capture has not
+    executed when the capture ends, and belongs to that graph's replays only."""
+    global _capture_id_out
+    import ctypes
+
+    if _capture_id_out is None:
+        _capture_id_out = ctypes.c_ulonglong(0)
+    rc = _lib.load().wx_stream_capture_id(stream, ctypes.byref(_capture_id_out))
+    if rc < 0:
+        _lib.check(rc)
+    return int(_capture_id_out.value) if rc == 1 else 0
+
+
 def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
     if t is None or t.numel() == 0:
         return None
@@ -661,23 +679,28 @@ def dual_swiglu_ffn_packed(x_tiled: torch.Tensor, num_rows: int, expert_offsets:
     return out
 
 
-_ffn_scratch = {}  # (device index, stream handle) -> (tiled activations, intermediate), grown on demand
+_ffn_scratch = {}  # (device index, stream handle, capturing) -> (tiled activations, intermediate, capture id)
 
 
 def _ffn_buffers(device: torch.device, stream: int, x_elems: int, h_elems: int):
     """The tiled-activation and intermediate buffers of the block forward, one pair per device and stream: the
     layers of a model run one after the other on a stream, so they can all work in the same two buffers (a pair per
     block would hold 0.45 GB per layer at 29 184 tokens).  Calls that overlap on one stream's pair from two threads
-    race, like any two launches writing one buffer."""
-    key = (device.index, stream)
+    race, like any two launches writing one buffer.  Under HIP graph capture the pair belongs to that capture (its
+    memory comes from the graph's pool and its replays write it): eager calls never share it, and a later capture on
+    the same stream replaces it."""
+    cap = capture_id(stream)
+    key = (device.index, stream, cap != 0)
     hit = _ffn_scratch.get(key)
+    if hit is not None and hit[2] != cap:
+        hit = None  # another capture's pair
     if hit is None or hit[0].numel() < x_elems or hit[1].numel() < h_elems:
         if hit is not None:
             x_elems, h_elems = max(x_elems, hit[0].numel()), max(h_elems, hit[1].numel())
         hit = (torch.empty(x_elems, dtype=torch.bfloat16, device=device),
-               torch.empty(h_elems, dtype=torch.bfloat16, device=device))
+               torch.empty(h_elems, dtype=torch.bfloat16, device=device), cap)
         _ffn_scratch[key] = hit
-    return hit
+    return hit[0], hit[1]
 
 
 def release_ffn_buffers() -> None:
