@@ -5,6 +5,7 @@ torch is used for allocation and stream lookup only; every computation is a HIP 
 Nothing here falls back to PyTorch math: without the library, or with CPU tensors, calls raise.
 """
 
+import ctypes
 import os
 import warnings
 from typing import List, Optional, Tuple
@@ -52,22 +53,15 @@ def _stream(t: torch.Tensor) -> int:
     return torch.cuda.current_stream(t.device).cuda_stream
 
 
-_capture_id_out = None
-
-
 def capture_id(stream: int) -> int:
     """Id of the HIP graph capture `stream` is in, 0 when it is not being captured.  State kept between calls (the
     cached token partition, the shared work buffers) is keyed on it: what is recorded during a capture has not
     executed when the capture ends, and belongs to that graph's replays only."""
-    global _capture_id_out
-    import ctypes
-
-    if _capture_id_out is None:
-        _capture_id_out = ctypes.c_ulonglong(0)
-    rc = _lib.load().wx_stream_capture_id(stream, ctypes.byref(_capture_id_out))
+    out = ctypes.c_ulonglong(0)  # per call: the library call runs without the interpreter lock
+    rc = _lib.load().wx_stream_capture_id(stream, ctypes.byref(out))
     if rc < 0:
         _lib.check(rc)
-    return int(_capture_id_out.value) if rc == 1 else 0
+    return int(out.value) if rc == 1 else 0
 
 
 def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
