@@ -519,10 +519,11 @@ def backward_measurement(dev, x, weights, m0):
 
 
 def training_step_measurement(dev, x, token_types, weights):
-    """Forward + backward of the drop-in SparseMoeBlock (wallx_mi355/moe.py) on the config 3 batch: the fused forward,
-    then the block's own backward (gate / up recomputed, SwiGLU derivative in one elementwise kernel, dX and dW of
-    all three projections of both experts as dual GEMMs in their K-major layouts).  FLOPs counted as 3 x forward
-    (the recompute, one third more, is not counted)."""
+    """Forward + backward of the drop-in SparseMoeBlock (wallx_mi355/moe.py) on the config 3 batch: the fused forward
+    (which keeps the gate / up projections), then the block's own backward (SwiGLU derivative in one elementwise
+    kernel, dX and dW of all three projections of both experts as dual GEMMs in their K-major layouts).  FLOPs
+    counted as 3 x forward.  Also timed with the VL expert frozen, the reference's freeze_vlm fine-tuning mode
+    (qwen_vl_act_trainer.py:530-536): its three weight gradients leave the launches."""
     import torch
     from types import SimpleNamespace
     from wallx_mi355 import moe
@@ -557,6 +558,10 @@ def training_step_measurement(dev, x, token_types, weights):
     flops = 6.0 * H * ((x.shape[0] - m1) * inters[0] + m1 * inters[1])
     out = {"forward_ms": round(t_f, 3), "forward_backward_ms": round(t_s, 3),
            "tflops_counting_3x_forward": round(3 * flops / t_s / 1e9, 1)}
+    for prm in block.experts[0].parameters():
+        prm.requires_grad_(False)
+    t_fz, _ = event_ms(step, 5, warm=2)
+    out["forward_backward_ms_vl_expert_frozen"] = round(t_fz, 3)
     del block, xb, dy
     torch.cuda.empty_cache()
     return out

@@ -332,7 +332,8 @@ int wx_swiglu_bwd(const void* gate, const void* up, const void* dh, void* hmid, 
                   int64_t num_elems, wx_stream_t stream);
 /* The same with gate and up of ONE expert read from the K-tiled buffers wx_dual_swiglu_gate_up_keep filled:
  * gate_tiled / up_tiled point at that expert's tiled matrix of tiled_rows rows (its row count rounded up to 256) and
- * cols columns; dh and the three outputs are row-major [rows, cols].  cols a multiple of 64. */
+ * cols columns; dh and the three outputs are row-major [rows, cols].  cols a multiple of 64.  hmid may be NULL when
+ * the caller does not need it (the expert's down projection does not train). */
 int wx_swiglu_bwd_tiled(const void* gate_tiled, const void* up_tiled, int64_t tiled_rows, const void* dh, void* hmid,
                         void* dgate, void* dup, int64_t rows, int64_t cols, wx_stream_t stream);
 

@@ -629,3 +629,39 @@ def test_moe_block_backward_matches_autograd_of_the_plain_forward(dev, fused_ext
             scale = float(wref.grad.abs().max())
             err = float((got.float().cpu() - wref.grad).abs().max())
             assert err <= 0.03 * scale + 1e-3, f"expert {e} {name}: max err {err} at scale {scale}"
+
+
+@pytest.mark.parametrize("frozen_expert", [0, 1])
+def test_moe_block_backward_with_one_expert_frozen(dev, frozen_expert):
+    """Fine-tuning with one expert frozen (the reference's freeze_vlm mode trains `moe.experts.1.*` alone,
+    qwen_vl_act_trainer.py:530-536): the frozen expert's weights get no gradient (and its three weight-gradient
+    products leave the launches), every other gradient equals the one of the fully trainable block bit for bit."""
+    class Cfg:
+        experts = [{"hidden_size": 128, "intermediate_size": 320, "hidden_act": "silu"},
+                   {"hidden_size": 128, "intermediate_size": 128, "hidden_act": "silu"}]
+
+    g = torch.Generator().manual_seed(13)
+    block = moe.SparseMoeBlock(Cfg(), 2).to(torch.bfloat16)
+    with torch.no_grad():
+        for prm in block.parameters():
+            prm.copy_(_bf(prm.shape, g, 0.08))
+    block = block.to(dev)
+    x = _bf((1, 700, 128), g).to(dev)
+    types = (torch.rand(1, 700, generator=g) > 0.6).to(dev)
+    dy = _bf((1, 700, 128), g).to(dev)
+
+    def grads():
+        for prm in block.parameters():
+            prm.grad = None
+        xd = x.clone().requires_grad_(True)
+        block(xd, types).backward(dy)
+        return xd.grad, [[w.grad for w in e.weights()] for e in block.experts]
+
+    dx_all, w_all = grads()
+    for prm in block.experts[frozen_expert].parameters():
+        prm.requires_grad_(False)
+    dx, w = grads()
+    assert torch.equal(dx, dx_all)
+    assert all(t is None for t in w[frozen_expert])
+    for got, want in zip(w[1 - frozen_expert], w_all[1 - frozen_expert]):
+        assert got is not None and torch.equal(got, want)

@@ -57,7 +57,7 @@ __global__ __launch_bounds__(256) void swiglu_bwd_tiled_kernel(const unsigned ch
     u32x4 hv, dgv, duv;
     swiglu_bwd_8(*reinterpret_cast<const u32x4*>(gate_t + t_off), *reinterpret_cast<const u32x4*>(up_t + t_off),
                  __builtin_nontemporal_load(dh + rm), hv, dgv, duv);
-    __builtin_nontemporal_store(hv, hmid + rm);
+    if (hmid != nullptr) __builtin_nontemporal_store(hv, hmid + rm);
     __builtin_nontemporal_store(dgv, dgate + rm);
     __builtin_nontemporal_store(duv, dup + rm);
   }
@@ -110,8 +110,8 @@ extern "C" int wx_swiglu_bwd_tiled(const void* gate_tiled, const void* up_tiled,
   if (cols % 64 != 0 || tiled_rows % kBlkRows != 0)
     return fail(WX_ERR_UNSUPPORTED, "%s: cols must be a multiple of 64 and tiled_rows of 16", who);
   if (rows == 0 || cols == 0) return WX_OK;
-  if (!gate_tiled || !up_tiled || !dh || !hmid || !dgate || !dup) return fail(WX_ERR_INVALID_ARGUMENT, "%s: null pointer", who);
-  const void* all[6] = {gate_tiled, up_tiled, dh, hmid, dgate, dup};
+  if (!gate_tiled || !up_tiled || !dh || !dgate || !dup) return fail(WX_ERR_INVALID_ARGUMENT, "%s: null pointer", who);
+  const void* all[6] = {gate_tiled, up_tiled, dh, hmid, dgate, dup};  // hmid may be null: that output is not wanted
   for (const void* ptr : all)
     if (reinterpret_cast<uintptr_t>(ptr) & 15) return fail(WX_ERR_INVALID_ARGUMENT, "%s: buffers must be 16-byte aligned", who);
   const int64_t units = (rows + kBlkRows - 1) / kBlkRows * (cols / 64) * 2;

@@ -88,13 +88,24 @@ class _RoutingCache(threading.local):
 _routing_cache = _RoutingCache()
 
 
-def _dual(a0, a1, w0, w1, n0, n1, trans_a, trans_b):
+def _dual(a0, a1, w0, w1, n0, n1, trans_a, trans_b, want=(True, True)):
+    """Both experts' products in one launch; an expert whose result nobody asked for (want[e] False) is given an empty
+    row range, leaves the launch's tile list, and comes back as None."""
+    ref = a0 if a0 is not None else a1
+
+    def absent(n):  # operands of an empty problem with n output columns (either may have been left out by the caller)
+        return ref.new_empty((0, 0)), ref.new_empty((n, 0) if trans_b else (0, n))
+
+    if not want[0]:
+        a0, w0 = absent(n0)
+    if not want[1]:
+        a1, w1 = absent(n1)
     m0 = a0.size(1) if trans_a else a0.size(0)
     m1 = a1.size(1) if trans_a else a1.size(0)
     o0 = torch.empty(m0, n0, dtype=torch.bfloat16, device=a0.device)
     o1 = torch.empty(m1, n1, dtype=torch.bfloat16, device=a0.device)
     native.asym_dual_gmm(a0, a1, w0, w1, o0, o1, trans_a, trans_b)
-    return o0, o1
+    return (o0 if want[0] else None), (o1 if want[1] else None)
 
 
 class _MoeBlockFunction(torch.autograd.Function):
@@ -117,10 +128,12 @@ class _MoeBlockFunction(torch.autograd.Function):
         I0, I1 = weights[0].size(0), weights[3].size(0)
         ctx.keep = I0 % 64 == 0 and I1 % 64 == 0
         # weights that train are repacked on every forward: writes through `.data` (master-weight or EMA copies) do
-        # not move the version counter a cached copy would be checked against
+        # not move the version counter a cached copy would be checked against.  Frozen ones keep their packed copies.
+        frozen = tuple(not n for n in ctx.needs_input_grad[5:11])
         if ctx.keep:
             y, gate_keep, up_keep, scratch["hmid"] = native.dual_swiglu_ffn_keep(
-                scratch["x_tiled"], T, expert_offsets, w, hmid=scratch.get("hmid"), out_row_id=sorted_row_id)
+                scratch["x_tiled"], T, expert_offsets, w, hmid=scratch.get("hmid"), out_row_id=sorted_row_id,
+                frozen=frozen)
             if sorted_row_id is None:
                 y = native.unpermute(y, row_id_map, torch.tensor([]), T, 1)
             ctx.save_for_backward(x, row_id_map, expert_offsets, gate_keep, up_keep, *weights)
@@ -128,9 +141,9 @@ class _MoeBlockFunction(torch.autograd.Function):
         ctx.save_for_backward(x, row_id_map, expert_offsets, *weights)
         if sorted_row_id is not None:
             return native.dual_swiglu_ffn(scratch["x_tiled"], T, expert_offsets, w, hmid=scratch.get("hmid"),
-                                          out_row_id=sorted_row_id, cache_packed=False)
+                                          out_row_id=sorted_row_id, cache_packed=frozen)
         y_sorted = native.dual_swiglu_ffn(scratch["x_tiled"], T, expert_offsets, w, hmid=scratch.get("hmid"),
-                                          cache_packed=False)
+                                          cache_packed=frozen)
         return native.unpermute(y_sorted, row_id_map, torch.tensor([]), T, 1)
 
     @staticmethod
@@ -140,6 +153,7 @@ class _MoeBlockFunction(torch.autograd.Function):
         else:
             x, row_id_map, expert_offsets, g0, u0, d0, g1, u1, d1 = ctx.saved_tensors
         T, H = x.shape
+        need = ctx.needs_input_grad
         o = expert_offsets.cpu().tolist()
         m0, m1 = o[1] - o[0], o[2] - o[1]
         xs = native.permute_rows(x.detach(), row_id_map, 1, T)
@@ -151,21 +165,23 @@ class _MoeBlockFunction(torch.autograd.Function):
         if ctx.keep:
             pad0 = (m0 + 255) // 256 * 256
             pad1 = (m1 + 255) // 256 * 256
-            hm0, dg0, du0 = native.swiglu_bwd_tiled(gate_keep, up_keep, 0, pad0, dh0)
-            hm1, dg1, du1 = native.swiglu_bwd_tiled(gate_keep, up_keep, pad0 * I0, pad1, dh1)
+            # the forward's hmid in row-major form is read by the down projection's weight gradient only
+            hm0, dg0, du0 = native.swiglu_bwd_tiled(gate_keep, up_keep, 0, pad0, dh0, want_hmid=need[7])
+            hm1, dg1, du1 = native.swiglu_bwd_tiled(gate_keep, up_keep, pad0 * I0, pad1, dh1, want_hmid=need[10])
         else:
             ga0, ga1 = _dual(x0, x1, g0, g1, I0, I1, False, True)
             up0, up1 = _dual(x0, x1, u0, u1, I0, I1, False, True)
             hm0, dg0, du0 = native.swiglu_bwd(ga0, up0, dh0)
             hm1, dg1, du1 = native.swiglu_bwd(ga1, up1, dh1)
-        need = ctx.needs_input_grad
         grads = [None] * 6
+        # weight gradients only of the experts that train: fine-tuning with the VL side frozen (the reference's
+        # freeze_vlm mode trains `moe.experts.1.*` alone, qwen_vl_act_trainer.py:530-536) skips the three large ones
         if need[5] or need[8]:  # gate weights
-            grads[0], grads[3] = _dual(dg0, dg1, x0, x1, H, H, True, False)
+            grads[0], grads[3] = _dual(dg0, dg1, x0, x1, H, H, True, False, want=(need[5], need[8]))
         if need[6] or need[9]:  # up weights
-            grads[1], grads[4] = _dual(du0, du1, x0, x1, H, H, True, False)
+            grads[1], grads[4] = _dual(du0, du1, x0, x1, H, H, True, False, want=(need[6], need[9]))
         if need[7] or need[10]:  # down weights
-            grads[2], grads[5] = _dual(dy0, dy1, hm0, hm1, I0, I1, True, False)
+            grads[2], grads[5] = _dual(dy0, dy1, hm0, hm1, I0, I1, True, False, want=(need[7], need[10]))
         dx = None
         if need[0]:
             # dX = dG Wg + dU Wu: the second product accumulates onto the first in its epilogue (bf16 + bf16, rounded

@@ -789,14 +789,16 @@ def packed_block_forward(experts: PackedExperts, x: torch.Tensor, row_id_map: to
 
 def dual_swiglu_ffn_keep(x_tiled: torch.Tensor, num_rows: int, expert_offsets: torch.Tensor, weights,
                          hmid: Optional[torch.Tensor] = None, host_rows=None,
-                         out_row_id: Optional[torch.Tensor] = None):
+                         out_row_id: Optional[torch.Tensor] = None, frozen=None):
     """dual_swiglu_ffn for a forward pass whose backward follows: the gate / up launch also stores the two
     projections (K-tiled, the intermediate's geometry) so the backward need not run them again.  The weights are
-    packed afresh (they train).  Returns (out, gate_keep, up_keep, hmid)."""
+    packed afresh (they train), except those flagged in `frozen` (six booleans in the order gate0, up0, down0, gate1,
+    up1, down1), whose packed copies are cached like an inference forward's.  Returns (out, gate_keep, up_keep, hmid)."""
     _need_cuda("x_tiled", x_tiled)
     (g0, u0, d0), (g1, u1, d1) = weights
     H, I0, I1 = g0.size(1), g0.size(0), g1.size(0)
-    packed = [pack_weight(w, cache=False) for w in (g0, u0, d0, g1, u1, d1)]
+    cached = tuple(frozen) if frozen is not None else (False,) * 6
+    packed = [pack_weight(w, cache=c) for w, c in zip((g0, u0, d0, g1, u1, d1), cached)]
     dev = x_tiled.device
     need = padded_sorted_rows(num_rows) * max(I0, I1)
     if hmid is None or hmid.numel() < need or hmid.dtype != torch.bfloat16:
@@ -816,16 +818,18 @@ def dual_swiglu_ffn_keep(x_tiled: torch.Tensor, num_rows: int, expert_offsets: t
 
 
 def swiglu_bwd_tiled(gate_keep: torch.Tensor, up_keep: torch.Tensor, elem_offset: int, tiled_rows: int,
-                     dh: torch.Tensor):
+                     dh: torch.Tensor, want_hmid: bool = True):
     """(hmid, dgate, dup), row-major like dh [rows, cols], of h = silu(gate) * up for one expert whose gate / up
     projections sit K-tiled in the buffers dual_swiglu_ffn_keep returned, at element offset `elem_offset`, as a
-    matrix of `tiled_rows` rows (the expert's row count rounded up to 256)."""
+    matrix of `tiled_rows` rows (the expert's row count rounded up to 256).  hmid is None (and not computed) without
+    want_hmid: only the down projection's weight gradient reads it."""
     _need_cuda("dh", dh)
     if dh.dtype != torch.bfloat16 or gate_keep.dtype != torch.bfloat16 or up_keep.dtype != torch.bfloat16:
         raise RuntimeError("All tensors must be BFloat16 for this kernel")
     dh = dh.contiguous()
     rows, cols = dh.shape
-    hm, dg, du = torch.empty_like(dh), torch.empty_like(dh), torch.empty_like(dh)
+    hm = torch.empty_like(dh) if want_hmid else None
+    dg, du = torch.empty_like(dh), torch.empty_like(dh)
     if rows == 0:
         return hm, dg, du
     with _DeviceGuard(dh):
@@ -842,7 +846,7 @@ def dual_swiglu_ffn(x_tiled: torch.Tensor, num_rows: int, expert_offsets: torch.
 
     x_tiled: result of permute_rows_tiled for num_rows tokens; expert_offsets int32 [3] ON THE DEVICE (from
     partition()); weights = ((gate0, up0, down0), (gate1, up1, down1)) in nn.Linear layout (packed here; the
-    packed copies are cached per tensor unless cache_packed is False).  host_rows: optional (rows of expert 0, rows
+    packed copies are cached per tensor unless cache_packed is False, or per weight where it is six booleans).  host_rows: optional (rows of expert 0, rows
     of expert 1) as host integers, when the caller has them
     anyway; they only spare the library a second, empty launch when it cannot tell which tile shape fits.
     out_row_id: optional int32 [num_rows] CUDA tensor, the partition's sorted_row_id; with it the result comes back
@@ -855,6 +859,7 @@ def dual_swiglu_ffn(x_tiled: torch.Tensor, num_rows: int, expert_offsets: torch.
     if tuple(g0.shape) != (I0, H) or tuple(u0.shape) != (I0, H) or tuple(d0.shape) != (H, I0) or \
             tuple(g1.shape) != (I1, H) or tuple(u1.shape) != (I1, H) or tuple(d1.shape) != (H, I1):
         raise RuntimeError("expert weight shapes are inconsistent with hidden size")
-    packed = [pack_weight(w, cache=cache_packed) for w in (g0, u0, d0, g1, u1, d1)]
+    cached = tuple(cache_packed) if isinstance(cache_packed, (tuple, list)) else (bool(cache_packed),) * 6
+    packed = [pack_weight(w, cache=c) for w, c in zip((g0, u0, d0, g1, u1, d1), cached)]
     return dual_swiglu_ffn_packed(x_tiled, num_rows, expert_offsets, packed, (H, I0, I1), hmid, out, host_rows,
                                   out_row_id)
