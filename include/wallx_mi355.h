@@ -325,7 +325,7 @@ int wx_unpermute_rows_add_rmsnorm(const void* y, const void* residual, void* out
                                   int64_t num_tokens, int64_t num_cols, wx_stream_t stream);
 
 /* Elementwise backward of h = silu(g) * u inside an expert FFN (act.py:79-82; the reference leaves it to autograd):
- * from gate, up (the two projections, recomputed) and dh (gradient w.r.t. h) in one pass:
+ * from gate, up (the two projections, kept by the forward or recomputed) and dh (gradient w.r.t. h) in one pass:
  * hmid = bf16(bf16(silu(g)) * u) as the forward fed it to the down projection, dgate = dh * u * s * (1 + g * (1 - s))
  * with s = sigmoid(g), dup = dh * silu(g).  bf16 in and out, fp32 math; num_elems a multiple of 8. */
 int wx_swiglu_bwd(const void* gate, const void* up, const void* dh, void* hmid, void* dgate, void* dup,

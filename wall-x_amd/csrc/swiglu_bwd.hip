@@ -1,6 +1,6 @@
 // Elementwise backward of the SwiGLU inside an expert FFN, h = silu(g) * u (act.py:79-82), for the block's training
-// path.  One pass reads gate, up (the recomputed projections) and dh (the gradient arriving from the down
-// projection) and writes the three tensors the remaining GEMMs need:
+// path.  One pass reads gate, up (the two projections, kept by the forward or recomputed) and dh (the gradient
+// arriving from the down projection) and writes the three tensors the remaining GEMMs need:
 //   hmid  = bf16(bf16(silu(g)) * u)           what the forward fed to the down projection (its eager rounding)
 //   dgate = dh * u * s * (1 + g * (1 - s))    with s = sigmoid(g)
 //   dup   = dh * silu(g)

@@ -2,10 +2,11 @@
 
 The reference's SparseMoeBlock permutes the tokens, loops over the experts in Python (six cuBLAS GEMMs,
 four elementwise kernels and two slice copies per layer, bounds read from CPU tensors) and unpermutes.
-Here one layer is: partition (2 small launches, reusable across layers) -> row scatter into the K-tiled
-activation layout -> gate/up + SwiGLU for both experts (1 launch) -> down for both experts (1 launch) -> row
-gather.  Expert weights are packed into the same K-tiled layout once and cached.  The per-expert row ranges
-stay on the device (expert_offsets from the partition), so nothing synchronises with the host.
+Here one layer is: partition (1 or 2 small launches, once per forward: every layer reuses it) -> row gather into
+the K-tiled activation layout -> gate/up + SwiGLU for both experts (1 launch) -> down for both experts (1 launch)
+whose stores put each row at its token's position (and add the layer's residual when asked to).  Expert weights
+are packed into the same K-tiled layout once and cached.  The per-expert row ranges stay on the device
+(expert_offsets from the partition), so nothing synchronises with the host.
 
 Parameter names match the reference (``experts.{e}.{gate,up,down}_proj.weight``), so its checkpoints load.
 """
