@@ -254,9 +254,11 @@ def main():
         side("ceilings", ceiling_measurements, dev, x, weights, m0)
     if not args.ops_only and not args.no_prefill:
         del x_tiled, hmid, x_sorted, y_sorted, y
-        side("prefill", prefill_measurement, dev, args.prefill_mask, False)
-        # the same forward with the q / k / v projection and M-RoPE as one launch of this library's GEMM
-        side("prefill_qkv_rope_in_gemm_epilogue", prefill_measurement, dev, args.prefill_mask, True)
+        # the harness as it stands: q / k / v projection with bias and M-RoPE in one launch of this library's GEMM, the
+        # o projection with its residual add on the same kernel
+        side("prefill", prefill_measurement, dev, args.prefill_mask, True)
+        # the same forward with both projections on the vendor GEMM (F.linear / addmm) and M-RoPE as its own pass
+        side("prefill_vendor_projections", prefill_measurement, dev, args.prefill_mask, False)
 
     traffic, traffic_source = measured_traffic("gate_up")
     result = {
@@ -613,14 +615,15 @@ def ceiling_measurements(dev, x, weights, m0):
     return out
 
 
-def prefill_measurement(dev, mask, fuse_qkv_rope=False):
+def prefill_measurement(dev, mask, native_projections=True):
     """BASELINE config 5: one prefill of 16 x 912 tokens through a randomly initialised 36-layer decoder of the
-    Qwen2.5-VL-3B shape with the dual-expert FFN in every layer; attention, projections and norms on PyTorch."""
+    Qwen2.5-VL-3B shape with the dual-expert FFN in every layer; attention on PyTorch, the projections on this
+    library's GEMM (native_projections) or the vendor's."""
     import torch
     from wallx_mi355 import harness
 
     model = harness.PrefillHarness(device=dev, mask="causal" if mask == "causal" else "action_block",
-                                   fuse_qkv_rope=fuse_qkv_rope)
+                                   fuse_qkv_rope=native_projections, o_proj_native=native_projections)
     ids, grid, types = harness.config5_inputs(16, dev)
     suffix = 32 if mask == "action_block" else None  # config 5: the 32 action tokens close every row
     if suffix is not None and not (bool(types[:, -suffix:].all()) and not bool(types[:, :-suffix].any())):
@@ -641,8 +644,9 @@ def prefill_measurement(dev, mask, fuse_qkv_rope=False):
     del model
     torch.cuda.empty_cache()
     return {
-        "qkv_projection": "this library's GEMM with bias and M-RoPE in its epilogue (wx_qkv_rope_proj)" if fuse_qkv_rope
-                          else "vendor GEMM (F.linear), then the M-RoPE kernel",
+        "projections": "this library's GEMM: q / k / v with bias and M-RoPE in its epilogue (wx_qkv_rope_proj), o with "
+                       "the residual add in its epilogue (wx_dual_gemm_add)" if native_projections
+                       else "vendor GEMM (F.linear, addmm); M-RoPE as its own kernel",
         "workload": "config 5 (BASELINE.json configs[4]): 36 layers, hidden 2048, 16 q / 2 kv heads x 128, experts "
                     "11008 / 1024, 16 x 912 tokens (32 action each), bf16, random init, rms eps 1e-6, mask " +
                     {"action_block": "causal + bidirectional action block (act.py:616-637) as two maskless attention calls",

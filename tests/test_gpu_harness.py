@@ -53,7 +53,8 @@ def test_prefill_harness_matches_plain_forward(dev, mask_mode, fuse, suffix, qkv
     from wallx_mi355 import harness
 
     h = harness.PrefillHarness(n_layers=2, hidden=256, n_q=4, n_kv=2, head_dim=128, inter=(512, 256), vocab=151936,
-                               device=dev, seed=3, mask=mask_mode, keep_dense=True, fuse=fuse, fuse_qkv_rope=qkv)
+                               device=dev, seed=3, mask=mask_mode, keep_dense=True, fuse=fuse, fuse_qkv_rope=qkv,
+                               o_proj_native=qkv)
     row = wl.vla_row_tokens(n_images=1, image_tokens=16, lead_text=5, tail_text=9, n_action=8)
     ids = torch.tensor([row, row, row], dtype=torch.int64, device=dev)
     grid = torch.tensor([[1, 8, 8]] * 3, dtype=torch.int64, device=dev)
@@ -99,10 +100,19 @@ def test_config5_full_shape_piece_by_piece(dev):
                       act[torch.randperm(act.numel(), generator=g)[:12]], act[:2], act[-2:]])
     for li in layers:
         c = cap[li]
-        # M-RoPE inside the forward (cos / sin evaluated in the kernel from the position ids): two batch rows in full
+        # M-RoPE inside the forward (cos / sin evaluated on the device from the position ids): two batch rows in full.
+        # With the rotation in the projection's epilogue (the default) q and k before the rotation exist nowhere on
+        # the device: the oracle projects the captured layer input with the layer's weights itself.
         for b in (0, 15):
-            rq, rk = oracle.mrope_apply_ref(c["q_in"][b:b + 1].cpu(), c["k_in"][b:b + 1].cpu(), cos[:, b:b + 1],
-                                            sin[:, b:b + 1], list(wl.MROPE_SECTION))
+            if "q_in" in c:
+                q_in, k_in = c["q_in"][b:b + 1].cpu(), c["k_in"][b:b + 1].cpu()
+            else:
+                lay = h.layers[li]
+                qkv = torch.nn.functional.linear(c["x_in"][b].float().cpu(), lay["wqkv"].float().cpu(),
+                                                 lay["bqkv"].float().cpu()).to(torch.bfloat16)
+                q_in = qkv[:, :h.n_q * 128].reshape(1, -1, h.n_q, 128).transpose(1, 2)
+                k_in = qkv[:, h.n_q * 128:(h.n_q + h.n_kv) * 128].reshape(1, -1, h.n_kv, 128).transpose(1, 2)
+            rq, rk = oracle.mrope_apply_ref(q_in, k_in, cos[:, b:b + 1], sin[:, b:b + 1], list(wl.MROPE_SECTION))
             for got, ref, what in ((c["q_out"][b:b + 1], rq, "q"), (c["k_out"][b:b + 1], rk, "k")):
                 err = (got.float().cpu() - ref.float()).abs()
                 assert bool((err <= 2e-2 + 1e-2 * ref.float().abs()).all()), f"layer {li} M-RoPE {what}: {float(err.max())}"

@@ -8,8 +8,8 @@
 //
 // Workgroup tile 256 x 256, K step 32, one workgroup per CU: eight wavefronts (two per SIMD) as 2 x 4, wave tile
 // 128 x 64 = 4 x 2 MFMA 32x32x16 accumulator blocks (128 accumulator registers per lane), of which one per SIMD
-// issues the global -> LDS loads; the projection that rotates heads in its epilogue runs the same tile with four
-// wavefronts as 2 x 2 (wave tile 128 x 128, 256 accumulator registers).  Problems whose 256 x 256
+// issues the global -> LDS loads; the projection that rotates heads in its epilogue runs the same tile with the
+// wavefronts as 4 x 2 (wave tile 64 x 128: a wavefront holds whole heads).  Problems whose 256 x 256
 // tiles would leave most CUs idle (a denoise step of a few thousand action tokens) run the same kernel with a
 // 128 x 128 tile, two workgroups per CU.  A ragged last round of the fused FFN launches (tiles left over after the
 // whole rounds of one tile per CU) runs in that small shape too, in a second launch, when it then fits the chip in
@@ -24,12 +24,14 @@
 //   generic  (wx_dual_gemm)            A, B, C row-major; loads touch 16 rows x 64 bytes per instruction.  An
 //                                      operand stored with K as its slow dimension (A as [k, m], B as [k, n]: the
 //                                      backward GEMMs) is loaded as K rows of 256 columns and transposed by the LDS
-//                                      reads (ds_read_b64_tr_b16), so no layout needs a transposed copy.
+//                                      reads (ds_read_b64_tr_b16), so no layout needs a transposed copy.  An
+//                                      addend of C's shape can be summed in the epilogue (wx_dual_gemm_add).
 //   gate/up  (wx_dual_swiglu_gate_up)  A = K-tiled activations, B = K-tiled gate and up weights (the B tile is 128
 //                                      gate rows + 128 up rows of the same output columns, so gate and up of an
 //                                      output element meet in one lane), C = K-tiled intermediate, SwiGLU epilogue.
 //   down     (wx_dual_down_proj)       A = K-tiled intermediate, B = K-tiled down weights, C row-major; with a row
-//                                      id list the rows go straight to their token positions (the unpermute).
+//                                      id list the rows go straight to their token positions (the unpermute), and
+//                                      a residual matrix can be added there on the way (the layer's closing add).
 //   qkv+rope (wx_qkv_rope_proj)        A, B, C row-major like the generic mode, one group; bias and the rotary
 //                                      embedding of the q and k heads are applied to the accumulators.
 // With K-tiled operands every load instruction moves one contiguous KiB (tiled_layout.h).
@@ -69,7 +71,7 @@ struct TileShape {
   static constexpr int kLoadsB = kLoadRowsB / 16;     // ... and B
   static constexpr int kSlotBytesA = BM * kRowBytes;  // bytes of A per K step
   static constexpr int kSlotBytesB = BN * kRowBytes;
-  static constexpr int kStageBytes = FN >= 4 ? 8192 : 2048;  // per-wave staging for the epilogue
+  static constexpr int kStageBytes = FN >= 4 ? (kWaves > 4 ? 4096 : 8192) : 2048;  // per-wave staging for the epilogue
   static constexpr int kLdsBytes = kStages * (kSlotBytesA + kSlotBytesB) + kWaves * kStageBytes;
   static constexpr int kWgPerCu = kLdsBytes <= 80 * 1024 && FM * FN * 16 <= 128 ? 2 : 1;
   static_assert(kLdsBytes <= 160 * 1024, "LDS budget");
@@ -89,9 +91,12 @@ using BigTile8 = TileShape<256, 256, 2, 4, 4>;
 // measure 6 % slower on a denoise step; timestamps inside that kernel put 254 ns on a K step whose 8 MFMAs per
 // wavefront need 110, and 169 ns with the loads taken out.)
 using SmallTile = TileShape<128, 128, 4, 2, 4>;
-// The large tile of a launch: BigTile8, except where the epilogue needs a wavefront to hold whole 128-column heads.
+// the same eight wavefronts as 4 x 2: wave tile 64 x 128, for the epilogue that needs a wavefront to hold whole
+// 128-column heads (the rotation partner of a channel is 64 columns away)
+using BigTile8Q = TileShape<256, 256, 4, 2, 4>;
+// The large tile of a launch.
 template <int MODE>
-using BigTileFor = std::conditional_t<MODE == 3 /* kQkvRope */, BigTile, BigTile8>;
+using BigTileFor = std::conditional_t<MODE == 3 /* kQkvRope */, BigTile8Q, BigTile8>;
 // the shape that runs the ragged last round of a launch (see tail_split_point): BigTile cut in four.  (Cut in two,
 // 256 x 128 with one workgroup per CU, measures the same.)
 using TailTile = SmallTile;
@@ -743,7 +748,7 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
         // head; channel d of the head sits in block d / 32 at lane d % 32, so its rotation partner d +/- 64 is two
         // blocks away in the same lane.  Evaluated like eager bf16 code: the projection (with its bias) rounded once,
         // then q * cos + rotate_half(q) * sin with each product and the sum rounded (vl.py:771-772).
-        static_assert(FN == 4 && FM * 32 == 128, "a wavefront covers whole heads of 128 channels");
+        static_assert(FN == 4, "a wavefront covers whole heads of 128 channels");
         const int col_w = S.col0 + wn * 128;  // first output column of this wavefront's head
         const bool live = wn * 128 < S.cols_left;
         float bias_v[4] = {0.f, 0.f, 0.f, 0.f};
@@ -1201,7 +1206,8 @@ extern "C" int wx_qkv_rope_proj(const void* x, const void* weight, const void* b
   p.rope_table = rope_table;
   p.rope_cols = (n_q_heads + n_kv_heads) * head_dim;
   // the large tile only: its wavefronts cover whole heads (the small tile's 64 columns would split a rotation pair)
-  hipLaunchKernelGGL((dual_gemm_kernel<kQkvRope, BigTile, false, false>), dim3(device_cu_count()), dim3(BigTile::kThreads),
+  using Tile = BigTileFor<kQkvRope>;
+  hipLaunchKernelGGL((dual_gemm_kernel<kQkvRope, Tile, false, false>), dim3(device_cu_count()), dim3(Tile::kThreads),
                      0, as_stream(stream), p);
   return check_launch("dual_gemm_kernel<qkv_rope>");
 }

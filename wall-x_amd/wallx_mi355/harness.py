@@ -1,7 +1,8 @@
 """Prefill harness for BASELINE config 5: a randomly initialised decoder with the Qwen2.5-VL-3B shape and the
 dual VL / action expert FFN in every layer (act.py:172-273, 397-530), with every layer's permute, grouped GEMM,
-M-RoPE and the position builder replaced by the MI355X kernels.  RMSNorm, the QKV / O projections and attention
-stay on PyTorch-ROCm (attention = F.scaled_dot_product_attention), as the configuration prescribes.
+M-RoPE and the position builder replaced by the MI355X kernels.  Attention stays on PyTorch-ROCm
+(F.scaled_dot_product_attention), as the configuration prescribes; the QKV / O projections run on this library's
+GEMM by default (they carry the rotary embedding and the residual add in their epilogues) or on the vendor's.
 
 This is a measurement harness, not a model port: no KV cache, no generation, no losses; one forward over a
 batch of full sequences (prefill).  What it states explicitly:
@@ -17,8 +18,10 @@ batch of full sequences (prefill).  What it states explicitly:
     evaluates cos/sin from the position ids in the kernel (no [3, B, S, D] tables) and leaves q / k token-major,
     and the attention residual is added by the o-projection GEMM; `fuse=False` keeps all of these as separate
     PyTorch ops,
-  * `fuse_qkv_rope=True` replaces the vendor GEMM of the q / k / v projection and the rope kernel by one launch of
-    this library's GEMM with bias and M-RoPE in its epilogue (vl.py:955-964).
+  * `fuse_qkv_rope=True` (default) replaces the vendor GEMM of the q / k / v projection and the rope kernel by one
+    launch of this library's GEMM with bias and M-RoPE in its epilogue (vl.py:955-964); `o_proj_native=True`
+    (default) runs the o projection with the residual add on this library's row-major GEMM.  With both False the
+    projections are vendor GEMMs.
 """
 
 from contextlib import contextmanager
@@ -66,11 +69,14 @@ class PrefillHarness:
     def __init__(self, n_layers: int = 36, hidden: int = wl.HIDDEN, n_q: int = wl.N_Q_HEADS, n_kv: int = wl.N_KV_HEADS,
                  head_dim: int = wl.HEAD_DIM, inter=(wl.INTER_VL, wl.INTER_ACT), vocab: int = 151936,
                  eps: float = 1e-6, device="cuda:0", seed: int = 0, mask: str = "causal", keep_dense: bool = False,
-                 fuse: bool = True, fuse_qkv_rope: bool = False):
+                 fuse: bool = True, fuse_qkv_rope: bool = True, o_proj_native: bool = True):
         self.dev = torch.device(device)
         # the q / k / v projection with M-RoPE in its epilogue (one launch of this library's GEMM kernel) instead of
         # the vendor GEMM followed by the rope kernel; needs fuse=True (token-major q / k) and head_dim 128
         self.fuse_qkv_rope = fuse_qkv_rope and fuse and head_dim == 128
+        # the o projection with the attention residual added in its epilogue on this library's row-major GEMM
+        # (wx_dual_gemm_add, second group empty) instead of the vendor's addmm; needs fuse=True
+        self.o_proj_native = o_proj_native and fuse
         self.n_layers, self.hidden, self.n_q, self.n_kv, self.head_dim = n_layers, hidden, n_q, n_kv, head_dim
         self.inter, self.eps, self.mask_mode, self.fuse = inter, eps, mask, fuse
         g = torch.Generator(device=self.dev).manual_seed(seed)
@@ -98,6 +104,10 @@ class PrefillHarness:
                 layer["experts"] = None
             self.layers.append(layer)
         self.final_ln = torch.ones(hidden, dtype=torch.bfloat16, device=self.dev)
+        # operands of the empty second group of the o projection's launch
+        self._none = (torch.empty(0, n_q * head_dim, dtype=torch.bfloat16, device=self.dev),
+                      torch.empty(8, n_q * head_dim, dtype=torch.bfloat16, device=self.dev),
+                      torch.empty(0, 8, dtype=torch.bfloat16, device=self.dev))
         self.inv_freq = wl.text_inv_freq(head_dim).to(self.dev)
         self._hmid: Optional[torch.Tensor] = None
         self._x_tiled: Optional[torch.Tensor] = None
@@ -232,9 +242,15 @@ class PrefillHarness:
                 else:
                     a = F.scaled_dot_product_attention(q, k, v, attn_mask=attn_mask, is_causal=attn_mask is None,
                                                        enable_gqa=True)
-            with timer.section("o_proj_torch"):
+            with timer.section("o_proj" if self.o_proj_native else "o_proj_torch"):
                 a2d = a.transpose(1, 2).reshape(B * S, nq * D)  # a view when attention kept the token-major layout
-                if self.fuse:
+                if self.o_proj_native:  # residual in the GEMM's epilogue (rounded product + residual, like eager)
+                    res = h.view(B * S, H)
+                    h = torch.empty_like(res)
+                    native.asym_dual_gmm(a2d, self._none[0], layer["wo"], self._none[1], h, self._none[2], False, True,
+                                         add_expert0=res)
+                    h = h.view(B, S, H)
+                elif self.fuse:
                     h = torch.addmm(h.view(B * S, H), a2d, layer["wo"].t()).view(B, S, H)  # residual in the GEMM
                 else:
                     h = h + F.linear(a2d, layer["wo"]).view(B, S, H)
