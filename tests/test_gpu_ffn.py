@@ -665,3 +665,33 @@ def test_moe_block_backward_with_one_expert_frozen(dev, frozen_expert):
     assert all(t is None for t in w[frozen_expert])
     for got, want in zip(w[1 - frozen_expert], w_all[1 - frozen_expert]):
         assert got is not None and torch.equal(got, want)
+
+
+def test_moe_block_under_bf16_autocast_takes_fp32_input(dev):
+    """Under bf16 autocast (the reference trains that way, train_qact.py:65) the nn.Linear layers of the reference block
+    take an fp32 input and answer in bf16; the drop-in does the same, forward and backward.  Outside autocast an fp32
+    input is refused."""
+    class Cfg:
+        experts = [{"hidden_size": 128, "intermediate_size": 256, "hidden_act": "silu"},
+                   {"hidden_size": 128, "intermediate_size": 64, "hidden_act": "silu"}]
+
+    g = torch.Generator().manual_seed(14)
+    block = moe.SparseMoeBlock(Cfg(), 2).to(torch.bfloat16)
+    with torch.no_grad():
+        for prm in block.parameters():
+            prm.copy_(_bf(prm.shape, g, 0.08))
+    block = block.to(dev)
+    x32 = _bf((1, 300, 128), g).float().to(dev).requires_grad_(True)
+    types = (torch.rand(1, 300, generator=g) > 0.5).to(dev)
+    with pytest.raises(RuntimeError):
+        block(x32, types)
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        y = block(x32, types)
+    assert y.dtype == torch.bfloat16
+    y.float().sum().backward()
+    assert x32.grad is not None and x32.grad.dtype == torch.float32
+    xb = x32.detach().to(torch.bfloat16).requires_grad_(True)
+    yb = block(xb, types)
+    assert torch.equal(y, yb)
+    yb.float().sum().backward()
+    assert torch.equal(x32.grad, xb.grad.float())

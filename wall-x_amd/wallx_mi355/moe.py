@@ -250,7 +250,13 @@ class SparseMoeBlock(nn.Module):
         batch, seq, hidden = hidden_states.shape
         x = hidden_states.reshape(-1, hidden)
         if x.dtype != torch.bfloat16:
-            raise RuntimeError("All tensors must be BFloat16 for this kernel")
+            # under bf16 autocast (the reference trains with accelerate's mixed_precision="bf16", train_qact.py:65) the
+            # nn.Linear layers this block replaces would take an fp32 input and answer in bf16: do the same
+            if x.is_floating_point() and torch.is_autocast_enabled("cuda") and \
+                    torch.get_autocast_dtype("cuda") == torch.bfloat16:
+                x = x.to(torch.bfloat16)
+            else:
+                raise RuntimeError("All tensors must be BFloat16 for this kernel")
         T = x.size(0)
         host_rows = self._host_rows(start_indices, end_indices, T)
         if routing is None:
