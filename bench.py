@@ -298,6 +298,12 @@ def main():
     }
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(x_cpu, types_cpu, w_cpu, args.cpu_seqs, H, I0, I1)
+        if isinstance(extra.get("prefill"), dict) and "tokens_per_s" in extra["prefill"]:
+            # the same prefill priced on the host cores (a bounded sample: one layer timed, 36 charged)
+            try:
+                extra["prefill"]["cpu_baseline"] = cpu_prefill_baseline()
+            except Exception as exc:  # noqa: BLE001 - the message goes into the report
+                extra["prefill"]["cpu_baseline"] = {"error": f"{type(exc).__name__}: {exc}"[:300]}
     print(json.dumps(result), flush=True)
 
 
@@ -722,6 +728,55 @@ def cpu_baseline(x_cpu, types_cpu, w_cpu, n_seq, H, I0, I1):
                   f"median of 5 runs after 2 warm-ups, {best * 1e3:.0f} ms per run; single_thread_value: first "
                   f"sequence ({tokens1} tokens), 1 thread, median of 3 runs after 1 warm-up, {best1 * 1e3:.0f} ms per run",
     }
+
+
+def cpu_prefill_baseline(n_layers_timed=2):
+    """The config 5 prefill on the host cores, for scale next to `extra.prefill`: the CPU oracle's pieces (RMSNorm,
+    M-RoPE, the dual-expert block) with torch's CPU linear layers and attention between them, fp32, at the full
+    16 x 912 batch.  A bounded sample: ONE decoder layer is timed n_layers_timed times after a warm-up and the forward
+    is priced as 36 such layers (embedding lookup and the last-token head are left out, well under 1 %)."""
+    import torch
+    import torch.nn.functional as F
+    import oracle
+    from wallx_mi355 import workloads as wl
+
+    g = torch.Generator().manual_seed(0)
+    H, nq, nkv, D, inter = wl.HIDDEN, wl.N_Q_HEADS, wl.N_KV_HEADS, wl.HEAD_DIM, (wl.INTER_VL, wl.INTER_ACT)
+    ids, grid = wl.config2_tokens(batch=16, tail_text=96)
+    types = ids == wl.ACTION_TOKEN_ID
+    B, S = ids.shape
+    pos, _ = oracle.rope_index_ref(ids, 2, wl.IMAGE_TOKEN_ID, wl.VIDEO_TOKEN_ID, wl.VISION_START_TOKEN_ID, 2,
+                                   image_grid_thw=grid)
+    cos, sin = oracle.rotary_cos_sin_ref(pos, wl.text_inv_freq(D), torch.float32)
+    w = lambda *shape: torch.randn(*shape, generator=g) * 0.02  # noqa: E731
+    ln = torch.ones(H)
+    wqkv, bqkv, wo = w((nq + 2 * nkv) * D, H), w((nq + 2 * nkv) * D), w(H, nq * D)
+    experts = [(w(i, H), w(i, H), w(H, i)) for i in inter]
+    causal = torch.ones(S, S, dtype=torch.bool).tril()
+    mask = causal[None, None] | (types[:, None, :, None] & types[:, None, None, :])  # act.py:616-637
+    h = torch.randn(B, S, H, generator=g)
+
+    def layer(h):
+        x = oracle.rms_norm_ref(h, ln, 1e-6)
+        q, k, v = F.linear(x, wqkv, bqkv).split([nq * D, nkv * D, nkv * D], dim=-1)
+        q, k, v = (t.view(B, S, -1, D).transpose(1, 2) for t in (q, k, v))
+        q, k = oracle.mrope_apply_ref(q, k, cos, sin, list(wl.MROPE_SECTION))
+        rep = nq // nkv
+        a = F.scaled_dot_product_attention(q, k.repeat_interleave(rep, 1), v.repeat_interleave(rep, 1), attn_mask=mask)
+        h = h + F.linear(a.transpose(1, 2).reshape(B, S, nq * D), wo)
+        return h + oracle.sparse_moe_block_ref(oracle.rms_norm_ref(h, ln, 1e-6), types, experts, eager_rounding=False)
+
+    with torch.no_grad():
+        layer(h)
+        times = []
+        for _ in range(n_layers_timed):
+            t0 = time.perf_counter()
+            layer(h)
+            times.append(time.perf_counter() - t0)
+    per_layer = statistics.median(times)
+    return {"tokens_per_s": round(B * S / (36 * per_layer), 1), "cores": torch.get_num_threads(),
+            "sample": f"one decoder layer at the full 16 x 912 batch (fp32, dense boolean attention mask), median of "
+                      f"{n_layers_timed} runs after a warm-up: {per_layer * 1e3:.0f} ms; the forward priced as 36 layers"}
 
 
 if __name__ == "__main__":
