@@ -380,6 +380,14 @@ def side_measurements(dev, iters):
     pos_bytes = 2.0 * 2 * tokens * D * (wl.N_Q_HEADS + wl.N_KV_HEADS) + 3.0 * 8 * tokens
     out["mrope_from_positions_us"] = round(t * 1e3, 2)
     out["mrope_from_positions_GBps"] = round(pos_bytes / t / 1e6, 1)
+    # ... and with cos/sin read from the packed table (256 bytes per token, built once per forward for all layers)
+    table = native.mrope_table(pos, inv, wl.MROPE_SECTION)
+    t, _ = event_ms(lambda: native.rope_from_table(q, k, table, qo, ko, sec2), iters, batch=10)
+    tab_bytes = 2.0 * 2 * tokens * D * (wl.N_Q_HEADS + wl.N_KV_HEADS) + 4.0 * tokens * (D // 2)
+    out["mrope_from_packed_table_us"] = round(t * 1e3, 2)
+    out["mrope_from_packed_table_GBps"] = round(tab_bytes / t / 1e6, 1)
+    t, _ = event_ms(lambda: native.mrope_table(pos, inv, wl.MROPE_SECTION), iters)
+    out["mrope_table_build_us"] = round(t * 1e3, 2)
 
     def build_tables():
         fr = pos.float()[..., None] * inv

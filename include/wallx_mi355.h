@@ -261,6 +261,18 @@ int wx_mrope_apply_positions(const void* q, const void* k, const int64_t* positi
 int wx_mrope_table(const int64_t* position_ids, const float* inv_freq, int64_t batch, int64_t seq, int head_dim,
                    const int mrope_section[3], int layout /* wx_mrope_layout */, uint32_t* table,
                    wx_stream_t stream);
+
+/* wx_mrope_apply / wx_mrope_apply_bwd (backward != 0) with cos and sin read from the packed table of wx_mrope_table
+ * instead of the two [3, B, S, D] tables: 256 bytes per token where the selected channels of three planes of two
+ * tables touch twelve cache lines.  bf16; layouts whose channels d and d + D/2 share a plane (WX_MROPE_HF); heads as
+ * for wx_mrope_apply_positions.  The table is built once per forward and serves every layer.  Results equal
+ * wx_mrope_apply_positions bit for bit (the same device cos / sin).  No counterpart in the reference beyond the rope
+ * op itself (ops.py:402-497, vl.py:731-773). */
+int wx_mrope_apply_packed(const void* q, const void* k, const uint32_t* table, void* q_out, void* k_out,
+                          int64_t batch, int64_t seq, int n_q_heads, int n_kv_heads, int head_dim,
+                          const int64_t q_strides[3], const int64_t k_strides[3], const int64_t qo_strides[3],
+                          const int64_t ko_strides[3], const int mrope_section[3], int layout, int dtype,
+                          int backward, wx_stream_t stream);
 int wx_qkv_rope_proj(const void* x, const void* weight, const void* bias, const uint32_t* rope_table, void* out,
                      int64_t num_tokens, int64_t hidden, int n_q_heads, int n_kv_heads, int head_dim,
                      wx_stream_t stream);

@@ -194,6 +194,48 @@ def test_mrope_from_positions_refuses_what_it_cannot_do(dev):
                                            pos[:, :, :5].to(dev), inv_freq, [16, 24, 24])
 
 
+def test_mrope_from_packed_table_equals_the_positions_path(dev):
+    """multimodal_rope_from_table reads cos / sin from the packed table of multimodal_rope_table (256 bytes per token,
+    built once per forward); the table holds what the positions path evaluates per thread (the same device sincosf on
+    the same angle, rounded to bf16), so forward and backward equal that path bit for bit -- at config 2's full size,
+    through strided views, and for a short ragged sequence -- and the oracle within the stated tolerance."""
+    ids, grid = wl.config2_tokens()
+    pos, _ = oracle.rope_index_ref(ids, 2, wl.IMAGE_TOKEN_ID, wl.VIDEO_TOKEN_ID, wl.VISION_START_TOKEN_ID, 2,
+                                   image_grid_thw=grid)
+    inv_freq = wl.text_inv_freq()
+    q, k = wl.qk_inputs(16, 896)
+    sec = list(wl.MROPE_SECTION)
+    cases = [(q.transpose(1, 2), k.transpose(1, 2), pos)]  # [B, H, S, D] views of token-major memory
+    q2, k2, pos2 = _pos_inputs(3, 37, torch.bfloat16, 31)
+    cases.append((q2.transpose(1, 2).contiguous(), k2.transpose(1, 2).contiguous(), pos2))
+    for qt, kt, p_ in cases:
+        table = ops.multimodal_rope_table(p_.to(dev), inv_freq.to(dev), sec)
+        qd, kd = qt.to(dev).requires_grad_(True), kt.to(dev).requires_grad_(True)
+        tq, tk = ops.multimodal_rope_from_table(qd, kd, table, sec)
+        pq, pk = ops.multimodal_rope_from_positions(qt.to(dev), kt.to(dev), p_.to(dev), inv_freq.to(dev), sec)
+        assert _n_diff(tq.detach(), pq.cpu()) == 0 and _n_diff(tk.detach(), pk.cpu()) == 0
+        cos, sin = oracle.rotary_cos_sin_ref(p_, inv_freq, torch.bfloat16)
+        rq, rk = oracle.mrope_apply_ref(qt, kt, cos, sin, sec, "hf")
+        _close(tq.detach(), rq)
+        _close(tk.detach(), rk)
+        g = torch.Generator(device=dev).manual_seed(5)
+        gq = torch.randn(tq.shape, device=dev, generator=g).to(torch.bfloat16)
+        gk = torch.randn(tk.shape, device=dev, generator=g).to(torch.bfloat16)
+        torch.autograd.backward([tq, tk], [gq, gk])
+        bq, bk = torch.empty_like(gq), torch.empty_like(gk)
+        native.rope_from_positions(gq, gk, p_.to(dev), inv_freq.to(dev), bq, bk, [2 * v for v in sec], backward=True)
+        assert _n_diff(qd.grad, bq.cpu()) == 0 and _n_diff(kd.grad, bk.cpu()) == 0
+    # what it cannot do is refused: fp16 (the table is bf16), the csrc layout (its half-channels take different planes)
+    table = ops.multimodal_rope_table(pos2.to(dev), inv_freq.to(dev), sec)
+    qh, kh = cases[1][0].to(dev), cases[1][1].to(dev)
+    with pytest.raises(RuntimeError):
+        native.rope_from_table(qh.half(), kh.half(), table, torch.empty_like(qh.half()), torch.empty_like(kh.half()),
+                               [2 * v for v in sec])
+    with pytest.raises(RuntimeError, match="different position planes"):
+        native.rope_from_table(qh, kh, table, torch.empty_like(qh), torch.empty_like(kh), [2 * v for v in sec],
+                               layout="csrc")
+
+
 def test_extension_level_rope_uses_the_cuda_kernels_layout(dev):
     """wallx_csrc.rope / rope_bwd stand in for the reference's extension (csrc/ops.cu:11-21), whose kernel maps
     channels d < 32 -> t, d < 80 -> h, else w (csrc/rope.cu:104-117): called the way the reference's own ops.py

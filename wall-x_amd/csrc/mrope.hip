@@ -181,11 +181,17 @@ __device__ __forceinline__ u32x4 partner_chunk(const u32x4& v, int half_lanes) {
 }
 
 // L = lanes per head when known at compile time (16), 0 = any power of two up to 64 (runtime).
-// POS: no cos/sin tables; `cos_t` is position_ids int64 [3, n_tokens] and `sin_t` is inv_freq fp32 [head_dim / 2].
-// The thread evaluates cos/sin of its channels itself, the way the table builder does (vl.py:679-712): the angle
-// is the fp32 product position * inv_freq (channels d and d + head_dim/2 share a frequency), cos and sin are
-// taken in fp32 and rounded to the storage type.
-template <int DT, bool BWD, int L, bool POS>
+// SRC says where cos / sin come from:
+//   kSrcTables     the two [3, n_tokens, head_dim] tables of the reference op;
+//   kSrcPositions  no tables: `cos_t` is position_ids int64 [3, n_tokens] and `sin_t` is inv_freq fp32 [head_dim / 2].
+//                  The thread evaluates cos/sin of its channels itself, the way the table builder does
+//                  (vl.py:679-712): the angle is the fp32 product position * inv_freq (channels d and d + head_dim/2
+//                  share a frequency), cos and sin are taken in fp32 and rounded to the storage type;
+//   kSrcPacked     `cos_t` is the packed table of wx_mrope_table, uint32 [n_tokens, head_dim / 2] (bf16 cos | bf16 sin
+//                  << 16 of the plane each channel pair takes): 256 bytes per token instead of the 12 cache lines the
+//                  selected channels of three planes of two tables touch.  bf16 only.
+enum { kSrcTables = 0, kSrcPositions = 1, kSrcPacked = 2 };
+template <int DT, bool BWD, int L, int SRC>
 __global__ __launch_bounds__(256) void mrope_rows_kernel(
     const void* __restrict__ q, const void* __restrict__ k, const void* __restrict__ cos_t,
     const void* __restrict__ sin_t, void* __restrict__ q_out, void* __restrict__ k_out, int64_t n_tokens,
@@ -210,7 +216,15 @@ __global__ __launch_bounds__(256) void mrope_rows_kernel(
   const int64_t hq_out = sqo.h * Elem<DT>::kBytes, hk_out = sko.h * Elem<DT>::kBytes;
 
   u32x4 c_raw, s_raw;
-  if constexpr (POS) {
+  if constexpr (SRC == kSrcPacked) {
+    static_assert(DT == WX_BF16, "the packed table holds bf16 pairs");
+    const uint32_t* t = static_cast<const uint32_t*>(cos_t) + token * (head_dim / 2) + (hi ? d0 - head_dim / 2 : d0);
+    const u32x4 t0 = *reinterpret_cast<const u32x4*>(t), t1 = *reinterpret_cast<const u32x4*>(t + 4);
+    c_raw = u32x4{(t0[0] & 0xffffu) | (t0[1] << 16), (t0[2] & 0xffffu) | (t0[3] << 16),
+                  (t1[0] & 0xffffu) | (t1[1] << 16), (t1[2] & 0xffffu) | (t1[3] << 16)};
+    s_raw = u32x4{(t0[0] >> 16) | (t0[1] & 0xffff0000u), (t0[2] >> 16) | (t0[3] & 0xffff0000u),
+                  (t1[0] >> 16) | (t1[1] & 0xffff0000u), (t1[2] >> 16) | (t1[3] & 0xffff0000u)};
+  } else if constexpr (SRC == kSrcPositions) {
     const int64_t pos = static_cast<const int64_t*>(cos_t)[ax.axis[d0] * n_tokens + token];
     const float* inv_freq = static_cast<const float*>(sin_t) + (hi ? d0 - head_dim / 2 : d0);
     const float pf = static_cast<float>(pos);
@@ -304,21 +318,23 @@ int build_axis_table(const int sec[3], int head_dim, int layout, AxisTable& ax) 
   return WX_OK;
 }
 
-// POS: cos_t / sin_t carry position_ids / inv_freq (see mrope_rows_kernel)
-template <bool BWD, bool POS = false>
+// SRC: what cos_t / sin_t carry (see mrope_rows_kernel)
+template <bool BWD, int SRC = kSrcTables>
 int launch(const void* q, const void* k, const void* cos_t, const void* sin_t, void* q_out, void* k_out,
            int64_t batch, int64_t seq, int n_q, int n_kv, int head_dim, const int64_t* sq, const int64_t* sk,
            const int64_t* sqo, const int64_t* sko, const int sec[3], int layout, int dtype, wx_stream_t stream) {
-  const char* who = POS ? (BWD ? "wx_mrope_apply_positions(backward)" : "wx_mrope_apply_positions")
-                        : (BWD ? "wx_mrope_apply_bwd" : "wx_mrope_apply");
+  const char* who = SRC == kSrcPositions ? (BWD ? "wx_mrope_apply_positions(backward)" : "wx_mrope_apply_positions")
+                    : SRC == kSrcPacked  ? (BWD ? "wx_mrope_apply_packed(backward)" : "wx_mrope_apply_packed")
+                                         : (BWD ? "wx_mrope_apply_bwd" : "wx_mrope_apply");
   if (batch < 0 || seq < 0 || n_q < 0 || n_kv < 0) return fail(WX_ERR_INVALID_ARGUMENT, "%s: negative size", who);
   if (head_dim <= 0 || head_dim % 16 != 0 || head_dim > kMaxHeadDim)
     return fail(WX_ERR_UNSUPPORTED, "%s: head_dim %d must be a multiple of 16 and <= %d", who, head_dim, kMaxHeadDim);
   if (!sq || !sk || !sqo || !sko || !sec) return fail(WX_ERR_INVALID_ARGUMENT, "%s: null stride/section", who);
   const int64_t n_tokens = batch * seq;
   if (n_tokens == 0 || n_q + n_kv == 0) return WX_OK;
-  if (!cos_t || !sin_t || (n_q && (!q || !q_out)) || (n_kv && (!k || !k_out)))
+  if (!cos_t || (SRC != kSrcPacked && !sin_t) || (n_q && (!q || !q_out)) || (n_kv && (!k || !k_out)))
     return fail(WX_ERR_INVALID_ARGUMENT, "%s: null pointer", who);
+  if (SRC == kSrcPacked && dtype != WX_BF16) return fail(WX_ERR_UNSUPPORTED, "%s: the packed table is bf16", who);
   const int align = dtype == WX_F32 ? 4 : 8;  // elements per 16 bytes
   const int64_t* all[4] = {sq, sk, sqo, sko};
   for (auto* st : all)
@@ -326,6 +342,12 @@ int launch(const void* q, const void* k, const void* cos_t, const void* sin_t, v
       if (st[i] % align != 0) return fail(WX_ERR_UNSUPPORTED, "%s: strides must keep rows 16-byte aligned", who);
   AxisTable ax{};
   if (int rc = build_axis_table(sec, head_dim, layout, ax)) return rc;
+  if constexpr (SRC == kSrcPacked) {
+    for (int d = 0; d < head_dim / 2; ++d)
+      if (ax.axis[d] != ax.axis[d + head_dim / 2])
+        return fail(WX_ERR_UNSUPPORTED, "%s: channels %d and %d take different position planes in this layout", who, d,
+                    d + head_dim / 2);
+  }
   const Strides a{sq[0], sq[1], sq[2]}, b{sk[0], sk[1], sk[2]}, c{sqo[0], sqo[1], sqo[2]}, d{sko[0], sko[1], sko[2]};
   hipStream_t s = as_stream(stream);
   // Row form: 16-byte chunks per head must be a power of two that divides the workgroup, and no section boundary
@@ -339,18 +361,22 @@ int launch(const void* q, const void* k, const void* cos_t, const void* sin_t, v
     if ((threads + 255) / 256 > 0x7fffffffll) return fail(WX_ERR_UNSUPPORTED, "%s: too many tokens", who);
     const dim3 grid(static_cast<unsigned>((threads + 255) / 256)), block(256);
 #define WX_LAUNCH_ROWS(DT, L)                                                                                       \
-  hipLaunchKernelGGL((mrope_rows_kernel<DT, BWD, L, POS>), grid, block, 0, s, q, k, cos_t, sin_t, q_out, k_out, n_tokens, \
+  hipLaunchKernelGGL((mrope_rows_kernel<DT, BWD, L, SRC>), grid, block, 0, s, q, k, cos_t, sin_t, q_out, k_out, n_tokens, \
                      seq, n_q, n_kv, head_dim, a, b, c, d, ax)
-    switch (dtype) {
-      case WX_F32: WX_LAUNCH_ROWS(WX_F32, 0); break;
-      case WX_F16: if (lanes == 16) WX_LAUNCH_ROWS(WX_F16, 16); else WX_LAUNCH_ROWS(WX_F16, 0); break;
-      case WX_BF16: if (lanes == 16) WX_LAUNCH_ROWS(WX_BF16, 16); else WX_LAUNCH_ROWS(WX_BF16, 0); break;
-      default: return fail(WX_ERR_UNSUPPORTED, "%s: dtype %d", who, dtype);
+    if constexpr (SRC == kSrcPacked) {
+      if (lanes == 16) WX_LAUNCH_ROWS(WX_BF16, 16); else WX_LAUNCH_ROWS(WX_BF16, 0);
+    } else {
+      switch (dtype) {
+        case WX_F32: WX_LAUNCH_ROWS(WX_F32, 0); break;
+        case WX_F16: if (lanes == 16) WX_LAUNCH_ROWS(WX_F16, 16); else WX_LAUNCH_ROWS(WX_F16, 0); break;
+        case WX_BF16: if (lanes == 16) WX_LAUNCH_ROWS(WX_BF16, 16); else WX_LAUNCH_ROWS(WX_BF16, 0); break;
+        default: return fail(WX_ERR_UNSUPPORTED, "%s: dtype %d", who, dtype);
+      }
     }
 #undef WX_LAUNCH_ROWS
     return check_launch(who);
   }
-  if constexpr (POS) {
+  if constexpr (SRC != kSrcTables) {
     return fail(WX_ERR_UNSUPPORTED,
                 "%s: needs a head of 2..64 16-byte chunks (a power of two) and sections that end on chunk boundaries; "
                 "build the cos/sin tables and call wx_mrope_apply instead", who);
@@ -421,12 +447,29 @@ extern "C" int wx_mrope_apply_positions(const void* q, const void* k, const int6
                                         const int64_t ko_strides[3], const int mrope_section[3], int layout,
                                         int dtype, int backward, wx_stream_t stream) {
   if (backward)
-    return wx::launch<true, true>(q, k, position_ids, inv_freq, q_out, k_out, batch, seq, n_q_heads, n_kv_heads,
+    return wx::launch<true, wx::kSrcPositions>(q, k, position_ids, inv_freq, q_out, k_out, batch, seq, n_q_heads, n_kv_heads,
                                   head_dim, q_strides, k_strides, qo_strides, ko_strides, mrope_section, layout, dtype,
                                   stream);
-  return wx::launch<false, true>(q, k, position_ids, inv_freq, q_out, k_out, batch, seq, n_q_heads, n_kv_heads,
+  return wx::launch<false, wx::kSrcPositions>(q, k, position_ids, inv_freq, q_out, k_out, batch, seq, n_q_heads, n_kv_heads,
                                  head_dim, q_strides, k_strides, qo_strides, ko_strides, mrope_section, layout, dtype,
                                  stream);
+}
+
+extern "C" int wx_mrope_apply_packed(const void* q, const void* k, const uint32_t* table, void* q_out, void* k_out,
+                                     int64_t batch, int64_t seq, int n_q_heads, int n_kv_heads, int head_dim,
+                                     const int64_t q_strides[3], const int64_t k_strides[3],
+                                     const int64_t qo_strides[3], const int64_t ko_strides[3],
+                                     const int mrope_section[3], int layout, int dtype, int backward,
+                                     wx_stream_t stream) {
+  if (reinterpret_cast<uintptr_t>(table) & 15)
+    return wx::fail(WX_ERR_INVALID_ARGUMENT, "wx_mrope_apply_packed: the table must be 16-byte aligned");
+  if (backward)
+    return wx::launch<true, wx::kSrcPacked>(q, k, table, nullptr, q_out, k_out, batch, seq, n_q_heads, n_kv_heads,
+                                            head_dim, q_strides, k_strides, qo_strides, ko_strides, mrope_section,
+                                            layout, dtype, stream);
+  return wx::launch<false, wx::kSrcPacked>(q, k, table, nullptr, q_out, k_out, batch, seq, n_q_heads, n_kv_heads,
+                                           head_dim, q_strides, k_strides, qo_strides, ko_strides, mrope_section,
+                                           layout, dtype, stream);
 }
 
 extern "C" int wx_mrope_table(const int64_t* position_ids, const float* inv_freq, int64_t batch, int64_t seq,

@@ -48,6 +48,8 @@ PROTOTYPES = {
     "wx_mrope_apply_positions": (_i32, [_vp] * 6 + [_i64, _i64, _i32, _i32, _i32] + [_c.POINTER(_i64)] * 4
                                  + [_c.POINTER(_i32), _i32, _i32, _i32, _vp]),
     "wx_mrope_table": (_i32, [_vp, _vp, _i64, _i64, _i32, _c.POINTER(_i32), _i32, _vp, _vp]),
+    "wx_mrope_apply_packed": (_i32, [_vp] * 5 + [_i64, _i64, _i32, _i32, _i32] + [_c.POINTER(_i64)] * 4
+                              + [_c.POINTER(_i32), _i32, _i32, _i32, _vp]),
     "wx_qkv_rope_proj": (_i32, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i32, _i32, _i32, _vp]),
     "wx_rope_index_workspace_bytes": (_sz, [_i64, _i64]),
     "wx_rope_index": (_i32, [_vp, _vp, _vp, _i64, _vp, _i64, _vp, _i64, _i64, _i32, _i64, _i64, _i64, _f32,

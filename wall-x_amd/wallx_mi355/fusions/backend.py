@@ -68,6 +68,11 @@ def rope_from_positions(q, k, position_ids, inv_freq, q_out, k_out, mrope_sectio
                                       layout)
 
 
+def rope_from_table(q, k, table, q_out, k_out, mrope_section_doubled, backward=False, layout: str = "hf") -> None:
+    """No counterpart in backend.py: the rope op reading the packed cos/sin table of mrope_table."""
+    return native.rope_from_table(q, k, table, q_out, k_out, mrope_section_doubled, backward, layout)
+
+
 def mrope_table(position_ids, inv_freq, mrope_section, layout: str = "hf"):
     """No counterpart in backend.py: the packed cos/sin table the projection below reads (vl.py:679-712)."""
     return native.mrope_table(position_ids, inv_freq, mrope_section, layout)

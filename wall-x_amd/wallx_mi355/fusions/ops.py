@@ -306,6 +306,51 @@ def multimodal_rope_table(position_ids, inv_freq, mrope_section):
     return backend.mrope_table(position_ids, inv_freq.to(torch.float32), list(mrope_section))
 
 
+class MultimodalRoPEFromTable(torch.autograd.Function):
+    """multimodal_rope with cos / sin read from the packed table of multimodal_rope_table (built once per forward,
+    256 bytes per token, shared by all layers) instead of the two [3, B, S, D] tables; bf16, PyTorch-path layout."""
+
+    @staticmethod
+    def forward(ctx, q, k, table, mrope_section):
+        for name, t in (("q", q), ("k", k), ("table", table)):
+            if t.is_cpu:
+                raise RuntimeError(f"[Error] The input `{name}` of multimodal_rope op is on the device: CPU!")
+        if len(mrope_section) != 3:
+            raise RuntimeError("[Error] The input `mrope_section` of multimodal_rope op must be a list of 3 integers!")
+        if q.stride(-1) != 1:
+            warnings.warn("The input `q` of multimodal_rope op is discontiguous!")
+            q = q.contiguous()
+        if k.stride(-1) != 1:
+            warnings.warn("The input `k` of multimodal_rope op is discontiguous!")
+            k = k.contiguous()
+        doubled = [2 * int(v) for v in mrope_section]
+        q_out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+        k_out = torch.empty(k.shape, dtype=k.dtype, device=k.device)
+        backend.rope_from_table(q, k, table, q_out, k_out, doubled)
+        ctx.save_for_backward(table)
+        ctx.mrope_section_doubled = doubled
+        return q_out, k_out
+
+    @staticmethod
+    def backward(ctx, grad_q_out, grad_k_out):
+        (table,) = ctx.saved_tensors
+        want_q, want_k = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+        if not (want_q or want_k):
+            return None, None, None, None
+        if grad_q_out.stride(-1) != 1:
+            grad_q_out = grad_q_out.contiguous()
+        if grad_k_out.stride(-1) != 1:
+            grad_k_out = grad_k_out.contiguous()
+        gq = torch.empty(grad_q_out.shape, dtype=grad_q_out.dtype, device=grad_q_out.device)
+        gk = torch.empty(grad_k_out.shape, dtype=grad_k_out.dtype, device=grad_k_out.device)
+        backend.rope_from_table(grad_q_out, grad_k_out, table, gq, gk, ctx.mrope_section_doubled, backward=True)
+        return (gq if want_q else None), (gk if want_k else None), None, None
+
+
+def multimodal_rope_from_table(q, k, table, mrope_section):
+    return MultimodalRoPEFromTable.apply(q, k, table, mrope_section)
+
+
 def qkv_projection_with_rope(hidden_states, qkv_weight, qkv_bias, rope_table, num_heads, num_key_value_heads,
                              head_dim=128):
     """Not in the reference's op set: the first lines of the attention forward (vl.py:955-964) as one launch.

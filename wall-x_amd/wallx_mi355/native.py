@@ -351,6 +351,30 @@ def rope_from_positions(q, k, position_ids, inv_freq, q_out, k_out, mrope_sectio
                   _bhsd_strides(k_out), section, _layout_code(layout), _dtype_code(q), int(bool(backward)), _stream(q))
 
 
+def rope_from_table(q, k, table, q_out, k_out, mrope_section_doubled, backward: bool = False,
+                    layout: str = "hf") -> None:
+    """M-RoPE with cos / sin read from the packed table of mrope_table (int32 [B * S, D / 2], built once per forward
+    for all layers).  bf16; same results as rope_from_positions, bit for bit.  With backward=True, q/k carry the
+    output gradients and q_out/k_out receive the input gradients."""
+    for name, t in (("q", q), ("k", k), ("table", table), ("q_out", q_out), ("k_out", k_out)):
+        _need_cuda(name, t)
+    if len(mrope_section_doubled) != 3:
+        raise RuntimeError("mrope_section_doubled must have 3 entries")
+    B, Hq, S, D = q.shape
+    Hk = k.size(1)
+    if tuple(k.shape) != (B, Hk, S, D) or tuple(q_out.shape) != tuple(q.shape) or tuple(k_out.shape) != tuple(k.shape):
+        raise RuntimeError("q/k/q_out/k_out shapes are inconsistent")
+    if tuple(table.shape) != (B * S, D // 2) or table.dtype != torch.int32 or not table.is_contiguous():
+        raise RuntimeError(f"table must be a contiguous int32 [{B * S}, {D // 2}] tensor from mrope_table")
+    if not (q.dtype == k.dtype == q_out.dtype == k_out.dtype == torch.bfloat16):
+        raise RuntimeError("All tensors must be BFloat16 for this kernel")
+    section = _lib.i32x3([int(v) // 2 for v in mrope_section_doubled])
+    with _DeviceGuard(q):
+        _lib.call("wx_mrope_apply_packed", _ptr(q), _ptr(k), _ptr(table), _ptr(q_out), _ptr(k_out), B, S, Hq, Hk, D,
+                  _bhsd_strides(q), _bhsd_strides(k), _bhsd_strides(q_out), _bhsd_strides(k_out), section,
+                  _layout_code(layout), _dtype_code(q), int(bool(backward)), _stream(q))
+
+
 def mrope_table(position_ids: torch.Tensor, inv_freq: torch.Tensor, mrope_section, layout: str = "hf") -> torch.Tensor:
     """Packed rotary table for qkv_rope_proj: int32 [B * S, D / 2], entry = bf16 cos | bf16 sin << 16 of
     position_ids[plane(d)] * inv_freq[d] (vl.py:679-712 rounded to bf16).  position_ids [3, B, S] int64, inv_freq
