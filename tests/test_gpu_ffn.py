@@ -35,6 +35,7 @@ GEMM_SHAPES = [
     (129, 136, 200, 0, 64, 64),          # empty action group, K tail
     (0, 64, 64, 0, 64, 64),              # nothing to do
     (3000, 3080, 96, 200, 264, 160),     # enough 256 x 256 tiles to take the large-tile kernel, ragged everywhere
+    (5000, 4104, 96, 300, 520, 160),     # 346 large tiles: more than one round of one tile per CU
     (40, 64, 0, 24, 72, 64),             # empty contraction: the output is zeros
 ]
 
@@ -99,6 +100,7 @@ def test_dual_gemm_all_transposes_and_autograd(dev):
     # m0, n0, k0, m1, n1, k1
     (72, 96, 64, 40, 56, 128),            # small tiles
     (3000, 3080, 96, 200, 264, 160),      # large tiles, ragged everywhere
+    (5000, 4104, 96, 304, 520, 160),      # more than a round of large tiles
     (264, 520, 2048, 0, 64, 64),          # long contraction, empty second problem
 ])
 def test_dual_gemm_k_major_layouts_through_the_c_abi(dev, shape):
