@@ -244,7 +244,7 @@ class SparseMoeBlock(nn.Module):
 
         Two optional caller fusions (the decoder layer around this block, act.py:256-265):
         pre_norm=(weight, eps) applies the post-attention RMSNorm to hidden_states inside the permute, and
-        residual=True returns hidden_states + block(...) with the add done inside the unpermute.  With both, the
+        residual=True returns hidden_states + block(...) with the add done in the down launch's stores.  With both, the
         layer's `residual = h; h = norm(h); h = moe(h); h = residual + h` is `h = moe(h, ..., pre_norm, True)`.
         """
         batch, seq, hidden = hidden_states.shape
