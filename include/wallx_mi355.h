@@ -38,6 +38,17 @@ typedef enum { WX_I32 = 0, WX_I64 = 1, WX_U8 = 2 /* torch.bool */ } wx_itype;
 typedef enum { WX_MROPE_HF = 0, WX_MROPE_CSRC = 1 } wx_mrope_layout;
 
 const char* wx_last_error_string(void);
+/* Which kernels the last wx_dual_gemm / wx_dual_gemm_add call on the calling thread launched, as a bit set (0 before
+ * the first call and after a call that launched nothing).  No counterpart in the reference; for tests and callers that
+ * want to assert the code path rather than time it: a problem that should run on the matrix cores must not have gone
+ * to the plain FMA kernel. */
+enum {
+  WX_GEMM_PATH_MFMA = 1,      /* the MFMA kernel (either tile shape) */
+  WX_GEMM_PATH_ZERO_FILL = 2, /* an empty contraction (k == 0): its output was filled with zeros */
+  WX_GEMM_PATH_FMA = 4,       /* the plain FMA kernel (K-major operands of 4 GiB or more) */
+  WX_GEMM_PATH_ADD_COPY = 8   /* an empty contraction with an addend: the addend was copied to the output */
+};
+int wx_last_gemm_path(void);
 int wx_abi_version(void);
 /* 1 and *id = the capture's id when `stream` is being captured into a HIP graph, 0 and *id = 0 when it is not
  * (negative on error).  No counterpart in the reference; for hosts that keep results between calls (a cached token
@@ -68,14 +79,19 @@ int wx_partition_build(const void* ids, int id_type /* wx_itype */, int64_t num_
  * status codes as wx_partition_build minus the workspace pair: the per-segment histograms go to a 1 MiB device
  * array built into the library (one copy per GPU, held until the process ends), which covers every size the
  * partition takes (up to 2^31 - 1 expanded tokens; larger counts are refused with WX_ERR_UNSUPPORTED, a count whose
- * histograms would not fit with WX_ERR_WORKSPACE).  The call allocates nothing and does not synchronise.  The first
- * call on a device looks up the array's address (hipGetSymbolAddress); make that call outside graph capture.
+ * histograms would not fit with WX_ERR_WORKSPACE).  The call allocates nothing and does not synchronise.  The
+ * array's address is looked up once per device (hipGetSymbolAddress) by wx_partition_noalloc_init(), or by the first
+ * call on that device when it is not being captured; a first use from inside a stream capture is refused with
+ * WX_ERR_INVALID_ARGUMENT (call the init function, with the device current, before capturing).
  * All calls on one GPU share the array: calls that overlap there (different streams or threads) race -- order them
  * on one stream.  Nothing in the array needs clearing between calls (every word read is written first). */
 int wx_partition_build_noalloc(const void* ids, int id_type /* wx_itype */, int64_t num_tokens, int num_topk,
                                int num_experts, int64_t num_out_tokens, int32_t* row_id_map,
                                int32_t* sorted_row_id, int32_t* expert_offsets, int32_t* status,
                                wx_stream_t stream);
+/* Set-up of wx_partition_build_noalloc for the current device: resolves the address of the built-in scratch array.
+ * Idempotent, launches nothing; it has no counterpart in the reference either. */
+int wx_partition_noalloc_init(void);
 
 /* Row scatter of the permute op: out[row_id_map[k*T + t], :] = x[t, :] for every k with a map entry
  * != -1.  Replaces moe_permute_topK_kernel, forward branch (csrc/permute.cu:156-262, 294-305).
@@ -248,24 +264,30 @@ int wx_mrope_apply_positions(const void* q, const void* k, const int64_t* positi
 /* The attention block's q / k / v projections with the rotary embedding in the GEMM's epilogue: replaces
  * q_proj / k_proj / v_proj (nn.Linear with bias, vl.py:821-832, 955-957) followed by the rope op
  * (vl.py:962-964, ops.py:402-497) -- one launch, and q / k are not written and read again for the rotation.
- * wx_mrope_table builds what the epilogue reads: table[token][d], d < head_dim / 2, = bf16 cos | bf16 sin << 16 of
- * position_ids[plane(d)][token] * inv_freq[d] (fp32 angle, fp32 cos / sin, rounded to bf16 as vl.py:679-712 does);
- * position_ids [3, B, S] int64, inv_freq [head_dim / 2] fp32, table uint32 [B * S, head_dim / 2].  Channels d and
- * d + head_dim / 2 must share a position plane: true for WX_MROPE_HF, refused (WX_ERR_UNSUPPORTED) for WX_MROPE_CSRC.
+ * wx_mrope_table builds what the epilogue reads: table[token][d], d < W, = bf16 cos | bf16 sin << 16 of
+ * position_ids[plane(d)][token] * inv_freq[d mod head_dim / 2] (fp32 angle, fp32 cos / sin, rounded to bf16 as
+ * vl.py:679-712 does); position_ids [3, B, S] int64, inv_freq [head_dim / 2] fp32, table uint32 [B * S, W].
+ * W = wx_mrope_table_width(head_dim, mrope_section, layout): head_dim / 2 when channels d and d + head_dim / 2 share a
+ * position plane (WX_MROPE_HF: one entry serves both), head_dim when they do not (WX_MROPE_CSRC: one entry per
+ * channel); negative status on bad arguments.
  * wx_qkv_rope_proj: out [num_tokens, (n_q + 2 n_kv) * head_dim] = x [num_tokens, hidden] @ weight^T + bias, weight
  * [(n_q + 2 n_kv) * head_dim, hidden] = the three nn.Linear weights stacked q, k, v (row-major, read in place), bias
  * likewise or NULL; the q and k heads (the first (n_q + n_kv) * head_dim columns) come out rotated:
  * head[d] * cos[d] + rotate_half(head)[d] * sin[d], evaluated like eager bf16 code (the projection rounded once, every
  * product and the sum rounded).  bf16; head_dim must be 128 (a wavefront's 128 output columns are one head), hidden a
- * multiple of 8.  Row t of the table belongs to row t of x. */
+ * multiple of 8.  Row t of the table belongs to row t of x; table_width is the W the table was built with (either
+ * layout is served: with WX_MROPE_HF this is the eager attention path of vl.py:860-862 / 1075-1077, with WX_MROPE_CSRC
+ * the flash-attention class's rope op, vl.py:962-964 on csrc/rope.cu:104-117). */
+int wx_mrope_table_width(int head_dim, const int mrope_section[3], int layout /* wx_mrope_layout */);
 int wx_mrope_table(const int64_t* position_ids, const float* inv_freq, int64_t batch, int64_t seq, int head_dim,
                    const int mrope_section[3], int layout /* wx_mrope_layout */, uint32_t* table,
                    wx_stream_t stream);
 
 /* wx_mrope_apply / wx_mrope_apply_bwd (backward != 0) with cos and sin read from the packed table of wx_mrope_table
- * instead of the two [3, B, S, D] tables: 256 bytes per token where the selected channels of three planes of two
- * tables touch twelve cache lines.  bf16; layouts whose channels d and d + D/2 share a plane (WX_MROPE_HF); heads as
- * for wx_mrope_apply_positions.  The table is built once per forward and serves every layer.  Results equal
+ * instead of the two [3, B, S, D] tables: 256 bytes per token (512 for WX_MROPE_CSRC, whose table has one entry per
+ * channel) where the selected channels of three planes of two tables touch twelve cache lines.  bf16; `layout` and
+ * `mrope_section` must be the ones the table was built with; heads as for wx_mrope_apply_positions.  The table is
+ * built once per forward and serves every layer.  Results equal
  * wx_mrope_apply_positions bit for bit (the same device cos / sin).  No counterpart in the reference beyond the rope
  * op itself (ops.py:402-497, vl.py:731-773). */
 int wx_mrope_apply_packed(const void* q, const void* k, const uint32_t* table, void* q_out, void* k_out,
@@ -273,9 +295,9 @@ int wx_mrope_apply_packed(const void* q, const void* k, const uint32_t* table, v
                           const int64_t q_strides[3], const int64_t k_strides[3], const int64_t qo_strides[3],
                           const int64_t ko_strides[3], const int mrope_section[3], int layout, int dtype,
                           int backward, wx_stream_t stream);
-int wx_qkv_rope_proj(const void* x, const void* weight, const void* bias, const uint32_t* rope_table, void* out,
-                     int64_t num_tokens, int64_t hidden, int n_q_heads, int n_kv_heads, int head_dim,
-                     wx_stream_t stream);
+int wx_qkv_rope_proj(const void* x, const void* weight, const void* bias, const uint32_t* rope_table,
+                     int table_width, void* out, int64_t num_tokens, int64_t hidden, int n_q_heads, int n_kv_heads,
+                     int head_dim, wx_stream_t stream);
 
 /* ------------------------------------------------------------------------------------------------
  * 3D position ids.  Replaces get_rope_index (csrc/rope_index.cu:464-569) with the semantics of the

@@ -18,7 +18,9 @@ How each function is pinned (tests/test_oracle_*.py):
   permute_ref / unpermute_ref      brute-force stable partition on tiny inputs,
                                    round-trip identity, permutation invariants
   dual_gemm_ref / swiglu_ffn_ref   float64 numpy contraction on small shapes,
-                                   linearity, zero-row groups
+                                   linearity, zero-row groups; the gelu / relu
+                                   gated forms and a three-expert block against a
+                                   float64 scalar-loop evaluation with math.erf
   mrope_apply_ref                  textbook rotate-half RoPE when t == h == w,
                                    identity at position 0, per-pair norm
                                    preservation, transformers' same-lineage
@@ -61,7 +63,7 @@ from .permute import (  # noqa: F401
     unpermute_bwd_ref,
     expert_offsets_ref,
 )
-from .ffn import dual_gemm_ref, swiglu_ffn_ref, swiglu_bwd_ref, sparse_moe_block_ref  # noqa: F401
+from .ffn import activation_ref, dual_gemm_ref, swiglu_ffn_ref, swiglu_bwd_ref, sparse_moe_block_ref  # noqa: F401
 from .mrope import (  # noqa: F401
     rotate_half_ref,
     mrope_axis_map,

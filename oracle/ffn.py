@@ -29,8 +29,23 @@ def dual_gemm_ref(in0, in1, w0, w1, trans_a: bool = False, trans_b: bool = False
     return outs[0], outs[1]
 
 
-def swiglu_ffn_ref(x, gate_w, up_w, down_w, eager_rounding: bool = True):
-    """down(silu(gate(x)) * up(x)) with nn.Linear weights [out, in] (act.py:74-82).
+def activation_ref(name: str):
+    """The gating function named by an expert's `hidden_act` (act.py:73,77 looks the name up in transformers'
+    ACT2FN): written out here for the names a wall-x style config can carry."""
+    table = {
+        "silu": F.silu,
+        "swish": F.silu,
+        "gelu": F.gelu,  # the exact (erf) form
+        "gelu_new": lambda t: F.gelu(t, approximate="tanh"),
+        "gelu_pytorch_tanh": lambda t: F.gelu(t, approximate="tanh"),
+        "relu": F.relu,
+    }
+    return table[name]
+
+
+def swiglu_ffn_ref(x, gate_w, up_w, down_w, eager_rounding: bool = True, act: str = "silu"):
+    """down(act(gate(x)) * up(x)) with nn.Linear weights [out, in] (act.py:74-82); act = the expert's
+    `hidden_act`, silu in wall-x's own configuration.
 
     eager_rounding=True reproduces the reference's op-by-op evaluation in the
     activation dtype: every F.linear / silu / multiply result is rounded to
@@ -39,16 +54,17 @@ def swiglu_ffn_ref(x, gate_w, up_w, down_w, eager_rounding: bool = True):
     throughout and rounds once at the end.
     """
     dt = x.dtype
+    fn = activation_ref(act)
     x32 = x.to(torch.float32)
     g = x32 @ gate_w.to(torch.float32).t()
     u = x32 @ up_w.to(torch.float32).t()
     if eager_rounding:
         g = g.to(dt).to(torch.float32)
         u = u.to(dt).to(torch.float32)
-        a = F.silu(g).to(dt).to(torch.float32)
+        a = fn(g).to(dt).to(torch.float32)
         h = (a * u).to(dt).to(torch.float32)
     else:
-        h = F.silu(g) * u
+        h = fn(g) * u
     y = h @ down_w.to(torch.float32).t()
     return y.to(dt)
 
@@ -69,11 +85,12 @@ def swiglu_bwd_ref(gate, up, dh):
     return hm, dg.to(dt), du.to(dt)
 
 
-def sparse_moe_block_ref(hidden, experts_indices, weights, eager_rounding: bool = True):
+def sparse_moe_block_ref(hidden, experts_indices, weights, eager_rounding: bool = True, acts=None):
     """SparseMoeBlock.forward (act.py:105-162).
 
     hidden [B, S, H]; experts_indices [B, S] (bool or integer expert id);
-    weights = [(gate_w, up_w, down_w), ...] per expert.  Permute groups the rows
+    weights = [(gate_w, up_w, down_w), ...] per expert (any number of experts);
+    acts = each expert's `hidden_act` (default: silu for all).  Permute groups the rows
     by expert (stable), each expert runs on its contiguous row range
     [start_e, end_e) (act.py:142-154; ranges from act.py:1274-1283), rows of
     experts with no tokens stay zero (act.py:139), unpermute restores the order
@@ -91,6 +108,6 @@ def sparse_moe_block_ref(hidden, experts_indices, weights, eager_rounding: bool 
         s, t = off[e], off[e + 1]
         if s == t:
             continue
-        out[s:t] = swiglu_ffn_ref(permuted[s:t], gw, uw, dw, eager_rounding)
+        out[s:t] = swiglu_ffn_ref(permuted[s:t], gw, uw, dw, eager_rounding, "silu" if acts is None else acts[e])
     y = unpermute_ref(out, row_id_map)
     return y.view(B, S, H)

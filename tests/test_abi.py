@@ -84,11 +84,20 @@ def test_argument_errors_without_a_gpu():
     assert lib.wx_dual_swiglu_gate_up_keep(*([None] * 9), 4, 64, 64, 64, None, None) == -1
     assert lib.wx_dual_down_proj_residual(*([None] * 6), 4, 64, 64, 64, None, None, None) == -1  # null pointers
     assert lib.wx_dual_down_proj_residual(*([None] * 6), 0, 64, 64, 64, None, None, None) == 0   # nothing to do
-    assert lib.wx_qkv_rope_proj(None, None, None, None, None, 4, 64, 1, 1, 96, None) == -2
+    assert lib.wx_qkv_rope_proj(None, None, None, None, 48, None, 4, 64, 1, 1, 96, None) == -2
     assert b"head_dim" in lib.wx_last_error_string()
-    assert lib.wx_qkv_rope_proj(None, None, None, None, None, 4, 64, 1, 1, 128, None) == -1
-    assert lib.wx_mrope_table(None, None, 1, 4, 128, _lib.i32x3((16, 24, 24)), _lib.WX_MROPE_CSRC, None, None) == -2
-    assert b"different position planes" in lib.wx_last_error_string()
+    assert lib.wx_qkv_rope_proj(None, None, None, None, 64, None, 4, 64, 1, 1, 128, None) == -1  # null pointers
+    assert lib.wx_qkv_rope_proj(None, None, None, None, 96, None, 4, 64, 1, 1, 128, None) == -1
+    assert b"table_width" in lib.wx_last_error_string()
+    # entries per token of the packed rotary table: one per channel pair when d and d + D/2 share a position plane
+    # (the PyTorch path's layout), one per channel when they do not (the CUDA kernel's layout)
+    sec = _lib.i32x3((16, 24, 24))
+    assert lib.wx_mrope_table_width(128, sec, _lib.WX_MROPE_HF) == 64
+    assert lib.wx_mrope_table_width(128, sec, _lib.WX_MROPE_CSRC) == 128
+    assert lib.wx_mrope_table_width(128, _lib.i32x3((64, 0, 0)), _lib.WX_MROPE_CSRC) == 64  # one plane: the maps agree
+    assert lib.wx_mrope_table_width(128, _lib.i32x3((16, 24, 25)), _lib.WX_MROPE_HF) == -1
+    assert lib.wx_mrope_table(None, None, 1, 4, 128, sec, _lib.WX_MROPE_CSRC, None, None) == -1  # null pointers
+    assert lib.wx_partition_build_noalloc(None, 0, 4, 200, 2, 0, None, None, None, None, None) == -2
     # M-RoPE from positions: shapes the row kernel cannot take are refused, not routed elsewhere
     st = _lib.i64x3((128 * 4, 128, 128 * 4))
     assert lib.wx_mrope_apply_positions(None, None, None, None, None, None, 1, 4, 2, 1, 128, st, st, st, st,

@@ -81,6 +81,34 @@ def test_checkpoint_to_block_forward(dev, tmp_path, dense, pack_only):
                 block(x.to(dev).requires_grad_(True), types.to(dev))
 
 
+def test_loading_into_a_block_that_kept_its_dense_weights_beside_the_packed_ones(dev):
+    """pack_for_inference(free_dense=False) leaves a block with both forms; a later load must not leave it running the
+    old packed weights."""
+    torch.manual_seed(0)
+    block = moe.SparseMoeBlock(_Cfg(), 2).to(torch.bfloat16).to(dev)
+    block.pack_for_inference(free_dense=False)
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(1, 120, H, generator=g).to(torch.bfloat16)
+    types = torch.rand(1, 120, generator=g) > 0.5
+    with torch.no_grad():
+        before = block(x.to(dev), types.to(dev))
+    sd = {}
+    for e, inter in enumerate(INTER):
+        for proj, shape in (("gate", (inter, H)), ("up", (inter, H)), ("down", (H, inter))):
+            sd[checkpoint.expert_weight_key(0, e, proj)] = (torch.randn(shape, generator=g) * 0.05).to(torch.bfloat16)
+    assert checkpoint.load_expert_weights(sd, {0: block}) == {0: 6}
+    assert block._packed is not None  # packed again, from the new values
+    with torch.no_grad():
+        after = block(x.to(dev), types.to(dev))
+    ws = [tuple(sd[checkpoint.expert_weight_key(0, e, p)] for p in ("gate", "up", "down")) for e in range(2)]
+    _close(after, oracle.sparse_moe_block_ref(x, types, ws))
+    assert int((after != before).sum()) > 0
+    # a block whose dense copies were released has nothing to load into: refused, not silently skipped
+    block.pack_for_inference(free_dense=True)
+    with pytest.raises(ValueError, match="checkpoint shape"):
+        checkpoint.load_expert_weights(sd, {0: block})
+
+
 def test_weight_written_through_data_after_a_forward(dev):
     """`.data` writes do not move torch's version counter.  A block whose weights train repacks on every forward, so
     it sees them; a frozen block needs native.invalidate_packed()."""

@@ -5,7 +5,7 @@ import pytest
 import torch
 
 import oracle
-from wallx_mi355 import moe, native, workloads as wl
+from wallx_mi355 import _lib, moe, native, workloads as wl
 from wallx_mi355.fusions import ops
 
 pytestmark = pytest.mark.gpu
@@ -164,7 +164,8 @@ def test_dual_gemm_add_accumulates_onto_an_addend(dev, trans_a, trans_b):
 def test_empty_contraction_of_one_expert_keeps_the_other_on_the_mfma_kernel(dev):
     """A weight gradient dW = dY^T X has k = the expert's token count: a batch without action tokens gives k1 = 0
     next to the VL expert's full-size contraction.  The empty one must come out as zeros and the other must not be
-    dragged onto the plain FMA kernel (two orders of magnitude slower), checked through the launch's duration."""
+    dragged onto the plain FMA kernel (two orders of magnitude slower), checked through the library's record of the
+    kernels the call launched (wx_last_gemm_path)."""
     g = torch.Generator().manual_seed(17)
     m0, n0, k0, m1, n1 = 2048, 2048, 4096, 512, 256
     a0, w0 = _bf((k0, m0), g).to(dev), _bf((k0, n0), g, 0.05).to(dev)      # trans_a: A stored [k, m]; B stored [k, n]
@@ -176,14 +177,11 @@ def test_empty_contraction_of_one_expert_keeps_the_other_on_the_mfma_kernel(dev)
     rows = torch.arange(0, m0, 61)
     ref = a0[:, rows.to(dev)].float().cpu().t() @ w0.float().cpu()
     _close(o0[rows.to(dev)], ref.to(torch.bfloat16), what="expert 0 beside an empty contraction")
-    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    start.record()
-    for _ in range(5):
-        native.asym_dual_gmm(a0, a1, w0, w1, o0, o1, True, False)
-    stop.record()
-    stop.synchronize()
-    per_call_ms = start.elapsed_time(stop) / 5
-    assert per_call_ms < 1.0, f"{per_call_ms:.2f} ms for 34 GFLOP: not the MFMA kernel"
+    # which kernels the call launched, from the library's own record of its last dual GEMM on this thread
+    path = _lib.load().wx_last_gemm_path()
+    assert path == _lib.WX_GEMM_PATH_MFMA | _lib.WX_GEMM_PATH_ZERO_FILL, f"launched {path:#x}: not MFMA + zero fill"
+    native.asym_dual_gmm(a0, a0[:, :m1], w0, w0[:, :n1].contiguous(), o0, o1, True, False)  # both contractions full
+    assert _lib.load().wx_last_gemm_path() == _lib.WX_GEMM_PATH_MFMA
 
 
 def test_dual_gemm_rejects_what_the_reference_rejects(dev):
@@ -368,6 +366,88 @@ def test_moe_block_module_is_a_drop_in(dev):
     assert y.shape == (2, 100, 256)
     _close(y, ref, what="block")
     assert int((y != y2).sum()) == 0
+
+
+@pytest.mark.parametrize("inters,acts", [((384, 128, 256), ("gelu", "silu", "gelu_pytorch_tanh")),
+                                         ((256, 64), ("gelu", "relu")), ((192, 320, 64, 128), ("silu",) * 4)])
+def test_moe_block_with_other_expert_lists_runs_on_the_generic_ops(dev, inters, acts):
+    """`SparseMoeBlock(config, num_experts)` accepts any expert list (act.py:71-77, 99-103, 142-154).  Three experts,
+    four experts, gelu / relu gating: the block runs permute -> pairs of experts as dual GEMMs with the activation as a
+    torch op -> unpermute, forward against the oracle and backward against autograd of the oracle's expression."""
+    from types import SimpleNamespace
+
+    E, H = len(inters), 256
+    cfg = SimpleNamespace(experts=[dict(hidden_size=H, intermediate_size=i, hidden_act=a) for i, a in zip(inters, acts)])
+    torch.manual_seed(3)
+    block = moe.SparseMoeBlock(cfg, E).to(torch.bfloat16)
+    with torch.no_grad():
+        for prm in block.parameters():
+            prm.mul_(2.0)  # nn.Linear's default init is small at these sizes: give the activations a visible range
+    g = torch.Generator().manual_seed(5)
+    x = _bf((2, 150, H), g)
+    ids = torch.randint(0, E, (2, 150), generator=g)
+    ids[ids == 1] = 0 if E == 3 else 1  # with three experts the middle one gets no tokens (act.py:144-145)
+    weights = [tuple(w.detach().clone() for w in e.weights()) for e in block.experts]
+    ref = oracle.sparse_moe_block_ref(x, ids, weights, acts=acts)
+    block = block.to(dev)
+    counts = torch.bincount(ids.reshape(-1), minlength=E)
+    end = torch.cumsum(counts, 0)
+    start = end - counts  # the caller's CPU row ranges (act.py:1274-1283)
+    with torch.no_grad():
+        y = block(x.to(dev), ids.to(dev), start, end)
+        y_dev_ranges = block(x.to(dev), ids.to(dev))  # without them: the partition's offsets are read back
+    _close(y, ref, what="generic block")
+    assert torch.equal(y, y_dev_ranges)
+    # backward: gradients of sum(y * dy) against autograd of the oracle in fp32 on the same (bf16-valued) weights
+    xd = x.to(dev).requires_grad_(True)
+    dy = _bf((2, 150, H), g)
+    block(xd, ids.to(dev), start, end).backward(dy.to(dev))
+    x32 = x.float().requires_grad_(True)
+    w32 = [tuple(t.float().requires_grad_(True) for t in w) for w in weights]
+    oracle.sparse_moe_block_ref(x32, ids, w32, eager_rounding=False, acts=acts).backward(dy.float())
+
+    def close_grad(got, want, what):
+        got, want = got.float().cpu(), want.float()
+        scale = float(want.abs().max()) + 1e-6
+        assert float((got - want).abs().max()) <= 3e-2 * scale, f"{what}: {float((got - want).abs().max())} vs scale {scale}"
+
+    close_grad(xd.grad, x32.grad, "dx")
+    for e in range(E):
+        for prm, want, name in zip(block.experts[e].weights(), w32[e], ("gate", "up", "down")):
+            if int(counts[e]) == 0:
+                assert prm.grad is None or float(prm.grad.abs().max()) == 0.0
+            else:
+                close_grad(prm.grad, want.grad, f"expert {e} {name}")
+
+
+def test_moe_block_under_inference_mode(dev):
+    """Tensors made under torch.inference_mode() have no version counter: the block must neither read one nor reuse
+    anything it could only have validated against one."""
+    class Cfg:
+        experts = [{"hidden_size": 256, "intermediate_size": 512, "hidden_act": "silu"},
+                   {"hidden_size": 256, "intermediate_size": 128, "hidden_act": "silu"}]
+
+    torch.manual_seed(0)
+    block = moe.SparseMoeBlock(Cfg(), 2).to(torch.bfloat16).to(dev)
+    weights = [tuple(w.detach().cpu().clone() for w in e.weights()) for e in block.experts]
+    g = torch.Generator().manual_seed(1)
+    x = _bf((1, 300, 256), g)
+    types = torch.rand(1, 300, generator=g) > 0.7
+    with torch.inference_mode():
+        types_d = types.to(dev)  # made inside inference mode, like a model's own `input_ids == action_token`
+        n0 = int((~types).sum())
+        start, end = torch.tensor([0, n0]), torch.tensor([n0, 300])
+        y = block(x.to(dev), types_d, start, end)
+        _close(y, oracle.sparse_moe_block_ref(x, types, weights), what="inference mode")
+        types_d[0, :40] = ~types_d[0, :40]  # an in-place change nothing records: the next call must partition again
+        types2 = types.clone()
+        types2[0, :40] = ~types2[0, :40]
+        y2 = block(x.to(dev), types_d)
+        _close(y2, oracle.sparse_moe_block_ref(x, types2, weights), what="inference mode, changed types")
+        # the functional form with weights made inside inference mode
+        w_inf = [tuple(t.to(dev) for t in w) for w in weights]
+        y3, _ = moe.moe_layer_forward(x.view(-1, 256).to(dev), types_d.view(-1), w_inf)
+        assert torch.equal(y3.view_as(y2), y2)
 
 
 def test_config1_golden_shapes_in_bf16(dev):

@@ -194,11 +194,14 @@ def test_mrope_from_positions_refuses_what_it_cannot_do(dev):
                                            pos[:, :, :5].to(dev), inv_freq, [16, 24, 24])
 
 
-def test_mrope_from_packed_table_equals_the_positions_path(dev):
-    """multimodal_rope_from_table reads cos / sin from the packed table of multimodal_rope_table (256 bytes per token,
-    built once per forward); the table holds what the positions path evaluates per thread (the same device sincosf on
+@pytest.mark.parametrize("layout", ["hf", "csrc"])
+def test_mrope_from_packed_table_equals_the_positions_path(dev, layout):
+    """multimodal_rope_from_table reads cos / sin from the packed table of multimodal_rope_table (256 bytes per token
+    for the PyTorch path's layout, 512 for the CUDA kernel's, whose channels d and d + 64 take different planes; built
+    once per forward); the table holds what the positions path evaluates per thread (the same device sincosf on
     the same angle, rounded to bf16), so forward and backward equal that path bit for bit -- at config 2's full size,
-    through strided views, and for a short ragged sequence -- and the oracle within the stated tolerance."""
+    through strided views, and for a short ragged sequence with distinct t / h / w positions -- and the oracle of the
+    same layout within the stated tolerance."""
     ids, grid = wl.config2_tokens()
     pos, _ = oracle.rope_index_ref(ids, 2, wl.IMAGE_TOKEN_ID, wl.VIDEO_TOKEN_ID, wl.VISION_START_TOKEN_ID, 2,
                                    image_grid_thw=grid)
@@ -209,13 +212,14 @@ def test_mrope_from_packed_table_equals_the_positions_path(dev):
     q2, k2, pos2 = _pos_inputs(3, 37, torch.bfloat16, 31)
     cases.append((q2.transpose(1, 2).contiguous(), k2.transpose(1, 2).contiguous(), pos2))
     for qt, kt, p_ in cases:
-        table = ops.multimodal_rope_table(p_.to(dev), inv_freq.to(dev), sec)
+        table = ops.multimodal_rope_table(p_.to(dev), inv_freq.to(dev), sec, layout)
+        assert tuple(table.shape) == (p_.shape[1] * p_.shape[2], 64 if layout == "hf" else 128)
         qd, kd = qt.to(dev).requires_grad_(True), kt.to(dev).requires_grad_(True)
-        tq, tk = ops.multimodal_rope_from_table(qd, kd, table, sec)
-        pq, pk = ops.multimodal_rope_from_positions(qt.to(dev), kt.to(dev), p_.to(dev), inv_freq.to(dev), sec)
+        tq, tk = ops.multimodal_rope_from_table(qd, kd, table, sec, layout)
+        pq, pk = ops.multimodal_rope_from_positions(qt.to(dev), kt.to(dev), p_.to(dev), inv_freq.to(dev), sec, layout)
         assert _n_diff(tq.detach(), pq.cpu()) == 0 and _n_diff(tk.detach(), pk.cpu()) == 0
         cos, sin = oracle.rotary_cos_sin_ref(p_, inv_freq, torch.bfloat16)
-        rq, rk = oracle.mrope_apply_ref(qt, kt, cos, sin, sec, "hf")
+        rq, rk = oracle.mrope_apply_ref(qt, kt, cos, sin, sec, layout)
         _close(tq.detach(), rq)
         _close(tk.detach(), rk)
         g = torch.Generator(device=dev).manual_seed(5)
@@ -223,17 +227,18 @@ def test_mrope_from_packed_table_equals_the_positions_path(dev):
         gk = torch.randn(tk.shape, device=dev, generator=g).to(torch.bfloat16)
         torch.autograd.backward([tq, tk], [gq, gk])
         bq, bk = torch.empty_like(gq), torch.empty_like(gk)
-        native.rope_from_positions(gq, gk, p_.to(dev), inv_freq.to(dev), bq, bk, [2 * v for v in sec], backward=True)
+        native.rope_from_positions(gq, gk, p_.to(dev), inv_freq.to(dev), bq, bk, [2 * v for v in sec], backward=True,
+                                   layout=layout)
         assert _n_diff(qd.grad, bq.cpu()) == 0 and _n_diff(kd.grad, bk.cpu()) == 0
-    # what it cannot do is refused: fp16 (the table is bf16), the csrc layout (its half-channels take different planes)
-    table = ops.multimodal_rope_table(pos2.to(dev), inv_freq.to(dev), sec)
+    # what it cannot do is refused: fp16 (the table is bf16), a table built for the other layout (its width differs)
+    table = ops.multimodal_rope_table(pos2.to(dev), inv_freq.to(dev), sec, layout)
     qh, kh = cases[1][0].to(dev), cases[1][1].to(dev)
     with pytest.raises(RuntimeError):
         native.rope_from_table(qh.half(), kh.half(), table, torch.empty_like(qh.half()), torch.empty_like(kh.half()),
-                               [2 * v for v in sec])
-    with pytest.raises(RuntimeError, match="different position planes"):
+                               [2 * v for v in sec], layout=layout)
+    with pytest.raises(RuntimeError, match="same mrope_section and layout"):
         native.rope_from_table(qh, kh, table, torch.empty_like(qh), torch.empty_like(kh), [2 * v for v in sec],
-                               layout="csrc")
+                               layout="csrc" if layout == "hf" else "hf")
 
 
 def test_extension_level_rope_uses_the_cuda_kernels_layout(dev):

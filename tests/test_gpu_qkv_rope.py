@@ -1,6 +1,7 @@
 """GPU parity of the q / k / v projection with M-RoPE in the GEMM epilogue (vl.py:955-964 as one launch) against the
-oracle: an fp32 linear layer rounded to bf16, then mrope_apply_ref in eager bf16 (the PyTorch path's layout).
-Tolerance |x - ref| <= 2e-2 + 1e-2 |ref|."""
+oracle: an fp32 linear layer rounded to bf16, then mrope_apply_ref in eager bf16, in both channel layouts (the
+PyTorch path's, vl.py:763-769, and the CUDA kernel's, csrc/rope.cu:104-117, which the flash-attention class of
+vl.py:962-964 runs).  Tolerance |x - ref| <= 2e-2 + 1e-2 |ref|."""
 
 import pytest
 import torch
@@ -21,7 +22,7 @@ def _close(got, ref, what):
     assert not bad.any(), f"{what}: {int(bad.sum())} of {bad.numel()} outside tolerance, max abs err {float(err.max())}"
 
 
-def _reference(x, w, b, pos, nq, nkv, rows=None):
+def _reference(x, w, b, pos, nq, nkv, rows=None, layout="hf"):
     """(q, k, v) [B, H, S, D] from the oracle; rows: optional token subset (flattened indices) to evaluate."""
     B, S, H = x.shape
     D = 128
@@ -37,13 +38,14 @@ def _reference(x, w, b, pos, nq, nkv, rows=None):
     q = q.reshape(B, S, nq, D).transpose(1, 2)
     k = k.reshape(B, S, nkv, D).transpose(1, 2)
     v = v.reshape(B, S, nkv, D).transpose(1, 2)
-    rq, rk = oracle.mrope_apply_ref(q, k, cos, sin, list(wl.MROPE_SECTION), "hf", eager_rounding=True)
+    rq, rk = oracle.mrope_apply_ref(q, k, cos, sin, list(wl.MROPE_SECTION), layout, eager_rounding=True)
     return rq, rk, v
 
 
+@pytest.mark.parametrize("layout", ["hf", "csrc"])
 @pytest.mark.parametrize("B,S,H,nq,nkv,with_bias", [(2, 300, 512, 4, 2, True), (1, 37, 256, 2, 1, False),
                                                    (3, 256, 1024, 3, 1, True), (1, 1, 64, 1, 1, True)])
-def test_qkv_rope_projection(dev, B, S, H, nq, nkv, with_bias):
+def test_qkv_rope_projection(dev, B, S, H, nq, nkv, with_bias, layout):
     g = torch.Generator().manual_seed(B * 1000 + S)
     x = torch.randn(B, S, H, generator=g).to(torch.bfloat16)
     n = (nq + 2 * nkv) * 128
@@ -51,13 +53,14 @@ def test_qkv_rope_projection(dev, B, S, H, nq, nkv, with_bias):
     b = (torch.randn(n, generator=g) * 0.5).to(torch.bfloat16) if with_bias else None
     pos = torch.stack([torch.randint(0, 60, (B, S), generator=g), torch.randint(100, 160, (B, S), generator=g),
                        torch.randint(300, 360, (B, S), generator=g)])  # distinct planes
-    table = ops.multimodal_rope_table(pos.to(dev), wl.text_inv_freq().to(dev), wl.MROPE_SECTION)
-    assert table.shape == (B * S, 64) and table.dtype == torch.int32
+    width = 64 if layout == "hf" else 128  # the CUDA kernel's layout rotates d and d + 64 by different planes
+    table = ops.multimodal_rope_table(pos.to(dev), wl.text_inv_freq().to(dev), wl.MROPE_SECTION, layout)
+    assert table.shape == (B * S, width) and table.dtype == torch.int32
     # the table itself: bf16 cos / sin of the oracle's builder, packed
     cos, sin = oracle.rotary_cos_sin_ref(pos, wl.text_inv_freq(), torch.bfloat16)
-    amap = oracle.mrope_axis_map(wl.MROPE_SECTION, 128, "hf")[:64]
-    cos_sel = cos[amap, :, :, torch.arange(64)].permute(1, 2, 0).reshape(B * S, 64)
-    sin_sel = sin[amap, :, :, torch.arange(64)].permute(1, 2, 0).reshape(B * S, 64)
+    amap = oracle.mrope_axis_map(wl.MROPE_SECTION, 128, layout)[:width]
+    cos_sel = cos[amap, :, :, torch.arange(width)].permute(1, 2, 0).reshape(B * S, width)
+    sin_sel = sin[amap, :, :, torch.arange(width)].permute(1, 2, 0).reshape(B * S, width)
     tb = table.cpu()
     got_cos = (tb << 16).view(torch.float32)
     got_sin = (tb & -65536).view(torch.float32)
@@ -66,7 +69,10 @@ def test_qkv_rope_projection(dev, B, S, H, nq, nkv, with_bias):
     assert bool(((got_cos - cos_sel.float()).abs() <= 2.0 ** -7).all()) and bool(((got_sin - sin_sel.float()).abs() <= 2.0 ** -7).all())
     q, k, v = ops.qkv_projection_with_rope(x.to(dev), w.to(dev), None if b is None else b.to(dev), table, nq, nkv)
     assert q.shape == (B, nq, S, 128) and k.shape == (B, nkv, S, 128) and v.shape == (B, nkv, S, 128)
-    rq, rk, rv = _reference(x, w, b, pos, nq, nkv)
+    rq, rk, rv = _reference(x, w, b, pos, nq, nkv, layout=layout)
+    if layout == "csrc":  # the two layouts must not coincide on these positions (distinct planes)
+        hq, _, _ = _reference(x, w, b, pos, nq, nkv, layout="hf")
+        assert not torch.equal(hq, rq)
     _close(q, rq, "q")
     _close(k, rk, "k")
     _close(v, rv, "v")
@@ -74,7 +80,7 @@ def test_qkv_rope_projection(dev, B, S, H, nq, nkv, with_bias):
     qkv = F.linear(x.to(dev), w.to(dev), None if b is None else b.to(dev))
     q2, k2, _ = qkv.split([nq * 128, nkv * 128, nkv * 128], dim=-1)
     gq, gk = ops.multimodal_rope_from_positions(q2.reshape(B, S, nq, 128).transpose(1, 2), k2.reshape(B, S, nkv, 128).transpose(1, 2),
-                                                pos.to(dev), wl.text_inv_freq().to(dev), list(wl.MROPE_SECTION))
+                                                pos.to(dev), wl.text_inv_freq().to(dev), list(wl.MROPE_SECTION), layout)
     _close(q, gq.cpu(), "q vs two-step path")
     _close(k, gk.cpu(), "k vs two-step path")
 
@@ -103,10 +109,8 @@ def test_qkv_rope_projection_config5_shape(dev):
 def test_qkv_rope_rejects_what_it_cannot_do(dev):
     lib = _lib.load()
     pos = torch.zeros(3, 1, 4, dtype=torch.int64, device=dev)
-    with pytest.raises(RuntimeError, match="different position planes"):
-        native.mrope_table(pos, wl.text_inv_freq().to(dev), wl.MROPE_SECTION, layout="csrc")
     p = pos.data_ptr()
-    assert lib.wx_qkv_rope_proj(p, p, None, p, p, 4, 64, 1, 1, 64, None) == -2
+    assert lib.wx_qkv_rope_proj(p, p, None, p, 32, p, 4, 64, 1, 1, 64, None) == -2
     assert b"head_dim" in lib.wx_last_error_string()
     x = torch.zeros(1, 4, 64, dtype=torch.bfloat16, device=dev).requires_grad_(True)
     with pytest.raises(RuntimeError, match="no backward"):

@@ -116,6 +116,45 @@ def test_moe_block_matches_per_token_evaluation():
     assert torch.allclose(y0.view(-1, H), oracle.swiglu_ffn_ref(x.view(-1, H), *ws[0].as_tuple()), atol=1e-6)
 
 
+def test_gated_ffn_with_other_activations_and_three_experts_against_a_scalar_loop():
+    """`hidden_act` other than silu and an expert list of any length (act.py:71-77, 99-103, 142-154): the block
+    against a float64 evaluation token by token, with gelu written through math.erf, the tanh form through math.tanh
+    and relu through max -- nothing of the oracle's own expression is reused."""
+    import math
+
+    scalar = {
+        "gelu": lambda v: 0.5 * v * (1.0 + math.erf(v / math.sqrt(2.0))),
+        "gelu_pytorch_tanh": lambda v: 0.5 * v * (1.0 + math.tanh(math.sqrt(2.0 / math.pi) * (v + 0.044715 * v ** 3))),
+        "relu": lambda v: max(v, 0.0),
+        "silu": lambda v: v / (1.0 + math.exp(-v)),
+    }
+    g = torch.Generator().manual_seed(21)
+    B, S, H = 2, 9, 8
+    inters, acts = (6, 4, 10), ("gelu", "relu", "gelu_pytorch_tanh")
+    x = torch.randn(B, S, H, generator=g)
+    ids = torch.randint(0, 3, (B, S), generator=g)
+    ws = [wl.expert_weights(H, i, torch.float32, g, 0.5).as_tuple() for i in inters]
+    y = oracle.sparse_moe_block_ref(x, ids, ws, eager_rounding=False, acts=acts).double()
+    for b in range(B):
+        for s_ in range(S):
+            e = int(ids[b, s_])
+            gw, uw, dw = (t.double().tolist() for t in ws[e])
+            xv = x[b, s_].double().tolist()
+            hidden = []
+            for i in range(inters[e]):
+                gate = sum(a * w for a, w in zip(xv, gw[i]))
+                up = sum(a * w for a, w in zip(xv, uw[i]))
+                hidden.append(scalar[acts[e]](gate) * up)
+            for o in range(H):
+                want = sum(h * w for h, w in zip(hidden, dw[o]))
+                assert abs(float(y[b, s_, o]) - want) <= 1e-5 + 1e-5 * abs(want), (b, s_, o)
+    # the named functions themselves, on a grid of arguments
+    t = torch.linspace(-6, 6, 49, dtype=torch.float64)
+    for name, fn in scalar.items():
+        got = oracle.activation_ref(name)(t)
+        assert torch.allclose(got, torch.tensor([fn(float(v)) for v in t], dtype=torch.float64), rtol=1e-9, atol=1e-12)
+
+
 # ----------------------------------------------------------------------------- M-RoPE
 def _cos_sin(pos, dtype=torch.float32):
     return oracle.rotary_cos_sin_ref(pos, wl.text_inv_freq(), dtype)

@@ -49,6 +49,12 @@ def test_noalloc_partition_equals_the_workspace_entry_point_twice_in_a_row(dev):
         assert torch.equal(flat[s1.long()], torch.sort(flat, stable=True).values)
 
 
+def test_noalloc_init_is_idempotent(dev):
+    lib = _lib.load()
+    assert lib.wx_partition_noalloc_init() == 0
+    assert lib.wx_partition_noalloc_init() == 0
+
+
 def test_noalloc_partition_rejects_what_does_not_fit(dev):
     lib = _lib.load()
     p = torch.zeros(8, dtype=torch.int32, device=dev).data_ptr()

@@ -13,6 +13,10 @@ int fail(int code, const char* fmt, ...);
 // hipGetLastError() after a launch; WX_OK or WX_ERR_LAUNCH with the HIP error text recorded.
 int check_launch(const char* what);
 
+// Bits of wx_last_gemm_path() for the calling thread: cleared at the start of a dual GEMM call, set as it launches.
+void gemm_path_reset();
+void gemm_path_note(int bit);
+
 inline hipStream_t as_stream(wx_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
 
 constexpr int kWave = 64;

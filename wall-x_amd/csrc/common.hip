@@ -16,6 +16,10 @@ int fail(int code, const char* fmt, ...) {
   return code;
 }
 
+static thread_local int g_gemm_path = 0;
+void gemm_path_reset() { g_gemm_path = 0; }
+void gemm_path_note(int bit) { g_gemm_path |= bit; }
+
 int check_launch(const char* what) {
   hipError_t e = hipGetLastError();
   if (e == hipSuccess) return WX_OK;
@@ -39,6 +43,7 @@ int device_cu_count() {
 }  // namespace wx
 
 extern "C" const char* wx_last_error_string(void) { return wx::g_error; }
+extern "C" int wx_last_gemm_path(void) { return wx::g_gemm_path; }
 extern "C" int wx_abi_version(void) { return 1; }
 
 extern "C" int wx_stream_capture_id(wx_stream_t stream, unsigned long long* id) {

@@ -137,11 +137,12 @@ struct Params {
   // closing residual add.  May be the output itself.
   const __bf16* residual;
   // kQkvRope only (group 0 is the projection, row-major operands): bias[n] (may be null), the packed rotary table
-  // [m, 64] (bf16 cos | bf16 sin << 16 per token and channel pair) and the number of leading output columns that are
-  // rotated (whole heads of 128: the q and k heads; the v heads behind them only take the bias).
+  // [m, rope_width] (bf16 cos | bf16 sin << 16 per token and channel: rope_width 64 when channels d and d + 64 share
+  // an entry, 128 when every channel has its own) and the number of leading output columns that are rotated (whole
+  // heads of 128: the q and k heads; the v heads behind them only take the bias).
   const __bf16* bias;
   const uint32_t* rope_table;
-  int rope_cols;
+  int rope_cols, rope_width;
   // kGateUp only (training): when set, the two projections themselves (rounded to bf16, before the SwiGLU) are
   // stored as well, K-tiled with the geometry of the intermediate, so that a backward pass need not recompute them.
   __bf16* keep_gate;
@@ -757,29 +758,32 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
           for (int j = 0; j < 4; ++j) bias_v[j] = static_cast<float>(p.bias[col_w + j * 32 + el32]);
         }
         const bool rotate = live && col_w < p.rope_cols;  // wave-uniform: q and k heads rotate, v heads do not
+        const bool full = p.rope_width == 128;  // uniform: channels d and d + 64 have entries of their own
 #pragma unroll
         for (int i = 0; i < FM; ++i) {
-          uint32_t cs[16][2];
-          if (rotate) {
+#pragma unroll
+          for (int jp = 0; jp < 2; ++jp) {
+            // cos | sin of this lane's channel d = 32 jp + lane % 32 (and of d + 64 when they differ) for its 16 rows
+            uint32_t cs_lo[16], cs_hi[16];
+            if (rotate) {
+#pragma unroll
+              for (int r = 0; r < 16; ++r) {
+                const int row = wm * (FM * 32) + i * 32 + 8 * (r >> 2) + 4 * elhi + (r & 3);
+                const bool in = row < S.rows;
+                const uint32_t* t = p.rope_table + static_cast<int64_t>(S.row0 + (in ? row : 0)) * p.rope_width + jp * 32 + el32;
+                cs_lo[r] = t[0];
+                cs_hi[r] = full ? t[64] : cs_lo[r];
+              }
+            }
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-              const int row = wm * (FM * 32) + i * 32 + 8 * (r >> 2) + 4 * elhi + (r & 3);
-              const bool in = row < S.rows;
-              const uint32_t* t = p.rope_table + static_cast<int64_t>(S.row0 + (in ? row : 0)) * 64 + el32;
-              cs[r][0] = t[0];
-              cs[r][1] = t[32];
-            }
-          }
-#pragma unroll
-          for (int r = 0; r < 16; ++r) {
-#pragma unroll
-            for (int jp = 0; jp < 2; ++jp) {
               const float lo = round_bf16(acc[i][jp][r] + bias_v[jp]);
               const float hi = round_bf16(acc[i][jp + 2][r] + bias_v[jp + 2]);
               if (rotate) {
-                const float c = __uint_as_float(cs[r][jp] << 16), sn = __uint_as_float(cs[r][jp] & 0xffff0000u);
-                acc[i][jp][r] = round_bf16(lo * c) - round_bf16(hi * sn);
-                acc[i][jp + 2][r] = round_bf16(hi * c) + round_bf16(lo * sn);
+                const float c_lo = __uint_as_float(cs_lo[r] << 16), s_lo = __uint_as_float(cs_lo[r] & 0xffff0000u);
+                const float c_hi = __uint_as_float(cs_hi[r] << 16), s_hi = __uint_as_float(cs_hi[r] & 0xffff0000u);
+                acc[i][jp][r] = round_bf16(lo * c_lo) - round_bf16(hi * s_lo);
+                acc[i][jp + 2][r] = round_bf16(hi * c_hi) + round_bf16(lo * s_hi);
               } else {
                 acc[i][jp][r] = lo;
                 acc[i][jp + 2][r] = hi;
@@ -1108,6 +1112,7 @@ int dual_gemm_impl(const void* in0, const void* in1, const void* w0, const void*
                    const void* add0, const void* add1, int64_t m0, int64_t n0, int64_t k0, int64_t m1, int64_t n1,
                    int64_t k1, int trans_a, int trans_b, wx_stream_t stream) {
   const void* adds[2] = {add0, add1};
+  gemm_path_reset();
   const bool k_in_rows = trans_a && !trans_b;  // A [k, m] and B [k, n]
   if (int rc = check_dims("wx_dual_gemm", m0, n0, k0, k_in_rows)) return rc;
   if (int rc = check_dims("wx_dual_gemm", m1, n1, k1, k_in_rows)) return rc;
@@ -1147,6 +1152,7 @@ int dual_gemm_impl(const void* in0, const void* in1, const void* w0, const void*
       if (adds[e] != ptrs[e][2] &&
           hipMemcpyAsync(const_cast<void*>(ptrs[e][2]), adds[e], static_cast<size_t>(m) * n * 2, hipMemcpyDeviceToDevice, s) != hipSuccess)
         return fail(WX_ERR_LAUNCH, "wx_dual_gemm_add: copy of the addend failed");
+      gemm_path_note(WX_GEMM_PATH_ADD_COPY);
       p.g[e].m = 0;
       continue;
     }
@@ -1155,6 +1161,7 @@ int dual_gemm_impl(const void* in0, const void* in1, const void* w0, const void*
     hipLaunchKernelGGL(zero_fill_kernel, dim3(static_cast<unsigned>(want < cap ? want : cap)), dim3(256), 0, s,
                        static_cast<u32x4*>(const_cast<void*>(ptrs[e][2])), n16);
     if (int rc = check_launch("zero_fill_kernel")) return rc;
+    gemm_path_note(WX_GEMM_PATH_ZERO_FILL);
     p.g[e].m = 0;
   }
   if ((p.g[0].m == 0 || n0 == 0) && (p.g[1].m == 0 || n1 == 0)) return WX_OK;
@@ -1168,23 +1175,28 @@ int dual_gemm_impl(const void* in0, const void* in1, const void* w0, const void*
   if (fits) {
     const int64_t tiles = ceil_div(mm0, BigTile::BM) * ceil_div(n0, BigTile::BN) + ceil_div(mm1, BigTile::BM) * ceil_div(n1, BigTile::BN);
     const char* who = "dual_gemm_kernel<generic>";
+    gemm_path_note(WX_GEMM_PATH_MFMA);
     if (!trans_a && trans_b) return launch_mfma<kGeneric, false, false>(p, tiles, tiles, s, who);
     if (!trans_a && !trans_b) return launch_mfma<kGeneric, false, true>(p, tiles, tiles, s, who);
     if (trans_a && trans_b) return launch_mfma<kGeneric, true, false>(p, tiles, tiles, s, who);
     return launch_mfma<kGeneric, true, true>(p, tiles, tiles, s, who);
   }
+  gemm_path_note(WX_GEMM_PATH_FMA);
   hipLaunchKernelGGL(dual_gemm_reference_layout_kernel, dim3(device_cu_count() * 4), dim3(256), 0, s, p, trans_a, trans_b);
   return check_launch("dual_gemm_reference_layout_kernel");
 }
 }  // namespace
 
 extern "C" int wx_qkv_rope_proj(const void* x, const void* weight, const void* bias, const uint32_t* rope_table,
-                                void* out, int64_t num_tokens, int64_t hidden, int n_q_heads, int n_kv_heads,
-                                int head_dim, wx_stream_t stream) {
+                                int table_width, void* out, int64_t num_tokens, int64_t hidden, int n_q_heads,
+                                int n_kv_heads, int head_dim, wx_stream_t stream) {
   const char* who = "wx_qkv_rope_proj";
   if (n_q_heads < 0 || n_kv_heads < 0) return fail(WX_ERR_INVALID_ARGUMENT, "%s: negative head count", who);
   if (head_dim != 128)
     return fail(WX_ERR_UNSUPPORTED, "%s: head_dim %d; the epilogue rotates heads of 128 channels", who, head_dim);
+  if (table_width != head_dim / 2 && table_width != head_dim)
+    return fail(WX_ERR_INVALID_ARGUMENT, "%s: table_width %d must be %d (channels d and d + %d share an entry) or %d", who,
+                table_width, head_dim / 2, head_dim / 2, head_dim);
   const int64_t n = static_cast<int64_t>(n_q_heads + 2 * n_kv_heads) * head_dim;
   if (int rc = check_dims(who, num_tokens, n, hidden)) return rc;
   if (num_tokens == 0 || n == 0) return WX_OK;
@@ -1205,6 +1217,7 @@ extern "C" int wx_qkv_rope_proj(const void* x, const void* weight, const void* b
   p.bias = static_cast<const __bf16*>(bias);
   p.rope_table = rope_table;
   p.rope_cols = (n_q_heads + n_kv_heads) * head_dim;
+  p.rope_width = table_width;
   // the large tile only: its wavefronts cover whole heads (the small tile's 64 columns would split a rotation pair)
   using Tile = BigTileFor<kQkvRope>;
   hipLaunchKernelGGL((dual_gemm_kernel<kQkvRope, Tile, false, false>), dim3(device_cu_count()), dim3(Tile::kThreads),

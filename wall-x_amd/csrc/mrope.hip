@@ -187,9 +187,11 @@ __device__ __forceinline__ u32x4 partner_chunk(const u32x4& v, int half_lanes) {
 //                  The thread evaluates cos/sin of its channels itself, the way the table builder does
 //                  (vl.py:679-712): the angle is the fp32 product position * inv_freq (channels d and d + head_dim/2
 //                  share a frequency), cos and sin are taken in fp32 and rounded to the storage type;
-//   kSrcPacked     `cos_t` is the packed table of wx_mrope_table, uint32 [n_tokens, head_dim / 2] (bf16 cos | bf16 sin
-//                  << 16 of the plane each channel pair takes): 256 bytes per token instead of the 12 cache lines the
-//                  selected channels of three planes of two tables touch.  bf16 only.
+//   kSrcPacked     `cos_t` is the packed table of wx_mrope_table, uint32 [n_tokens, W] (bf16 cos | bf16 sin << 16 of
+//                  the plane each channel takes): W = head_dim / 2 when channels d and d + head_dim / 2 share a plane
+//                  (256 bytes per token instead of the 12 cache lines the selected channels of three planes of two
+//                  tables touch), W = head_dim when they do not (one entry per channel); `sin_t` carries W as a
+//                  pointer-sized integer.  bf16 only.
 enum { kSrcTables = 0, kSrcPositions = 1, kSrcPacked = 2 };
 template <int DT, bool BWD, int L, int SRC>
 __global__ __launch_bounds__(256) void mrope_rows_kernel(
@@ -218,7 +220,8 @@ __global__ __launch_bounds__(256) void mrope_rows_kernel(
   u32x4 c_raw, s_raw;
   if constexpr (SRC == kSrcPacked) {
     static_assert(DT == WX_BF16, "the packed table holds bf16 pairs");
-    const uint32_t* t = static_cast<const uint32_t*>(cos_t) + token * (head_dim / 2) + (hi ? d0 - head_dim / 2 : d0);
+    const int width = static_cast<int>(reinterpret_cast<uintptr_t>(sin_t));
+    const uint32_t* t = static_cast<const uint32_t*>(cos_t) + token * width + ((hi && width != head_dim) ? d0 - head_dim / 2 : d0);
     const u32x4 t0 = *reinterpret_cast<const u32x4*>(t), t1 = *reinterpret_cast<const u32x4*>(t + 4);
     c_raw = u32x4{(t0[0] & 0xffffu) | (t0[1] << 16), (t0[2] & 0xffffu) | (t0[3] << 16),
                   (t1[0] & 0xffffu) | (t1[1] << 16), (t1[2] & 0xffffu) | (t1[3] << 16)};
@@ -318,6 +321,15 @@ int build_axis_table(const int sec[3], int head_dim, int layout, AxisTable& ax) 
   return WX_OK;
 }
 
+// Entries per token of the packed table: head_dim / 2 when every channel d shares its position plane with channel
+// d + head_dim / 2 (the PyTorch path's layout, vl.py:763-769: one entry serves both), head_dim otherwise (the CUDA
+// kernel's layout, csrc/rope.cu:104-117: one entry per channel).
+int packed_table_width(const AxisTable& ax, int head_dim) {
+  for (int d = 0; d < head_dim / 2; ++d)
+    if (ax.axis[d] != ax.axis[d + head_dim / 2]) return head_dim;
+  return head_dim / 2;
+}
+
 // SRC: what cos_t / sin_t carry (see mrope_rows_kernel)
 template <bool BWD, int SRC = kSrcTables>
 int launch(const void* q, const void* k, const void* cos_t, const void* sin_t, void* q_out, void* k_out,
@@ -343,10 +355,8 @@ int launch(const void* q, const void* k, const void* cos_t, const void* sin_t, v
   AxisTable ax{};
   if (int rc = build_axis_table(sec, head_dim, layout, ax)) return rc;
   if constexpr (SRC == kSrcPacked) {
-    for (int d = 0; d < head_dim / 2; ++d)
-      if (ax.axis[d] != ax.axis[d + head_dim / 2])
-        return fail(WX_ERR_UNSUPPORTED, "%s: channels %d and %d take different position planes in this layout", who, d,
-                    d + head_dim / 2);
+    // the table's width follows from the layout exactly as in wx_mrope_table; it travels in the unused `sin_t` slot
+    sin_t = reinterpret_cast<const void*>(static_cast<uintptr_t>(packed_table_width(ax, head_dim)));
   }
   const Strides a{sq[0], sq[1], sq[2]}, b{sk[0], sk[1], sk[2]}, c{sqo[0], sqo[1], sqo[2]}, d{sko[0], sko[1], sko[2]};
   hipStream_t s = as_stream(stream);
@@ -401,21 +411,22 @@ int launch(const void* q, const void* k, const void* cos_t, const void* sin_t, v
   }
 }
 
-// Packed rotary table for the projection kernel that rotates q and k in its epilogue: entry [token][d], d <
-// head_dim / 2, holds cos (low half) and sin (high half) of position[plane(d)] * inv_freq[d], rounded to bf16 like
-// the table builder's output (vl.py:679-712).  Channels d and d + head_dim / 2 must take the same plane, which is the
-// case for the PyTorch path's layout (vl.py:763-769) and not for the CUDA kernel's (csrc/rope.cu:104-117).
+// Packed rotary table for the projection kernel that rotates q and k in its epilogue and for the packed form of the
+// apply kernel: entry [token][d], d < width, holds cos (low half) and sin (high half) of
+// position[plane(d)] * inv_freq[d mod half], rounded to bf16 like the table builder's output (vl.py:679-712).
+// width = half when channels d and d + half take the same plane (the PyTorch path's layout, vl.py:763-769), else
+// 2 * half, one entry per channel (the CUDA kernel's layout, csrc/rope.cu:104-117).
 __global__ __launch_bounds__(256) void mrope_table_kernel(const int64_t* __restrict__ pos,
                                                           const float* __restrict__ inv_freq,
                                                           uint32_t* __restrict__ out, int64_t n_tokens, int half,
-                                                          AxisTable ax) {
+                                                          int width, AxisTable ax) {
   const int64_t gid = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-  if (gid >= n_tokens * half) return;
-  const int64_t token = gid / half;
-  const int d = static_cast<int>(gid - token * half);
+  if (gid >= n_tokens * width) return;
+  const int64_t token = gid / width;
+  const int d = static_cast<int>(gid - token * width);
   const float pf = static_cast<float>(pos[ax.axis[d] * n_tokens + token]);
   float sv, cv;
-  sincosf(__fmul_rn(pf, inv_freq[d]), &sv, &cv);
+  sincosf(__fmul_rn(pf, inv_freq[d >= half ? d - half : d]), &sv, &cv);
   out[gid] = f32_to_bf16_bits(cv) | (f32_to_bf16_bits(sv) << 16);
 }
 
@@ -484,15 +495,23 @@ extern "C" int wx_mrope_table(const int64_t* position_ids, const float* inv_freq
   AxisTable ax{};
   if (int rc = build_axis_table(mrope_section, head_dim, layout, ax)) return rc;
   const int half = head_dim / 2;
-  for (int d = 0; d < half; ++d)
-    if (ax.axis[d] != ax.axis[d + half])
-      return fail(WX_ERR_UNSUPPORTED, "%s: channels %d and %d take different position planes in this layout; the "
-                  "packed table (and the projection that rotates in its epilogue) needs them equal", who, d, d + half);
-  const int64_t n = batch * seq * half;
+  const int width = packed_table_width(ax, head_dim);
+  const int64_t n = batch * seq * width;
   if (n == 0) return WX_OK;
   if (!position_ids || !inv_freq || !table) return fail(WX_ERR_INVALID_ARGUMENT, "%s: null pointer", who);
   if ((n + 255) / 256 > 0x7fffffffll) return fail(WX_ERR_UNSUPPORTED, "%s: too many tokens", who);
   hipLaunchKernelGGL(mrope_table_kernel, dim3(static_cast<unsigned>((n + 255) / 256)), dim3(256), 0, as_stream(stream),
-                     position_ids, inv_freq, table, batch * seq, half, ax);
+                     position_ids, inv_freq, table, batch * seq, half, width, ax);
   return check_launch(who);
+}
+
+extern "C" int wx_mrope_table_width(int head_dim, const int mrope_section[3], int layout) {
+  using namespace wx;
+  const char* who = "wx_mrope_table_width";
+  if (head_dim <= 0 || head_dim % 16 != 0 || head_dim > kMaxHeadDim)
+    return fail(WX_ERR_UNSUPPORTED, "%s: head_dim %d must be a multiple of 16 and <= %d", who, head_dim, kMaxHeadDim);
+  if (!mrope_section) return fail(WX_ERR_INVALID_ARGUMENT, "%s: null section", who);
+  AxisTable ax{};
+  if (int rc = build_axis_table(mrope_section, head_dim, layout, ax)) return rc;
+  return packed_table_width(ax, head_dim);
 }

@@ -614,12 +614,19 @@ constexpr int kMaxDevices = 64;
 std::mutex g_scratch_mutex;
 int32_t* g_scratch_ptr[kMaxDevices] = {};
 
-int static_scratch(int32_t** out) {
+// `capturing`: the call that asks is being recorded into a HIP graph.  The address lookup is a runtime call that does
+// not belong inside a capture (it can fail there, or end the capture), so a first use on a device from inside one is
+// refused with a message that says what to do instead.
+int static_scratch(int32_t** out, bool capturing) {
   int dev = -1;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices)
     return fail(WX_ERR_LAUNCH, "wx_partition_build_noalloc: no current device (or its index is %d or above)", kMaxDevices);
   std::lock_guard<std::mutex> lock(g_scratch_mutex);
   if (g_scratch_ptr[dev] == nullptr) {
+    if (capturing)
+      return fail(WX_ERR_INVALID_ARGUMENT,
+                  "wx_partition_build_noalloc: first use on device %d comes from inside a stream capture; call "
+                  "wx_partition_noalloc_init() (or make one call) on this device before capturing", dev);
     void* p = nullptr;
     const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
     if (e != hipSuccess || p == nullptr)
@@ -648,10 +655,20 @@ extern "C" int wx_partition_build_noalloc(const void* ids, int id_type, int64_t 
     return fail(WX_ERR_WORKSPACE, "wx_partition_build_noalloc: %lld expanded tokens need %zu bytes of histograms, the built-in scratch has %zu",
                 static_cast<long long>(num_tokens * num_topk), wx_partition_workspace_bytes(num_tokens * num_topk), kScratchBytes);
   int32_t* hist = nullptr;
-  if (int rc = static_scratch(&hist)) return rc;
+  hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(as_stream(stream), &cap) != hipSuccess) {
+    (void)hipGetLastError();
+    cap = hipStreamCaptureStatusNone;
+  }
+  if (int rc = static_scratch(&hist, cap != hipStreamCaptureStatusNone)) return rc;
   return partition_launch("wx_partition_build_noalloc", ids, id_type, num_tokens, num_topk, num_experts,
                           num_out_tokens, row_id_map, sorted_row_id, expert_offsets, status, hist, kScratchBytes,
                           as_stream(stream));
+}
+
+extern "C" int wx_partition_noalloc_init(void) {
+  int32_t* hist = nullptr;
+  return static_scratch(&hist, false);
 }
 
 extern "C" int wx_permute_rows(const void* x, void* out, const int32_t* row_id_map, int64_t num_tokens,

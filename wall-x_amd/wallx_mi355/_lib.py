@@ -15,6 +15,7 @@ LIB_PATH = os.environ.get("WALLX_MI355_LIB") or os.path.join(_HERE, "libwallx_mi
 WX_F32, WX_F16, WX_BF16 = 0, 1, 2
 WX_I32, WX_I64, WX_U8 = 0, 1, 2
 WX_MROPE_HF, WX_MROPE_CSRC = 0, 1
+WX_GEMM_PATH_MFMA, WX_GEMM_PATH_ZERO_FILL, WX_GEMM_PATH_FMA, WX_GEMM_PATH_ADD_COPY = 1, 2, 4, 8
 
 _c = ctypes
 _vp, _i64, _i32, _sz, _f32 = _c.c_void_p, _c.c_int64, _c.c_int, _c.c_size_t, _c.c_float
@@ -22,11 +23,13 @@ _vp, _i64, _i32, _sz, _f32 = _c.c_void_p, _c.c_int64, _c.c_int, _c.c_size_t, _c.
 # name -> (restype, argtypes); mirrors include/wallx_mi355.h one to one
 PROTOTYPES = {
     "wx_last_error_string": (_c.c_char_p, []),
+    "wx_last_gemm_path": (_i32, []),
     "wx_abi_version": (_i32, []),
     "wx_stream_capture_id": (_i32, [_vp, ctypes.POINTER(ctypes.c_ulonglong)]),
     "wx_partition_workspace_bytes": (_sz, [_i64]),
     "wx_partition_build": (_i32, [_vp, _i32, _i64, _i32, _i32, _i64, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     "wx_partition_build_noalloc": (_i32, [_vp, _i32, _i64, _i32, _i32, _i64, _vp, _vp, _vp, _vp, _vp]),
+    "wx_partition_noalloc_init": (_i32, []),
     "wx_permute_rows": (_i32, [_vp, _vp, _vp, _i64, _i32, _i64, _i32, _vp]),
     "wx_unpermute_rows": (_i32, [_vp, _vp, _vp, _vp, _i64, _i32, _i64, _i32, _vp]),
     "wx_unpermute_rows_bwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i32, _i64, _i32, _vp]),
@@ -47,10 +50,11 @@ PROTOTYPES = {
                            + [_c.POINTER(_i32), _i32, _i32, _vp]),
     "wx_mrope_apply_positions": (_i32, [_vp] * 6 + [_i64, _i64, _i32, _i32, _i32] + [_c.POINTER(_i64)] * 4
                                  + [_c.POINTER(_i32), _i32, _i32, _i32, _vp]),
+    "wx_mrope_table_width": (_i32, [_i32, _c.POINTER(_i32), _i32]),
     "wx_mrope_table": (_i32, [_vp, _vp, _i64, _i64, _i32, _c.POINTER(_i32), _i32, _vp, _vp]),
     "wx_mrope_apply_packed": (_i32, [_vp] * 5 + [_i64, _i64, _i32, _i32, _i32] + [_c.POINTER(_i64)] * 4
                               + [_c.POINTER(_i32), _i32, _i32, _i32, _vp]),
-    "wx_qkv_rope_proj": (_i32, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i32, _i32, _i32, _vp]),
+    "wx_qkv_rope_proj": (_i32, [_vp, _vp, _vp, _vp, _i32, _vp, _i64, _i64, _i32, _i32, _i32, _vp]),
     "wx_rope_index_workspace_bytes": (_sz, [_i64, _i64]),
     "wx_rope_index": (_i32, [_vp, _vp, _vp, _i64, _vp, _i64, _vp, _i64, _i64, _i32, _i64, _i64, _i64, _f32,
                              _vp, _vp, _vp, _vp, _sz, _vp]),

@@ -59,7 +59,10 @@ def load_expert_weights(source, blocks: Mapping[int, torch.nn.Module], dense_as_
     ``moe.experts.*`` key must receive all six tensors; a layer that only has dense ``mlp.*`` keys must receive
     expert 0's three (the action expert then keeps its initialisation, as in the trainer).  Shapes are checked, and
     so is the dtype of the block's parameters: the kernels are bf16 only.  Cached K-tiled copies of the touched
-    parameters are dropped, so the next forward packs the new values.
+    parameters are dropped, so the next forward packs the new values.  A block that was packed for inference with
+    its nn.Linear copies kept (`pack_for_inference(free_dense=False)`) would go on running its old packed weights:
+    its packed set is dropped before the copy and rebuilt from the new values at the end.  A block whose nn.Linear
+    copies were released cannot be loaded into (its parameters are empty: the shape check raises).
     pack_only=True finishes with `block.pack_for_inference()` on every block: the weights are packed into the
     K-tiled layout and the nn.Linear copies released (forward-only blocks, half the expert memory).
     """
@@ -68,6 +71,7 @@ def load_expert_weights(source, blocks: Mapping[int, torch.nn.Module], dense_as_
     items = source.items() if isinstance(source, Mapping) else iter_safetensors(source)
     loaded: Dict[int, set] = {layer: set() for layer in blocks}
     moe_format: Dict[int, bool] = {layer: False for layer in blocks}
+    repack = set()  # layers whose block held a packed set next to its nn.Linear copies
     for layer, block in blocks.items():
         for e in block.experts:
             for w in e.weights():
@@ -89,6 +93,9 @@ def load_expert_weights(source, blocks: Mapping[int, torch.nn.Module], dense_as_
         param = getattr(block.experts[expert], f"{proj}_proj").weight
         if tuple(param.shape) != tuple(tensor.shape):
             raise ValueError(f"{key}: checkpoint shape {tuple(tensor.shape)} != module shape {tuple(param.shape)}")
+        if getattr(block, "_packed", None) is not None:
+            block._packed = None  # built from the values about to be overwritten
+            repack.add(layer)
         with torch.no_grad():
             param.copy_(tensor.to(device=param.device, dtype=param.dtype))
         native.invalidate_packed(param)
@@ -103,4 +110,7 @@ def load_expert_weights(source, blocks: Mapping[int, torch.nn.Module], dense_as_
     if pack_only:
         for block in blocks.values():
             block.pack_for_inference(free_dense=True)
+    else:
+        for layer in sorted(repack):
+            blocks[layer].pack_for_inference(free_dense=False)
     return {layer: len(got) for layer, got in loaded.items()}

@@ -297,21 +297,24 @@ def multimodal_rope_from_positions(q, k, position_ids, inv_freq, mrope_section, 
     return MultimodalRoPEFromPositions.apply(q, k, position_ids, inv_freq, mrope_section, layout)
 
 
-def multimodal_rope_table(position_ids, inv_freq, mrope_section):
-    """The packed cos/sin table `qkv_projection_with_rope` reads: build it once per forward from the position ids
-    (it replaces the [3, B, S, D] tables of Qwen2_5_VLRotaryEmbedding.forward, vl.py:679-712) and hand it to every
-    layer.  PyTorch-path channel layout (vl.py:763-769)."""
+def multimodal_rope_table(position_ids, inv_freq, mrope_section, layout="hf"):
+    """The packed cos/sin table `qkv_projection_with_rope` and `multimodal_rope_from_table` read: build it once per
+    forward from the position ids (it replaces the [3, B, S, D] tables of Qwen2_5_VLRotaryEmbedding.forward,
+    vl.py:679-712) and hand it to every layer.  layout="hf": the channel -> plane map of the PyTorch path
+    (vl.py:763-769; channels d and d + D/2 share an entry, [B*S, D/2]); layout="csrc": that of the reference's CUDA
+    kernel (csrc/rope.cu:104-117; one entry per channel, [B*S, D])."""
     if position_ids.is_cpu or inv_freq.is_cpu:
         raise RuntimeError("[Error] The inputs of multimodal_rope_table are on the device: CPU!")
-    return backend.mrope_table(position_ids, inv_freq.to(torch.float32), list(mrope_section))
+    return backend.mrope_table(position_ids, inv_freq.to(torch.float32), list(mrope_section), layout)
 
 
 class MultimodalRoPEFromTable(torch.autograd.Function):
     """multimodal_rope with cos / sin read from the packed table of multimodal_rope_table (built once per forward,
-    256 bytes per token, shared by all layers) instead of the two [3, B, S, D] tables; bf16, PyTorch-path layout."""
+    256 or 512 bytes per token, shared by all layers) instead of the two [3, B, S, D] tables; bf16; `layout` as given
+    to multimodal_rope_table."""
 
     @staticmethod
-    def forward(ctx, q, k, table, mrope_section):
+    def forward(ctx, q, k, table, mrope_section, layout="hf"):
         for name, t in (("q", q), ("k", k), ("table", table)):
             if t.is_cpu:
                 raise RuntimeError(f"[Error] The input `{name}` of multimodal_rope op is on the device: CPU!")
@@ -326,9 +329,10 @@ class MultimodalRoPEFromTable(torch.autograd.Function):
         doubled = [2 * int(v) for v in mrope_section]
         q_out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
         k_out = torch.empty(k.shape, dtype=k.dtype, device=k.device)
-        backend.rope_from_table(q, k, table, q_out, k_out, doubled)
+        backend.rope_from_table(q, k, table, q_out, k_out, doubled, layout=layout)
         ctx.save_for_backward(table)
         ctx.mrope_section_doubled = doubled
+        ctx.layout = layout
         return q_out, k_out
 
     @staticmethod
@@ -336,19 +340,20 @@ class MultimodalRoPEFromTable(torch.autograd.Function):
         (table,) = ctx.saved_tensors
         want_q, want_k = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
         if not (want_q or want_k):
-            return None, None, None, None
+            return None, None, None, None, None
         if grad_q_out.stride(-1) != 1:
             grad_q_out = grad_q_out.contiguous()
         if grad_k_out.stride(-1) != 1:
             grad_k_out = grad_k_out.contiguous()
         gq = torch.empty(grad_q_out.shape, dtype=grad_q_out.dtype, device=grad_q_out.device)
         gk = torch.empty(grad_k_out.shape, dtype=grad_k_out.dtype, device=grad_k_out.device)
-        backend.rope_from_table(grad_q_out, grad_k_out, table, gq, gk, ctx.mrope_section_doubled, backward=True)
-        return (gq if want_q else None), (gk if want_k else None), None, None
+        backend.rope_from_table(grad_q_out, grad_k_out, table, gq, gk, ctx.mrope_section_doubled, backward=True,
+                                layout=ctx.layout)
+        return (gq if want_q else None), (gk if want_k else None), None, None, None
 
 
-def multimodal_rope_from_table(q, k, table, mrope_section):
-    return MultimodalRoPEFromTable.apply(q, k, table, mrope_section)
+def multimodal_rope_from_table(q, k, table, mrope_section, layout="hf"):
+    return MultimodalRoPEFromTable.apply(q, k, table, mrope_section, layout)
 
 
 def qkv_projection_with_rope(hidden_states, qkv_weight, qkv_bias, rope_table, num_heads, num_key_value_heads,

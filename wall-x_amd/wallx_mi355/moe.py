@@ -22,16 +22,34 @@ from torch import nn
 from . import _lib, native
 
 
+def activation(name: str):
+    """The gating function a config names in `hidden_act` (the reference looks it up in transformers' ACT2FN,
+    act.py:73-77): that table when transformers is importable, else the handful of names torch covers."""
+    try:
+        from transformers.activations import ACT2FN
+    except Exception:  # noqa: BLE001 - transformers absent or broken: the local table below
+        ACT2FN = None
+    if ACT2FN is not None and name in ACT2FN:
+        return ACT2FN[name]
+    F = torch.nn.functional
+    table = {"silu": F.silu, "swish": F.silu, "gelu": F.gelu, "relu": F.relu, "tanh": torch.tanh,
+             "sigmoid": torch.sigmoid, "gelu_new": lambda t: F.gelu(t, approximate="tanh"),
+             "gelu_pytorch_tanh": lambda t: F.gelu(t, approximate="tanh")}
+    if name not in table:
+        raise KeyError(f"unknown hidden_act {name!r}")
+    return table[name]
+
+
 class ExpertMLP(nn.Module):
-    """Weights of one SwiGLU expert, laid out like BlockSparseMLP (act.py:67-82)."""
+    """Weights of one gated expert, laid out like BlockSparseMLP (act.py:67-82).  The fused kernels implement silu
+    gating; an expert with another `hidden_act` makes its block run on the generic ops (see SparseMoeBlock)."""
 
     def __init__(self, config: dict):
         super().__init__()
         self.hidden_size = config["hidden_size"]
         self.intermediate_size = config["intermediate_size"]
         self.hidden_act = config.get("hidden_act", "silu")
-        if self.hidden_act != "silu":
-            raise ValueError(f"the fused expert kernel implements silu gating only, got {self.hidden_act!r}")
+        self.act_fn = activation(self.hidden_act)
         self.gate_proj = nn.Linear(self.hidden_size, self.intermediate_size, bias=False)
         self.up_proj = nn.Linear(self.hidden_size, self.intermediate_size, bias=False)
         self.down_proj = nn.Linear(self.intermediate_size, self.hidden_size, bias=False)
@@ -48,6 +66,16 @@ class Routing:
     expert_offsets: torch.Tensor  # int32 [E + 1] on the device
     num_tokens: int
     sorted_row_id: Optional[torch.Tensor] = None  # int32 [T]: token at each sorted position (inverse map)
+    host_offsets: Optional[list] = None  # expert_offsets read back to the host (generic path only, once per routing)
+
+
+def _version_of(t: torch.Tensor):
+    """The tensor's version counter, or None for a tensor that has none (one created under torch.inference_mode():
+    reading `_version` of such a tensor raises).  State derived from a tensor without a counter is never reused:
+    nothing would tell a write to it from no write."""
+    if t.is_inference():
+        return None
+    return t._version
 
 
 class _RoutingCache(threading.local):
@@ -57,33 +85,50 @@ class _RoutingCache(threading.local):
     each layer's block would partition it again.  The cache answers with the previous result when the caller passes
     the very same tensor object (so its memory cannot have been recycled for other data), unmodified (same version
     counter), on the same stream and for the same expert count: one partition per forward without any change to
-    the reference's model code.  The partition's scratch buffers are kept here too, per device."""
+    the reference's model code.  A tensor without a version counter (made under torch.inference_mode()) is partitioned
+    on every call.  The partition's scratch buffers are kept here too, per device and stream."""
 
     def __init__(self):
         self.ref = None
         self.key = None
         self.routing = None
-        self.workspace = {}  # (device, capture id) -> [histograms, status word]
+        self.workspace = {}  # (device, stream, capture id) -> [histograms, status word]
 
     def lookup(self, ids: torch.Tensor, num_experts: int):
         stream = torch.cuda.current_stream(ids.device).cuda_stream if ids.is_cuda else 0
         # a partition recorded during a HIP graph capture has not run when the capture ends: it answers lookups of
         # that capture only (its id is part of the key; 0 outside captures)
-        key = (ids._version, ids.shape, ids.dtype, ids.device, num_experts, stream, native.capture_id(stream))
-        if self.ref is not None and self.ref() is ids and self.key == key:
+        version = _version_of(ids)
+        key = (version, ids.shape, ids.dtype, ids.device, num_experts, stream, native.capture_id(stream))
+        if version is not None and self.ref is not None and self.ref() is ids and self.key == key:
             return self.routing
         flat = ids.reshape(-1)
-        # the scratch pair of a capture stays with its graph (a fresh one per capture); eager calls share one per device
-        ws_key = (ids.device, key[-1])
+        ws_key = partition_workspace_key(ids.device, stream, key[-1])
         row_id_map, offsets, inverse, ws = native.partition(flat, num_experts, 0, self.workspace.get(ws_key),
                                                             want_sorted=True)
-        if key[-1] != 0:
-            for k in [k for k in self.workspace if k[1] not in (0, key[-1])]:
+        self.store_workspace(ws_key, ws)
+        routing = Routing(row_id_map, offsets, flat.numel(), inverse)
+        if version is None:  # nothing to check a later call against: answer this call only
+            self.ref = self.key = self.routing = None
+            return routing
+        self.ref, self.key, self.routing = weakref.ref(ids), key, routing
+        return routing
+
+    def store_workspace(self, ws_key, ws) -> None:
+        """Keeps the partition's scratch pair under its key.  The pair of a capture stays with its graph (a fresh one
+        per capture, the pairs of earlier captures are dropped); eager calls keep one per device and stream, so two
+        forwards issued on different streams never count into the same histograms."""
+        if ws_key[2] != 0:
+            for k in [k for k in self.workspace if k[2] not in (0, ws_key[2])]:
+                del self.workspace[k]
+        if len(self.workspace) >= 64 and ws_key not in self.workspace:
+            for k in [k for k in self.workspace if k[2] == 0]:
                 del self.workspace[k]
         self.workspace[ws_key] = ws
-        self.ref, self.key = weakref.ref(ids), key
-        self.routing = Routing(row_id_map, offsets, flat.numel(), inverse)
-        return self.routing
+
+
+def partition_workspace_key(device, stream: int, capture: int):
+    return (device, stream, capture)
 
 
 _routing_cache = _RoutingCache()
@@ -196,16 +241,21 @@ class _MoeBlockFunction(torch.autograd.Function):
 
 
 class SparseMoeBlock(nn.Module):
-    """Same constructor and forward signature as the reference block (act.py:85-162)."""
+    """Same constructor and forward signature as the reference block (act.py:85-162).
+
+    wall-x's own configuration -- two silu-gated experts of one hidden size -- runs the fused dual-expert path.  Any
+    other `config.experts` list (another expert count, another `hidden_act`) runs the same block on this library's
+    generic ops instead: `ops.permute`, then per pair of experts `ops.asym_dual_gmm` for the gate, up and down
+    projections with the activation as a torch op between them, then `ops.unpermute` (all differentiable)."""
 
     def __init__(self, config, num_experts: int):
         super().__init__()
-        if num_experts != 2:
-            raise ValueError("the dual-expert kernel runs exactly two experts (VL and action)")
         self.num_experts = num_experts
         self.experts = nn.ModuleList([ExpertMLP(config.experts[i]) for i in range(num_experts)])
+        self._fused = (num_experts == 2 and all(e.hidden_act in ("silu", "swish") for e in self.experts) and
+                       self.experts[0].hidden_size == self.experts[1].hidden_size)
         self._dims = (self.experts[0].hidden_size, self.experts[0].intermediate_size,
-                      self.experts[1].intermediate_size)
+                      self.experts[1].intermediate_size) if self._fused else None
         self._hmid: Optional[torch.Tensor] = None      # training path only; inference shares buffers per stream
         self._x_tiled: Optional[torch.Tensor] = None
         self._packed: Optional[native.PackedExperts] = None  # set by pack_for_inference()
@@ -221,6 +271,9 @@ class SparseMoeBlock(nn.Module):
         """Packs the six projection weights into the K-tiled layout the kernels read and, with free_dense, releases
         the nn.Linear copies (the parameters stay registered, emptied, so the module tree keeps its shape): half the
         expert memory of a block that holds both.  The block is forward-only afterwards; load weights first."""
+        if not self._fused:
+            raise RuntimeError("pack_for_inference: only the fused dual-expert configuration (two silu experts) has a "
+                               "packed form; this block runs on the generic ops")
         flat = [w for e in self.experts for w in e.weights()]
         if any(w.numel() == 0 for w in flat):
             raise RuntimeError("pack_for_inference: the nn.Linear weights were already released")
@@ -258,6 +311,9 @@ class SparseMoeBlock(nn.Module):
             else:
                 raise RuntimeError("All tensors must be BFloat16 for this kernel")
         T = x.size(0)
+        if not self._fused:
+            return self._forward_generic(x, experts_indices, start_indices, end_indices, routing, pre_norm,
+                                         residual).view(batch, seq, hidden)
         host_rows = self._host_rows(start_indices, end_indices, T)
         if routing is None:
             routing = _routing_cache.lookup(experts_indices, self.num_experts)
@@ -286,16 +342,17 @@ class SparseMoeBlock(nn.Module):
         builds them once per forward, act.py:1274-1283, and hands them to all 36 layers)."""
         if start_indices is None or end_indices is None or start_indices.is_cuda or end_indices.is_cuda:
             return None
+        versions = (_version_of(start_indices), _version_of(end_indices))
+        tracked = None not in versions  # tensors made under inference_mode have no counter: read them every call
         hit = self._rows_seen
-        if hit is not None and hit[0] is start_indices and hit[1] is end_indices and \
-                hit[2] == (start_indices._version, end_indices._version, num_tokens):
+        if tracked and hit is not None and hit[0] is start_indices and hit[1] is end_indices and \
+                hit[2] == (*versions, num_tokens):
             return hit[3]
         counts = (end_indices - start_indices).tolist()
         rows = None
         if len(counts) == 2 and min(counts) >= 0 and sum(counts) == num_tokens:
             rows = _lib.i64x2(counts)
-        self._rows_seen = (start_indices, end_indices, (start_indices._version, end_indices._version, num_tokens),
-                           rows)
+        self._rows_seen = (start_indices, end_indices, (*versions, num_tokens), rows) if tracked else None
         return rows
 
     def _forward_training(self, x, routing, flat, pre_norm, residual):
@@ -311,6 +368,59 @@ class SparseMoeBlock(nn.Module):
         y = _MoeBlockFunction.apply(xin, routing.row_id_map, routing.expert_offsets, routing.sorted_row_id,
                                     scratch, *flat)
         self._x_tiled = scratch["x_tiled"]
+        return x + y if residual else y
+
+    def _forward_generic(self, x, experts_indices, start_indices, end_indices, routing, pre_norm, residual):
+        """Any expert list (act.py:105-162 as written): permute -> per pair of experts the three projections as
+        dual GEMMs with the activation between them -> unpermute.  Row ranges come from the caller's CPU tensors when
+        given (act.py:1274-1283), else from the partition's offsets, read back once per routing."""
+        from .fusions import ops
+
+        E, T = self.num_experts, x.size(0)
+        xin = x
+        if pre_norm is not None:
+            norm_weight, eps = pre_norm
+            xin = torch.nn.functional.rms_norm(x, (x.size(1),), norm_weight, eps)
+        bounds = None
+        if start_indices is not None and end_indices is not None and not start_indices.is_cuda \
+                and not end_indices.is_cuda:
+            starts, ends = start_indices.tolist(), end_indices.tolist()
+            if len(starts) == E and len(ends) == E:
+                bounds = list(zip((int(v) for v in starts), (int(v) for v in ends)))
+        if bounds is None:
+            if routing is None:
+                routing = _routing_cache.lookup(experts_indices, E)
+            if routing.host_offsets is None:
+                routing.host_offsets = routing.expert_offsets.cpu().tolist()
+            off = routing.host_offsets
+            bounds = [(off[e], off[e + 1]) for e in range(E)]
+        if T == 0:
+            return xin + x if residual else xin
+        ids = experts_indices.reshape(-1)
+        permuted, row_id_map = ops.permute(xin, ids if ids.dtype == torch.int32 else ids.to(torch.int32))
+        final = torch.zeros_like(permuted)  # rows no expert range covers stay zero (act.py:139)
+        for e in range(0, E, 2):
+            a, b = self.experts[e], self.experts[e + 1] if e + 1 < E else None
+            ra, rb = bounds[e], bounds[e + 1] if b is not None else (0, 0)
+            if ra[0] == ra[1] and rb[0] == rb[1]:
+                continue  # act.py:144-145
+            xa = permuted[ra[0]:ra[1]]
+            if b is not None:
+                xb, wb, act_b = permuted[rb[0]:rb[1]], b.weights(), b.act_fn
+            else:  # an odd expert count: the last launch's second problem is empty
+                xb = permuted.new_empty((0, a.hidden_size))
+                wb = (permuted.new_empty((8, a.hidden_size)), permuted.new_empty((8, a.hidden_size)),
+                      permuted.new_empty((a.hidden_size, 8)))
+                act_b = a.act_fn
+            wa = a.weights()
+            ga, gb = ops.asym_dual_gmm(xa, xb, wa[0], wb[0], trans_b=True)
+            ua, ub = ops.asym_dual_gmm(xa, xb, wa[1], wb[1], trans_b=True)
+            ya, yb = ops.asym_dual_gmm(a.act_fn(ga) * ua, act_b(gb) * ub, wa[2], wb[2], trans_b=True)
+            if ra[0] != ra[1]:
+                final[ra[0]:ra[1]] = ya
+            if rb[0] != rb[1]:
+                final[rb[0]:rb[1]] = yb
+        y = ops.unpermute(final, row_id_map)
         return x + y if residual else y
 
     def _forward_scatter(self, x, routing, experts, host_rows, pre_norm, residual):
@@ -336,8 +446,9 @@ def _experts_for(weights) -> "native.PackedExperts":
     once per set of tensors and reused while those tensor objects keep their storage and version counters."""
     flat = (*weights[0], *weights[1])
     key = tuple(map(id, flat))
-    state = tuple((w.data_ptr(), w._version) for w in flat)
-    hit = _functional_experts.get(key)
+    state = tuple((w.data_ptr(), _version_of(w)) for w in flat)
+    tracked = all(v is not None for _, v in state)  # weights made under inference_mode: packed on every call
+    hit = _functional_experts.get(key) if tracked else None
     if hit is not None and hit[0] == state and all(r() is w for r, w in zip(hit[1], flat)):
         return hit[2]
     g0, u0, d0, g1, u1, d1 = flat
@@ -345,7 +456,9 @@ def _experts_for(weights) -> "native.PackedExperts":
     if tuple(u0.shape) != (I0, H) or tuple(d0.shape) != (H, I0) or tuple(g1.shape) != (I1, H) or \
             tuple(u1.shape) != (I1, H) or tuple(d1.shape) != (H, I1):
         raise RuntimeError("expert weight shapes are inconsistent with hidden size")
-    experts = native.PackedExperts([native.pack_weight(w) for w in flat], (H, I0, I1))
+    experts = native.PackedExperts([native.pack_weight(w, cache=tracked) for w in flat], (H, I0, I1))
+    if not tracked:
+        return experts
     if len(_functional_experts) >= 64:
         _functional_experts.clear()
     # the entry (and with it the packed copies) goes when any of the six tensors does
@@ -364,11 +477,12 @@ def moe_layer_forward(x: torch.Tensor, token_types: torch.Tensor, weights, routi
     work buffers are the per-stream pair every block shares, so `hmid` is accepted for compatibility and not used.
     """
     if routing is None:
-        ws_key = (token_types.device, native.capture_id(torch.cuda.current_stream(token_types.device).cuda_stream))
+        stream = torch.cuda.current_stream(token_types.device).cuda_stream
+        ws_key = partition_workspace_key(token_types.device, stream, native.capture_id(stream))
         ws = workspace if workspace is not None else _routing_cache.workspace.get(ws_key)
         row_id_map, offsets, inverse, ws = native.partition(token_types.reshape(-1), 2, 0, ws, want_sorted=True)
         if workspace is None:
-            _routing_cache.workspace[ws_key] = ws
+            _routing_cache.store_workspace(ws_key, ws)
         routing = Routing(row_id_map, offsets, x.size(0), inverse)
     experts = _experts_for(weights)
     rows = None if host_rows is None else _lib.i64x2(host_rows)

@@ -353,9 +353,10 @@ def rope_from_positions(q, k, position_ids, inv_freq, q_out, k_out, mrope_sectio
 
 def rope_from_table(q, k, table, q_out, k_out, mrope_section_doubled, backward: bool = False,
                     layout: str = "hf") -> None:
-    """M-RoPE with cos / sin read from the packed table of mrope_table (int32 [B * S, D / 2], built once per forward
-    for all layers).  bf16; same results as rope_from_positions, bit for bit.  With backward=True, q/k carry the
-    output gradients and q_out/k_out receive the input gradients."""
+    """M-RoPE with cos / sin read from the packed table of mrope_table (int32 [B * S, D / 2] for "hf", [B * S, D] for
+    "csrc"; built once per forward for all layers with the same section and layout).  bf16; same results as
+    rope_from_positions, bit for bit.  With backward=True, q/k carry the output gradients and q_out/k_out receive
+    the input gradients."""
     for name, t in (("q", q), ("k", k), ("table", table), ("q_out", q_out), ("k_out", k_out)):
         _need_cuda(name, t)
     if len(mrope_section_doubled) != 3:
@@ -364,22 +365,31 @@ def rope_from_table(q, k, table, q_out, k_out, mrope_section_doubled, backward: 
     Hk = k.size(1)
     if tuple(k.shape) != (B, Hk, S, D) or tuple(q_out.shape) != tuple(q.shape) or tuple(k_out.shape) != tuple(k.shape):
         raise RuntimeError("q/k/q_out/k_out shapes are inconsistent")
-    if tuple(table.shape) != (B * S, D // 2) or table.dtype != torch.int32 or not table.is_contiguous():
-        raise RuntimeError(f"table must be a contiguous int32 [{B * S}, {D // 2}] tensor from mrope_table")
+    section = _lib.i32x3([int(v) // 2 for v in mrope_section_doubled])
+    width = _table_width(D, section, layout)
+    if tuple(table.shape) != (B * S, width) or table.dtype != torch.int32 or not table.is_contiguous():
+        raise RuntimeError(f"table must be a contiguous int32 [{B * S}, {width}] tensor from mrope_table with the same "
+                           f"mrope_section and layout ({layout!r})")
     if not (q.dtype == k.dtype == q_out.dtype == k_out.dtype == torch.bfloat16):
         raise RuntimeError("All tensors must be BFloat16 for this kernel")
-    section = _lib.i32x3([int(v) // 2 for v in mrope_section_doubled])
     with _DeviceGuard(q):
         _lib.call("wx_mrope_apply_packed", _ptr(q), _ptr(k), _ptr(table), _ptr(q_out), _ptr(k_out), B, S, Hq, Hk, D,
                   _bhsd_strides(q), _bhsd_strides(k), _bhsd_strides(q_out), _bhsd_strides(k_out), section,
                   _layout_code(layout), _dtype_code(q), int(bool(backward)), _stream(q))
 
 
+def _table_width(head_dim: int, section_c, layout: str) -> int:
+    width = _lib.load().wx_mrope_table_width(int(head_dim), section_c, _layout_code(layout))
+    if width < 0:
+        _lib.check(width)
+    return int(width)
+
+
 def mrope_table(position_ids: torch.Tensor, inv_freq: torch.Tensor, mrope_section, layout: str = "hf") -> torch.Tensor:
-    """Packed rotary table for qkv_rope_proj: int32 [B * S, D / 2], entry = bf16 cos | bf16 sin << 16 of
-    position_ids[plane(d)] * inv_freq[d] (vl.py:679-712 rounded to bf16).  position_ids [3, B, S] int64, inv_freq
-    [D / 2] fp32, mrope_section the three (un-doubled) section sizes.  Only layouts whose channels d and d + D / 2
-    share a position plane ("hf")."""
+    """Packed rotary table for qkv_rope_proj and rope_from_table: int32 [B * S, W], entry = bf16 cos | bf16 sin << 16
+    of position_ids[plane(d)] * inv_freq[d mod D / 2] (vl.py:679-712 rounded to bf16).  position_ids [3, B, S] int64,
+    inv_freq [D / 2] fp32, mrope_section the three (un-doubled) section sizes.  W = D / 2 for layout "hf" (channels d
+    and d + D / 2 share a position plane and an entry), W = D for "csrc" (one entry per channel)."""
     _need_cuda("position_ids", position_ids)
     _need_cuda("inv_freq", inv_freq)
     if position_ids.dim() != 3 or position_ids.size(0) != 3 or position_ids.dtype != torch.int64:
@@ -391,10 +401,11 @@ def mrope_table(position_ids: torch.Tensor, inv_freq: torch.Tensor, mrope_sectio
     _, B, S = position_ids.shape
     half = inv_freq.numel()
     position_ids, inv_freq = position_ids.contiguous(), inv_freq.contiguous()
-    table = torch.empty((B * S, half), dtype=torch.int32, device=position_ids.device)
+    section = _lib.i32x3([int(v) for v in mrope_section])
+    table = torch.empty((B * S, _table_width(2 * half, section, layout)), dtype=torch.int32, device=position_ids.device)
     with _DeviceGuard(position_ids):
-        _lib.call("wx_mrope_table", _ptr(position_ids), _ptr(inv_freq), B, S, 2 * half,
-                  _lib.i32x3([int(v) for v in mrope_section]), _layout_code(layout), _ptr(table), _stream(position_ids))
+        _lib.call("wx_mrope_table", _ptr(position_ids), _ptr(inv_freq), B, S, 2 * half, section, _layout_code(layout),
+                  _ptr(table), _stream(position_ids))
     return table
 
 
@@ -402,8 +413,9 @@ def qkv_rope_proj(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Te
                   n_q_heads: int, n_kv_heads: int, head_dim: int = 128, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """x [..., hidden] @ weight^T + bias with M-RoPE applied to the q and k heads in the GEMM's epilogue
     (vl.py:955-964 in one launch).  weight [(n_q + 2 n_kv) * head_dim, hidden] = q, k, v weights stacked, bias likewise
-    or None, table from mrope_table (one row per row of x).  Returns [..., (n_q + 2 n_kv) * head_dim]: columns
-    [0, n_q D) are the rotated q heads, the next n_kv D the rotated k heads, the last n_kv D the v heads."""
+    or None, table from mrope_table (one row per row of x; its width says whether channels d and d + D / 2 share an
+    entry, so either channel layout is served).  Returns [..., (n_q + 2 n_kv) * head_dim]: columns [0, n_q D) are the
+    rotated q heads, the next n_kv D the rotated k heads, the last n_kv D the v heads."""
     for name, t in (("x", x), ("weight", weight), ("table", table)):
         _need_cuda(name, t)
     if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16 or (bias is not None and bias.dtype != torch.bfloat16):
@@ -418,16 +430,18 @@ def qkv_rope_proj(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Te
     if not x2.is_contiguous():
         x2 = x2.contiguous()
     T = x2.size(0)
-    if table.dtype != torch.int32 or tuple(table.shape) != (T, head_dim // 2):
-        raise RuntimeError(f"table must be int32 [{T}, {head_dim // 2}] (mrope_table of the same tokens)")
+    if table.dtype != torch.int32 or table.dim() != 2 or table.size(0) != T or \
+            table.size(1) not in (head_dim // 2, head_dim):
+        raise RuntimeError(f"table must be int32 [{T}, {head_dim // 2}] or [{T}, {head_dim}] (mrope_table of the same "
+                           "tokens)")
     weight = weight.contiguous()
     table = table.contiguous()
     bias = None if bias is None else bias.contiguous()
     if out is None or out.dtype != torch.bfloat16 or out.numel() != T * n or not out.is_contiguous() or out.device != x.device:
         out = torch.empty((T, n), dtype=torch.bfloat16, device=x.device)
     with _DeviceGuard(x2):
-        _lib.call("wx_qkv_rope_proj", _ptr(x2), _ptr(weight), _ptr(bias), _ptr(table), _ptr(out), T, hidden,
-                  int(n_q_heads), int(n_kv_heads), int(head_dim), _stream(x2))
+        _lib.call("wx_qkv_rope_proj", _ptr(x2), _ptr(weight), _ptr(bias), _ptr(table), int(table.size(1)), _ptr(out), T,
+                  hidden, int(n_q_heads), int(n_kv_heads), int(head_dim), _stream(x2))
     return out.view(*x.shape[:-1], n)
 
 
@@ -572,9 +586,11 @@ def pack_weight(w: torch.Tensor, cache: bool = True) -> torch.Tensor:
     if w.dtype != torch.bfloat16 or w.dim() != 2:
         raise RuntimeError("expert weights must be 2-D BFloat16 tensors")
     key = id(w)
+    if w.is_inference():
+        cache = False  # a tensor made under torch.inference_mode() has no version counter to check a cached copy against
     if not cache:
         _packed_cache.pop(key, None)
-    state = (w.data_ptr(), w._version, tuple(w.shape), w.device)
+    state = (w.data_ptr(), None if not cache else w._version, tuple(w.shape), w.device)
     if cache:
         hit = _packed_cache.get(key)
         if hit is not None and hit[0]() is w and hit[1] == state:
