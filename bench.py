@@ -43,9 +43,13 @@ def parse():
                          "dense mask), or plain causal")
     ap.add_argument("--cpu-seqs", type=int, default=32, help="sequences of the batch the CPU baseline runs (32 = all)")
     ap.add_argument("--kernel-loop", default=None,
-                    choices=["gate_up", "down", "down_unpermute", "permute", "permute_plain", "unpermute", "partition", "copy"],
+                    choices=["gate_up", "down", "down_unpermute", "permute", "permute_plain", "unpermute", "partition", "copy",
+                             "mrope", "mrope_packed", "mrope_copy", "config2_index"],
                     help="profiling aid: run only this kernel --steps times (no JSON line); 'copy' is a plain "
-                         "device-to-device copy of the [T, H] activations, the known-size yardstick for HBM counters")
+                         "device-to-device copy of the [T, H] activations, the known-size yardstick for HBM counters; "
+                         "'mrope' / 'mrope_packed' are the M-RoPE apply at config 2 from the two tables / from the "
+                         "packed table, 'mrope_copy' a device copy of q and k of the same shape, 'config2_index' the "
+                         "three index builders and the packed-table builder at config 2")
     ap.add_argument("--kernel-shape", default="config3", choices=["config3", "denoise"],
                     help="with --kernel-loop: the batch the kernel runs on -- config 3 (29184 tokens, 28160 VL + 1024 "
                          "action) or config 4's denoise step (2048 action tokens, VL group empty)")
@@ -86,6 +90,9 @@ def main():
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.kernel_loop in ("mrope", "mrope_packed", "mrope_copy", "config2_index"):
+        config2_kernel_loop(dev, args.kernel_loop, args.steps)
+        return
     H, I0, I1 = wl.HIDDEN, wl.INTER_VL, wl.INTER_ACT
     B, S, NA = 32, 912, 32
     T = B * S
@@ -298,6 +305,11 @@ def main():
     }
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(x_cpu, types_cpu, w_cpu, args.cpu_seqs, H, I0, I1)
+        if not args.ops_only:
+            try:  # the config 2 ops (M-RoPE apply and the index builders) on the host cores, beside their GPU figures
+                extra["cpu_baseline_config2"] = cpu_baseline_config2()
+            except Exception as exc:  # noqa: BLE001 - the message goes into the report
+                extra["cpu_baseline_config2"] = {"error": f"{type(exc).__name__}: {exc}"[:300]}
         if isinstance(extra.get("prefill"), dict) and "tokens_per_s" in extra["prefill"]:
             # the same prefill priced on the host cores (a bounded sample: one layer timed, 36 charged)
             try:
@@ -399,6 +411,98 @@ def side_measurements(dev, iters):
     return out
 
 
+def config2_inputs(dev):
+    """The config 2 tensors on the device: token ids and grids, position ids, cos / sin tables, q / k as [B, H, S, D]
+    views of token-major memory, contiguous outputs, the packed rotary table."""
+    import torch
+    from wallx_mi355 import native, workloads as wl
+    from wallx_mi355.fusions import ops
+
+    ids_cpu, grid_cpu = wl.config2_tokens()
+    ids, grid = ids_cpu.to(dev), grid_cpu.to(dev)
+    args = (2, wl.IMAGE_TOKEN_ID, wl.VIDEO_TOKEN_ID, wl.VISION_START_TOKEN_ID, 2)
+    pos, _ = ops.get_rope_index(ids, *args, image_grid_thw=grid)
+    B, S, D = ids.shape[0], ids.shape[1], wl.HEAD_DIM
+    inv = wl.text_inv_freq().to(dev)
+    freqs = pos.float()[..., None] * inv
+    emb = torch.cat((freqs, freqs), -1)
+    cos, sin = emb.cos().to(torch.bfloat16), emb.sin().to(torch.bfloat16)
+    q = torch.randn(B, S, wl.N_Q_HEADS, D, device=dev).to(torch.bfloat16).transpose(1, 2)
+    k = torch.randn(B, S, wl.N_KV_HEADS, D, device=dev).to(torch.bfloat16).transpose(1, 2)
+    qo = torch.empty(B, wl.N_Q_HEADS, S, D, dtype=torch.bfloat16, device=dev)
+    ko = torch.empty(B, wl.N_KV_HEADS, S, D, dtype=torch.bfloat16, device=dev)
+    table = native.mrope_table(pos, inv, wl.MROPE_SECTION)
+    return dict(ids_cpu=ids_cpu, grid_cpu=grid_cpu, ids=ids, grid=grid, args=args, pos=pos, inv=inv, cos=cos, sin=sin,
+                q=q, k=k, qo=qo, ko=ko, table=table, sec2=[2 * v for v in wl.MROPE_SECTION])
+
+
+def config2_kernel_loop(dev, which, steps):
+    """--kernel-loop for the config 2 kernels (profiling aid, no JSON line)."""
+    import torch
+    from wallx_mi355 import native, workloads as wl
+    from wallx_mi355.fusions import ops
+
+    c = config2_inputs(dev)
+    grid32 = c["grid"].to(torch.int32)
+    inv_v = wl.vision_inv_freq().to(dev)
+    torch.cuda.synchronize()
+    for _ in range(steps):
+        if which == "mrope":
+            native.rope(c["q"], c["k"], c["cos"], c["sin"], c["qo"], c["ko"], c["sec2"], layout="hf")
+        elif which == "mrope_packed":
+            native.rope_from_table(c["q"], c["k"], c["table"], c["qo"], c["ko"], c["sec2"])
+        elif which == "mrope_copy":  # the same q / k bytes through the runtime's copy: the yardstick for the counters
+            c["qo"].copy_(c["q"])
+            c["ko"].copy_(c["k"])
+        else:
+            ops.get_rope_index(c["ids"], *c["args"], image_grid_thw=c["grid"])
+            native.rot_pos_emb(inv_v, c["grid"], 2, grid_thw_host=c["grid_cpu"])
+            native.get_window_index(grid32, 2, 4, 14, 4, grid_thw_host=c["grid_cpu"])
+            native.mrope_table(c["pos"], c["inv"], wl.MROPE_SECTION)
+    torch.cuda.synchronize()
+
+
+def cpu_baseline_config2():
+    """The config 2 ops on the host cores, beside the GPU figures of `extra`: the oracle's restatements of
+    apply_multimodal_rotary_pos_emb (vl.py:731-773, eager bf16 like the reference), get_rope_index (act.py:929-1149),
+    rot_pos_emb and get_window_index (vl.py:473-547) at the full config 2 sizes.  Median of 5 runs after a warm-up, on
+    the threads torch uses on this box (the index builders are Python / single-threaded torch code either way)."""
+    import torch
+    import oracle
+    from wallx_mi355 import workloads as wl
+
+    def med_us(fn, runs=5):
+        fn()
+        ts = []
+        for _ in range(runs):
+            t0 = time.perf_counter()
+            fn()
+            ts.append(time.perf_counter() - t0)
+        return round(statistics.median(ts) * 1e6, 1)
+
+    ids, grid = wl.config2_tokens()
+    args = (2, wl.IMAGE_TOKEN_ID, wl.VIDEO_TOKEN_ID, wl.VISION_START_TOKEN_ID, 2)
+    pos, _ = oracle.rope_index_ref(ids, *args, image_grid_thw=grid)
+    cos, sin = oracle.rotary_cos_sin_ref(pos, wl.text_inv_freq(), torch.bfloat16)
+    q, k = wl.qk_inputs(ids.shape[0], ids.shape[1])
+    qt, kt = q.transpose(1, 2), k.transpose(1, 2)
+    sec = list(wl.MROPE_SECTION)
+    inv_v = wl.vision_inv_freq()
+    tokens, D = ids.numel(), wl.HEAD_DIM
+    rope_bytes = 2.0 * 2 * tokens * D * (wl.N_Q_HEADS + wl.N_KV_HEADS) + 2.0 * 2 * tokens * D
+    t_rope = med_us(lambda: oracle.mrope_apply_ref(qt, kt, cos, sin, sec))
+    return {
+        "mrope_us": t_rope, "mrope_GBps": round(rope_bytes / t_rope / 1e3, 2),
+        "cos_sin_tables_us": med_us(lambda: oracle.rotary_cos_sin_ref(pos, wl.text_inv_freq(), torch.bfloat16)),
+        "rope_index_us": med_us(lambda: oracle.rope_index_ref(ids, *args, image_grid_thw=grid)),
+        "rot_pos_emb_us": med_us(lambda: oracle.rot_pos_emb_ref(inv_v, grid, 2)),
+        "window_index_us": med_us(lambda: oracle.window_index_ref(grid, 112, 2, 14, 4)),
+        "cores": torch.get_num_threads(), "kind": "port",
+        "sample": "the oracle's functions at the full config 2 sizes (16 x 896 tokens, 48 grids of 1 x 32 x 32, q "
+                  "[14336, 16, 128] and k [14336, 2, 128] bf16), median of 5 runs after a warm-up",
+    }
+
+
 def cold_measurements(dev, x, row_id_map, T, H, row_bytes, iters):
     """The bandwidth kernels with operands that are NOT resident in the 256 MB memory-side cache: each call works
     on the next of several buffer sets whose total size is above 1 GB, so every byte comes from and goes to HBM.
@@ -480,6 +584,7 @@ def config4_measurement(dev, weights):
         out[name]["us_drop_in_block_same_token_types"] = round(tb * 1e3, 1)            # one call, GPU idle before it
         out[name]["us_per_layer_drop_in_block_36_calls_back_to_back"] = round(tbb * 1e3, 1)  # as a decoder issues them
         if n_vl == 0:
+            out[name]["kernels_us"] = denoise_kernel_times(dev, x, types, weights)
             # the denoise loop repeats this shape 10 x 36 times per action chunk: record 36 layers once into a HIP
             # graph (the entry points neither allocate nor synchronise) and time its replays
             layers = 36
@@ -504,6 +609,50 @@ def config4_measurement(dev, weights):
             out[name]["us_per_layer_eager_shared_routing"] = round(te * 1e3 / layers, 1)
             out[name]["us_per_layer_hip_graph_replay"] = round(tg * 1e3 / layers, 1)
     return out
+
+
+def denoise_kernel_times(dev, x, types, weights):
+    """The launches of one denoise layer by themselves (HIP events, 20 back-to-back launches per event pair): tiled
+    permute, gate/up + SwiGLU, down with the unpermute in its stores, the host handing over the row counts (one
+    dispatch each), and what fraction of the bf16 MFMA peak the two GEMM launches reach."""
+    import torch
+    from wallx_mi355 import _lib, native
+
+    T, H = x.shape
+    (g0, u0, d0), (g1, u1, d1) = weights
+    I0, I1 = g0.shape[0], g1.shape[0]
+    packed = [native.pack_weight(w) for w in (g0, u0, d0, g1, u1, d1)]
+    rmap, off, inv, _ = native.partition(types, 2, 0, None, want_sorted=True)
+    rows_pad = native.padded_sorted_rows(T)
+    x_tiled = torch.empty(rows_pad * H, dtype=torch.bfloat16, device=dev)
+    hmid = torch.empty(rows_pad * max(I0, I1), dtype=torch.bfloat16, device=dev)
+    y = torch.empty_like(x)
+    n_act = int(types.sum())
+    rows = _lib.i64x2((T - n_act, n_act))
+    stream = torch.cuda.current_stream().cuda_stream
+    p = [t.data_ptr() for t in packed]
+
+    def permute():
+        _lib.call("wx_permute_rows_tiled", x.data_ptr(), x_tiled.data_ptr(), rmap.data_ptr(), inv.data_ptr(),
+                  off.data_ptr(), T, H, stream)
+
+    def gate_up():
+        _lib.call("wx_dual_swiglu_gate_up", x_tiled.data_ptr(), hmid.data_ptr(), off.data_ptr(), p[0], p[1], p[3], p[4],
+                  T, H, I0, I1, rows, stream)
+
+    def down():
+        _lib.call("wx_dual_down_proj", hmid.data_ptr(), y.data_ptr(), off.data_ptr(), p[2], p[5], T, H, I0, I1, rows,
+                  inv.data_ptr(), stream)
+
+    permute(); gate_up(); down()
+    t_p, _ = event_ms(permute, 20, warm=3, batch=20)
+    t_g, _ = event_ms(gate_up, 20, warm=3, batch=20)
+    t_d, _ = event_ms(down, 20, warm=3, batch=20)
+    f_g, f_d = 4.0 * H * n_act * I1, 2.0 * H * n_act * I1
+    return {"permute_tiled": round(t_p * 1e3, 2), "gate_up_swiglu": round(t_g * 1e3, 2),
+            "down_with_unpermute": round(t_d * 1e3, 2),
+            "gate_up_frac_mfma_peak": round(f_g / t_g / 1e9 / PEAK_BF16_TFLOPS, 3),
+            "down_frac_mfma_peak": round(f_d / t_d / 1e9 / PEAK_BF16_TFLOPS, 3)}
 
 
 def backward_measurement(dev, x, weights, m0):
@@ -624,8 +773,26 @@ def ceiling_measurements(dev, x, weights, m0):
     o2 = torch.empty(m0, H, dtype=torch.bfloat16, device=dev)
     t, _ = event_ms(lambda: torch.matmul(hm, d0.t(), out=o2), 10)
     out["hipblaslt_down_shape_tflops"] = round(2.0 * m0 * I0 * H / t / 1e9, 1)
-    out["note"] = ("same GPU, same run; hipBLASLt numbers are plain GEMMs of the VL expert on the benchmark's tensors "
-                   "(no SwiGLU, no second expert, rows already contiguous)")
+    del o2, hm
+    # the denoise step of config 4 (2048 action tokens on the 1024-wide expert): gate and up as one 2048 x 2048 x 2048
+    # product, down as 2048 x 2048 x 1024, on the action expert's tensors; many launches per event pair, so that
+    # launch gaps stay out of a figure of a few tens of microseconds
+    (g1, u1, d1) = weights[1]
+    I1 = g1.shape[0]
+    xa = x[:2048].contiguous()
+    wgu1 = torch.cat((g1, u1), 0)
+    oa = torch.empty(2048, 2 * I1, dtype=torch.bfloat16, device=dev)
+    t, _ = event_ms(lambda: torch.matmul(xa, wgu1.t(), out=oa), 20, batch=20)
+    out["hipblaslt_denoise_gate_up_shape_us"] = round(t * 1e3, 2)
+    out["hipblaslt_denoise_gate_up_shape_tflops"] = round(4.0 * 2048 * I1 * H / t / 1e9, 1)
+    ha = oa[:, :I1].contiguous()
+    ob = torch.empty(2048, H, dtype=torch.bfloat16, device=dev)
+    t, _ = event_ms(lambda: torch.matmul(ha, d1.t(), out=ob), 20, batch=20)
+    out["hipblaslt_denoise_down_shape_us"] = round(t * 1e3, 2)
+    out["hipblaslt_denoise_down_shape_tflops"] = round(2.0 * 2048 * I1 * H / t / 1e9, 1)
+    out["note"] = ("same GPU, same run; hipBLASLt numbers are plain GEMMs on the benchmark's tensors (no SwiGLU, one "
+                   "expert, rows already contiguous): the VL expert's two shapes at config 3 (28160 rows), and the "
+                   "action expert's two shapes at config 4's denoise step (2048 rows)")
     return out
 
 

@@ -96,7 +96,7 @@ using SmallTile = TileShape<128, 128, 4, 2, 4>;
 using BigTile8Q = TileShape<256, 256, 4, 2, 4>;
 // The large tile of a launch.
 template <int MODE>
-using BigTileFor = std::conditional_t<MODE == 3 /* kQkvRope */, BigTile8Q, BigTile8>;
+using BigTileFor = std::conditional_t<MODE == 3 || MODE == 4 /* kQkvRope, kQkvRopeFull */, BigTile8Q, BigTile8>;
 // the shape that runs the ragged last round of a launch (see tail_split_point): BigTile cut in four.  (Cut in two,
 // 256 x 128 with one workgroup per CU, measures the same.)
 using TailTile = SmallTile;
@@ -104,7 +104,9 @@ using TailTile = SmallTile;
 constexpr int kXcds = 8;
 constexpr int kGroupM = 8;                     // tile rows per patch in the tile order
 
-enum Mode { kGeneric = 0, kGateUp = 1, kDown = 2, kQkvRope = 3 };
+// kQkvRopeFull: kQkvRope reading a rotary table with one entry per channel (an instantiation of its own: both table
+// forms in one kernel cost the K loop registers)
+enum Mode { kGeneric = 0, kGateUp = 1, kDown = 2, kQkvRope = 3, kQkvRopeFull = 4 };
 
 struct Group {
   const __bf16* a;   // generic: [m, k] row-major (lda).  tiled: base of the K-tiled matrix
@@ -744,7 +746,7 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
         }
       }
     } else {
-      if constexpr (MODE == kQkvRope) {
+      if constexpr (MODE == kQkvRope || MODE == kQkvRopeFull) {
         // Bias and rotary embedding on the accumulators, before they are staged.  A wavefront's 128 columns are one
         // head; channel d of the head sits in block d / 32 at lane d % 32, so its rotation partner d +/- 64 is two
         // blocks away in the same lane.  Evaluated like eager bf16 code: the projection (with its bias) rounded once,
@@ -758,35 +760,70 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
           for (int j = 0; j < 4; ++j) bias_v[j] = static_cast<float>(p.bias[col_w + j * 32 + el32]);
         }
         const bool rotate = live && col_w < p.rope_cols;  // wave-uniform: q and k heads rotate, v heads do not
-        const bool full = p.rope_width == 128;  // uniform: channels d and d + 64 have entries of their own
+        if constexpr (MODE == kQkvRope) {  // channels d and d + 64 share a table entry (64 per token)
 #pragma unroll
-        for (int i = 0; i < FM; ++i) {
-#pragma unroll
-          for (int jp = 0; jp < 2; ++jp) {
-            // cos | sin of this lane's channel d = 32 jp + lane % 32 (and of d + 64 when they differ) for its 16 rows
-            uint32_t cs_lo[16], cs_hi[16];
+          for (int i = 0; i < FM; ++i) {
+            // cos | sin of this lane's channels 32 jp + lane % 32 (shared with the channel 64 further) for its 16 rows:
+            // all 32 loads go out before the first is used
+            uint32_t cs[16][2];
             if (rotate) {
 #pragma unroll
               for (int r = 0; r < 16; ++r) {
                 const int row = wm * (FM * 32) + i * 32 + 8 * (r >> 2) + 4 * elhi + (r & 3);
                 const bool in = row < S.rows;
-                const uint32_t* t = p.rope_table + static_cast<int64_t>(S.row0 + (in ? row : 0)) * p.rope_width + jp * 32 + el32;
-                cs_lo[r] = t[0];
-                cs_hi[r] = full ? t[64] : cs_lo[r];
+                const uint32_t* t = p.rope_table + static_cast<int64_t>(S.row0 + (in ? row : 0)) * 64 + el32;
+                cs[r][0] = t[0];
+                cs[r][1] = t[32];
               }
             }
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-              const float lo = round_bf16(acc[i][jp][r] + bias_v[jp]);
-              const float hi = round_bf16(acc[i][jp + 2][r] + bias_v[jp + 2]);
+#pragma unroll
+              for (int jp = 0; jp < 2; ++jp) {
+                const float lo = round_bf16(acc[i][jp][r] + bias_v[jp]);
+                const float hi = round_bf16(acc[i][jp + 2][r] + bias_v[jp + 2]);
+                if (rotate) {
+                  const float c = __uint_as_float(cs[r][jp] << 16), sn = __uint_as_float(cs[r][jp] & 0xffff0000u);
+                  acc[i][jp][r] = round_bf16(lo * c) - round_bf16(hi * sn);
+                  acc[i][jp + 2][r] = round_bf16(hi * c) + round_bf16(lo * sn);
+                } else {
+                  acc[i][jp][r] = lo;
+                  acc[i][jp + 2][r] = hi;
+                }
+              }
+            }
+          }
+        } else {
+          // one table entry per channel (128 per token): the same walk, one half of the channel pairs at a time (32
+          // entries in flight)
+#pragma unroll
+          for (int i = 0; i < FM; ++i) {
+#pragma unroll
+            for (int jp = 0; jp < 2; ++jp) {
+              uint32_t cs[16][2];  // [row][0]: channel 32 jp + lane % 32, [1]: the channel 64 further
               if (rotate) {
-                const float c_lo = __uint_as_float(cs_lo[r] << 16), s_lo = __uint_as_float(cs_lo[r] & 0xffff0000u);
-                const float c_hi = __uint_as_float(cs_hi[r] << 16), s_hi = __uint_as_float(cs_hi[r] & 0xffff0000u);
-                acc[i][jp][r] = round_bf16(lo * c_lo) - round_bf16(hi * s_lo);
-                acc[i][jp + 2][r] = round_bf16(hi * c_hi) + round_bf16(lo * s_hi);
-              } else {
-                acc[i][jp][r] = lo;
-                acc[i][jp + 2][r] = hi;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                  const int row = wm * (FM * 32) + i * 32 + 8 * (r >> 2) + 4 * elhi + (r & 3);
+                  const bool in = row < S.rows;
+                  const uint32_t* t = p.rope_table + static_cast<int64_t>(S.row0 + (in ? row : 0)) * 128 + jp * 32 + el32;
+                  cs[r][0] = t[0];
+                  cs[r][1] = t[64];
+                }
+              }
+#pragma unroll
+              for (int r = 0; r < 16; ++r) {
+                const float lo = round_bf16(acc[i][jp][r] + bias_v[jp]);
+                const float hi = round_bf16(acc[i][jp + 2][r] + bias_v[jp + 2]);
+                if (rotate) {
+                  const float c_lo = __uint_as_float(cs[r][0] << 16), s_lo = __uint_as_float(cs[r][0] & 0xffff0000u);
+                  const float c_hi = __uint_as_float(cs[r][1] << 16), s_hi = __uint_as_float(cs[r][1] & 0xffff0000u);
+                  acc[i][jp][r] = round_bf16(lo * c_lo) - round_bf16(hi * s_lo);
+                  acc[i][jp + 2][r] = round_bf16(hi * c_hi) + round_bf16(lo * s_hi);
+                } else {
+                  acc[i][jp][r] = lo;
+                  acc[i][jp + 2][r] = hi;
+                }
               }
             }
           }
@@ -1220,8 +1257,12 @@ extern "C" int wx_qkv_rope_proj(const void* x, const void* weight, const void* b
   p.rope_width = table_width;
   // the large tile only: its wavefronts cover whole heads (the small tile's 64 columns would split a rotation pair)
   using Tile = BigTileFor<kQkvRope>;
-  hipLaunchKernelGGL((dual_gemm_kernel<kQkvRope, Tile, false, false>), dim3(device_cu_count()), dim3(Tile::kThreads),
-                     0, as_stream(stream), p);
+  if (table_width == head_dim)
+    hipLaunchKernelGGL((dual_gemm_kernel<kQkvRopeFull, Tile, false, false>), dim3(device_cu_count()),
+                       dim3(Tile::kThreads), 0, as_stream(stream), p);
+  else
+    hipLaunchKernelGGL((dual_gemm_kernel<kQkvRope, Tile, false, false>), dim3(device_cu_count()), dim3(Tile::kThreads),
+                       0, as_stream(stream), p);
   return check_launch("dual_gemm_kernel<qkv_rope>");
 }
 

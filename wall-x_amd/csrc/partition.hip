@@ -348,13 +348,15 @@ __global__ __launch_bounds__(kMoverWaves* kWave) void permute_rows_tiled_gather_
 // blocks, for rows (lane >> 3) and (lane >> 3) + 8 of the row block, so a load instruction touches 8 rows x one whole
 // cache line instead of 16 rows x half a line, and a store instruction writes two 512-byte runs (the upper or lower
 // 8 rows of the two blocks).  Needs an even number of column blocks.
+// `split`: wavefronts per 16-row block (each takes that share of the column-block pairs); the host raises it for small
+// token counts so that the launch still has a few wavefronts per SIMD to cover the latency of its dependent loads.
 __global__ __launch_bounds__(kMoverWaves* kWave) void permute_rows_tiled_gather128_kernel(
     const u32x4* __restrict__ x, unsigned char* __restrict__ out, const int32_t* __restrict__ sorted_row_id,
-    const int32_t* __restrict__ expert_offsets, int64_t num_tokens, int64_t col_blocks, int64_t row_blocks) {
+    const int32_t* __restrict__ expert_offsets, int64_t num_tokens, int64_t col_blocks, int64_t row_blocks, int split) {
   const int lane = lane_id();
   const int64_t wave = static_cast<int64_t>(blockIdx.x) * kMoverWaves + threadIdx.x / kWave;
-  const int64_t rb = wave / kGatherSplit;
-  const int part = static_cast<int>(wave % kGatherSplit);
+  const int64_t rb = wave / split;
+  const int part = static_cast<int>(wave % split);
   if (rb >= row_blocks) return;
   const int32_t o0 = expert_offsets[0], o1 = expert_offsets[1], o2 = expert_offsets[2];
   const int64_t pad0 = round_up_256(o1 - o0);
@@ -377,7 +379,7 @@ __global__ __launch_bounds__(kMoverWaves* kWave) void permute_rows_tiled_gather1
     dst_off[h] = r * 64 + (((c8 & 3) ^ ((r >> 2) & 3)) << 4);
   }
   const int64_t pairs = col_blocks / 2;
-  const int64_t per = (pairs + kGatherSplit - 1) / kGatherSplit;
+  const int64_t per = (pairs + split - 1) / split;
   const int64_t p0 = part * per, p1 = p0 + per < pairs ? p0 + per : pairs;
   unsigned char* base = out + (rb << 10) + (((c8 >> 2) * row_blocks) << 10);  // block kb or kb + 1 of the pair
   const u32x4 zero = {0, 0, 0, 0};
@@ -694,17 +696,26 @@ extern "C" int wx_permute_rows_tiled(const void* x, void* out_tiled, const int32
   if (expert_offsets == nullptr) return fail(WX_ERR_INVALID_ARGUMENT, "wx_permute_rows_tiled: null expert_offsets");
   const int64_t row_blocks = padded_sorted_rows(num_tokens) / kBlkRows;
   if (sorted_row_id != nullptr) {
-    const int64_t waves = row_blocks * kGatherSplit;
-    const dim3 grid(static_cast<unsigned>((waves + kMoverWaves - 1) / kMoverWaves)), block(kMoverWaves * kWave);
+    const dim3 block(kMoverWaves * kWave);
 #ifndef WX_GATHER128
 #define WX_GATHER128 1
 #endif
     if (WX_GATHER128 && (num_cols / kBlkCols) % 2 == 0) {
-      hipLaunchKernelGGL(permute_rows_tiled_gather128_kernel, grid, block, 0, as_stream(stream),
-                         static_cast<const u32x4*>(x), static_cast<unsigned char*>(out_tiled), sorted_row_id,
-                         expert_offsets, num_tokens, num_cols / kBlkCols, row_blocks);
+      // kGatherSplit wavefronts per row block suit tens of thousands of tokens; a few thousand tokens would leave
+      // most SIMDs with one wavefront or none, each walking a chain of dependent loads: split the row blocks
+      // further, up to eight wavefronts per CU's worth or one pair of column blocks per two wavefronts' iteration
+      const int64_t pairs = num_cols / kBlkCols / 2;
+      int split = kGatherSplit;
+      while (row_blocks * split < 8ll * device_cu_count() && 2 * split <= pairs / 2) split *= 2;
+      const int64_t gather_waves = row_blocks * split;
+      hipLaunchKernelGGL(permute_rows_tiled_gather128_kernel, dim3(static_cast<unsigned>((gather_waves + kMoverWaves - 1) / kMoverWaves)),
+                         block, 0, as_stream(stream), static_cast<const u32x4*>(x),
+                         static_cast<unsigned char*>(out_tiled), sorted_row_id, expert_offsets, num_tokens,
+                         num_cols / kBlkCols, row_blocks, split);
       return check_launch("permute_rows_tiled_gather128_kernel");
     }
+    const int64_t waves = row_blocks * kGatherSplit;
+    const dim3 grid(static_cast<unsigned>((waves + kMoverWaves - 1) / kMoverWaves));
     hipLaunchKernelGGL(permute_rows_tiled_gather_kernel, grid, block, 0, as_stream(stream), static_cast<const u32x4*>(x),
                        static_cast<unsigned char*>(out_tiled), sorted_row_id, expert_offsets, num_tokens,
                        num_cols / kBlkCols, row_blocks);
