@@ -50,6 +50,10 @@ def parse():
                          "'mrope' / 'mrope_packed' are the M-RoPE apply at config 2 from the two tables / from the "
                          "packed table, 'mrope_copy' a device copy of q and k of the same shape, 'config2_index' the "
                          "three index builders and the packed-table builder at config 2")
+    ap.add_argument("--kernel-data", default="normal", choices=["normal", "zeros"],
+                    help="with --kernel-loop: the benchmark's normally distributed activations and weights, or all-zero "
+                         "ones (same launches and cycle counts, far less switching activity: the pair shows which clock "
+                         "the chip holds under each)")
     ap.add_argument("--kernel-shape", default="config3", choices=["config3", "denoise"],
                     help="with --kernel-loop: the batch the kernel runs on -- config 3 (29184 tokens, 28160 VL + 1024 "
                          "action) or config 4's denoise step (2048 action tokens, VL group empty)")
@@ -166,6 +170,9 @@ def main():
         down_unpermute()
 
     if args.kernel_loop:
+        if args.kernel_data == "zeros":
+            for t in (x, pg0, pu0, pd0, pg1, pu1, pd1):
+                t.zero_()
         permute(); gate_up(); down()
         fn = {"gate_up": gate_up, "down": down, "down_unpermute": down_unpermute, "permute": permute,
               "permute_plain": permute_plain,

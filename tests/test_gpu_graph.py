@@ -180,3 +180,58 @@ def test_prefill_forward_graph_replays_match_eager(dev):
         want = h.forward(ids, grid, ids == wl.ACTION_TOKEN_ID)
         torch.cuda.synchronize()
         assert torch.equal(got, want), f"replay {it} differs from the eager forward"
+
+
+def test_row_counts_reach_the_host_without_a_sync_and_captures_ignore_them(dev):
+    """An eager partition starts an asynchronous copy of expert_offsets to pinned host memory; once it has landed,
+    later layers hand the row counts to the GEMM entry points (one dispatch each instead of one per tile shape).  The
+    result is the same either way, a partition made under capture has no such copy, and a capture that uses an eager
+    routing still records the launches that decide on the device (its replays follow new offsets)."""
+    g = torch.Generator(device=dev).manual_seed(23)
+    hidden, inters = 1024, (1536, 512)
+    weights = _weights(dev, hidden, inters, g)
+    T, n_act = 2048, 2048
+    x = torch.randn(T, hidden, device=dev, generator=g).to(torch.bfloat16)
+    types = torch.ones(T, dtype=torch.bool, device=dev)
+    y_first, routing = moe.moe_layer_forward(x, types, weights)  # the copy cannot be checked for yet: device decides
+    assert routing.host_rows is not None
+    torch.cuda.synchronize()
+    rows = routing.rows_when_ready()
+    assert rows is not None and list(rows) == [T - n_act, n_act]
+    y_host, _ = moe.moe_layer_forward(x, types, weights, routing=routing)  # now with the counts from the host
+    assert int((y_first != y_host).sum()) == 0
+
+    # a capture on an eager routing: the offsets change before the replay, and the replay follows them
+    types_static = types.clone()
+    x_static = x.clone()
+    rmap, off, inv, _ = native.partition(types_static, 2, 0, None, want_sorted=True)
+    static_routing = moe.Routing(rmap, off, T, inv)
+    static_routing.host_rows = native.HostRows(off, T)
+    for e in weights:
+        for w in e:
+            native.pack_weight(w)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        moe.moe_layer_forward(x_static, types_static, weights, routing=static_routing)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    assert static_routing.rows_when_ready() is not None
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out_static, _ = moe.moe_layer_forward(x_static, types_static, weights, routing=static_routing)
+        captured, _ = moe.moe_layer_forward(x_static, types_static, weights)
+    assert _.host_rows is None  # partitioned under capture: nothing has run, nothing to read back
+    for n_vl in (0, 700):
+        new_types = torch.ones(T, dtype=torch.bool, device=dev)
+        new_types[:n_vl] = False
+        types_static.copy_(new_types)
+        # the eager routing's tensors are rewritten in place by a new partition, as a caller with static buffers would
+        r2, o2, i2, _ws = native.partition(types_static, 2, 0, None, want_sorted=True)
+        rmap.copy_(r2); off.copy_(o2); inv.copy_(i2)
+        graph.replay()
+        got, got_captured = out_static.clone(), captured.clone()
+        torch.cuda.synchronize()
+        want, _r = moe.moe_layer_forward(x, new_types, weights)
+        torch.cuda.synchronize()
+        assert int((got != want).sum()) == 0 and int((got_captured != want).sum()) == 0

@@ -67,6 +67,11 @@ class Routing:
     num_tokens: int
     sorted_row_id: Optional[torch.Tensor] = None  # int32 [T]: token at each sorted position (inverse map)
     host_offsets: Optional[list] = None  # expert_offsets read back to the host (generic path only, once per routing)
+    host_rows: Optional["native.HostRows"] = None  # the offsets' asynchronous copy to the host (eager partitions only)
+
+    def rows_when_ready(self):
+        """Per-expert row counts as _lib.i64x2 once the partition's asynchronous read-back has landed, else None."""
+        return None if self.host_rows is None else self.host_rows.ready()
 
 
 def _version_of(t: torch.Tensor):
@@ -108,6 +113,8 @@ class _RoutingCache(threading.local):
                                                             want_sorted=True)
         self.store_workspace(ws_key, ws)
         routing = Routing(row_id_map, offsets, flat.numel(), inverse)
+        if key[-1] == 0 and num_experts == 2:  # not under capture: the offsets start their way to the host
+            routing.host_rows = native.HostRows(offsets, flat.numel())
         if version is None:  # nothing to check a later call against: answer this call only
             self.ref = self.key = self.routing = None
             return routing
@@ -333,8 +340,8 @@ class SparseMoeBlock(nn.Module):
         if routing.sorted_row_id is None:
             return self._forward_scatter(x, routing, experts, host_rows, pre_norm, residual).view(batch, seq, hidden)
         return native.packed_block_forward(experts, x, routing.row_id_map, routing.sorted_row_id,
-                                           routing.expert_offsets, host_rows, pre_norm, residual
-                                           ).view(batch, seq, hidden)
+                                           routing.expert_offsets, host_rows, pre_norm, residual,
+                                           routing.rows_when_ready).view(batch, seq, hidden)
 
     def _host_rows(self, start_indices, end_indices, num_tokens):
         """The per-expert row counts as a host int64[2] when the caller's CPU tensors give them, else None.  The
@@ -484,11 +491,13 @@ def moe_layer_forward(x: torch.Tensor, token_types: torch.Tensor, weights, routi
         if workspace is None:
             _routing_cache.store_workspace(ws_key, ws)
         routing = Routing(row_id_map, offsets, x.size(0), inverse)
+        if ws_key[2] == 0:
+            routing.host_rows = native.HostRows(offsets, x.size(0))
     experts = _experts_for(weights)
     rows = None if host_rows is None else _lib.i64x2(host_rows)
     if routing.sorted_row_id is not None:  # the down launch stores every row at its token's position
         y = native.packed_block_forward(experts, x, routing.row_id_map, routing.sorted_row_id,
-                                        routing.expert_offsets, rows)
+                                        routing.expert_offsets, rows, rows_when_ready=routing.rows_when_ready)
         return y, routing
     x_tiled = native.permute_rows_tiled(x, routing.row_id_map, routing.expert_offsets, None, None)
     y_sorted = native.dual_swiglu_ffn_packed(x_tiled, x.size(0), routing.expert_offsets, experts.tensors,

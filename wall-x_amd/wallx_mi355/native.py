@@ -713,6 +713,36 @@ def dual_swiglu_ffn_packed(x_tiled: torch.Tensor, num_rows: int, expert_offsets:
     return out
 
 
+class HostRows:
+    """The partition's expert_offsets on their way to the host without a synchronisation: an asynchronous copy into
+    pinned memory, queued behind the partition on its stream, and an event behind the copy.  `ready()` answers None
+    until the event has completed and the per-expert row counts as _lib.i64x2 afterwards, so the layers of a forward
+    that are queued after the copy has landed hand the counts to the GEMM entry points and get one dispatch each
+    instead of one per tile shape (act.py:1274-1283 gives the reference's caller the same numbers on the host)."""
+
+    __slots__ = ("pinned", "event", "rows", "num_tokens")
+
+    def __init__(self, expert_offsets: torch.Tensor, num_tokens: int):
+        self.pinned = torch.empty(3, dtype=torch.int32, pin_memory=True)
+        self.pinned.copy_(expert_offsets[:3], non_blocking=True)
+        self.event = torch.cuda.Event()
+        self.event.record(torch.cuda.current_stream(expert_offsets.device))
+        self.rows = None
+        self.num_tokens = num_tokens
+
+    def ready(self):
+        if self.rows is None:
+            if self.event is None or not self.event.query():
+                return None
+            o = self.pinned.tolist()
+            self.event = None
+            counts = (o[1] - o[0], o[2] - o[1])
+            if min(counts) < 0 or sum(counts) != self.num_tokens:
+                return None  # rows were dropped (num_out_tokens) or the offsets are not a two-expert split
+            self.rows = _lib.i64x2(counts)
+        return self.rows
+
+
 _ffn_scratch = {}  # (device index, stream handle, capturing) -> (tiled activations, intermediate, capture id)
 
 
@@ -734,7 +764,7 @@ def _ffn_buffers(device: torch.device, stream: int, x_elems: int, h_elems: int):
         hit = (torch.empty(x_elems, dtype=torch.bfloat16, device=device),
                torch.empty(h_elems, dtype=torch.bfloat16, device=device), cap)
         _ffn_scratch[key] = hit
-    return hit[0], hit[1]
+    return hit[0], hit[1], cap
 
 
 def release_ffn_buffers() -> None:
@@ -781,11 +811,13 @@ class PackedExperts:
 
 def packed_block_forward(experts: PackedExperts, x: torch.Tensor, row_id_map: torch.Tensor,
                          sorted_row_id: torch.Tensor, expert_offsets: torch.Tensor, host_rows_c=None,
-                         pre_norm=None, residual: bool = False) -> torch.Tensor:
+                         pre_norm=None, residual: bool = False, rows_when_ready=None) -> torch.Tensor:
     """One block forward on packed weights, in token order: [RMSNorm ->] permute -> gate/up + SwiGLU -> down with
     the unpermute [and the residual add, + x] in its stores.  x [T, hidden] bf16; the three routing tensors are the partition's
-    (int32, on x's device); host_rows_c is None or _lib.i64x2((rows of expert 0, rows of expert 1)).  The work
-    buffers are shared per stream (see _ffn_buffers); the result is a new tensor."""
+    (int32, on x's device); host_rows_c is None or _lib.i64x2((rows of expert 0, rows of expert 1)).  Without it,
+    `rows_when_ready` (a callable returning such a pair or None: the partition's own read-back of expert_offsets, see
+    HostRows) is asked outside HIP graph captures; a capture always records the launches that decide on the device.
+    The work buffers are shared per stream (see _ffn_buffers); the result is a new tensor."""
     dev = x.device
     if dev != experts.device or x.dtype != torch.bfloat16 or x.dim() != 2 or x.shape[1] != experts.hidden:
         raise RuntimeError("x must be a [tokens, hidden] BFloat16 tensor on the device of the packed weights")
@@ -803,7 +835,9 @@ def packed_block_forward(experts: PackedExperts, x: torch.Tensor, row_id_map: to
     lib = _lib.load()
     stream = torch.cuda.current_stream(dev).cuda_stream
     x_elems, h_elems = experts.sizes(T)
-    x_tiled, hmid = _ffn_buffers(dev, stream, x_elems, h_elems)
+    x_tiled, hmid, cap = _ffn_buffers(dev, stream, x_elems, h_elems)
+    if host_rows_c is None and rows_when_ready is not None and cap == 0:
+        host_rows_c = rows_when_ready()
     H, I0, I1 = experts.hidden, experts.inter0, experts.inter1
     xt, hm, off, srt = x_tiled.data_ptr(), hmid.data_ptr(), expert_offsets.data_ptr(), sorted_row_id.data_ptr()
     with _DeviceGuard(x):
