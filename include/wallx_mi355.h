@@ -357,6 +357,25 @@ int wx_unpermute_rows_add(const void* y, const void* residual, void* out, const 
 int wx_unpermute_rows_add_rmsnorm(const void* y, const void* residual, void* out, void* normed,
                                   const void* weight, float eps, const int32_t* row_id_map,
                                   int64_t num_tokens, int64_t num_cols, wx_stream_t stream);
+/* The training step's side of the two fusions above (the reference trains through act.py:256-265 with autograd):
+ * wx_rmsnorm_permute_rows = the same RMSNorm followed by wx_permute_rows at topK 1 -- out_sorted[p] = weight *
+ * rmsnorm(x[sorted_row_id[p]]), row-major in expert-sorted order: the normed rows the experts' weight gradients
+ * contract over, recomputed in the backward instead of kept by the forward.
+ * wx_unpermute_rows_rmsnorm_bwd = backward of "normed = weight * rmsnorm(x); sorted = permute(normed)" for the
+ * gradient grad_sorted of the sorted rows (wx_unpermute_rows_bwd at topK 1, then the norm's backward), in one pass:
+ *   grad_x[t] = (add[t] +) inv * (g w - xhat * mean(g w xhat)),  g = grad_sorted[row_id_map[t]] (0 where the map holds
+ *   -1), xhat = x[t] * inv, inv = rsqrt(mean(x[t]^2) + eps), fp32 math and one rounding;  `add` (optional, [T, H]) is
+ *   the gradient that reaches x along the residual branch (act.py:256,265: the layer's output gradient itself);
+ *   grad_weight[c] = sum over t of g[c] * bf16(xhat[c]), fp32 accumulation, bf16 [H].
+ * workspace: wx_rmsnorm_bwd_workspace_bytes(num_cols) bytes of device memory (per-wavefront partial sums of
+ * grad_weight).  num_cols: a multiple of 8, at most 4096. */
+int wx_rmsnorm_permute_rows(const void* x, const void* weight, float eps, void* out_sorted,
+                            const int32_t* sorted_row_id, int64_t num_tokens, int64_t num_cols, wx_stream_t stream);
+size_t wx_rmsnorm_bwd_workspace_bytes(int64_t num_cols);
+int wx_unpermute_rows_rmsnorm_bwd(const void* grad_sorted, const void* x, const void* weight, float eps,
+                                  const void* add, void* grad_x, void* grad_weight, const int32_t* row_id_map,
+                                  int64_t num_tokens, int64_t num_cols, void* workspace, size_t workspace_bytes,
+                                  wx_stream_t stream);
 
 /* Elementwise backward of h = silu(g) * u inside an expert FFN (act.py:79-82; the reference leaves it to autograd):
  * from gate, up (the two projections, kept by the forward or recomputed) and dh (gradient w.r.t. h) in one pass:

@@ -673,7 +673,9 @@ def test_swiglu_bwd_kernel(dev, shape):
 @pytest.mark.parametrize("n_tok,inters", [(203, (256, 64)), (700, (192, 96)), (700, (320, 128))])
 def test_moe_block_backward_matches_autograd_of_the_plain_forward(dev, fused_extras, n_tok, inters):
     """Gradients of the block (inputs and all six weights) against torch autograd through the oracle's fp32
-    forward; with fused_extras the layer's RMSNorm and residual ride along (PyTorch ops under autograd).
+    forward; with fused_extras the layer's RMSNorm and residual ride along (inside the permute and the down launch's
+    stores in the forward, inside the unpermute of the input gradient in the backward) and the norm weight's
+    gradient is checked as well.
     Intermediate sizes that are multiples of 64 take the path that keeps the gate / up projections of the forward
     (one and several 256-row tiles per expert); (192, 96) takes the one that recomputes them."""
     class Cfg:
@@ -692,7 +694,8 @@ def test_moe_block_backward_matches_autograd_of_the_plain_forward(dev, fused_ext
     # reference: fp32 leaves, oracle forward, torch autograd
     xr = x.float().requires_grad_(True)
     wr = [tuple(w.detach().float().requires_grad_(True) for w in e.weights()) for e in block.experts]
-    hin = oracle.rms_norm_ref(xr, nw.float(), 1e-6) if fused_extras else xr
+    nwr = nw.float().requires_grad_(True)
+    hin = oracle.rms_norm_ref(xr, nwr, 1e-6) if fused_extras else xr
     yr = oracle.sparse_moe_block_ref(hin, types, wr, eager_rounding=False)
     if fused_extras:
         yr = xr + yr
@@ -700,11 +703,16 @@ def test_moe_block_backward_matches_autograd_of_the_plain_forward(dev, fused_ext
     # kernels
     block = block.to(dev)
     xd = x.to(dev).requires_grad_(True)
-    kw = dict(pre_norm=(nw.to(dev), 1e-6), residual=True) if fused_extras else {}
+    nwd = nw.to(dev).requires_grad_(True)
+    kw = dict(pre_norm=(nwd, 1e-6), residual=True) if fused_extras else {}
     yd = block(xd, types.to(dev), **kw)
     _close(yd, yr.detach(), atol=3e-2, rtol=2e-2, what="forward under autograd")
     yd.backward(dy.to(dev))
     _close(xd.grad, xr.grad, atol=3e-2, rtol=3e-2, what="grad of the input")
+    if fused_extras:
+        scale = float(nwr.grad.abs().max())
+        err = float((nwd.grad.float().cpu() - nwr.grad).abs().max())
+        assert err <= 0.03 * scale + 1e-3, f"norm weight: max err {err} at scale {scale}"
     for e in range(2):
         for name, wref in zip(("gate", "up", "down"), wr[e]):
             got = getattr(block.experts[e], f"{name}_proj").weight.grad

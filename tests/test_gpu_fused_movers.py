@@ -92,6 +92,54 @@ def test_unpermute_add_rmsnorm(dev, T, H):
     assert float((got != ref_norm).float().mean()) < 0.02
 
 
+@pytest.mark.parametrize("T,H,n_act", [(300, 256, 37), (912, 2048, 32), (7, 8, 7), (33, 1000, 0), (20, 4096, 11)])
+def test_rmsnorm_permute_rows(dev, T, H, n_act):
+    """The normed rows in expert-sorted order, row-major: the oracle's RMSNorm followed by its permute, up to the
+    rounding-boundary steps the fp32 sum of squares (another accumulation order) allows."""
+    g = torch.Generator().manual_seed(T + 3 * H)
+    x = _bf((T, H), g, 2.0)
+    w = (1.0 + 0.1 * torch.randn(H, generator=g)).to(torch.bfloat16)
+    types = torch.zeros(T, dtype=torch.bool)
+    types[torch.randperm(T, generator=g)[:n_act]] = True
+    ref, _, _ = oracle.permute_ref(oracle.rms_norm_ref(x, w, 1e-6), types)
+    _, _, inv, _ = native.partition(types.to(dev), 2, 0, None, want_sorted=True)
+    got = native.rmsnorm_permute_rows(x.to(dev), w.to(dev), 1e-6, inv).cpu().float()
+    ref = ref.float()
+    bad = (got - ref).abs() > 2.0 ** -6 * ref.abs() + 1e-6
+    assert not bad.any(), f"{int(bad.sum())} of {bad.numel()} differ by more than two bf16 steps"
+    assert float((got != ref).float().mean()) < 0.02
+
+
+@pytest.mark.parametrize("with_add", [False, True])
+@pytest.mark.parametrize("T,H,n_act", [(300, 256, 37), (912, 2048, 32), (7, 8, 7), (33, 1000, 0), (3000, 1024, 800)])
+def test_unpermute_rmsnorm_bwd(dev, T, H, n_act, with_add):
+    """Backward of permute(weight * rmsnorm(x)) for a gradient of the sorted rows, against torch autograd of the
+    oracle's RMSNorm and permute in fp32 (the kernel rounds its result once, to bf16): the input gradient, with and
+    without the residual branch's gradient summed in, and the weight gradient."""
+    g = torch.Generator().manual_seed(T * 7 + H)
+    x = _bf((T, H), g, 2.0)
+    w = (1.0 + 0.1 * torch.randn(H, generator=g)).to(torch.bfloat16)
+    gs = _bf((T, H), g)  # gradient w.r.t. the sorted, normed rows
+    add = _bf((T, H), g) if with_add else None
+    types = torch.zeros(T, dtype=torch.bool)
+    types[torch.randperm(T, generator=g)[:n_act]] = True
+    xr, wr = x.float().requires_grad_(True), w.float().requires_grad_(True)
+    sorted_ref, _, _ = oracle.permute_ref(oracle.rms_norm_ref(xr, wr, 1e-6), types)
+    loss = (sorted_ref * gs.float()).sum()
+    if with_add:
+        loss = loss + (xr * add.float()).sum()
+    loss.backward()
+    rmap, _, _, _ = native.partition(types.to(dev), 2, 0, None, want_sorted=False)
+    gx, gw = native.unpermute_rmsnorm_bwd(gs.to(dev), x.to(dev), w.to(dev), 1e-6, rmap,
+                                          add=None if add is None else add.to(dev))
+    ref = xr.grad
+    err = (gx.cpu().float() - ref).abs()
+    assert not (err > 2.0 ** -7 * ref.abs() + 2e-3 * float(ref.abs().mean())).any(), float(err.max())
+    scale = float(wr.grad.abs().max())
+    werr = float((gw.cpu().float() - wr.grad).abs().max())
+    assert werr <= 2.0 ** -7 * scale + 1e-3 * scale, f"weight gradient: max err {werr} at scale {scale}"
+
+
 def test_moe_block_with_both_fusions(dev):
     """h + block(RMSNorm(h)) through the module's fused path against the same module fed by separate PyTorch ops."""
     from types import SimpleNamespace

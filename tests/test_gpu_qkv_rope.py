@@ -112,7 +112,55 @@ def test_qkv_rope_rejects_what_it_cannot_do(dev):
     p = pos.data_ptr()
     assert lib.wx_qkv_rope_proj(p, p, None, p, 32, p, 4, 64, 1, 1, 64, None) == -2
     assert b"head_dim" in lib.wx_last_error_string()
-    x = torch.zeros(1, 4, 64, dtype=torch.bfloat16, device=dev).requires_grad_(True)
-    with pytest.raises(RuntimeError, match="no backward"):
-        ops.qkv_projection_with_rope(x, torch.zeros(384, 64, dtype=torch.bfloat16, device=dev), None,
-                                     torch.zeros(4, 64, dtype=torch.int32, device=dev), 1, 1)
+
+
+@pytest.mark.parametrize("layout", ["hf", "csrc"])
+@pytest.mark.parametrize("B,S,H,nq,nkv,with_bias", [(2, 200, 512, 4, 2, True), (1, 37, 256, 2, 1, False)])
+def test_qkv_rope_projection_backward(dev, B, S, H, nq, nkv, with_bias, layout):
+    """Gradients of the fused projection against torch autograd of the fp32 expression it fuses (linear, then the
+    oracle's M-RoPE in fp32 on the same cos / sin): d hidden, d weight, d bias for a random cotangent on q, k and v.
+    The fused op rounds the forward and the rotated gradient to bf16 like the eager bf16 path, so the comparison
+    carries the GEMM tolerance, scaled to each gradient's magnitude."""
+    g = torch.Generator().manual_seed(B * 77 + S)
+    D = 128
+    n = (nq + 2 * nkv) * D
+    x = torch.randn(B, S, H, generator=g).to(torch.bfloat16)
+    w = (torch.randn(n, H, generator=g) * 0.05).to(torch.bfloat16)
+    b = (torch.randn(n, generator=g) * 0.5).to(torch.bfloat16) if with_bias else None
+    pos = torch.stack([torch.randint(0, 60, (B, S), generator=g), torch.randint(100, 160, (B, S), generator=g),
+                       torch.randint(300, 360, (B, S), generator=g)])
+    cq = torch.randn(B, nq, S, D, generator=g).to(torch.bfloat16)
+    ck = torch.randn(B, nkv, S, D, generator=g).to(torch.bfloat16)
+    cv = torch.randn(B, nkv, S, D, generator=g).to(torch.bfloat16)
+    # reference: fp32 autograd through linear and the oracle's rotation
+    xr, wr = x.float().requires_grad_(True), w.float().requires_grad_(True)
+    br = None if b is None else b.float().requires_grad_(True)
+    cos, sin = oracle.rotary_cos_sin_ref(pos, wl.text_inv_freq(), torch.bfloat16)
+    qkv = F.linear(xr, wr, br)
+    q, k, v = qkv.split([nq * D, nkv * D, nkv * D], dim=-1)
+    q = q.reshape(B, S, nq, D).transpose(1, 2)
+    k = k.reshape(B, S, nkv, D).transpose(1, 2)
+    v = v.reshape(B, S, nkv, D).transpose(1, 2)
+    rq, rk = oracle.mrope_apply_ref(q, k, cos.float(), sin.float(), list(wl.MROPE_SECTION), layout)
+    ((rq * cq.float()).sum() + (rk * ck.float()).sum() + (v * cv.float()).sum()).backward()
+    # fused op
+    xd, wd = x.to(dev).requires_grad_(True), w.to(dev).requires_grad_(True)
+    bd = None if b is None else b.to(dev).requires_grad_(True)
+    table = ops.multimodal_rope_table(pos.to(dev), wl.text_inv_freq().to(dev), wl.MROPE_SECTION, layout)
+    gq, gk, gv = ops.qkv_projection_with_rope(xd, wd, bd, table, nq, nkv, mrope_section=wl.MROPE_SECTION)
+    torch.autograd.backward([gq, gk, gv], [cq.to(dev), ck.to(dev), cv.to(dev)])
+
+    def close(got, ref, what):
+        got, ref = got.float().cpu(), ref.float()
+        s = float(ref.pow(2).mean().sqrt())
+        bad = (got - ref).abs() > 2e-2 * s + 1e-2 * ref.abs()
+        assert not bad.any(), f"{what}: {int(bad.sum())} of {bad.numel()} outside tolerance (rms {s})"
+
+    close(xd.grad, xr.grad, "d hidden_states")
+    close(wd.grad, wr.grad, "d qkv_weight")
+    if b is not None:
+        close(bd.grad, br.grad, "d qkv_bias")
+    # the forward under autograd is the same launch as without it
+    with torch.no_grad():
+        q0, k0, v0 = ops.qkv_projection_with_rope(x.to(dev), w.to(dev), None if b is None else b.to(dev), table, nq, nkv)
+    assert torch.equal(q0, gq) and torch.equal(k0, gk) and torch.equal(v0, gv)

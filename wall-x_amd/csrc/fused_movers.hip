@@ -3,6 +3,10 @@
 //   unpermute_add           unpermute + residual add
 //   unpermute_add_rmsnorm   the same, and the RMSNorm that reads the sum next (the following layer's
 //                           input_layernorm, act.py:240, or the final norm, act.py:506) as a second output
+//   rmsnorm_permute_rows    the same norm with a row-major, expert-sorted result (what the weight gradients of a
+//                           training step contract over), and
+//   unpermute_rmsnorm_bwd   unpermute of the gradient w.r.t. the normed rows + the norm's backward (+ the residual
+//                           branch's gradient), with per-wavefront partial sums of the norm weight's gradient
 // Each replaces two (three) passes over [T, H] by one.  bf16 only (the FFN kernels' type).
 //
 // RMSNorm follows the reference module op by op: x in fp32, variance = mean(x^2), x * rsqrt(variance + eps),
@@ -239,6 +243,159 @@ __global__ __launch_bounds__(256) void unpermute_add_rmsnorm_kernel(
   }
 }
 
+// out[pos] = weight * rmsnorm(x[sorted_row_id[pos]]), row-major in expert-sorted order; one wavefront per row, the
+// row held in registers.  The same arithmetic as the tiled form above.
+template <int NV>
+__global__ __launch_bounds__(256) void rmsnorm_permute_rows_kernel(
+    const u32x4* __restrict__ x, const u32x4* __restrict__ weight, float eps, u32x4* __restrict__ out,
+    const int32_t* __restrict__ sorted_row_id, int64_t num_tokens, int vec_per_row) {
+  const int lane = threadIdx.x & 63;
+  const int64_t wave = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
+  const int64_t n_waves = static_cast<int64_t>(gridDim.x) * 4;
+  for (int64_t pos = wave; pos < num_tokens; pos += n_waves) {
+    const int32_t tok = sorted_row_id[pos];
+    const bool live = tok >= 0 && tok < num_tokens;
+    const u32x4* src = x + static_cast<int64_t>(live ? tok : 0) * vec_per_row;
+    u32x4 a[NV];
+    float ss = 0.f;
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+      const int cc = lane + u * 64;
+      a[u] = (cc < vec_per_row && live) ? ld16(src + cc) : u32x4{0, 0, 0, 0};
+    }
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+      float f[8];
+      unpack16<WX_BF16>(a[u], f);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ss += f[e] * f[e];
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) ss += __shfl_xor(ss, off);
+    const float inv = __frsqrt_rn(ss / static_cast<float>(vec_per_row * 8) + eps);
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+      const int cc = lane + u * 64;
+      if (cc < vec_per_row) {
+        float f[8], w[8];
+        unpack16<WX_BF16>(a[u], f);
+        unpack16<WX_BF16>(weight[cc], w);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) f[e] = w[e] * round_bf16(f[e] * inv);  // pack16 rounds the product
+        st16(out + pos * vec_per_row + cc, pack16<WX_BF16>(f));
+      }
+    }
+  }
+}
+
+// Backward of  y[row_id_map[t]] = weight * rmsnorm(x[t])  for the gradient g of the sorted rows:
+//   dx[t] = (add[t] +) inv * (g w - xhat * mean(g w xhat)),  xhat = x[t] * inv,  inv = rsqrt(mean(x[t]^2) + eps)
+// in fp32 with one rounding at the store (a dropped token, map entry -1, has g = 0), and
+//   dw_partial[wavefront] = sum over the wavefront's rows of g * round_bf16(xhat)   (the forward's rounded xhat),
+// fp32 [number of wavefronts, H]; a second kernel adds the partials up.  One wavefront per token row.
+template <int NV>
+__global__ __launch_bounds__(256) void unpermute_rmsnorm_bwd_kernel(
+    const u32x4* __restrict__ g_sorted, const u32x4* __restrict__ x, const u32x4* __restrict__ weight, float eps,
+    const u32x4* __restrict__ add, u32x4* __restrict__ dx, float* __restrict__ dw_partial,
+    const int32_t* __restrict__ row_id_map, int64_t num_tokens, int vec_per_row) {
+  const int lane = threadIdx.x & 63;
+  const int64_t wave = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
+  const int64_t n_waves = static_cast<int64_t>(gridDim.x) * 4;
+  float dw[NV][8];
+#pragma unroll
+  for (int u = 0; u < NV; ++u)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) dw[u][e] = 0.f;
+  for (int64_t t = wave; t < num_tokens; t += n_waves) {
+    const int32_t src_row = row_id_map[t];
+    const u32x4* gsrc = g_sorted + static_cast<int64_t>(src_row < 0 ? 0 : src_row) * vec_per_row;
+    u32x4 xv[NV], gv[NV], av[NV];
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+      const int cc = lane + u * 64;
+      const bool in = cc < vec_per_row;
+      xv[u] = in ? ld16(x + t * vec_per_row + cc) : u32x4{0, 0, 0, 0};
+      gv[u] = (in && src_row >= 0) ? ld16(gsrc + cc) : u32x4{0, 0, 0, 0};
+      av[u] = (in && add != nullptr) ? ld16(add + t * vec_per_row + cc) : u32x4{0, 0, 0, 0};
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+      float f[8];
+      unpack16<WX_BF16>(xv[u], f);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ss += f[e] * f[e];
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) ss += __shfl_xor(ss, off);
+    const float inv = __frsqrt_rn(ss / static_cast<float>(vec_per_row * 8) + eps);
+    float dot = 0.f;  // sum of g w xhat over the row
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+      const int cc = lane + u * 64;
+      if (cc < vec_per_row) {
+        float xf[8], gf[8], w[8];
+        unpack16<WX_BF16>(xv[u], xf);
+        unpack16<WX_BF16>(gv[u], gf);
+        unpack16<WX_BF16>(weight[cc], w);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float xhat = xf[e] * inv;
+          dw[u][e] += gf[e] * round_bf16(xhat);
+          dot += gf[e] * w[e] * xhat;
+        }
+      }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) dot += __shfl_xor(dot, off);
+    const float mean = dot / static_cast<float>(vec_per_row * 8);
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+      const int cc = lane + u * 64;
+      if (cc < vec_per_row) {
+        float xf[8], gf[8], af[8], w[8];
+        unpack16<WX_BF16>(xv[u], xf);
+        unpack16<WX_BF16>(gv[u], gf);
+        unpack16<WX_BF16>(av[u], af);
+        unpack16<WX_BF16>(weight[cc], w);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) af[e] += inv * (gf[e] * w[e] - xf[e] * inv * mean);
+        st16(dx + t * vec_per_row + cc, pack16<WX_BF16>(af));
+      }
+    }
+  }
+  float* mine = dw_partial + wave * (static_cast<int64_t>(vec_per_row) * 8);
+#pragma unroll
+  for (int u = 0; u < NV; ++u) {
+    const int cc = lane + u * 64;
+    if (cc < vec_per_row) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) mine[cc * 8 + e] = dw[u][e];
+    }
+  }
+}
+
+// dw[c] = sum over p of partial[p][c], rounded to bf16.  A workgroup takes 64 columns; its four wavefronts split the
+// partial rows and meet in LDS.
+__global__ __launch_bounds__(256) void column_sums_kernel(const float* __restrict__ partial, __bf16* __restrict__ dw,
+                                                          int64_t n_partials, int64_t cols) {
+  __shared__ float s_sum[4][64];
+  const int lane = threadIdx.x & 63, part = threadIdx.x >> 6;
+  const int64_t c = static_cast<int64_t>(blockIdx.x) * 64 + lane;
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  if (c < cols) {
+    int64_t p = part;
+    for (; p + 12 < n_partials; p += 16) {
+#pragma unroll
+      for (int u = 0; u < 4; ++u) acc[u] += partial[(p + 4 * u) * cols + c];
+    }
+    for (; p < n_partials; p += 4) acc[0] += partial[p * cols + c];
+  }
+  s_sum[part][lane] = (acc[0] + acc[1]) + (acc[2] + acc[3]);
+  __syncthreads();
+  if (part == 0 && c < cols) dw[c] = static_cast<__bf16>((s_sum[0][lane] + s_sum[1][lane]) + (s_sum[2][lane] + s_sum[3][lane]));
+}
+
 }  // namespace
 }  // namespace wx
 
@@ -344,4 +501,86 @@ extern "C" int wx_unpermute_rows_add_rmsnorm(const void* y, const void* residual
   }
 #undef WX_CASE
   return check_launch("unpermute_add_rmsnorm_kernel");
+}
+
+extern "C" int wx_rmsnorm_permute_rows(const void* x, const void* weight, float eps, void* out_sorted,
+                                       const int32_t* sorted_row_id, int64_t num_tokens, int64_t num_cols,
+                                       wx_stream_t stream) {
+  const char* who = "wx_rmsnorm_permute_rows";
+  if (num_tokens < 0 || num_cols <= 0) return fail(WX_ERR_INVALID_ARGUMENT, "%s: bad sizes", who);
+  if (num_cols % 8 != 0 || num_cols > 4096)
+    return fail(WX_ERR_UNSUPPORTED, "%s: num_cols (%lld) must be a multiple of 8 and at most 4096", who,
+                static_cast<long long>(num_cols));
+  if (!(eps >= 0.f)) return fail(WX_ERR_INVALID_ARGUMENT, "%s: eps must be non-negative", who);
+  if (num_tokens == 0) return WX_OK;
+  if (num_tokens > INT32_MAX) return fail(WX_ERR_UNSUPPORTED, "%s: more than 2^31-1 rows", who);
+  if (!x || !weight || !out_sorted || !sorted_row_id) return fail(WX_ERR_INVALID_ARGUMENT, "%s: null pointer", who);
+  if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(weight) | reinterpret_cast<uintptr_t>(out_sorted)) & 15)
+    return fail(WX_ERR_INVALID_ARGUMENT, "%s: buffers must be 16-byte aligned", who);
+  const int vec = static_cast<int>(num_cols / 8);
+  const int64_t want = (num_tokens + 3) / 4;
+  const int64_t cap = static_cast<int64_t>(device_cu_count()) * 8;
+  const dim3 grid(static_cast<unsigned>(want < cap ? want : cap)), block(256);
+  hipStream_t s = as_stream(stream);
+#define WX_CASE(N)                                                                                                   \
+  case N:                                                                                                            \
+    hipLaunchKernelGGL(rmsnorm_permute_rows_kernel<N>, grid, block, 0, s, static_cast<const u32x4*>(x),              \
+                       static_cast<const u32x4*>(weight), eps, static_cast<u32x4*>(out_sorted), sorted_row_id,       \
+                       num_tokens, vec);                                                                             \
+    break;
+  switch ((vec + 63) / 64) {
+    WX_CASE(1) WX_CASE(2) WX_CASE(3) WX_CASE(4) WX_CASE(5) WX_CASE(6) WX_CASE(7) WX_CASE(8)
+    default: return fail(WX_ERR_UNSUPPORTED, "%s: num_cols too large", who);
+  }
+#undef WX_CASE
+  return check_launch("rmsnorm_permute_rows_kernel");
+}
+
+extern "C" size_t wx_rmsnorm_bwd_workspace_bytes(int64_t num_cols) {
+  if (num_cols <= 0) return 0;
+  // one fp32 row of partial weight-gradient sums per wavefront of the largest grid the backward launches
+  return static_cast<size_t>(device_cu_count()) * 2 * 4 * static_cast<size_t>(num_cols) * sizeof(float);
+}
+
+extern "C" int wx_unpermute_rows_rmsnorm_bwd(const void* grad_sorted, const void* x, const void* weight, float eps,
+                                             const void* add, void* grad_x, void* grad_weight,
+                                             const int32_t* row_id_map, int64_t num_tokens, int64_t num_cols,
+                                             void* workspace, size_t workspace_bytes, wx_stream_t stream) {
+  const char* who = "wx_unpermute_rows_rmsnorm_bwd";
+  if (num_tokens < 0 || num_cols <= 0) return fail(WX_ERR_INVALID_ARGUMENT, "%s: bad sizes", who);
+  if (num_cols % 8 != 0 || num_cols > 4096)
+    return fail(WX_ERR_UNSUPPORTED, "%s: num_cols (%lld) must be a multiple of 8 and at most 4096", who,
+                static_cast<long long>(num_cols));
+  if (!(eps >= 0.f)) return fail(WX_ERR_INVALID_ARGUMENT, "%s: eps must be non-negative", who);
+  if (num_tokens > INT32_MAX) return fail(WX_ERR_UNSUPPORTED, "%s: more than 2^31-1 rows", who);
+  if (!grad_weight || !workspace) return fail(WX_ERR_INVALID_ARGUMENT, "%s: null pointer", who);
+  if (num_tokens > 0 && (!grad_sorted || !x || !weight || !grad_x || !row_id_map))
+    return fail(WX_ERR_INVALID_ARGUMENT, "%s: null pointer", who);
+  if ((reinterpret_cast<uintptr_t>(grad_sorted) | reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(weight) |
+       reinterpret_cast<uintptr_t>(add) | reinterpret_cast<uintptr_t>(grad_x) | reinterpret_cast<uintptr_t>(workspace)) & 15)
+    return fail(WX_ERR_INVALID_ARGUMENT, "%s: buffers must be 16-byte aligned", who);
+  if (workspace_bytes < wx_rmsnorm_bwd_workspace_bytes(num_cols))
+    return fail(WX_ERR_INVALID_ARGUMENT, "%s: workspace too small (see wx_rmsnorm_bwd_workspace_bytes)", who);
+  const int vec = static_cast<int>(num_cols / 8);
+  const int64_t want = (num_tokens + 3) / 4;
+  const int64_t cap = static_cast<int64_t>(device_cu_count()) * 2;  // bounded by the workspace: one partial row per wavefront
+  const int64_t blocks = want < cap ? (want > 0 ? want : 1) : cap;
+  const dim3 grid(static_cast<unsigned>(blocks)), block(256);
+  hipStream_t s = as_stream(stream);
+#define WX_CASE(N)                                                                                                   \
+  case N:                                                                                                            \
+    hipLaunchKernelGGL(unpermute_rmsnorm_bwd_kernel<N>, grid, block, 0, s, static_cast<const u32x4*>(grad_sorted),   \
+                       static_cast<const u32x4*>(x), static_cast<const u32x4*>(weight), eps,                        \
+                       static_cast<const u32x4*>(add), static_cast<u32x4*>(grad_x), static_cast<float*>(workspace), \
+                       row_id_map, num_tokens, vec);                                                                 \
+    break;
+  switch ((vec + 63) / 64) {
+    WX_CASE(1) WX_CASE(2) WX_CASE(3) WX_CASE(4) WX_CASE(5) WX_CASE(6) WX_CASE(7) WX_CASE(8)
+    default: return fail(WX_ERR_UNSUPPORTED, "%s: num_cols too large", who);
+  }
+#undef WX_CASE
+  if (int rc = check_launch("unpermute_rmsnorm_bwd_kernel")) return rc;
+  hipLaunchKernelGGL(column_sums_kernel, dim3(static_cast<unsigned>((num_cols + 63) / 64)), dim3(256), 0, s,
+                     static_cast<const float*>(workspace), static_cast<__bf16*>(grad_weight), blocks * 4, num_cols);
+  return check_launch("column_sums_kernel");
 }

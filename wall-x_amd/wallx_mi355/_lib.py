@@ -63,6 +63,9 @@ PROTOTYPES = {
     "wx_rmsnorm_permute_rows_tiled": (_i32, [_vp, _vp, _f32, _vp, _vp, _vp, _i64, _i64, _vp]),
     "wx_unpermute_rows_add": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _vp]),
     "wx_unpermute_rows_add_rmsnorm": (_i32, [_vp, _vp, _vp, _vp, _vp, _f32, _vp, _i64, _i64, _vp]),
+    "wx_rmsnorm_permute_rows": (_i32, [_vp, _vp, _f32, _vp, _vp, _i64, _i64, _vp]),
+    "wx_rmsnorm_bwd_workspace_bytes": (_sz, [_i64]),
+    "wx_unpermute_rows_rmsnorm_bwd": (_i32, [_vp, _vp, _vp, _f32, _vp, _vp, _vp, _vp, _i64, _i64, _vp, _sz, _vp]),
     "wx_swiglu_bwd": (_i32, [_vp] * 6 + [_i64, _vp]),
     "wx_swiglu_bwd_tiled": (_i32, [_vp, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _vp]),
 }

@@ -356,8 +356,51 @@ def multimodal_rope_from_table(q, k, table, mrope_section, layout="hf"):
     return MultimodalRoPEFromTable.apply(q, k, table, mrope_section, layout)
 
 
+class QkvProjectionWithRoPE(torch.autograd.Function):
+    """The fused projection under autograd.  Forward: one launch (backend.qkv_rope_proj).  Backward, for the gradient
+    `g` of the [B, S, (Hq + 2 Hkv) D] result: the adjoint rotation of g's q and k heads from the same packed table
+    (backend.rope_from_table(backward=True), what ops.py:463-493 gives the separate rope op), in place of a copy of
+    g; then d hidden = g W and d W = g^T hidden as dual-GEMM launches on the row-major operands (the transposition
+    happens inside the kernel) and d bias = the column sums of g (fp32 accumulation, like nn.Linear's)."""
+
+    @staticmethod
+    def forward(ctx, hidden_states, qkv_weight, qkv_bias, rope_table, nq, nkv, D, mrope_section, layout):
+        out = backend.qkv_rope_proj(hidden_states, qkv_weight, qkv_bias, rope_table, nq, nkv, D)
+        ctx.save_for_backward(hidden_states, qkv_weight, rope_table)
+        ctx.heads = (nq, nkv, D)
+        ctx.rope = ([2 * int(v) for v in mrope_section], layout)
+        ctx.has_bias = qkv_bias is not None
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        hidden_states, weight, table = ctx.saved_tensors
+        nq, nkv, D = ctx.heads
+        doubled, layout = ctx.rope
+        B, S, H = hidden_states.shape
+        N = (nq + 2 * nkv) * D
+        g = grad_out.to(torch.bfloat16).contiguous().clone().view(B, S, N)  # rotated back in place below
+        gq = g[..., :nq * D].view(B, S, nq, D).transpose(1, 2)
+        gk = g[..., nq * D:(nq + nkv) * D].view(B, S, nkv, D).transpose(1, 2)
+        backend.rope_from_table(gq, gk, table, gq, gk, doubled, backward=True, layout=layout)
+        g2, x2 = g.view(B * S, N), hidden_states.reshape(B * S, H)
+        none = g2.new_empty((0, 0))
+        want_x, want_w, want_b = ctx.needs_input_grad[0], ctx.needs_input_grad[1], ctx.needs_input_grad[2]
+        dx = dw = db = None
+        if want_x:  # [T, N] @ [N, H]: the weight is read as stored, K-major
+            dx = torch.empty(B * S, H, dtype=torch.bfloat16, device=g.device)
+            backend.asym_dual_gmm_separated(g2, none, weight, g2.new_empty((0, H)), dx, g2.new_empty((0, H)), False, False)
+            dx = dx.view(B, S, H)
+        if want_w:  # [T, N]^T @ [T, H]: both operands K-major
+            dw = torch.empty(N, H, dtype=torch.bfloat16, device=g.device)
+            backend.asym_dual_gmm_separated(g2, none, x2, g2.new_empty((0, H)), dw, g2.new_empty((0, H)), True, False)
+        if want_b and ctx.has_bias:
+            db = g2.sum(0, dtype=torch.float32).to(torch.bfloat16)
+        return dx, dw, db, None, None, None, None, None, None
+
+
 def qkv_projection_with_rope(hidden_states, qkv_weight, qkv_bias, rope_table, num_heads, num_key_value_heads,
-                             head_dim=128):
+                             head_dim=128, mrope_section=(16, 24, 24), layout=None):
     """Not in the reference's op set: the first lines of the attention forward (vl.py:955-964) as one launch.
 
         q = q_proj(h).view(B, S, Hq, D).transpose(1, 2); k, v likewise; q, k = multimodal_rope(q, k, cos, sin, sec)
@@ -366,17 +409,29 @@ def qkv_projection_with_rope(hidden_states, qkv_weight, qkv_bias, rope_table, nu
     along the output dimension (torch.cat((q_proj.weight, k_proj.weight, v_proj.weight)), once per module);
     rope_table from multimodal_rope_table for the same tokens.  Returns (q [B, Hq, S, D], k [B, Hkv, S, D],
     v [B, Hkv, S, D]) as views of one [B, S, (Hq + 2 Hkv) D] buffer (token-major memory, what attention kernels
-    take through strides), q and k rotated.  Forward only (inference / prefill)."""
+    take through strides), q and k rotated.  The table's width tells the channel layout it was built for: D / 2
+    entries per token reproduce the eager attention class (vl.py:860-862 on the PyTorch rope, vl.py:731-773), D
+    entries the flash-attention class, whose rope op runs the CUDA kernel's layout (vl.py:962-964 on
+    csrc/rope.cu:104-117).  Differentiable in hidden_states, qkv_weight and qkv_bias; the backward rotates the
+    gradient with `mrope_section` / `layout` (the ones the table was built with; layout defaults to the one the
+    table's width implies)."""
     if hidden_states.is_cpu:
         raise RuntimeError("[Error] The input `hidden_states` of qkv_projection_with_rope op is on the device: CPU!")
     if hidden_states.dim() != 3:
         raise RuntimeError("[Error] hidden_states must be [batch, seq, hidden]")
-    if torch.is_grad_enabled() and (hidden_states.requires_grad or qkv_weight.requires_grad):
-        raise RuntimeError("qkv_projection_with_rope has no backward: use the separate projections and multimodal_rope "
-                           "under autograd")
     B, S, _ = hidden_states.shape
     D, nq, nkv = head_dim, num_heads, num_key_value_heads
-    out = backend.qkv_rope_proj(hidden_states, qkv_weight, qkv_bias, rope_table, nq, nkv, D)
+    needs_grad = torch.is_grad_enabled() and (hidden_states.requires_grad or qkv_weight.requires_grad or
+                                              (qkv_bias is not None and qkv_bias.requires_grad))
+    if needs_grad:
+        if len(mrope_section) != 3:
+            raise RuntimeError("[Error] The input `mrope_section` of multimodal_rope op must be a list of 3 integers!")
+        if layout is None:
+            layout = "hf" if rope_table.size(-1) == D // 2 else "csrc"
+        out = QkvProjectionWithRoPE.apply(hidden_states, qkv_weight, qkv_bias, rope_table, nq, nkv, D,
+                                          tuple(mrope_section), layout)
+    else:
+        out = backend.qkv_rope_proj(hidden_states, qkv_weight, qkv_bias, rope_table, nq, nkv, D)
     q, k, v = out.split([nq * D, nkv * D, nkv * D], dim=-1)
     return (q.view(B, S, nq, D).transpose(1, 2), k.view(B, S, nkv, D).transpose(1, 2),
             v.view(B, S, nkv, D).transpose(1, 2))

@@ -162,55 +162,85 @@ def _dual(a0, a1, w0, w1, n0, n1, trans_a, trans_b, want=(True, True)):
 
 
 class _MoeBlockFunction(torch.autograd.Function):
-    """permute -> both experts' SwiGLU FFN -> unpermute with a backward (act.py:105-162 under autograd).
+    """[RMSNorm ->] permute -> both experts' SwiGLU FFN -> unpermute [+ residual] with a backward (act.py:105-162,
+    and the decoder layer's lines around it, act.py:256-265, under autograd).
 
     Forward is the fused path; its gate / up launch also keeps the two projections (the reference's autograd keeps
-    them too, along with act_fn(gate) and the product, act.py:79-82).  Backward runs every remaining contraction of
-    both experts as one dual GEMM each: dHm = dY Wd, dWd = dY^T Hm, dX = dG Wg + dU Wu (the second product added onto
-    the first in its epilogue), dWg = dG^T X, dWu = dU^T X,
+    them too, along with act_fn(gate) and the product, act.py:79-82).  With a norm weight the post-attention RMSNorm
+    runs inside the permute, with `residual` the closing add inside the down launch's stores.  Backward runs every
+    remaining contraction of both experts as one dual GEMM each: dHm = dY Wd, dWd = dY^T Hm, dX = dG Wg + dU Wu (the
+    second product added onto the first in its epilogue), dWg = dG^T X, dWu = dU^T X,
     with the SwiGLU derivative (and Hm in row-major form) from one fused elementwise kernel per expert (fp32 math).
-    Intermediate sizes that are not multiples of 64 recompute the two projections instead.  The per-expert row
-    counts are read back from the device once per backward (the forward never synchronises)."""
+    The normed, sorted rows the weight gradients contract over are recomputed (one pass, where the plain block
+    permutes x), and the unpermute of dX carries the norm's backward and the residual branch's gradient (one pass,
+    which also sums the norm weight's gradient).  Intermediate sizes that are not multiples of 64 recompute the two
+    projections instead.  The per-expert row counts are read back from the device once per backward (the forward
+    never synchronises)."""
+
+    N_FIXED = 8  # inputs in front of the six weights
 
     @staticmethod
-    def forward(ctx, x, row_id_map, expert_offsets, sorted_row_id, scratch, *weights):
+    def forward(ctx, x, norm_weight, row_id_map, expert_offsets, sorted_row_id, scratch, eps, residual, *weights):
         T = x.size(0)
-        scratch["x_tiled"] = native.permute_rows_tiled(x, row_id_map, expert_offsets, scratch.get("x_tiled"),
-                                                       sorted_row_id)
+        if norm_weight is not None:
+            if sorted_row_id is None:
+                raise RuntimeError("pre_norm needs a routing with sorted_row_id (partition(..., want_sorted=True))")
+            scratch["x_tiled"] = native.rmsnorm_permute_rows_tiled(x, norm_weight, eps, expert_offsets, sorted_row_id,
+                                                                   scratch.get("x_tiled"))
+        else:
+            scratch["x_tiled"] = native.permute_rows_tiled(x, row_id_map, expert_offsets, scratch.get("x_tiled"),
+                                                           sorted_row_id)
         w = ((weights[0], weights[1], weights[2]), (weights[3], weights[4], weights[5]))
         I0, I1 = weights[0].size(0), weights[3].size(0)
         ctx.keep = I0 % 64 == 0 and I1 % 64 == 0
+        ctx.eps, ctx.residual, ctx.has_norm = eps, bool(residual), norm_weight is not None
+        ctx.has_sorted = sorted_row_id is not None
         # weights that train are repacked on every forward: writes through `.data` (master-weight or EMA copies) do
         # not move the version counter a cached copy would be checked against.  Frozen ones keep their packed copies.
-        frozen = tuple(not n for n in ctx.needs_input_grad[5:11])
+        n0 = _MoeBlockFunction.N_FIXED
+        frozen = tuple(not n for n in ctx.needs_input_grad[n0:n0 + 6])
+        res_in_stores = x if (residual and sorted_row_id is not None) else None
+        saved = [x, row_id_map, expert_offsets]
+        if ctx.has_norm:
+            saved.append(norm_weight)
+        if ctx.has_sorted:
+            saved.append(sorted_row_id)
         if ctx.keep:
             y, gate_keep, up_keep, scratch["hmid"] = native.dual_swiglu_ffn_keep(
                 scratch["x_tiled"], T, expert_offsets, w, hmid=scratch.get("hmid"), out_row_id=sorted_row_id,
-                frozen=frozen)
-            if sorted_row_id is None:
-                y = native.unpermute(y, row_id_map, torch.tensor([]), T, 1)
-            ctx.save_for_backward(x, row_id_map, expert_offsets, gate_keep, up_keep, *weights)
-            return y
-        ctx.save_for_backward(x, row_id_map, expert_offsets, *weights)
-        if sorted_row_id is not None:
-            return native.dual_swiglu_ffn(scratch["x_tiled"], T, expert_offsets, w, hmid=scratch.get("hmid"),
-                                          out_row_id=sorted_row_id, cache_packed=frozen)
-        y_sorted = native.dual_swiglu_ffn(scratch["x_tiled"], T, expert_offsets, w, hmid=scratch.get("hmid"),
-                                          cache_packed=frozen)
-        return native.unpermute(y_sorted, row_id_map, torch.tensor([]), T, 1)
+                frozen=frozen, residual=res_in_stores)
+            saved += [gate_keep, up_keep]
+        else:
+            y = native.dual_swiglu_ffn(scratch["x_tiled"], T, expert_offsets, w, hmid=scratch.get("hmid"),
+                                       out_row_id=sorted_row_id, cache_packed=frozen, residual=res_in_stores)
+        ctx.save_for_backward(*saved, *weights)
+        if sorted_row_id is None:
+            if residual:
+                return native.unpermute_add(y, x, row_id_map)
+            return native.unpermute(y, row_id_map, torch.tensor([]), T, 1)
+        return y
 
     @staticmethod
     def backward(ctx, dy):
-        if ctx.keep:
-            x, row_id_map, expert_offsets, gate_keep, up_keep, g0, u0, d0, g1, u1, d1 = ctx.saved_tensors
-        else:
-            x, row_id_map, expert_offsets, g0, u0, d0, g1, u1, d1 = ctx.saved_tensors
+        saved = list(ctx.saved_tensors)
+        x, row_id_map, expert_offsets = saved[:3]
+        del saved[:3]
+        norm_weight = saved.pop(0) if ctx.has_norm else None
+        sorted_row_id = saved.pop(0) if ctx.has_sorted else None
+        gate_keep, up_keep = (saved.pop(0), saved.pop(0)) if ctx.keep else (None, None)
+        g0, u0, d0, g1, u1, d1 = saved
         T, H = x.shape
-        need = ctx.needs_input_grad
+        n0 = _MoeBlockFunction.N_FIXED
+        need = (None,) * 5 + tuple(ctx.needs_input_grad[n0:n0 + 6])  # need[5..10]: the six weights
+        need_x, need_norm = ctx.needs_input_grad[0], ctx.has_norm and ctx.needs_input_grad[1]
         o = expert_offsets.cpu().tolist()
         m0, m1 = o[1] - o[0], o[2] - o[1]
-        xs = native.permute_rows(x.detach(), row_id_map, 1, T)
-        dys = native.permute_rows(dy.contiguous().to(torch.bfloat16), row_id_map, 1, T)
+        dy = dy.contiguous().to(torch.bfloat16)
+        if ctx.has_norm:  # the experts' input rows: normed, in sorted order
+            xs = native.rmsnorm_permute_rows(x.detach(), norm_weight.detach(), ctx.eps, sorted_row_id)
+        else:
+            xs = native.permute_rows(x.detach(), row_id_map, 1, T)
+        dys = native.permute_rows(dy, row_id_map, 1, T)
         x0, x1 = xs[:m0], xs[m0:m0 + m1]
         dy0, dy1 = dys[:m0], dys[m0:m0 + m1]
         I0, I1 = g0.size(0), g1.size(0)
@@ -235,16 +265,24 @@ class _MoeBlockFunction(torch.autograd.Function):
             grads[1], grads[4] = _dual(du0, du1, x0, x1, H, H, True, False, want=(need[6], need[9]))
         if need[7] or need[10]:  # down weights
             grads[2], grads[5] = _dual(dy0, dy1, hm0, hm1, I0, I1, True, False, want=(need[7], need[10]))
-        dx = None
-        if need[0]:
+        dx = dnorm = None
+        if need_x or need_norm:
             # dX = dG Wg + dU Wu: the second product accumulates onto the first in its epilogue (bf16 + bf16, rounded
             # once -- what the two eager ops and their add give)
             dxs = torch.empty(T, H, dtype=torch.bfloat16, device=x.device)
             d0_, d1_ = dxs[:m0], dxs[m0:m0 + m1]
             native.asym_dual_gmm(dg0, dg1, g0, g1, d0_, d1_, False, False)
             native.asym_dual_gmm(du0, du1, u0, u1, d0_, d1_, False, False, add_expert0=d0_, add_expert1=d1_)
-            dx = native.unpermute(dxs, row_id_map, torch.tensor([]), T, 1)
-        return (dx, None, None, None, None, *grads)
+            if ctx.has_norm:
+                dx, dnorm = native.unpermute_rmsnorm_bwd(dxs, x.detach(), norm_weight.detach(), ctx.eps, row_id_map,
+                                                         add=dy if ctx.residual else None)
+            elif ctx.residual:
+                dx = native.unpermute_add(dxs, dy, row_id_map)
+            else:
+                dx = native.unpermute(dxs, row_id_map, torch.tensor([]), T, 1)
+        elif ctx.residual and need_x:
+            dx = dy
+        return (dx if need_x else None, dnorm if need_norm else None, None, None, None, None, None, None, *grads)
 
 
 class SparseMoeBlock(nn.Module):
@@ -363,19 +401,17 @@ class SparseMoeBlock(nn.Module):
         return rows
 
     def _forward_training(self, x, routing, flat, pre_norm, residual):
-        # norm and residual stay PyTorch ops (autograd differentiates them), the block itself has its own backward
-        xin = x
-        if pre_norm is not None:
-            norm_weight, eps = pre_norm
-            xin = torch.nn.functional.rms_norm(x, (x.size(1),), norm_weight, eps)
+        # the norm runs inside the permute and the residual add inside the down launch's stores, as in the inference
+        # path; the autograd function's backward covers both
+        norm_weight, eps = pre_norm if pre_norm is not None else (None, 0.0)
         need = native.padded_sorted_rows(x.size(0)) * max(self._dims[1:])
         if self._hmid is None or self._hmid.numel() < need or self._hmid.device != x.device:
             self._hmid = torch.empty(need, dtype=torch.bfloat16, device=x.device)
         scratch = {"x_tiled": self._x_tiled, "hmid": self._hmid}
-        y = _MoeBlockFunction.apply(xin, routing.row_id_map, routing.expert_offsets, routing.sorted_row_id,
-                                    scratch, *flat)
+        y = _MoeBlockFunction.apply(x, norm_weight, routing.row_id_map, routing.expert_offsets,
+                                    routing.sorted_row_id, scratch, float(eps), bool(residual), *flat)
         self._x_tiled = scratch["x_tiled"]
-        return x + y if residual else y
+        return y
 
     def _forward_generic(self, x, experts_indices, start_indices, end_indices, routing, pre_norm, residual):
         """Any expert list (act.py:105-162 as written): permute -> per pair of experts the three projections as

@@ -678,11 +678,54 @@ def unpermute_add_rmsnorm(y_sorted: torch.Tensor, residual: torch.Tensor, row_id
     return out, normed
 
 
+def rmsnorm_permute_rows(x: torch.Tensor, weight: torch.Tensor, eps: float, sorted_row_id: torch.Tensor) -> torch.Tensor:
+    """weight * rmsnorm(x)[sorted_row_id]: the normed rows in expert-sorted order, row-major (one pass)."""
+    _need_cuda("x", x)
+    if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
+        raise RuntimeError("All tensors must be BFloat16 for this kernel")
+    x, weight = x.contiguous(), weight.contiguous()
+    T, H = x.shape
+    if weight.numel() != H or sorted_row_id.numel() < T or sorted_row_id.dtype != torch.int32:
+        raise RuntimeError("weight size must equal the hidden size, sorted_row_id must be int32 with one entry per row")
+    out = torch.empty_like(x)
+    with _DeviceGuard(x):
+        _lib.call("wx_rmsnorm_permute_rows", _ptr(x), _ptr(weight), float(eps), _ptr(out), _ptr(sorted_row_id), T, H,
+                  _stream(x))
+    return out
+
+
+def unpermute_rmsnorm_bwd(grad_sorted: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, eps: float,
+                          row_id_map: torch.Tensor, add: Optional[torch.Tensor] = None):
+    """Backward of `permute(weight * rmsnorm(x))` for the gradient of the sorted rows, in one pass (topK 1, bf16):
+    returns (grad_x [T, H] -- with `add`, a [T, H] gradient arriving along the residual branch, summed in -- and
+    grad_weight [H])."""
+    _need_cuda("grad_sorted", grad_sorted)
+    for t in (grad_sorted, x, weight) + ((add,) if add is not None else ()):
+        if t.dtype != torch.bfloat16:
+            raise RuntimeError("All tensors must be BFloat16 for this kernel")
+    grad_sorted, x, weight = grad_sorted.contiguous(), x.contiguous(), weight.contiguous()
+    T, H = x.shape
+    if grad_sorted.shape[1] != H or row_id_map.numel() < T or weight.numel() != H or \
+            (add is not None and tuple(add.shape) != (T, H)):
+        raise RuntimeError("shape mismatch between the sorted gradient, x, weight, add and row_id_map")
+    add = None if add is None else add.contiguous()
+    gx = torch.empty_like(x)
+    gw = torch.empty(H, dtype=torch.bfloat16, device=x.device)
+    nbytes = _lib.load().wx_rmsnorm_bwd_workspace_bytes(H)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
+    with _DeviceGuard(x):
+        _lib.call("wx_unpermute_rows_rmsnorm_bwd", _ptr(grad_sorted), _ptr(x), _ptr(weight), float(eps), _ptr(add),
+                  _ptr(gx), _ptr(gw), _ptr(row_id_map), T, H, ws.data_ptr(), nbytes, _stream(x))
+    return gx, gw
+
+
 def dual_swiglu_ffn_packed(x_tiled: torch.Tensor, num_rows: int, expert_offsets: torch.Tensor, packed, dims,
                            hmid: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
-                           host_rows=None, out_row_id: Optional[torch.Tensor] = None) -> torch.Tensor:
+                           host_rows=None, out_row_id: Optional[torch.Tensor] = None,
+                           residual: Optional[torch.Tensor] = None) -> torch.Tensor:
     """dual_swiglu_ffn on weights that are already K-tiled: packed = (gate0, up0, down0, gate1, up1, down1) from
-    pack_weight, dims = (hidden, inter0, inter1)."""
+    pack_weight, dims = (hidden, inter0, inter1).  residual (with out_row_id): a [num_rows, hidden] tensor in token
+    order added to the result in the down launch's stores."""
     _need_cuda("x_tiled", x_tiled)
     H, I0, I1 = (int(v) for v in dims)
     lib = _lib.load()
@@ -705,12 +748,30 @@ def dual_swiglu_ffn_packed(x_tiled: torch.Tensor, num_rows: int, expert_offsets:
         hmid = torch.empty(need, dtype=torch.bfloat16, device=dev)
     if out is None:
         out = torch.empty((num_rows, H), dtype=torch.bfloat16, device=dev)
+    if residual is not None:
+        _check_residual(residual, num_rows, H, dev, out_row_id)
     with _DeviceGuard(x_tiled):
-        _lib.call("wx_dual_swiglu_ffn", x_tiled.data_ptr(), _ptr(out), expert_offsets.data_ptr(), _ptr(packed[0]),
-                  _ptr(packed[1]), _ptr(packed[2]), _ptr(packed[3]), _ptr(packed[4]), _ptr(packed[5]),
-                  hmid.data_ptr(), int(num_rows), H, I0, I1, _lib.i64x2(host_rows), _ptr(out_row_id),
-                  _stream(x_tiled))
+        if residual is not None and num_rows:
+            _lib.call("wx_dual_swiglu_gate_up", x_tiled.data_ptr(), hmid.data_ptr(), expert_offsets.data_ptr(),
+                      _ptr(packed[0]), _ptr(packed[1]), _ptr(packed[3]), _ptr(packed[4]), int(num_rows), H, I0, I1,
+                      _lib.i64x2(host_rows), _stream(x_tiled))
+            _lib.call("wx_dual_down_proj_residual", hmid.data_ptr(), _ptr(out), residual.data_ptr(),
+                      expert_offsets.data_ptr(), _ptr(packed[2]), _ptr(packed[5]), int(num_rows), H, I0, I1,
+                      _lib.i64x2(host_rows), _ptr(out_row_id), _stream(x_tiled))
+        else:
+            _lib.call("wx_dual_swiglu_ffn", x_tiled.data_ptr(), _ptr(out), expert_offsets.data_ptr(), _ptr(packed[0]),
+                      _ptr(packed[1]), _ptr(packed[2]), _ptr(packed[3]), _ptr(packed[4]), _ptr(packed[5]),
+                      hmid.data_ptr(), int(num_rows), H, I0, I1, _lib.i64x2(host_rows), _ptr(out_row_id),
+                      _stream(x_tiled))
     return out
+
+
+def _check_residual(residual, num_rows, hidden, dev, out_row_id) -> None:
+    if out_row_id is None:
+        raise RuntimeError("a residual is added in token order: it needs out_row_id")
+    if residual.dtype != torch.bfloat16 or tuple(residual.shape) != (num_rows, hidden) or residual.device != dev or \
+            not residual.is_contiguous():
+        raise RuntimeError("residual must be a contiguous [num_rows, hidden] BFloat16 tensor on the activations' device")
 
 
 class HostRows:
@@ -863,7 +924,8 @@ def packed_block_forward(experts: PackedExperts, x: torch.Tensor, row_id_map: to
 
 def dual_swiglu_ffn_keep(x_tiled: torch.Tensor, num_rows: int, expert_offsets: torch.Tensor, weights,
                          hmid: Optional[torch.Tensor] = None, host_rows=None,
-                         out_row_id: Optional[torch.Tensor] = None, frozen=None):
+                         out_row_id: Optional[torch.Tensor] = None, frozen=None,
+                         residual: Optional[torch.Tensor] = None):
     """dual_swiglu_ffn for a forward pass whose backward follows: the gate / up launch also stores the two
     projections (K-tiled, the intermediate's geometry) so the backward need not run them again.  The weights are
     packed afresh (they train), except those flagged in `frozen` (six booleans in the order gate0, up0, down0, gate1,
@@ -882,12 +944,20 @@ def dual_swiglu_ffn_keep(x_tiled: torch.Tensor, num_rows: int, expert_offsets: t
     out = torch.empty((num_rows, H), dtype=torch.bfloat16, device=dev)
     if num_rows == 0:
         return out, gate_keep, up_keep, hmid
+    if residual is not None:
+        _check_residual(residual, num_rows, H, dev, out_row_id)
     with _DeviceGuard(x_tiled):
         _lib.call("wx_dual_swiglu_gate_up_keep", x_tiled.data_ptr(), hmid.data_ptr(), gate_keep.data_ptr(),
                   up_keep.data_ptr(), expert_offsets.data_ptr(), _ptr(packed[0]), _ptr(packed[1]), _ptr(packed[3]),
                   _ptr(packed[4]), int(num_rows), H, I0, I1, _lib.i64x2(host_rows), _stream(x_tiled))
-        _lib.call("wx_dual_down_proj", hmid.data_ptr(), _ptr(out), expert_offsets.data_ptr(), _ptr(packed[2]),
-                  _ptr(packed[5]), int(num_rows), H, I0, I1, _lib.i64x2(host_rows), _ptr(out_row_id), _stream(x_tiled))
+        if residual is not None:
+            _lib.call("wx_dual_down_proj_residual", hmid.data_ptr(), _ptr(out), residual.data_ptr(),
+                      expert_offsets.data_ptr(), _ptr(packed[2]), _ptr(packed[5]), int(num_rows), H, I0, I1,
+                      _lib.i64x2(host_rows), _ptr(out_row_id), _stream(x_tiled))
+        else:
+            _lib.call("wx_dual_down_proj", hmid.data_ptr(), _ptr(out), expert_offsets.data_ptr(), _ptr(packed[2]),
+                      _ptr(packed[5]), int(num_rows), H, I0, I1, _lib.i64x2(host_rows), _ptr(out_row_id),
+                      _stream(x_tiled))
     return out, gate_keep, up_keep, hmid
 
 
@@ -915,7 +985,7 @@ def swiglu_bwd_tiled(gate_keep: torch.Tensor, up_keep: torch.Tensor, elem_offset
 def dual_swiglu_ffn(x_tiled: torch.Tensor, num_rows: int, expert_offsets: torch.Tensor, weights,
                     hmid: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
                     host_rows=None, out_row_id: Optional[torch.Tensor] = None,
-                    cache_packed: bool = True) -> torch.Tensor:
+                    cache_packed: bool = True, residual: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Both experts' SwiGLU FFN over expert-sorted rows in two launches (act.py:79-82, 142-154).
 
     x_tiled: result of permute_rows_tiled for num_rows tokens; expert_offsets int32 [3] ON THE DEVICE (from
@@ -924,7 +994,8 @@ def dual_swiglu_ffn(x_tiled: torch.Tensor, num_rows: int, expert_offsets: torch.
     of expert 1) as host integers, when the caller has them
     anyway; they only spare the library a second, empty launch when it cannot tell which tile shape fits.
     out_row_id: optional int32 [num_rows] CUDA tensor, the partition's sorted_row_id; with it the result comes back
-    in token order (the unpermute happens in the down launch's stores).
+    in token order (the unpermute happens in the down launch's stores), and `residual` ([num_rows, hidden], token
+    order) is added there when given.
     Returns out [num_rows, hidden] bf16, in sorted order unless out_row_id is given.
     """
     (g0, u0, d0), (g1, u1, d1) = weights
@@ -936,4 +1007,4 @@ def dual_swiglu_ffn(x_tiled: torch.Tensor, num_rows: int, expert_offsets: torch.
     cached = tuple(cache_packed) if isinstance(cache_packed, (tuple, list)) else (bool(cache_packed),) * 6
     packed = [pack_weight(w, cache=c) for w, c in zip((g0, u0, d0, g1, u1, d1), cached)]
     return dual_swiglu_ffn_packed(x_tiled, num_rows, expert_offsets, packed, (H, I0, I1), hmid, out, host_rows,
-                                  out_row_id)
+                                  out_row_id, residual)
