@@ -588,8 +588,12 @@ def config4_measurement(dev, weights):
         with torch.no_grad():
             tb, _ = event_ms(lambda: block(x3, types2, start, end), 20, warm=5)
             tbb, _ = event_ms(lambda: block(x3, types2, start, end), 20, warm=5, batch=36)
+            # ... and by a caller that passes no CPU row ranges: the cached partition's own asynchronous read-back of
+            # expert_offsets supplies the row counts once it has landed
+            tbn, _ = event_ms(lambda: block(x3, types2), 20, warm=5, batch=36)
         out[name]["us_drop_in_block_same_token_types"] = round(tb * 1e3, 1)            # one call, GPU idle before it
         out[name]["us_per_layer_drop_in_block_36_calls_back_to_back"] = round(tbb * 1e3, 1)  # as a decoder issues them
+        out[name]["us_per_layer_drop_in_block_36_calls_without_row_ranges"] = round(tbn * 1e3, 1)
         if n_vl == 0:
             out[name]["kernels_us"] = denoise_kernel_times(dev, x, types, weights)
             # the denoise loop repeats this shape 10 x 36 times per action chunk: record 36 layers once into a HIP

@@ -193,8 +193,9 @@ def test_row_counts_reach_the_host_without_a_sync_and_captures_ignore_them(dev):
     T, n_act = 2048, 2048
     x = torch.randn(T, hidden, device=dev, generator=g).to(torch.bfloat16)
     types = torch.ones(T, dtype=torch.bool, device=dev)
-    y_first, routing = moe.moe_layer_forward(x, types, weights)  # the copy cannot be checked for yet: device decides
+    routing = moe._routing_cache.lookup(types, 2)  # what a block's forward does with its token types
     assert routing.host_rows is not None
+    y_first, _ = moe.moe_layer_forward(x, types, weights, routing=routing)  # most likely too early for the counts
     torch.cuda.synchronize()
     rows = routing.rows_when_ready()
     assert rows is not None and list(rows) == [T - n_act, n_act]
@@ -221,7 +222,8 @@ def test_row_counts_reach_the_host_without_a_sync_and_captures_ignore_them(dev):
     with torch.cuda.graph(graph):
         out_static, _ = moe.moe_layer_forward(x_static, types_static, weights, routing=static_routing)
         captured, _ = moe.moe_layer_forward(x_static, types_static, weights)
-    assert _.host_rows is None  # partitioned under capture: nothing has run, nothing to read back
+        in_capture = moe._routing_cache.lookup(types_static, 2)
+    assert in_capture.host_rows is None  # partitioned under capture: nothing has run, nothing to read back
     for n_vl in (0, 700):
         new_types = torch.ones(T, dtype=torch.bool, device=dev)
         new_types[:n_vl] = False

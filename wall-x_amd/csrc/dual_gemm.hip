@@ -71,7 +71,7 @@ struct TileShape {
   static constexpr int kLoadsB = kLoadRowsB / 16;     // ... and B
   static constexpr int kSlotBytesA = BM * kRowBytes;  // bytes of A per K step
   static constexpr int kSlotBytesB = BN * kRowBytes;
-  static constexpr int kStageBytes = FN >= 4 ? (kWaves > 4 ? 4096 : 8192) : 2048;  // per-wave staging for the epilogue
+  static constexpr int kStageBytes = FN >= 4 ? (kWaves > 4 || BM <= 128 ? 4096 : 8192) : 2048;  // per-wave staging for the epilogue
   static constexpr int kLdsBytes = kStages * (kSlotBytesA + kSlotBytesB) + kWaves * kStageBytes;
   static constexpr int kWgPerCu = kLdsBytes <= 80 * 1024 && FM * FN * 16 <= 128 ? 2 : 1;
   static_assert(kLdsBytes <= 160 * 1024, "LDS budget");
@@ -100,6 +100,11 @@ using BigTileFor = std::conditional_t<MODE == 3 || MODE == 4 /* kQkvRope, kQkvRo
 // the shape that runs the ragged last round of a launch (see tail_split_point): BigTile cut in four.  (Cut in two,
 // 256 x 128 with one workgroup per CU, measures the same.)
 using TailTile = SmallTile;
+// ... and for the projection that rotates heads: four wavefronts as 4 x 1, wave tile 32 x 128, so that a wavefront
+// still holds whole heads of 128 channels (all four load)
+using TailTileQ = TileShape<128, 128, 4, 1>;
+template <int MODE>
+using TailTileFor = std::conditional_t<MODE == 3 || MODE == 4 /* kQkvRope, kQkvRopeFull */, TailTileQ, TailTile>;
 
 constexpr int kXcds = 8;
 constexpr int kGroupM = 8;                     // tile rows per patch in the tile order
@@ -321,7 +326,7 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
   int total = tiles_m[0] * tiles_n[0] + tiles_m[1] * tiles_n[1];  // the host bounds this below 2^31
   // tail split: the first launch (256 x 256 tiles) stops at `split_at`; the second (this shape: 128 x 128)
   // takes virtual tiles [split_at, all) of the 256 x 256 tiling, kSubM x kSubN pieces each
-  constexpr bool kIsTail = std::is_same_v<TS, TailTile>, kIsBig = std::is_same_v<TS, BigTileFor<MODE>>;
+  constexpr bool kIsTail = std::is_same_v<TS, TailTileFor<MODE>>, kIsBig = std::is_same_v<TS, BigTileFor<MODE>>;
   constexpr int kSubM = BigTile::BM / BM, kSubN = BigTile::BN / BN;
   int big_m[2], big_n[2], split_at = 0, pieces = 0;
   if ((kIsBig && p.split == 1) || (kIsTail && p.split == 2)) {
@@ -1255,14 +1260,31 @@ extern "C" int wx_qkv_rope_proj(const void* x, const void* weight, const void* b
   p.rope_table = rope_table;
   p.rope_cols = (n_q_heads + n_kv_heads) * head_dim;
   p.rope_width = table_width;
-  // the large tile only: its wavefronts cover whole heads (the small tile's 64 columns would split a rotation pair)
+  // Tiles whose wavefronts cover whole heads only (a 64-column wave tile would split a rotation pair): the large
+  // tile, and for a ragged last round (see tail_split_point) a second launch of 128 x 128 tiles with 32 x 128 wave tiles
   using Tile = BigTileFor<kQkvRope>;
-  if (table_width == head_dim)
-    hipLaunchKernelGGL((dual_gemm_kernel<kQkvRopeFull, Tile, false, false>), dim3(device_cu_count()),
-                       dim3(Tile::kThreads), 0, as_stream(stream), p);
-  else
-    hipLaunchKernelGGL((dual_gemm_kernel<kQkvRope, Tile, false, false>), dim3(device_cu_count()), dim3(Tile::kThreads),
-                       0, as_stream(stream), p);
+  using Tail = TailTileFor<kQkvRope>;
+  const int cus = device_cu_count();
+  const int64_t tiles = ceil_div(num_tokens, Tile::BM) * ceil_div(n, Tile::BN);
+  const bool split = tiles < INT32_MAX && tail_split_point(static_cast<int>(tiles), 0, g.k, 0, cus) != tiles;
+  p.split = split ? 1 : 0;
+  p.split_cus = cus;
+  hipStream_t s = as_stream(stream);
+  if (table_width == head_dim) {
+    hipLaunchKernelGGL((dual_gemm_kernel<kQkvRopeFull, Tile, false, false>), dim3(cus), dim3(Tile::kThreads), 0, s, p);
+    if (split) {
+      p.split = 2;
+      hipLaunchKernelGGL((dual_gemm_kernel<kQkvRopeFull, Tail, false, false>), dim3(cus * Tail::kWgPerCu),
+                         dim3(Tail::kThreads), 0, s, p);
+    }
+  } else {
+    hipLaunchKernelGGL((dual_gemm_kernel<kQkvRope, Tile, false, false>), dim3(cus), dim3(Tile::kThreads), 0, s, p);
+    if (split) {
+      p.split = 2;
+      hipLaunchKernelGGL((dual_gemm_kernel<kQkvRope, Tail, false, false>), dim3(cus * Tail::kWgPerCu),
+                         dim3(Tail::kThreads), 0, s, p);
+    }
+  }
   return check_launch("dual_gemm_kernel<qkv_rope>");
 }
 

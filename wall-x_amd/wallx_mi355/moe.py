@@ -516,7 +516,9 @@ def moe_layer_forward(x: torch.Tensor, token_types: torch.Tensor, weights, routi
 
     x [T, H] bf16, token_types [T] (bool / int), weights ((g0,u0,d0),(g1,u1,d1)).  Returns (y [T, H], routing).
     Without `routing` the token types are partitioned on every call (pass the returned routing to the following
-    layers).  Frozen weights are packed once (see native.pack_weight for what invalidates the packed copies); the
+    layers; a caller that knows the per-expert row counts passes `host_rows` too -- unlike the block's cached
+    partition, this one starts no read-back of its own, which would cost a call that is not repeated more than it
+    saves).  Frozen weights are packed once (see native.pack_weight for what invalidates the packed copies); the
     work buffers are the per-stream pair every block shares, so `hmid` is accepted for compatibility and not used.
     """
     if routing is None:
@@ -527,8 +529,6 @@ def moe_layer_forward(x: torch.Tensor, token_types: torch.Tensor, weights, routi
         if workspace is None:
             _routing_cache.store_workspace(ws_key, ws)
         routing = Routing(row_id_map, offsets, x.size(0), inverse)
-        if ws_key[2] == 0:
-            routing.host_rows = native.HostRows(offsets, x.size(0))
     experts = _experts_for(weights)
     rows = None if host_rows is None else _lib.i64x2(host_rows)
     if routing.sorted_row_id is not None:  # the down launch stores every row at its token's position
