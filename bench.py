@@ -619,6 +619,27 @@ def config4_measurement(dev, weights):
             tg, _ = event_ms(graph.replay, 10, warm=3)
             out[name]["us_per_layer_eager_shared_routing"] = round(te * 1e3 / layers, 1)
             out[name]["us_per_layer_hip_graph_replay"] = round(tg * 1e3 / layers, 1)
+            # the same replay with an action expert of its own in every layer, as the model has them: 36 x 12.6 MB of
+            # weights no longer stay in the caches between layers, every layer streams its expert from HBM
+            (g0, u0, d0), (g1, u1, d1) = weights
+            per_layer = [((g0, u0, d0), tuple(w.clone() for w in (g1, u1, d1))) for _ in range(layers)]
+
+            def stack_distinct():
+                h = x
+                for wl_ in per_layer:
+                    h = moe.moe_layer_forward(h, types, wl_, routing=routing, host_rows=(n_vl, n_act))[0]
+                return h
+
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                stack_distinct()  # packs the 36 action experts outside the capture
+            torch.cuda.current_stream().wait_stream(side)
+            graph2 = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph2):
+                stack_distinct()
+            tg2, _ = event_ms(graph2.replay, 10, warm=3)
+            out[name]["us_per_layer_hip_graph_replay_36_distinct_action_experts"] = round(tg2 * 1e3 / layers, 1)
+            del graph2, per_layer
     return out
 
 
