@@ -377,6 +377,22 @@ int wx_unpermute_rows_rmsnorm_bwd(const void* grad_sorted, const void* x, const 
                                   int64_t num_tokens, int64_t num_cols, void* workspace, size_t workspace_bytes,
                                   wx_stream_t stream);
 
+/* One call for the block's forward as the decoder layer uses it (act.py:256-265 around act.py:105-162):
+ * [RMSNorm ->] permute into the K-tiled activations -> gate/up + SwiGLU -> down with every row stored at its token's
+ * position [+ residual].  Exactly the launches of wx_rmsnorm_permute_rows_tiled / wx_permute_rows_tiled,
+ * wx_dual_swiglu_gate_up and wx_dual_down_proj / wx_dual_down_proj_residual in that order, with their argument rules:
+ * a host that issues a layer per call (36 per forward, 360 per denoised action chunk) pays for one library call
+ * instead of three.  x, out: [num_rows, hidden] bf16 in token order; row_id_map, sorted_row_id, expert_offsets: the
+ * partition's outputs (sorted_row_id required); the six weights packed (wx_pack_tiled); x_tiled and hmid: work
+ * buffers of wx_tiled_bytes(wx_padded_sorted_rows(num_rows), hidden) bytes and wx_padded_sorted_rows(num_rows) *
+ * max(inter0, inter1) bf16; norm_weight: bf16 [hidden] or NULL (no norm); add_residual != 0 returns x + block(x). */
+int wx_moe_block_forward(const void* x, void* out, const int32_t* row_id_map, const int32_t* sorted_row_id,
+                         const int32_t* expert_offsets, const void* gate0, const void* up0, const void* down0,
+                         const void* gate1, const void* up1, const void* down1, void* x_tiled, void* hmid,
+                         int64_t num_rows, int64_t hidden, int64_t inter0, int64_t inter1,
+                         const int64_t* host_rows_per_expert, const void* norm_weight, float eps,
+                         int add_residual, wx_stream_t stream);
+
 /* Elementwise backward of h = silu(g) * u inside an expert FFN (act.py:79-82; the reference leaves it to autograd):
  * from gate, up (the two projections, kept by the forward or recomputed) and dh (gradient w.r.t. h) in one pass:
  * hmid = bf16(bf16(silu(g)) * u) as the forward fed it to the down projection, dgate = dh * u * s * (1 + g * (1 - s))

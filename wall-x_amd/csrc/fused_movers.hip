@@ -584,3 +584,29 @@ extern "C" int wx_unpermute_rows_rmsnorm_bwd(const void* grad_sorted, const void
                      static_cast<const float*>(workspace), static_cast<__bf16*>(grad_weight), blocks * 4, num_cols);
   return check_launch("column_sums_kernel");
 }
+
+extern "C" int wx_moe_block_forward(const void* x, void* out, const int32_t* row_id_map, const int32_t* sorted_row_id,
+                                    const int32_t* expert_offsets, const void* gate0, const void* up0,
+                                    const void* down0, const void* gate1, const void* up1, const void* down1,
+                                    void* x_tiled, void* hmid, int64_t num_rows, int64_t hidden, int64_t inter0,
+                                    int64_t inter1, const int64_t* host_rows_per_expert, const void* norm_weight,
+                                    float eps, int add_residual, wx_stream_t stream) {
+  const char* who = "wx_moe_block_forward";
+  if (num_rows < 0) return fail(WX_ERR_INVALID_ARGUMENT, "%s: negative row count", who);
+  if (num_rows == 0) return WX_OK;
+  if (!sorted_row_id) return fail(WX_ERR_INVALID_ARGUMENT, "%s: sorted_row_id is required", who);
+  if (int rc = norm_weight != nullptr
+                   ? wx_rmsnorm_permute_rows_tiled(x, norm_weight, eps, x_tiled, sorted_row_id, expert_offsets, num_rows,
+                                                   hidden, stream)
+                   : wx_permute_rows_tiled(x, x_tiled, row_id_map, sorted_row_id, expert_offsets, num_rows, hidden,
+                                           stream))
+    return rc;
+  if (int rc = wx_dual_swiglu_gate_up(x_tiled, hmid, expert_offsets, gate0, up0, gate1, up1, num_rows, hidden, inter0,
+                                      inter1, host_rows_per_expert, stream))
+    return rc;
+  if (add_residual)
+    return wx_dual_down_proj_residual(hmid, out, x, expert_offsets, down0, down1, num_rows, hidden, inter0, inter1,
+                                      host_rows_per_expert, sorted_row_id, stream);
+  return wx_dual_down_proj(hmid, out, expert_offsets, down0, down1, num_rows, hidden, inter0, inter1,
+                           host_rows_per_expert, sorted_row_id, stream);
+}

@@ -66,6 +66,7 @@ PROTOTYPES = {
     "wx_rmsnorm_permute_rows": (_i32, [_vp, _vp, _f32, _vp, _vp, _i64, _i64, _vp]),
     "wx_rmsnorm_bwd_workspace_bytes": (_sz, [_i64]),
     "wx_unpermute_rows_rmsnorm_bwd": (_i32, [_vp, _vp, _vp, _f32, _vp, _vp, _vp, _vp, _i64, _i64, _vp, _sz, _vp]),
+    "wx_moe_block_forward": (_i32, [_vp] * 13 + [_i64] * 4 + [_vp, _vp, _f32, _i32, _vp]),
     "wx_swiglu_bwd": (_i32, [_vp] * 6 + [_i64, _vp]),
     "wx_swiglu_bwd_tiled": (_i32, [_vp, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _vp]),
 }

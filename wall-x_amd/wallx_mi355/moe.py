@@ -99,12 +99,17 @@ class _RoutingCache(threading.local):
         self.routing = None
         self.workspace = {}  # (device, stream, capture id) -> [histograms, status word]
 
-    def lookup(self, ids: torch.Tensor, num_experts: int):
-        stream = torch.cuda.current_stream(ids.device).cuda_stream if ids.is_cuda else 0
+    def lookup(self, ids: torch.Tensor, num_experts: int, stream: Optional[int] = None, capture: Optional[int] = None):
+        """stream / capture: the current stream's handle and its capture id when the caller has looked them up already
+        (a block's forward needs both again for its work buffers)."""
+        if stream is None:
+            stream = torch.cuda.current_stream(ids.device).cuda_stream if ids.is_cuda else 0
+        if capture is None:
+            capture = native.capture_id(stream)
         # a partition recorded during a HIP graph capture has not run when the capture ends: it answers lookups of
         # that capture only (its id is part of the key; 0 outside captures)
         version = _version_of(ids)
-        key = (version, ids.shape, ids.dtype, ids.device, num_experts, stream, native.capture_id(stream))
+        key = (version, ids.shape, ids.dtype, ids.device, num_experts, stream, capture)
         if version is not None and self.ref is not None and self.ref() is ids and self.key == key:
             return self.routing
         flat = ids.reshape(-1)
@@ -360,8 +365,11 @@ class SparseMoeBlock(nn.Module):
             return self._forward_generic(x, experts_indices, start_indices, end_indices, routing, pre_norm,
                                          residual).view(batch, seq, hidden)
         host_rows = self._host_rows(start_indices, end_indices, T)
+        # the stream and its capture state, looked up once for the partition cache and the work buffers
+        stream = torch.cuda.current_stream(x.device).cuda_stream if x.is_cuda else 0
+        capture = native.capture_id(stream) if x.is_cuda else 0
         if routing is None:
-            routing = _routing_cache.lookup(experts_indices, self.num_experts)
+            routing = _routing_cache.lookup(experts_indices, self.num_experts, stream, capture)
         if routing.num_tokens != T:
             raise RuntimeError(f"routing was built for {routing.num_tokens} tokens, got {T}")
         grad = torch.is_grad_enabled()
@@ -379,7 +387,7 @@ class SparseMoeBlock(nn.Module):
             return self._forward_scatter(x, routing, experts, host_rows, pre_norm, residual).view(batch, seq, hidden)
         return native.packed_block_forward(experts, x, routing.row_id_map, routing.sorted_row_id,
                                            routing.expert_offsets, host_rows, pre_norm, residual,
-                                           routing.rows_when_ready).view(batch, seq, hidden)
+                                           routing.rows_when_ready, stream, capture).view(batch, seq, hidden)
 
     def _host_rows(self, start_indices, end_indices, num_tokens):
         """The per-expert row counts as a host int64[2] when the caller's CPU tensors give them, else None.  The

@@ -807,14 +807,15 @@ class HostRows:
 _ffn_scratch = {}  # (device index, stream handle, capturing) -> (tiled activations, intermediate, capture id)
 
 
-def _ffn_buffers(device: torch.device, stream: int, x_elems: int, h_elems: int):
+def _ffn_buffers(device: torch.device, stream: int, x_elems: int, h_elems: int, cap: Optional[int] = None):
     """The tiled-activation and intermediate buffers of the block forward, one pair per device and stream: the
     layers of a model run one after the other on a stream, so they can all work in the same two buffers (a pair per
     block would hold 0.45 GB per layer at 29 184 tokens).  Calls that overlap on one stream's pair from two threads
     race, like any two launches writing one buffer.  Under HIP graph capture the pair belongs to that capture (its
     memory comes from the graph's pool and its replays write it): eager calls never share it, and a later capture on
     the same stream replaces it."""
-    cap = capture_id(stream)
+    if cap is None:
+        cap = capture_id(stream)
     key = (device.index, stream, cap != 0)
     hit = _ffn_scratch.get(key)
     if hit is not None and hit[2] != cap:
@@ -872,13 +873,15 @@ class PackedExperts:
 
 def packed_block_forward(experts: PackedExperts, x: torch.Tensor, row_id_map: torch.Tensor,
                          sorted_row_id: torch.Tensor, expert_offsets: torch.Tensor, host_rows_c=None,
-                         pre_norm=None, residual: bool = False, rows_when_ready=None) -> torch.Tensor:
+                         pre_norm=None, residual: bool = False, rows_when_ready=None,
+                         stream: Optional[int] = None, capture: Optional[int] = None) -> torch.Tensor:
     """One block forward on packed weights, in token order: [RMSNorm ->] permute -> gate/up + SwiGLU -> down with
     the unpermute [and the residual add, + x] in its stores.  x [T, hidden] bf16; the three routing tensors are the partition's
     (int32, on x's device); host_rows_c is None or _lib.i64x2((rows of expert 0, rows of expert 1)).  Without it,
     `rows_when_ready` (a callable returning such a pair or None: the partition's own read-back of expert_offsets, see
     HostRows) is asked outside HIP graph captures; a capture always records the launches that decide on the device.
-    The work buffers are shared per stream (see _ffn_buffers); the result is a new tensor."""
+    The work buffers are shared per stream (see _ffn_buffers); the result is a new tensor.  stream / capture: x's
+    device's current stream handle and its capture id, when the caller has them already."""
     dev = x.device
     if dev != experts.device or x.dtype != torch.bfloat16 or x.dim() != 2 or x.shape[1] != experts.hidden:
         raise RuntimeError("x must be a [tokens, hidden] BFloat16 tensor on the device of the packed weights")
@@ -894,31 +897,25 @@ def packed_block_forward(experts: PackedExperts, x: torch.Tensor, row_id_map: to
     if T == 0:
         return out
     lib = _lib.load()
-    stream = torch.cuda.current_stream(dev).cuda_stream
+    if stream is None:
+        stream = torch.cuda.current_stream(dev).cuda_stream
     x_elems, h_elems = experts.sizes(T)
-    x_tiled, hmid, cap = _ffn_buffers(dev, stream, x_elems, h_elems)
+    x_tiled, hmid, cap = _ffn_buffers(dev, stream, x_elems, h_elems, capture)
     if host_rows_c is None and rows_when_ready is not None and cap == 0:
         host_rows_c = rows_when_ready()
     H, I0, I1 = experts.hidden, experts.inter0, experts.inter1
-    xt, hm, off, srt = x_tiled.data_ptr(), hmid.data_ptr(), expert_offsets.data_ptr(), sorted_row_id.data_ptr()
-    with _DeviceGuard(x):
-        if pre_norm is not None:
-            weight, eps = pre_norm
-            if weight.dtype != torch.bfloat16 or weight.numel() != H or weight.device != dev or \
-                    not weight.is_contiguous():
-                raise RuntimeError("the norm weight must be a contiguous BFloat16 tensor of the hidden size")
-            _lib.check(lib.wx_rmsnorm_permute_rows_tiled(x.data_ptr(), weight.data_ptr(), float(eps), xt, srt, off,
-                                                         T, H, stream))
-        else:
-            _lib.check(lib.wx_permute_rows_tiled(x.data_ptr(), xt, row_id_map.data_ptr(), srt, off, T, H, stream))
-        if residual:  # the add happens in the down launch's epilogue: the sorted result is never written
-            g0, u0, d0, g1, u1, d1 = experts.ptrs
-            _lib.check(lib.wx_dual_swiglu_gate_up(xt, hm, off, g0, u0, g1, u1, T, H, I0, I1, host_rows_c, stream))
-            _lib.check(lib.wx_dual_down_proj_residual(hm, out.data_ptr(), x.data_ptr(), off, d0, d1, T, H, I0, I1,
-                                                      host_rows_c, srt, stream))
-        else:
-            _lib.check(lib.wx_dual_swiglu_ffn(xt, out.data_ptr(), off, *experts.ptrs, hm, T, H, I0, I1,
-                                              host_rows_c, srt, stream))
+    norm_ptr, eps = None, 0.0
+    if pre_norm is not None:
+        weight, eps = pre_norm
+        if weight.dtype != torch.bfloat16 or weight.numel() != H or weight.device != dev or \
+                not weight.is_contiguous():
+            raise RuntimeError("the norm weight must be a contiguous BFloat16 tensor of the hidden size")
+        norm_ptr = weight.data_ptr()
+    with _DeviceGuard(x):  # one library call: [RMSNorm +] permute, gate/up, down with the unpermute [and the residual]
+        _lib.check(lib.wx_moe_block_forward(x.data_ptr(), out.data_ptr(), row_id_map.data_ptr(),
+                                            sorted_row_id.data_ptr(), expert_offsets.data_ptr(), *experts.ptrs,
+                                            x_tiled.data_ptr(), hmid.data_ptr(), T, H, I0, I1, host_rows_c, norm_ptr,
+                                            float(eps), int(bool(residual)), stream))
     return out
 
 
