@@ -159,3 +159,58 @@ def test_moe_block_with_both_fusions(dev):
         plain = h + block(oracle.rms_norm_ref(h.cpu(), w.cpu(), 1e-6).to(dev), types)
     err = (fused.float() - plain.float()).abs()
     assert not (err > 2e-2 + 1e-2 * plain.float().abs()).any(), float(err.max())
+
+
+@pytest.mark.parametrize("with_norm,with_residual", [(False, False), (True, False), (False, True), (True, True)])
+def test_block_forward_as_one_library_call_equals_its_launches(dev, with_norm, with_residual):
+    """wx_moe_block_forward through the C ABI against the entry points it is made of, called one by one on buffers of
+    their own: bit-equal, with and without the fused RMSNorm and residual add."""
+    from wallx_mi355 import _lib
+
+    g = torch.Generator().manual_seed(31)
+    T, H, I0, I1 = 700, 256, 384, 128
+    x = _bf((T, H), g, 2.0).to(dev)
+    nw = (1.0 + 0.1 * torch.randn(H, generator=g)).to(torch.bfloat16).to(dev)
+    types = (torch.rand(T, generator=g) < 0.2).to(dev)
+    ws = [(torch.randn(s, generator=g) * 0.05).to(torch.bfloat16).to(dev)
+          for s in ((I0, H), (I0, H), (H, I0), (I1, H), (I1, H), (H, I1))]
+    packed = [native.pack_weight(w, cache=False) for w in ws]
+    rmap, off, inv, _ = native.partition(types, 2, 0, None, want_sorted=True)
+    lib = _lib.load()
+    stream = torch.cuda.current_stream().cuda_stream
+    pad = native.padded_sorted_rows(T)
+    bufs = [(torch.empty(lib.wx_tiled_bytes(pad, H) // 2, dtype=torch.bfloat16, device=dev),
+             torch.empty(pad * max(I0, I1), dtype=torch.bfloat16, device=dev), torch.empty_like(x)) for _ in range(2)]
+    (xt, hm, out), (xt2, hm2, out2) = bufs
+    p = [t.data_ptr() for t in packed]
+    eps = 1e-6
+    _lib.call("wx_moe_block_forward", x.data_ptr(), out.data_ptr(), rmap.data_ptr(), inv.data_ptr(), off.data_ptr(),
+              p[0], p[1], p[2], p[3], p[4], p[5], xt.data_ptr(), hm.data_ptr(), T, H, I0, I1, None,
+              nw.data_ptr() if with_norm else None, eps, int(with_residual), stream)
+    if with_norm:
+        _lib.call("wx_rmsnorm_permute_rows_tiled", x.data_ptr(), nw.data_ptr(), eps, xt2.data_ptr(), inv.data_ptr(),
+                  off.data_ptr(), T, H, stream)
+    else:
+        _lib.call("wx_permute_rows_tiled", x.data_ptr(), xt2.data_ptr(), rmap.data_ptr(), inv.data_ptr(),
+                  off.data_ptr(), T, H, stream)
+    _lib.call("wx_dual_swiglu_gate_up", xt2.data_ptr(), hm2.data_ptr(), off.data_ptr(), p[0], p[1], p[3], p[4], T, H,
+              I0, I1, None, stream)
+    if with_residual:
+        _lib.call("wx_dual_down_proj_residual", hm2.data_ptr(), out2.data_ptr(), x.data_ptr(), off.data_ptr(), p[2],
+                  p[5], T, H, I0, I1, None, inv.data_ptr(), stream)
+    else:
+        _lib.call("wx_dual_down_proj", hm2.data_ptr(), out2.data_ptr(), off.data_ptr(), p[2], p[5], T, H, I0, I1, None,
+                  inv.data_ptr(), stream)
+    torch.cuda.synchronize()
+    assert torch.equal(out, out2)
+    # and against the oracle
+    hin = oracle.rms_norm_ref(x.cpu(), nw.cpu(), eps) if with_norm else x.cpu()
+    wc = [tuple(w.cpu() for w in ws[:3]), tuple(w.cpu() for w in ws[3:])]
+    ref = oracle.sparse_moe_block_ref(hin[None], types.cpu()[None], wc)[0].float()
+    if with_residual:
+        ref = (x.cpu().float() + ref).to(torch.bfloat16).float()
+    err = (out.cpu().float() - ref).abs()
+    assert not (err > 2e-2 + 1e-2 * ref.abs()).any(), float(err.max())
+    assert lib.wx_moe_block_forward(x.data_ptr(), out.data_ptr(), rmap.data_ptr(), None, off.data_ptr(), p[0], p[1],
+                                    p[2], p[3], p[4], p[5], xt.data_ptr(), hm.data_ptr(), T, H, I0, I1, None, None,
+                                    eps, 0, stream) == -1  # sorted_row_id is required
