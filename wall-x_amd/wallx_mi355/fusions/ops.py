@@ -359,8 +359,8 @@ def multimodal_rope_from_table(q, k, table, mrope_section, layout="hf"):
 class QkvProjectionWithRoPE(torch.autograd.Function):
     """The fused projection under autograd.  Forward: one launch (backend.qkv_rope_proj).  Backward, for the gradient
     `g` of the [B, S, (Hq + 2 Hkv) D] result: the adjoint rotation of g's q and k heads from the same packed table
-    (backend.rope_from_table(backward=True), what ops.py:463-493 gives the separate rope op), in place of a copy of
-    g; then d hidden = g W and d W = g^T hidden as dual-GEMM launches on the row-major operands (the transposition
+    (backend.rope_from_table(backward=True), what ops.py:463-493 gives the separate rope op) into a buffer of
+    g's shape, the v heads copied beside them; then d hidden = g W and d W = g^T hidden as dual-GEMM launches on the row-major operands (the transposition
     happens inside the kernel) and d bias = the column sums of g (fp32 accumulation, like nn.Linear's)."""
 
     @staticmethod
@@ -379,10 +379,15 @@ class QkvProjectionWithRoPE(torch.autograd.Function):
         doubled, layout = ctx.rope
         B, S, H = hidden_states.shape
         N = (nq + 2 * nkv) * D
-        g = grad_out.to(torch.bfloat16).contiguous().clone().view(B, S, N)  # rotated back in place below
-        gq = g[..., :nq * D].view(B, S, nq, D).transpose(1, 2)
-        gk = g[..., nq * D:(nq + nkv) * D].view(B, S, nkv, D).transpose(1, 2)
-        backend.rope_from_table(gq, gk, table, gq, gk, doubled, backward=True, layout=layout)
+        go = grad_out.to(torch.bfloat16).contiguous().view(B, S, N)
+        g = torch.empty_like(go)  # the gradient w.r.t. the projection's own output: q and k heads rotated back, v as is
+
+        def heads(t, first, count):
+            return t[..., first * D:(first + count) * D].view(B, S, count, D).transpose(1, 2)
+
+        backend.rope_from_table(heads(go, 0, nq), heads(go, nq, nkv), table, heads(g, 0, nq), heads(g, nq, nkv), doubled,
+                                backward=True, layout=layout)
+        g[..., (nq + nkv) * D:].copy_(go[..., (nq + nkv) * D:])
         g2, x2 = g.view(B * S, N), hidden_states.reshape(B * S, H)
         none = g2.new_empty((0, 0))
         want_x, want_w, want_b = ctx.needs_input_grad[0], ctx.needs_input_grad[1], ctx.needs_input_grad[2]
