@@ -251,19 +251,40 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
   static_assert(MODE == kGeneric || (!KA && !KB), "K-major operands exist in the generic mode only");
   // kStages ring slots per operand, each one K step (256 rows x 32 bf16).  Separate arrays let the compiler
   // see that a read of one slot never waits for a buffer load that targets another.
-  __shared__ __attribute__((aligned(1024))) unsigned char s_a0[kSlotBytesA];
-  __shared__ __attribute__((aligned(1024))) unsigned char s_a1[kSlotBytesA];
-  __shared__ __attribute__((aligned(1024))) unsigned char s_a2[kSlotBytesA];
-  __shared__ __attribute__((aligned(1024))) unsigned char s_b0[kSlotBytesB];
-  __shared__ __attribute__((aligned(1024))) unsigned char s_b1[kSlotBytesB];
-  __shared__ __attribute__((aligned(1024))) unsigned char s_b2[kSlotBytesB];
-  __shared__ __attribute__((aligned(1024))) unsigned char s_a3[kSlotBytesA];
-  __shared__ __attribute__((aligned(1024))) unsigned char s_b3[kSlotBytesB];
+  // Row-major operands with K contiguous (the NT layout of the generic mode): the ring's slots live in PAIRS.  A load instruction then fetches 8 rows x 128 bytes -- the K chunks of two consecutive K steps,
+  // i.e. whole cache lines -- where one slot's worth would be 16 rows x 64 bytes (sixteen half lines, which hold the
+  // loading wavefront's issue slot about twice as long).  A pair is one array of 1 KiB blocks, block = 8 rows x
+  // [512 bytes of the even step | 512 bytes of the odd step], so the instruction's 64 lanes land on consecutive LDS
+  // addresses; inside a step's half, rows are 64 bytes with the same chunk swizzle as everywhere else.
+  // (The projection that rotates heads reads row-major operands too and keeps the slot-by-slot ring: with pairs its
+  // launches measured 3 % slower inside a forward pass.)
+  constexpr bool kPair = MODE == kGeneric && !KA && !KB;
+  constexpr int kRingA = kPair ? 16 : kSlotBytesA, kRingB = kPair ? 16 : kSlotBytesB;  // the form not in use shrinks
+  constexpr int kPairA = kPair ? 2 * kSlotBytesA : 16, kPairB = kPair ? 2 * kSlotBytesB : 16;
+  constexpr int kRingAlign = kPair ? 16 : 1024, kPairAlign = kPair ? 1024 : 16;
+  __shared__ __attribute__((aligned(kRingAlign))) unsigned char s_a0[kRingA];
+  __shared__ __attribute__((aligned(kRingAlign))) unsigned char s_a1[kRingA];
+  __shared__ __attribute__((aligned(kRingAlign))) unsigned char s_a2[kRingA];
+  __shared__ __attribute__((aligned(kRingAlign))) unsigned char s_b0[kRingB];
+  __shared__ __attribute__((aligned(kRingAlign))) unsigned char s_b1[kRingB];
+  __shared__ __attribute__((aligned(kRingAlign))) unsigned char s_b2[kRingB];
+  __shared__ __attribute__((aligned(kRingAlign))) unsigned char s_a3[kRingA];
+  __shared__ __attribute__((aligned(kRingAlign))) unsigned char s_b3[kRingB];
+  __shared__ __attribute__((aligned(kPairAlign))) unsigned char s_pa0[kPairA];  // slots 0 and 1 of A
+  __shared__ __attribute__((aligned(kPairAlign))) unsigned char s_pa1[kPairA];  // slots 2 and 3
+  __shared__ __attribute__((aligned(kPairAlign))) unsigned char s_pb0[kPairB];
+  __shared__ __attribute__((aligned(kPairAlign))) unsigned char s_pb1[kPairB];
   __shared__ __attribute__((aligned(1024))) unsigned char s_out[kWaves * kStageBytes];
   // ring slot s of each operand (s is a constant after unrolling)
   static_assert(kStages == 4, "ring slots are declared one by one");
-  auto slot_a = [&](int s) -> unsigned char* { return s == 0 ? s_a0 : (s == 1 ? s_a1 : (s == 2 ? s_a2 : s_a3)); };
-  auto slot_b = [&](int s) -> unsigned char* { return s == 0 ? s_b0 : (s == 1 ? s_b1 : (s == 2 ? s_b2 : s_b3)); };
+  auto slot_a = [&](int s) -> unsigned char* {
+    if constexpr (kPair) return (s < 2 ? s_pa0 : s_pa1) + (s & 1) * 512;
+    else return s == 0 ? s_a0 : (s == 1 ? s_a1 : (s == 2 ? s_a2 : s_a3));
+  };
+  auto slot_b = [&](int s) -> unsigned char* {
+    if constexpr (kPair) return (s < 2 ? s_pb0 : s_pb1) + (s & 1) * 512;
+    else return s == 0 ? s_b0 : (s == 1 ? s_b1 : (s == 2 ? s_b2 : s_b3));
+  };
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keeps descriptors and LDS bases scalar
@@ -359,6 +380,18 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
 #pragma unroll
   for (int kk = 0; kk < 2; ++kk) frag_off[kk] = ((2 * kk + lhi) ^ sw) << 4;
   const int a_row_off = (wm * (FM * 32) + l32) * kRowBytes;
+  // paired slots: row r of a step's half sits at block r / 8 (1 KiB each), row r % 8 inside it
+  const int pair_lane_off = ((l32 >> 3) << 10) + ((l32 & 7) << 6);
+  const int a_pair_off = wm * (FM * 32) * 128 + pair_lane_off;
+  // paired loader: lane -> (row lane / 4 % 8 of the instruction's 8 rows, step half lane / 32, slot lane % 4)
+  constexpr int kPairLoadsA = kLoadRowsA / 8, kPairLoadsB = kLoadRowsB / 8;
+  const int pl_row = (lane >> 2) & 7, pl_half = lane >> 5, pl_slot = lane & 3;
+  // K chunk (of the 8 in a 128-byte line) this lane fetches in instruction i: the instruction's rows are 8 i + pl_row
+  // past a multiple of 32, and the slot holds chunk slot ^ ((row >> 2) & 3) of its step -- one value for even i, one
+  // for odd i, so a lane's byte offsets are two bases plus i times the (uniform) pitch of 8 rows
+  const int pair_chunk_even = 4 * pl_half + (pl_slot ^ ((pl_row >> 2) & 3));
+  const int pair_chunk_odd = 4 * pl_half + (pl_slot ^ (((pl_row >> 2) + 2) & 3));
+  auto pair_chunk = [&](int i) { return (i & 1) ? pair_chunk_odd : pair_chunk_even; };
   // B fragment j of this wave starts at LDS row b_row(j): plain tiles hold 256 weight rows; SwiGLU tiles hold 128
   // gate rows then the 128 up rows of the same output columns, and fragments [0, FN/2) are gate, [FN/2, FN) up
   auto b_row = [&](int j) {
@@ -383,7 +416,8 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
   struct Loader {   // where this wave's kLoadsA + kLoadsB loads per K step come from
     const __bf16 *a_base, *b_base;
     uint32_t a_bytes, b_bytes;        // readable bytes from the base (row-major) / from the current block (tiled)
-    uint32_t voff_a[kLoadsA], voff_b[kLoadsB];
+    uint32_t voff_a[kPair ? 2 : kLoadsA], voff_b[kPair ? 2 : kLoadsB];  // paired slots: [even i, odd i] of instruction 0
+    uint32_t pitch8_a, pitch8_b;      // paired slots: bytes between the rows of consecutive load instructions
     int64_t a_step, b_step;           // tiled: bytes between consecutive K steps
     // tiled: the load stream walks a tile's K steps in order, so the step's base and the bytes readable from it are
     // kept as running values (one add and one saturating subtract per step) instead of products with the step index
@@ -488,8 +522,15 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
       } else {
         L.a_base = G.a + static_cast<int64_t>(row0) * G.lda;
         L.a_bytes = static_cast<uint32_t>(rows_a) * G.lda * 2u;
+        if constexpr (kPair) {
+          const uint32_t row_off = static_cast<uint32_t>(wave * kLoadRowsA + pl_row) * G.lda * 2u;
+          L.voff_a[0] = row_off + pair_chunk_even * 16u;
+          L.voff_a[1] = row_off + pair_chunk_odd * 16u;
+          L.pitch8_a = 16u * static_cast<uint32_t>(G.lda);
+        } else {
 #pragma unroll
-        for (int i = 0; i < kLoadsA; ++i) L.voff_a[i] = static_cast<uint32_t>(ld_row0 + 16 * i) * G.lda * 2u + ld_chunk * 16u;
+          for (int i = 0; i < kLoadsA; ++i) L.voff_a[i] = static_cast<uint32_t>(ld_row0 + 16 * i) * G.lda * 2u + ld_chunk * 16u;
+        }
       }
       if constexpr (KB) {
         L.b_base = b_src + col0;
@@ -501,9 +542,16 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
       } else {
         L.b_base = b_src + static_cast<int64_t>(col0) * G.ldb;
         L.b_bytes = static_cast<uint32_t>(rows_b) * G.ldb * 2u;
-        const int b_ld_row0 = b_wave * kLoadRowsB + (lane >> 2);
+        if constexpr (kPair) {
+          const uint32_t row_off = static_cast<uint32_t>(b_wave * kLoadRowsB + pl_row) * G.ldb * 2u;
+          L.voff_b[0] = row_off + pair_chunk_even * 16u;
+          L.voff_b[1] = row_off + pair_chunk_odd * 16u;
+          L.pitch8_b = 16u * static_cast<uint32_t>(G.ldb);
+        } else {
+          const int b_ld_row0 = b_wave * kLoadRowsB + (lane >> 2);
 #pragma unroll
-        for (int i = 0; i < kLoadsB; ++i) L.voff_b[i] = static_cast<uint32_t>(b_ld_row0 + 16 * i) * G.ldb * 2u + ld_chunk * 16u;
+          for (int i = 0; i < kLoadsB; ++i) L.voff_b[i] = static_cast<uint32_t>(b_ld_row0 + 16 * i) * G.ldb * 2u + ld_chunk * 16u;
+        }
       }
     }
   };
@@ -514,7 +562,34 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
   // `Pending` carries what the B half needs across that gap, which may include a change of tile.
   struct Pending {
     __amdgpu_buffer_rsrc_t rb;
-    uint32_t voff_b[kLoadsB];
+    uint32_t voff_b[kPair ? 2 : kLoadsB];
+    uint32_t pitch8_b;  // paired slots
+  };
+  // Paired slots: the loads of K steps ks and ks + 1 (ks even) of this wave's rows, A here and B through `Pending`.
+  auto issue_pair_a = [&](Loader& L, int ks, unsigned char* pa, Pending& P) {
+    const int k0 = ks * BK;
+    const uint32_t adv = 2u * static_cast<uint32_t>(k0);
+    // as in issue_a: the base advances along K and keeps the absolute end of the readable range, so rows past the
+    // matrix read as zero; K chunks at or past the row end are pushed out of range lane by lane
+    const __amdgpu_buffer_rsrc_t ra = make_rsrc(L.a_base + k0, L.a_bytes > adv ? L.a_bytes - adv : 0u);
+    P.rb = make_rsrc(L.b_base + k0, L.b_bytes > adv ? L.b_bytes - adv : 0u);
+    const bool k_tail = k0 + 2 * BK > L.K;
+    const uint32_t oob_even = (k_tail && k0 + pair_chunk_even * 8 >= L.K) ? 0x80000000u : 0u;
+    const uint32_t oob_odd = (k_tail && k0 + pair_chunk_odd * 8 >= L.K) ? 0x80000000u : 0u;
+    P.voff_b[0] = L.voff_b[0] | oob_even;
+    P.voff_b[1] = L.voff_b[1] | oob_odd;
+    P.pitch8_b = L.pitch8_b;
+    const uint32_t va_even = L.voff_a[0] | oob_even, va_odd = L.voff_a[1] | oob_odd;
+#pragma unroll
+    for (int i = 0; i < kPairLoadsA; ++i)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, LDS_PTR(pa + (wave * kPairLoadsA + i) * 1024), 16,
+                                               ((i & 1) ? va_odd : va_even) + static_cast<uint32_t>(i) * L.pitch8_a, 0, 0, 0);
+  };
+  auto issue_pair_b = [&](const Pending& P, unsigned char* pb) {
+#pragma unroll
+    for (int i = 0; i < kPairLoadsB; ++i)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(P.rb, LDS_PTR(pb + (wave * kPairLoadsB + i) * 1024), 16,
+                                               P.voff_b[i & 1] + static_cast<uint32_t>(i) * P.pitch8_b, 0, 0, 0);
   };
   auto issue_a = [&](Loader& L, int ks, unsigned char* sa, Pending& P) {
     __amdgpu_buffer_rsrc_t ra;
@@ -581,10 +656,12 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
   };
   auto read_a = [&](const unsigned char* sa, int i, int kk) {
     if constexpr (KA) return read_k_major(sa, tr_base_a, BM * 2, i, kk);
+    else if constexpr (kPair) return *reinterpret_cast<const bf16x8*>(sa + a_pair_off + i * 32 * 128 + frag_off[kk]);
     else return *reinterpret_cast<const bf16x8*>(sa + a_row_off + i * 32 * kRowBytes + frag_off[kk]);
   };
   auto read_b = [&](const unsigned char* sb, int j, int kk) {
     if constexpr (KB) return read_k_major(sb, tr_base_b, BN * 2, j, kk);
+    else if constexpr (kPair) return *reinterpret_cast<const bf16x8*>(sb + b_row(j) * 128 + pair_lane_off + frag_off[kk]);
     else return *reinterpret_cast<const bf16x8*>(sb + b_row(j) * kRowBytes + b_lane_off + frag_off[kk]);
   };
   auto read_frags = [&](const unsigned char* sa, const unsigned char* sb, int kk, int set) {
@@ -659,6 +736,60 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
     read_frags(sa_n, sb_n, 0, 0);
     mma(1);
     schedule_after_barrier(with_loads);
+  };
+  // The same step on paired slots (step S of a ring round; slots 0, 1 are pair 0, slots 2, 3 pair 1).  A pair is
+  // free once its odd slot has been read, i.e. after the barrier of steps 1 and 3: its A refill (the K steps one ring
+  // round ahead) goes out there, its B refill at the start of the following step, and everything must have landed
+  // by the barrier two steps on, which is the only load still in flight then -- the counted wait becomes vmcnt(0) on
+  // odd steps and none on even ones.
+  auto schedule_pair = [&](auto n_before, auto n_after) {
+    constexpr int kB = decltype(n_before)::value, kA = decltype(n_after)::value;
+    constexpr int kMfma = FM * FN, kReads = FM + FN;
+    (void)kA;
+    constexpr int kCarry = kMfma / 2;
+    constexpr int kReadsPer = (kReads + kCarry - 1) / kCarry;
+    constexpr int kBd = kB > 0 ? kB : 1;
+    constexpr int kLoadEvery = kCarry / kBd > 0 ? kCarry / kBd : 1;
+    constexpr int kLoadsPer = kB > kCarry ? (kB + kCarry - 1) / kCarry : 1;
+#pragma unroll
+    for (int m = 0; m < kCarry; ++m) {
+      __builtin_amdgcn_sched_group_barrier(0x100, kReadsPer, 0);
+      if (kB > 0 && m % kLoadEvery == 0 && m / kLoadEvery * kLoadsPer < kB) __builtin_amdgcn_sched_group_barrier(0x020, kLoadsPer, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, kMfma - kCarry, 0);
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  auto schedule_pair_after = [&](auto n_after) {
+    constexpr int kA = decltype(n_after)::value;
+    constexpr int kMfma = FM * FN, kReads = FM + FN;
+    constexpr int kReadEvery = kMfma / kReads > 0 ? kMfma / kReads : 1;
+    constexpr int kReadsPer = kReads * kReadEvery > kMfma ? (kReads + kMfma - 1) / kMfma : 1;
+    constexpr int kAd = kA > 0 ? kA : 1;
+    constexpr int kLoadEvery = kMfma / kAd > 0 ? kMfma / kAd : 1;
+    constexpr int kLoadsPer = kA > kMfma ? (kA + kMfma - 1) / kMfma : 1;
+#pragma unroll
+    for (int m = 0; m < kMfma; ++m) {
+      if (kA > 0 && m % kLoadEvery == 0 && m / kLoadEvery * kLoadsPer < kA) __builtin_amdgcn_sched_group_barrier(0x020, kLoadsPer, 0);
+      if (m % kReadEvery == 0 && m / kReadEvery * kReadsPer < kReads) __builtin_amdgcn_sched_group_barrier(0x100, kReadsPer, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  auto k_step_pair = [&](auto with_loads, auto step_c, Loader& L, int ld_ks) {
+    constexpr bool LD = decltype(with_loads)::value;
+    constexpr int S = decltype(step_c)::value;
+    constexpr bool kOdd = (S & 1) != 0;
+    read_frags(slot_a(S), slot_b(S), 1, 1);
+    if constexpr (LD && !kOdd) issue_pair_b(pend, S == 0 ? s_pb1 : s_pb0);
+    mma(0);
+    schedule_pair(std::integral_constant<int, (LD && !kOdd) ? kPairLoadsB : 0>{}, std::integral_constant<int, 0>{});
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm((LD && kOdd) ? 0 : 63, 0));
+    barrier_no_fence();
+    if constexpr (LD && kOdd) issue_pair_a(L, ld_ks + (S == 1 ? 0 : 2), S == 1 ? s_pa0 : s_pa1, pend);
+    read_frags(slot_a((S + 1) % kStages), slot_b((S + 1) % kStages), 0, 0);
+    mma(1);
+    schedule_pair_after(std::integral_constant<int, (LD && kOdd) ? kPairLoadsA : 0>{});
   };
   // ---- epilogue ------------------------------------------------------------------------------------------
   // Accumulator register r of lane l holds row 8*(r/4) + 4*(l/32) + r%4, column l%32 of its 32x32 block.  Values
@@ -941,7 +1072,13 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
     Store S;
     if constexpr (LD) setup_loader(tc, L);
     setup_store(tc, S);
-    if constexpr (LD) {
+    if constexpr (LD && kPair) {
+      issue_pair_a(L, 0, s_pa0, pend);
+      issue_pair_b(pend, s_pb0);
+      issue_pair_a(L, 2, s_pa1, pend);  // this pair's B half goes out in the first K step
+      // pair 0 must be complete before its first fragments are read: pair 1's A half may remain in flight
+      __builtin_amdgcn_s_waitcnt(waitcnt_imm(kPairLoadsA, 15));
+    } else if constexpr (LD) {
 #pragma unroll
       for (int s = 0; s < kStages; ++s) {
         issue_a(L, s, slot_a(s), pend);
@@ -951,7 +1088,7 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
       __builtin_amdgcn_s_waitcnt(waitcnt_imm((kStages - 2) * kLoadsPerStep + kLoadsA, 15));
     }
     __syncthreads();
-    read_frags(s_a0, s_b0, 0, 0);
+    read_frags(slot_a(0), slot_b(0), 0, 0);
 
     while (have) {
 #pragma unroll
@@ -977,10 +1114,17 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
           }
           ld_ks = 0;
         }
+        if constexpr (kPair) {
+          k_step_pair(with_loads, std::integral_constant<int, 0>{}, L, ld_ks);
+          k_step_pair(with_loads, std::integral_constant<int, 1>{}, L, ld_ks);
+          k_step_pair(with_loads, std::integral_constant<int, 2>{}, L, ld_ks);
+          k_step_pair(with_loads, std::integral_constant<int, 3>{}, L, ld_ks);
+        } else {
 #pragma unroll
-        for (int s = 0; s < kStages; ++s)
-          k_step_as(with_loads, L, ld_ks + s, slot_a(s), slot_b(s), slot_a((s + 1) % kStages), slot_b((s + 1) % kStages),
-                    slot_b((s + kStages - 1) % kStages));
+          for (int s = 0; s < kStages; ++s)
+            k_step_as(with_loads, L, ld_ks + s, slot_a(s), slot_b(s), slot_a((s + 1) % kStages), slot_b((s + 1) % kStages),
+                      slot_b((s + kStages - 1) % kStages));
+        }
       }
       epilogue(done);
     }
