@@ -259,30 +259,34 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
   // (The projection that rotates heads reads row-major operands too and keeps the slot-by-slot ring: with pairs its
   // launches measured 3 % slower inside a forward pass.)
   constexpr bool kPair = MODE == kGeneric && !KA && !KB;
-  constexpr int kRingA = kPair ? 16 : kSlotBytesA, kRingB = kPair ? 16 : kSlotBytesB;  // the form not in use shrinks
-  constexpr int kPairA = kPair ? 2 * kSlotBytesA : 16, kPairB = kPair ? 2 * kSlotBytesB : 16;
-  constexpr int kRingAlign = kPair ? 16 : 1024, kPairAlign = kPair ? 1024 : 16;
-  __shared__ __attribute__((aligned(kRingAlign))) unsigned char s_a0[kRingA];
-  __shared__ __attribute__((aligned(kRingAlign))) unsigned char s_a1[kRingA];
-  __shared__ __attribute__((aligned(kRingAlign))) unsigned char s_a2[kRingA];
-  __shared__ __attribute__((aligned(kRingAlign))) unsigned char s_b0[kRingB];
-  __shared__ __attribute__((aligned(kRingAlign))) unsigned char s_b1[kRingB];
-  __shared__ __attribute__((aligned(kRingAlign))) unsigned char s_b2[kRingB];
-  __shared__ __attribute__((aligned(kRingAlign))) unsigned char s_a3[kRingA];
-  __shared__ __attribute__((aligned(kRingAlign))) unsigned char s_b3[kRingB];
-  __shared__ __attribute__((aligned(kPairAlign))) unsigned char s_pa0[kPairA];  // slots 0 and 1 of A
-  __shared__ __attribute__((aligned(kPairAlign))) unsigned char s_pa1[kPairA];  // slots 2 and 3
-  __shared__ __attribute__((aligned(kPairAlign))) unsigned char s_pb0[kPairB];
-  __shared__ __attribute__((aligned(kPairAlign))) unsigned char s_pb1[kPairB];
+  // NN (a row-major A beside a K-major B: dX, dHm, the op's default layout): A alone lives in pairs, B keeps its slots
+  constexpr bool kPairAOnly = MODE == kGeneric && !KA && KB;
+  constexpr bool kPA = kPair || kPairAOnly, kPB = kPair;
+  constexpr int kRingA = kPA ? 16 : kSlotBytesA, kRingB = kPB ? 16 : kSlotBytesB;  // the form not in use shrinks
+  constexpr int kPairA = kPA ? 2 * kSlotBytesA : 16, kPairB = kPB ? 2 * kSlotBytesB : 16;
+  constexpr int kRingAlignA = kPA ? 16 : 1024, kPairAlignA = kPA ? 1024 : 16;
+  constexpr int kRingAlignB = kPB ? 16 : 1024, kPairAlignB = kPB ? 1024 : 16;
+  __shared__ __attribute__((aligned(kRingAlignA))) unsigned char s_a0[kRingA];
+  __shared__ __attribute__((aligned(kRingAlignA))) unsigned char s_a1[kRingA];
+  __shared__ __attribute__((aligned(kRingAlignA))) unsigned char s_a2[kRingA];
+  __shared__ __attribute__((aligned(kRingAlignB))) unsigned char s_b0[kRingB];
+  __shared__ __attribute__((aligned(kRingAlignB))) unsigned char s_b1[kRingB];
+  __shared__ __attribute__((aligned(kRingAlignB))) unsigned char s_b2[kRingB];
+  __shared__ __attribute__((aligned(kRingAlignA))) unsigned char s_a3[kRingA];
+  __shared__ __attribute__((aligned(kRingAlignB))) unsigned char s_b3[kRingB];
+  __shared__ __attribute__((aligned(kPairAlignA))) unsigned char s_pa0[kPairA];  // slots 0 and 1 of A
+  __shared__ __attribute__((aligned(kPairAlignA))) unsigned char s_pa1[kPairA];  // slots 2 and 3
+  __shared__ __attribute__((aligned(kPairAlignB))) unsigned char s_pb0[kPairB];
+  __shared__ __attribute__((aligned(kPairAlignB))) unsigned char s_pb1[kPairB];
   __shared__ __attribute__((aligned(1024))) unsigned char s_out[kWaves * kStageBytes];
   // ring slot s of each operand (s is a constant after unrolling)
   static_assert(kStages == 4, "ring slots are declared one by one");
   auto slot_a = [&](int s) -> unsigned char* {
-    if constexpr (kPair) return (s < 2 ? s_pa0 : s_pa1) + (s & 1) * 512;
+    if constexpr (kPA) return (s < 2 ? s_pa0 : s_pa1) + (s & 1) * 512;
     else return s == 0 ? s_a0 : (s == 1 ? s_a1 : (s == 2 ? s_a2 : s_a3));
   };
   auto slot_b = [&](int s) -> unsigned char* {
-    if constexpr (kPair) return (s < 2 ? s_pb0 : s_pb1) + (s & 1) * 512;
+    if constexpr (kPB) return (s < 2 ? s_pb0 : s_pb1) + (s & 1) * 512;
     else return s == 0 ? s_b0 : (s == 1 ? s_b1 : (s == 2 ? s_b2 : s_b3));
   };
 
@@ -416,7 +420,7 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
   struct Loader {   // where this wave's kLoadsA + kLoadsB loads per K step come from
     const __bf16 *a_base, *b_base;
     uint32_t a_bytes, b_bytes;        // readable bytes from the base (row-major) / from the current block (tiled)
-    uint32_t voff_a[kPair ? 2 : kLoadsA], voff_b[kPair ? 2 : kLoadsB];  // paired slots: [even i, odd i] of instruction 0
+    uint32_t voff_a[kPA ? 2 : kLoadsA], voff_b[kPB ? 2 : kLoadsB];  // paired slots: [even i, odd i] of instruction 0
     uint32_t pitch8_a, pitch8_b;      // paired slots: bytes between the rows of consecutive load instructions
     int64_t a_step, b_step;           // tiled: bytes between consecutive K steps
     // tiled: the load stream walks a tile's K steps in order, so the step's base and the bytes readable from it are
@@ -522,7 +526,7 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
       } else {
         L.a_base = G.a + static_cast<int64_t>(row0) * G.lda;
         L.a_bytes = static_cast<uint32_t>(rows_a) * G.lda * 2u;
-        if constexpr (kPair) {
+        if constexpr (kPA) {
           const uint32_t row_off = static_cast<uint32_t>(wave * kLoadRowsA + pl_row) * G.lda * 2u;
           L.voff_a[0] = row_off + pair_chunk_even * 16u;
           L.voff_a[1] = row_off + pair_chunk_odd * 16u;
@@ -562,7 +566,7 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
   // `Pending` carries what the B half needs across that gap, which may include a change of tile.
   struct Pending {
     __amdgpu_buffer_rsrc_t rb;
-    uint32_t voff_b[kPair ? 2 : kLoadsB];
+    uint32_t voff_b[kPB ? 2 : kLoadsB];
     uint32_t pitch8_b;  // paired slots
   };
   // Paired slots: the loads of K steps ks and ks + 1 (ks even) of this wave's rows, A here and B through `Pending`.
@@ -572,13 +576,15 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
     // as in issue_a: the base advances along K and keeps the absolute end of the readable range, so rows past the
     // matrix read as zero; K chunks at or past the row end are pushed out of range lane by lane
     const __amdgpu_buffer_rsrc_t ra = make_rsrc(L.a_base + k0, L.a_bytes > adv ? L.a_bytes - adv : 0u);
-    P.rb = make_rsrc(L.b_base + k0, L.b_bytes > adv ? L.b_bytes - adv : 0u);
     const bool k_tail = k0 + 2 * BK > L.K;
     const uint32_t oob_even = (k_tail && k0 + pair_chunk_even * 8 >= L.K) ? 0x80000000u : 0u;
     const uint32_t oob_odd = (k_tail && k0 + pair_chunk_odd * 8 >= L.K) ? 0x80000000u : 0u;
-    P.voff_b[0] = L.voff_b[0] | oob_even;
-    P.voff_b[1] = L.voff_b[1] | oob_odd;
-    P.pitch8_b = L.pitch8_b;
+    if constexpr (kPB) {
+      P.rb = make_rsrc(L.b_base + k0, L.b_bytes > adv ? L.b_bytes - adv : 0u);
+      P.voff_b[0] = L.voff_b[0] | oob_even;
+      P.voff_b[1] = L.voff_b[1] | oob_odd;
+      P.pitch8_b = L.pitch8_b;
+    }
     const uint32_t va_even = L.voff_a[0] | oob_even, va_odd = L.voff_a[1] | oob_odd;
 #pragma unroll
     for (int i = 0; i < kPairLoadsA; ++i)
@@ -627,12 +633,16 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
       oob = (k_tail && k0 + ld_chunk * 8 >= L.K) ? 0x80000000u : 0u;
     }
     const uint32_t oob_a = KA ? 0u : oob, oob_b = KB ? 0u : oob;
+    if constexpr (!kPB) {
 #pragma unroll
-    for (int i = 0; i < kLoadsB; ++i) P.voff_b[i] = L.voff_b[i] | oob_b;
+      for (int i = 0; i < kLoadsB; ++i) P.voff_b[i] = L.voff_b[i] | oob_b;
+    }
+    if constexpr (!kPA) {  // (A in pairs: this call only prepares the step's B descriptor)
 #pragma unroll
-    for (int i = 0; i < kLoadsA; ++i)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, LDS_PTR(sa + (wave * kLoadRowsA + 16 * i) * kRowBytes), 16,
-                                               L.voff_a[i] | oob_a, 0, 0, 0);
+      for (int i = 0; i < kLoadsA; ++i)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, LDS_PTR(sa + (wave * kLoadRowsA + 16 * i) * kRowBytes), 16,
+                                                 L.voff_a[i] | oob_a, 0, 0, 0);
+    }
   };
   auto issue_b = [&](const Pending& P, unsigned char* sb) {
 #pragma unroll
@@ -656,12 +666,12 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
   };
   auto read_a = [&](const unsigned char* sa, int i, int kk) {
     if constexpr (KA) return read_k_major(sa, tr_base_a, BM * 2, i, kk);
-    else if constexpr (kPair) return *reinterpret_cast<const bf16x8*>(sa + a_pair_off + i * 32 * 128 + frag_off[kk]);
+    else if constexpr (kPA) return *reinterpret_cast<const bf16x8*>(sa + a_pair_off + i * 32 * 128 + frag_off[kk]);
     else return *reinterpret_cast<const bf16x8*>(sa + a_row_off + i * 32 * kRowBytes + frag_off[kk]);
   };
   auto read_b = [&](const unsigned char* sb, int j, int kk) {
     if constexpr (KB) return read_k_major(sb, tr_base_b, BN * 2, j, kk);
-    else if constexpr (kPair) return *reinterpret_cast<const bf16x8*>(sb + b_row(j) * 128 + pair_lane_off + frag_off[kk]);
+    else if constexpr (kPB) return *reinterpret_cast<const bf16x8*>(sb + b_row(j) * 128 + pair_lane_off + frag_off[kk]);
     else return *reinterpret_cast<const bf16x8*>(sb + b_row(j) * kRowBytes + b_lane_off + frag_off[kk]);
   };
   auto read_frags = [&](const unsigned char* sa, const unsigned char* sb, int kk, int set) {
@@ -762,7 +772,7 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
   };
   auto schedule_pair_after = [&](auto n_after) {
     constexpr int kA = decltype(n_after)::value;
-    constexpr int kMfma = FM * FN, kReads = FM + FN;
+    constexpr int kMfma = FM * FN, kReads = FM * (KA ? 2 : 1) + FN * (KB ? 2 : 1);
     constexpr int kReadEvery = kMfma / kReads > 0 ? kMfma / kReads : 1;
     constexpr int kReadsPer = kReads * kReadEvery > kMfma ? (kReads + kMfma - 1) / kMfma : 1;
     constexpr int kAd = kA > 0 ? kA : 1;
@@ -787,6 +797,28 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
     __builtin_amdgcn_s_waitcnt(waitcnt_imm((LD && kOdd) ? 0 : 63, 0));
     barrier_no_fence();
     if constexpr (LD && kOdd) issue_pair_a(L, ld_ks + (S == 1 ? 0 : 2), S == 1 ? s_pa0 : s_pa1, pend);
+    read_frags(slot_a((S + 1) % kStages), slot_b((S + 1) % kStages), 0, 0);
+    mma(1);
+    schedule_pair_after(std::integral_constant<int, (LD && kOdd) ? kPairLoadsA : 0>{});
+  };
+  // ... and with A alone in pairs (NN).  B keeps the slot-by-slot schedule of k_step_as (the refill of slot S - 1 at
+  // the start of step S, its descriptor prepared after the barrier of step S - 1), A the pairs' (after the barrier of
+  // odd steps).  In flight behind what the barrier of step S needs: the B refills of the two youngest steps, and on
+  // even steps the A pair issued one step ago as well.
+  auto k_step_mixed = [&](auto with_loads, auto step_c, Loader& L, int ld_ks) {
+    constexpr bool LD = decltype(with_loads)::value;
+    constexpr int S = decltype(step_c)::value;
+    constexpr bool kOdd = (S & 1) != 0;
+    read_frags(slot_a(S), slot_b(S), 1, 1);
+    if constexpr (LD) issue_b(pend, slot_b((S + kStages - 1) % kStages));
+    mma(0);
+    schedule_before_barrier(with_loads);
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(LD ? (kOdd ? 2 * kLoadsB : 2 * kLoadsB + kPairLoadsA) : 63, 0));
+    barrier_no_fence();
+    if constexpr (LD) {
+      issue_a(L, ld_ks + S, nullptr, pend);
+      if constexpr (kOdd) issue_pair_a(L, ld_ks + S - 1, S == 1 ? s_pa0 : s_pa1, pend);
+    }
     read_frags(slot_a((S + 1) % kStages), slot_b((S + 1) % kStages), 0, 0);
     mma(1);
     schedule_pair_after(std::integral_constant<int, (LD && kOdd) ? kPairLoadsA : 0>{});
@@ -1078,6 +1110,20 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
       issue_pair_a(L, 2, s_pa1, pend);  // this pair's B half goes out in the first K step
       // pair 0 must be complete before its first fragments are read: pair 1's A half may remain in flight
       __builtin_amdgcn_s_waitcnt(waitcnt_imm(kPairLoadsA, 15));
+    } else if constexpr (LD && kPairAOnly) {
+      // in the order the steps keep: A's first pair, B's slots 0 and 1, A's second pair, B's slot 2 (slot 3 goes out in
+      // the first K step)
+      issue_a(L, 0, nullptr, pend);
+      issue_pair_a(L, 0, s_pa0, pend);
+      issue_b(pend, slot_b(0));
+      issue_a(L, 1, nullptr, pend);
+      issue_b(pend, slot_b(1));
+      issue_pair_a(L, 2, s_pa1, pend);
+      issue_a(L, 2, nullptr, pend);
+      issue_b(pend, slot_b(2));
+      issue_a(L, 3, nullptr, pend);
+      // slot 0 of both operands must be complete: everything behind B's slot 0 may remain in flight
+      __builtin_amdgcn_s_waitcnt(waitcnt_imm(2 * kLoadsB + kPairLoadsA, 15));
     } else if constexpr (LD) {
 #pragma unroll
       for (int s = 0; s < kStages; ++s) {
@@ -1114,7 +1160,12 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
           }
           ld_ks = 0;
         }
-        if constexpr (kPair) {
+        if constexpr (kPairAOnly) {
+          k_step_mixed(with_loads, std::integral_constant<int, 0>{}, L, ld_ks);
+          k_step_mixed(with_loads, std::integral_constant<int, 1>{}, L, ld_ks);
+          k_step_mixed(with_loads, std::integral_constant<int, 2>{}, L, ld_ks);
+          k_step_mixed(with_loads, std::integral_constant<int, 3>{}, L, ld_ks);
+        } else if constexpr (kPair) {
           k_step_pair(with_loads, std::integral_constant<int, 0>{}, L, ld_ks);
           k_step_pair(with_loads, std::integral_constant<int, 1>{}, L, ld_ks);
           k_step_pair(with_loads, std::integral_constant<int, 2>{}, L, ld_ks);
