@@ -186,7 +186,7 @@ def test_block_forward_as_one_library_call_equals_its_launches(dev, with_norm, w
     eps = 1e-6
     _lib.call("wx_moe_block_forward", x.data_ptr(), out.data_ptr(), rmap.data_ptr(), inv.data_ptr(), off.data_ptr(),
               p[0], p[1], p[2], p[3], p[4], p[5], xt.data_ptr(), hm.data_ptr(), T, H, I0, I1, None,
-              nw.data_ptr() if with_norm else None, eps, int(with_residual), stream)
+              nw.data_ptr() if with_norm else None, eps, int(with_residual), None, stream)
     if with_norm:
         _lib.call("wx_rmsnorm_permute_rows_tiled", x.data_ptr(), nw.data_ptr(), eps, xt2.data_ptr(), inv.data_ptr(),
                   off.data_ptr(), T, H, stream)
@@ -213,4 +213,4 @@ def test_block_forward_as_one_library_call_equals_its_launches(dev, with_norm, w
     assert not (err > 2e-2 + 1e-2 * ref.abs()).any(), float(err.max())
     assert lib.wx_moe_block_forward(x.data_ptr(), out.data_ptr(), rmap.data_ptr(), None, off.data_ptr(), p[0], p[1],
                                     p[2], p[3], p[4], p[5], xt.data_ptr(), hm.data_ptr(), T, H, I0, I1, None, None,
-                                    eps, 0, stream) == -1  # sorted_row_id is required
+                                    eps, 0, None, stream) == -1  # sorted_row_id is required

@@ -235,10 +235,40 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
   return __builtin_bit_cast(uint32_t, v);
 }
 
+// One LDS array per (size, alignment, index).
+template <int BYTES, int ALIGN, int ID>
+__device__ __forceinline__ unsigned char* lds_array() {
+  __shared__ __attribute__((aligned(ALIGN))) unsigned char s[BYTES];
+  return s;
+}
+
+// The fused FFN launch: gate/up tiles (producers) and down tiles (consumers) in one grid.  A down tile of row block
+// rb reads the intermediate rows that the gate/up tiles of the same row block write, so it waits until `ready[rb]`
+// has reached the number of those tiles.  Workgroups are dispatched in index order and the producers come first, so
+// a consumer only ever waits for workgroups that are already running and never wait themselves; its wait is bounded
+// all the same (kFusedSpinLimit polls, then `*error` is set and the tile goes ahead).  The last consumer past the
+// wait of a row block clears its two counters, so a launch leaves the workspace as it found it: all zero.
+constexpr int kFusedMaxRowBlocks = 256;   // 128-row blocks per expert
+constexpr int kFusedSpinLimit = 1 << 20;
+constexpr int kFusedCounterStride = 64;   // ints between two counters: 256 bytes, so that the polls of different row
+                                          // blocks (and the producers' increments) spread over the memory channels
+struct FusedSync {
+  int* ready;     // [2 * kFusedMaxRowBlocks] x stride: gate/up tiles finished, by expert and row block
+  int* passed;    // [2 * kFusedMaxRowBlocks] x stride: down tiles past their wait
+  int* error;     // set to 1 when a wait ran into its bound
+  int need[2];    // gate/up tiles per row block of expert e
+  int consumers;  // down tiles per row block
+};
+
 // KA / KB (generic mode only): the operand is stored with K as its slow dimension -- A as [k, m], B as [k, n] --
 // and is transposed on the way from LDS to the MFMA registers.
-template <int MODE, typename TS, bool KA = false, bool KB = false>
-__global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(Params p) {
+//
+// The kernel's body is a function of its own so that one launch can run two of them side by side (the fused FFN
+// launch below: some workgroups run the gate/up form, the others the down form).  `wg` of `n_wg` is the workgroup's
+// place among those that share this body's tile list (blockIdx.x of gridDim.x in a plain launch).
+// ROLE: 0 = a plain launch; 1 / 2 = producer / consumer of a fused launch (see FusedSync).
+template <int MODE, typename TS, bool KA, bool KB, int ROLE>
+__device__ __forceinline__ void dual_gemm_body(const Params& p, const int wg, const int n_wg, const FusedSync& fs) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stub; the body uses gfx950-only builtins
   constexpr int BM = TS::BM, BN = TS::BN, FM = TS::FM, FN = TS::FN;
   constexpr int kWavesN = TS::kWavesN, kWaves = TS::kWaves;
@@ -266,19 +296,21 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
   constexpr int kPairA = kPA ? 2 * kSlotBytesA : 16, kPairB = kPB ? 2 * kSlotBytesB : 16;
   constexpr int kRingAlignA = kPA ? 16 : 1024, kPairAlignA = kPA ? 1024 : 16;
   constexpr int kRingAlignB = kPB ? 16 : 1024, kPairAlignB = kPB ? 1024 : 16;
-  __shared__ __attribute__((aligned(kRingAlignA))) unsigned char s_a0[kRingA];
-  __shared__ __attribute__((aligned(kRingAlignA))) unsigned char s_a1[kRingA];
-  __shared__ __attribute__((aligned(kRingAlignA))) unsigned char s_a2[kRingA];
-  __shared__ __attribute__((aligned(kRingAlignB))) unsigned char s_b0[kRingB];
-  __shared__ __attribute__((aligned(kRingAlignB))) unsigned char s_b1[kRingB];
-  __shared__ __attribute__((aligned(kRingAlignB))) unsigned char s_b2[kRingB];
-  __shared__ __attribute__((aligned(kRingAlignA))) unsigned char s_a3[kRingA];
-  __shared__ __attribute__((aligned(kRingAlignB))) unsigned char s_b3[kRingB];
-  __shared__ __attribute__((aligned(kPairAlignA))) unsigned char s_pa0[kPairA];  // slots 0 and 1 of A
-  __shared__ __attribute__((aligned(kPairAlignA))) unsigned char s_pa1[kPairA];  // slots 2 and 3
-  __shared__ __attribute__((aligned(kPairAlignB))) unsigned char s_pb0[kPairB];
-  __shared__ __attribute__((aligned(kPairAlignB))) unsigned char s_pb1[kPairB];
-  __shared__ __attribute__((aligned(1024))) unsigned char s_out[kWaves * kStageBytes];
+  // (one LDS object per (size, alignment, index): the two bodies of a fused launch name the same objects, so the
+  // launch needs the LDS of one of them)
+  unsigned char* const s_a0 = lds_array<kRingA, kRingAlignA, 0>();
+  unsigned char* const s_a1 = lds_array<kRingA, kRingAlignA, 1>();
+  unsigned char* const s_a2 = lds_array<kRingA, kRingAlignA, 2>();
+  unsigned char* const s_b0 = lds_array<kRingB, kRingAlignB, 3>();
+  unsigned char* const s_b1 = lds_array<kRingB, kRingAlignB, 4>();
+  unsigned char* const s_b2 = lds_array<kRingB, kRingAlignB, 5>();
+  unsigned char* const s_a3 = lds_array<kRingA, kRingAlignA, 6>();
+  unsigned char* const s_b3 = lds_array<kRingB, kRingAlignB, 7>();
+  unsigned char* const s_pa0 = lds_array<kPairA, kPairAlignA, 8>();  // slots 0 and 1 of A
+  unsigned char* const s_pa1 = lds_array<kPairA, kPairAlignA, 9>();  // slots 2 and 3
+  unsigned char* const s_pb0 = lds_array<kPairB, kPairAlignB, 10>();
+  unsigned char* const s_pb1 = lds_array<kPairB, kPairAlignB, 11>();
+  unsigned char* const s_out = lds_array<kWaves * kStageBytes, 1024, 12>();
   // ring slot s of each operand (s is a constant after unrolling)
   static_assert(kStages == 4, "ring slots are declared one by one");
   auto slot_a = [&](int s) -> unsigned char* {
@@ -436,6 +468,7 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
                             // an addend: its element under c_base; else null
     int rows, cols_left, ldc, nk;
     int row0, col0;         // first row / column of the tile inside its group's output
+    int row_block;          // fused launch: index of the tile's (expert, row block) counters
   };
 
   // K steps of a tile rounded up to whole ring rounds (padding steps read zeros).  The host never launches this
@@ -466,6 +499,7 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
     S.cols_left = G.n - col0;
     S.row0 = row0;
     S.col0 = col0;
+    S.row_block = tc.group * kFusedMaxRowBlocks + tc.tm;
     S.ldc = G.ldc;
     S.nk = padded_steps(G.k);
   };
@@ -649,6 +683,59 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
     for (int i = 0; i < kLoadsB; ++i)
       __builtin_amdgcn_raw_ptr_buffer_load_lds(P.rb, LDS_PTR(sb + (wave * kLoadRowsB + 16 * i) * kRowBytes), 16,
                                                P.voff_b[i], 0, 0, 0);
+  };
+
+  // Fused launch, consumer: the B half of K step `s` of a tile that has not started yet (s < kStages), leaving the
+  // loader's running values alone.
+  auto issue_b_ahead = [&](const Loader& L, int s, unsigned char* sb) {
+    uint32_t left = L.b_left;
+    for (int i = 0; i < s; ++i)
+      if (left != 0x7fffff00u) left = left > L.b_dec ? left - L.b_dec : 0u;
+    Pending P;
+    P.rb = make_rsrc(L.b_cur + s * L.b_step, s * BK < L.K ? left : 0u);
+#pragma unroll
+    for (int i = 0; i < kLoadsB; ++i) P.voff_b[i] = L.voff_b[i];
+    issue_b(P, sb);
+  };
+  // Fused launch, producer: this workgroup's tile of row block `rb` is in memory (its stores are write-through and
+  // every wavefront has waited for its own before the barrier); one lane counts the tile.
+  auto signal_consumers = [&](int rb) {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
+    __syncthreads();
+    if (tid == 0)
+      __hip_atomic_fetch_add(fs.ready + rb * kFusedCounterStride, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  };
+  // Fused launch, consumer: wait (bounded) until the producers of row block `rb` have all counted themselves.
+  // No cache is invalidated afterwards: the launch began with clean caches, and no line of a row block's
+  // intermediate is read anywhere before that row block is complete (its 1 KiB blocks belong to one producer tile
+  // each), so no cache can hold an older version of it.
+  int passed_before = 0;  // consumers of the row block that were past their wait before this one
+  auto wait_for_producers = [&](int rb, int group) {
+    if (tid == 0) {
+      const int need = fs.need[group];
+      const int* flag = fs.ready + rb * kFusedCounterStride;
+      int polls = 0;
+      while (__hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < need) {
+        if (++polls > kFusedSpinLimit) {
+          __hip_atomic_store(fs.error, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          break;
+        }
+        __builtin_amdgcn_s_sleep(2);
+      }
+      // counted here, looked at when the tile is done: the answer travels while the tile is computed
+      passed_before = __hip_atomic_fetch_add(fs.passed + rb * kFusedCounterStride, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    barrier_no_fence();  // (no wait for the counter's answer here)
+  };
+  // ... and once its tile is done: the consumer that was the last of its row block to get past the wait (the
+  // producers are done and every other consumer is past its wait as well) leaves the row block's counters at zero
+  // for the next launch
+  auto leave_row_block = [&](int rb) {
+    if (tid == 0 && passed_before == fs.consumers - 1) {
+      __hip_atomic_store(fs.ready + rb * kFusedCounterStride, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(fs.passed + rb * kFusedCounterStride, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
   };
 
   f32x16 acc[FM][FN];
@@ -906,7 +993,13 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
               if (col < S.cols_left) {
                 unsigned char* dst = reinterpret_cast<unsigned char*>(S.c_base) + keep_off[what] +
                                      ((static_cast<int64_t>(col / kBlkCols) * S.ldc + row / kBlkRows) << 10);
-                *reinterpret_cast<u32x4*>(dst + lane_e * 16) = v;
+                if constexpr (ROLE == 1) {
+                  // fused launch: written through to memory (agent-scope store), so that the tile is visible to
+                  // the other XCDs once the stores have completed, without a write-back of this XCD's L2
+                  __builtin_amdgcn_raw_buffer_store_b128(v, make_rsrc(dst, kBlkBytes), lane_e * 16, 0, 16 /* sc1 */);
+                } else {
+                  *reinterpret_cast<u32x4*>(dst + lane_e * 16) = v;
+                }
               }
             }
           }
@@ -1076,11 +1169,11 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
   // the next tile's data lands while this tile's results are stored.  After the last tile the stream continues
   // with an empty descriptor (every load out of range, nothing fetched), which keeps the in-flight accounting
   // of the waits uniform.
-  int next_t = blockIdx.x;
+  int next_t = wg;
   auto next_tile = [&](TileCoord& tc) {
     bool have = false;
     if (kIsTail && p.split == 2) {
-      for (; next_t < pieces && !have; next_t += gridDim.x) {
+      for (; next_t < pieces && !have; next_t += n_wg) {
         const int piece = next_t % (kSubM * kSubN);
         tile_coords(split_at + next_t / (kSubM * kSubN), big_m, big_n, tc);
         tc.tm = kSubM * tc.tm + piece / kSubN;
@@ -1090,7 +1183,7 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
       }
       return have;
     }
-    for (; next_t < padded && !have; next_t += gridDim.x) have = map_tile(next_t, total, tiles_m, tiles_n, tc);
+    for (; next_t < padded && !have; next_t += n_wg) have = map_tile(next_t, total, tiles_m, tiles_n, tc);
     return have;
   };
   TileCoord tc;
@@ -1104,7 +1197,25 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
     Store S;
     if constexpr (LD) setup_loader(tc, L);
     setup_store(tc, S);
-    if constexpr (LD && kPair) {
+    // Consumer of a fused launch: every tile starts from an empty ring.  The weights of the first ring slots are
+    // fetched at once, the intermediate only after the row block's producers have finished; then the ring is as the
+    // plain prologue leaves it (the last slot's B half goes out in the first K step), with every load landed.
+    auto consumer_prologue = [&]() {
+      static_assert(ROLE != 2 || TILED_IN, "the fused launch runs the tiled forms");
+      if constexpr (LD) {
+#pragma unroll
+        for (int s = 0; s + 1 < kStages; ++s) issue_b_ahead(L, s, slot_b(s));
+      }
+      wait_for_producers(S.row_block, tc.group);
+      if constexpr (LD) {
+#pragma unroll
+        for (int s = 0; s < kStages; ++s) issue_a(L, s, slot_a(s), pend);
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));
+      }
+    };
+    if constexpr (ROLE == 2) {
+      consumer_prologue();
+    } else if constexpr (LD && kPair) {
       issue_pair_a(L, 0, s_pa0, pend);
       issue_pair_b(pend, s_pb0);
       issue_pair_a(L, 2, s_pa1, pend);  // this pair's B half goes out in the first K step
@@ -1149,7 +1260,8 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
       for (int ks = 0; ks < nk; ks += kStages) {
         int ld_ks = ks + kStages;
         if (ld_ks == nk) {  // the loader moves on to the next tile (or to the empty descriptor)
-          have = next_tile(tc);
+          // (a consumer of a fused launch lets the ring run empty: its next tile has a wait of its own in front)
+          have = ROLE == 2 ? false : next_tile(tc);
           if (have) {
             if constexpr (LD) setup_loader(tc, L);
             setup_store(tc, S);
@@ -1178,6 +1290,18 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
         }
       }
       epilogue(done);
+      if constexpr (ROLE == 1) signal_consumers(done.row_block);
+      if constexpr (ROLE == 2) {
+        leave_row_block(done.row_block);
+        have = next_tile(tc);
+        if (have) {  // (one tile per consumer unless the host's row counts were not the device's)
+          if constexpr (LD) setup_loader(tc, L);
+          setup_store(tc, S);
+          consumer_prologue();
+          __syncthreads();
+          read_frags(slot_a(0), slot_b(0), 0, 0);
+        }
+      }
     }
   };
   if constexpr (!ASYM) {
@@ -1187,6 +1311,22 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
     else run(std::false_type{});
   }
 #endif
+}
+
+template <int MODE, typename TS, bool KA = false, bool KB = false>
+__global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(Params p) {
+  dual_gemm_body<MODE, TS, KA, KB, 0>(p, blockIdx.x, gridDim.x, FusedSync{});
+}
+
+// The fused FFN launch (see FusedSync): workgroups [0, producers) run the gate/up form on `pg`, the rest the down
+// form on `pd`, both in the small tile shape.  `producers` is a multiple of 8, so a workgroup's index among its
+// form's workgroups names the same XCD as its index in the grid.
+__global__ __launch_bounds__(SmallTile::kThreads, SmallTile::kWgPerCu) void ffn_fused_kernel(Params pg, Params pd,
+                                                                                             FusedSync fs,
+                                                                                             int producers) {
+  const int wg = blockIdx.x;
+  if (wg < producers) dual_gemm_body<kGateUp, SmallTile, false, false, 1>(pg, wg, producers, fs);
+  else dual_gemm_body<kDown, SmallTile, false, false, 2>(pd, wg - producers, static_cast<int>(gridDim.x) - producers, fs);
 }
 
 // ---- plain FMA tiles: any transpose combination, any k --------------------------------------------------------
@@ -1543,7 +1683,7 @@ int check_ffn(const char* who, const FfnArgs& a, bool need_gate_up, bool need_do
 }
 
 // hmid_e = silu(x_e @ gate_e^T) * (x_e @ up_e^T), K-tiled per expert
-int launch_gate_up(const FfnArgs& a, hipStream_t s) {
+Params gate_up_params(const FfnArgs& a) {
   Params p{};
   for (int e = 0; e < 2; ++e) {
     Group& g = p.g[e];
@@ -1560,6 +1700,11 @@ int launch_gate_up(const FfnArgs& a, hipStream_t s) {
   p.offsets = a.offsets;
   p.keep_gate = static_cast<__bf16*>(a.keep_gate);
   p.keep_up = static_cast<__bf16*>(a.keep_up);
+  return p;
+}
+
+int launch_gate_up(const FfnArgs& a, hipStream_t s) {
+  const Params p = gate_up_params(a);
   const int64_t t0 = ceil_div(a.inter[0], BigTile::BN / 2), t1 = ceil_div(a.inter[1], BigTile::BN / 2);
   if (a.host_rows != nullptr) {  // the caller knows the split: one launch of the right tile shape
     const int64_t by_expert[2] = {ceil_div(a.host_rows[0], BigTile::BM) * t0, ceil_div(a.host_rows[1], BigTile::BM) * t1};
@@ -1573,7 +1718,7 @@ int launch_gate_up(const FfnArgs& a, hipStream_t s) {
 }
 
 // out_e = hmid_e @ down_e^T, row-major, expert e's rows start at offsets[e]
-int launch_down(const FfnArgs& a, hipStream_t s) {
+Params down_params(const FfnArgs& a) {
   Params p{};
   for (int e = 0; e < 2; ++e) {
     Group& g = p.g[e];
@@ -1590,6 +1735,11 @@ int launch_down(const FfnArgs& a, hipStream_t s) {
   p.offsets = a.offsets;
   p.scatter = a.out_row_id;
   p.residual = static_cast<const __bf16*>(a.residual);
+  return p;
+}
+
+int launch_down(const FfnArgs& a, hipStream_t s) {
+  const Params p = down_params(a);
   const int64_t col_tiles = ceil_div(a.hidden, BigTile::BN);
   if (a.host_rows != nullptr) {
     const int64_t by_expert[2] = {ceil_div(a.host_rows[0], BigTile::BM) * col_tiles, ceil_div(a.host_rows[1], BigTile::BM) * col_tiles};
@@ -1600,7 +1750,66 @@ int launch_down(const FfnArgs& a, hipStream_t s) {
   return launch_mfma<kDown>(p, row_tiles * col_tiles, (row_tiles + 1) * col_tiles, s, "dual_gemm_kernel<down>");
 }
 
+// Both launches as one (ffn_fused_kernel), for the shapes where each is a single round of small tiles with the row
+// counts known on the host -- a denoise step.  Returns 1 when the shape is not of that kind (nothing launched).
+constexpr size_t kFusedWorkspaceInts = 4 * kFusedMaxRowBlocks * kFusedCounterStride + 1;  // ready, passed, then the error flag
+int launch_ffn_fused(const FfnArgs& a, int* ws, hipStream_t s) {
+  if (a.host_rows == nullptr || ws == nullptr || a.keep_gate != nullptr) return 1;
+  // (whatever the real split of the rows: the counters hold this many row blocks per expert)
+  if (a.rows > static_cast<int64_t>(kFusedMaxRowBlocks) * SmallTile::BM) return 1;
+  const int cus = device_cu_count();
+  int64_t gate_tiles = 0, down_tiles = 0;
+  int need[2] = {0, 0};
+  const int64_t down_cols = ceil_div(a.hidden, SmallTile::BN);
+  for (int e = 0; e < 2; ++e) {
+    const int64_t row_blocks = ceil_div(a.host_rows[e], SmallTile::BM);
+    need[e] = static_cast<int>(ceil_div(a.inter[e], SmallTile::BN / 2));
+    gate_tiles += row_blocks * need[e];
+    down_tiles += row_blocks * down_cols;
+  }
+  if (gate_tiles == 0 || gate_tiles > cus || down_tiles > cus) return 1;
+  Params pg = gate_up_params(a), pd = down_params(a);
+  pg.gate = pd.gate = 0;
+  pg.split = pd.split = 0;
+  FusedSync fs{};
+  fs.ready = ws;
+  fs.passed = ws + 2 * kFusedMaxRowBlocks * kFusedCounterStride;
+  fs.error = ws + 4 * kFusedMaxRowBlocks * kFusedCounterStride;
+  fs.need[0] = need[0];
+  fs.need[1] = need[1];
+  fs.consumers = static_cast<int>(down_cols);
+  const int producers = static_cast<int>((gate_tiles + kXcds - 1) / kXcds * kXcds);
+  const int consumers = static_cast<int>((down_tiles + kXcds - 1) / kXcds * kXcds);
+  hipLaunchKernelGGL(ffn_fused_kernel, dim3(producers + consumers), dim3(SmallTile::kThreads), 0, s, pg, pd, fs, producers);
+  return check_launch("ffn_fused_kernel");
+}
+
 }  // namespace
+
+extern "C" size_t wx_ffn_fused_workspace_bytes(void) { return kFusedWorkspaceInts * sizeof(int); }
+
+extern "C" int wx_dual_swiglu_ffn_fused(const void* x_tiled, void* out, const void* residual,
+                                        const int32_t* expert_offsets, const void* gate0, const void* up0,
+                                        const void* down0, const void* gate1, const void* up1, const void* down1,
+                                        void* hmid, int64_t num_rows, int64_t hidden, int64_t inter0, int64_t inter1,
+                                        const int64_t* host_rows_per_expert, const int32_t* out_row_id,
+                                        void* workspace, wx_stream_t stream) {
+  const char* who = "wx_dual_swiglu_ffn_fused";
+  FfnArgs a{x_tiled, {gate0, gate1}, {up0, up1}, {down0, down1}, out, hmid, host_rows_per_expert, expert_offsets,
+            num_rows, hidden, {inter0, inter1}, out_row_id};
+  if (int rc = check_ffn(who, a, true, true)) return rc;
+  if (num_rows == 0) return WX_OK;
+  if (residual != nullptr) {
+    if (!out_row_id) return fail(WX_ERR_INVALID_ARGUMENT, "%s: a residual needs out_row_id (the sum is formed in token order)", who);
+    if (reinterpret_cast<uintptr_t>(residual) & 15) return fail(WX_ERR_INVALID_ARGUMENT, "%s: residual must be 16-byte aligned", who);
+    a.residual = residual;
+  }
+  if (reinterpret_cast<uintptr_t>(workspace) & 3) return fail(WX_ERR_INVALID_ARGUMENT, "%s: workspace must be 4-byte aligned", who);
+  const int rc = launch_ffn_fused(a, static_cast<int*>(workspace), as_stream(stream));
+  if (rc <= 0) return rc;
+  if (int rc2 = launch_gate_up(a, as_stream(stream))) return rc2;
+  return launch_down(a, as_stream(stream));
+}
 
 extern "C" int wx_dual_swiglu_gate_up(const void* x_tiled, void* hmid, const int32_t* expert_offsets,
                                       const void* gate0, const void* up0, const void* gate1, const void* up1,

@@ -590,7 +590,7 @@ extern "C" int wx_moe_block_forward(const void* x, void* out, const int32_t* row
                                     const void* down0, const void* gate1, const void* up1, const void* down1,
                                     void* x_tiled, void* hmid, int64_t num_rows, int64_t hidden, int64_t inter0,
                                     int64_t inter1, const int64_t* host_rows_per_expert, const void* norm_weight,
-                                    float eps, int add_residual, wx_stream_t stream) {
+                                    float eps, int add_residual, void* ffn_workspace, wx_stream_t stream) {
   const char* who = "wx_moe_block_forward";
   if (num_rows < 0) return fail(WX_ERR_INVALID_ARGUMENT, "%s: negative row count", who);
   if (num_rows == 0) return WX_OK;
@@ -601,6 +601,10 @@ extern "C" int wx_moe_block_forward(const void* x, void* out, const int32_t* row
                    : wx_permute_rows_tiled(x, x_tiled, row_id_map, sorted_row_id, expert_offsets, num_rows, hidden,
                                            stream))
     return rc;
+  if (ffn_workspace != nullptr)  // one launch for both GEMMs where the shape allows it, else the two below
+    return wx_dual_swiglu_ffn_fused(x_tiled, out, add_residual ? x : nullptr, expert_offsets, gate0, up0, down0, gate1,
+                                    up1, down1, hmid, num_rows, hidden, inter0, inter1, host_rows_per_expert,
+                                    sorted_row_id, ffn_workspace, stream);
   if (int rc = wx_dual_swiglu_gate_up(x_tiled, hmid, expert_offsets, gate0, up0, gate1, up1, num_rows, hidden, inter0,
                                       inter1, host_rows_per_expert, stream))
     return rc;

@@ -40,6 +40,8 @@ PROTOTYPES = {
     "wx_pack_tiled": (_i32, [_vp, _vp, _i64, _i64, _vp]),
     "wx_permute_rows_tiled": (_i32, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _vp]),
     "wx_dual_swiglu_ffn": (_i32, [_vp] * 10 + [_i64] * 4 + [_vp, _vp, _vp]),
+    "wx_ffn_fused_workspace_bytes": (_sz, []),
+    "wx_dual_swiglu_ffn_fused": (_i32, [_vp] * 11 + [_i64] * 4 + [_vp, _vp, _vp, _vp]),
     "wx_dual_swiglu_gate_up": (_i32, [_vp] * 7 + [_i64] * 4 + [_vp, _vp]),
     "wx_dual_swiglu_gate_up_keep": (_i32, [_vp] * 9 + [_i64] * 4 + [_vp, _vp]),
     "wx_dual_down_proj": (_i32, [_vp] * 5 + [_i64] * 4 + [_vp, _vp, _vp]),
@@ -66,7 +68,7 @@ PROTOTYPES = {
     "wx_rmsnorm_permute_rows": (_i32, [_vp, _vp, _f32, _vp, _vp, _i64, _i64, _vp]),
     "wx_rmsnorm_bwd_workspace_bytes": (_sz, [_i64]),
     "wx_unpermute_rows_rmsnorm_bwd": (_i32, [_vp, _vp, _vp, _f32, _vp, _vp, _vp, _vp, _i64, _i64, _vp, _sz, _vp]),
-    "wx_moe_block_forward": (_i32, [_vp] * 13 + [_i64] * 4 + [_vp, _vp, _f32, _i32, _vp]),
+    "wx_moe_block_forward": (_i32, [_vp] * 13 + [_i64] * 4 + [_vp, _vp, _f32, _i32, _vp, _vp]),
     "wx_swiglu_bwd": (_i32, [_vp] * 6 + [_i64, _vp]),
     "wx_swiglu_bwd_tiled": (_i32, [_vp, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _vp]),
 }

@@ -804,7 +804,10 @@ class HostRows:
         return self.rows
 
 
-_ffn_scratch = {}  # (device index, stream handle, capturing) -> (tiled activations, intermediate, capture id)
+# The two GEMMs of a block forward as one launch where the shape allows it (wx_dual_swiglu_ffn_fused); off: always two.
+_one_launch_ffn = os.environ.get("WALLX_MI355_ONE_LAUNCH_FFN", "1") != "0"
+
+_ffn_scratch = {}  # (device index, stream handle, capturing) -> (tiled activations, intermediate, capture id, counters)
 
 
 def _ffn_buffers(device: torch.device, stream: int, x_elems: int, h_elems: int, cap: Optional[int] = None):
@@ -813,7 +816,8 @@ def _ffn_buffers(device: torch.device, stream: int, x_elems: int, h_elems: int, 
     block would hold 0.45 GB per layer at 29 184 tokens).  Calls that overlap on one stream's pair from two threads
     race, like any two launches writing one buffer.  Under HIP graph capture the pair belongs to that capture (its
     memory comes from the graph's pool and its replays write it): eager calls never share it, and a later capture on
-    the same stream replaces it."""
+    the same stream replaces it.  With them comes the zeroed counter workspace of the one-launch FFN
+    (wx_dual_swiglu_ffn_fused), which every launch leaves zero again."""
     if cap is None:
         cap = capture_id(stream)
     key = (device.index, stream, cap != 0)
@@ -823,10 +827,12 @@ def _ffn_buffers(device: torch.device, stream: int, x_elems: int, h_elems: int, 
     if hit is None or hit[0].numel() < x_elems or hit[1].numel() < h_elems:
         if hit is not None:
             x_elems, h_elems = max(x_elems, hit[0].numel()), max(h_elems, hit[1].numel())
+        counters = hit[3] if hit is not None and hit[2] == cap else \
+            torch.zeros(_lib.load().wx_ffn_fused_workspace_bytes() // 4 + 1, dtype=torch.int32, device=device)
         hit = (torch.empty(x_elems, dtype=torch.bfloat16, device=device),
-               torch.empty(h_elems, dtype=torch.bfloat16, device=device), cap)
+               torch.empty(h_elems, dtype=torch.bfloat16, device=device), cap, counters)
         _ffn_scratch[key] = hit
-    return hit[0], hit[1], cap
+    return hit[0], hit[1], cap, hit[3]
 
 
 def release_ffn_buffers() -> None:
@@ -900,7 +906,7 @@ def packed_block_forward(experts: PackedExperts, x: torch.Tensor, row_id_map: to
     if stream is None:
         stream = torch.cuda.current_stream(dev).cuda_stream
     x_elems, h_elems = experts.sizes(T)
-    x_tiled, hmid, cap = _ffn_buffers(dev, stream, x_elems, h_elems, capture)
+    x_tiled, hmid, cap, counters = _ffn_buffers(dev, stream, x_elems, h_elems, capture)
     if host_rows_c is None and rows_when_ready is not None and cap == 0:
         host_rows_c = rows_when_ready()
     H, I0, I1 = experts.hidden, experts.inter0, experts.inter1
@@ -915,7 +921,8 @@ def packed_block_forward(experts: PackedExperts, x: torch.Tensor, row_id_map: to
         _lib.check(lib.wx_moe_block_forward(x.data_ptr(), out.data_ptr(), row_id_map.data_ptr(),
                                             sorted_row_id.data_ptr(), expert_offsets.data_ptr(), *experts.ptrs,
                                             x_tiled.data_ptr(), hmid.data_ptr(), T, H, I0, I1, host_rows_c, norm_ptr,
-                                            float(eps), int(bool(residual)), stream))
+                                            float(eps), int(bool(residual)),
+                                            counters.data_ptr() if _one_launch_ffn else None, stream))
     return out
 
 
