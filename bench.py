@@ -563,7 +563,7 @@ def config4_measurement(dev, weights):
     VL group empty, (ii) a prefill of 4096 VL tokens plus n action tokens.  Activations N(0, 1); the weights are
     the benchmark's N(0, 0.02) tensors (timing does not depend on the weight scale)."""
     import torch
-    from wallx_mi355 import moe
+    from wallx_mi355 import moe, native
 
     H = weights[0][0].shape[1]
     I0, I1 = weights[0][0].shape[0], weights[1][0].shape[0]
@@ -626,6 +626,21 @@ def config4_measurement(dev, weights):
             tg, _ = event_ms(graph.replay, 10, warm=3)
             out[name]["us_per_layer_eager_shared_routing"] = round(te * 1e3 / layers, 1)
             out[name]["us_per_layer_hip_graph_replay"] = round(tg * 1e3 / layers, 1)
+            # the same graph with the layer as its three launches (permute, gate/up, down) instead of one
+            native.set_one_launch_ffn(False)
+            try:
+                side.wait_stream(torch.cuda.current_stream())
+                with torch.cuda.stream(side):
+                    stack()
+                torch.cuda.current_stream().wait_stream(side)
+                graph3 = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph3):
+                    stack()
+                tg3, _ = event_ms(graph3.replay, 10, warm=3)
+            finally:
+                native.set_one_launch_ffn(True)
+            out[name]["us_per_layer_hip_graph_replay_three_launches"] = round(tg3 * 1e3 / layers, 1)
+            del graph3
             # the same replay with an action expert of its own in every layer, as the model has them: 36 x 12.6 MB of
             # weights no longer stay in the caches between layers, every layer streams its expert from HBM
             (g0, u0, d0), (g1, u1, d1) = weights
@@ -683,15 +698,26 @@ def denoise_kernel_times(dev, x, types, weights):
         _lib.call("wx_dual_down_proj", hmid.data_ptr(), y.data_ptr(), off.data_ptr(), p[2], p[5], T, H, I0, I1, rows,
                   inv.data_ptr(), stream)
 
-    permute(); gate_up(); down()
+    counters = torch.zeros(_lib.load().wx_ffn_fused_workspace_bytes() // 4, dtype=torch.int32, device=dev)
+
+    def one_launch():  # the three of them as one launch: gate/up tiles read the token rows, down tiles wait for them
+        _lib.call("wx_dual_swiglu_ffn_fused", x.data_ptr(), x_tiled.data_ptr(), y.data_ptr(), None, off.data_ptr(), p[0],
+                  p[1], p[2], p[3], p[4], p[5], hmid.data_ptr(), T, H, I0, I1, rows, inv.data_ptr(), counters.data_ptr(),
+                  stream)
+
+    permute(); gate_up(); down(); one_launch()
     t_p, _ = event_ms(permute, 20, warm=3, batch=20)
     t_g, _ = event_ms(gate_up, 20, warm=3, batch=20)
     t_d, _ = event_ms(down, 20, warm=3, batch=20)
+    t_1, _ = event_ms(one_launch, 20, warm=3, batch=20)
     f_g, f_d = 4.0 * H * n_act * I1, 2.0 * H * n_act * I1
     return {"permute_tiled": round(t_p * 1e3, 2), "gate_up_swiglu": round(t_g * 1e3, 2),
             "down_with_unpermute": round(t_d * 1e3, 2),
             "gate_up_frac_mfma_peak": round(f_g / t_g / 1e9 / PEAK_BF16_TFLOPS, 3),
-            "down_frac_mfma_peak": round(f_d / t_d / 1e9 / PEAK_BF16_TFLOPS, 3)}
+            "down_frac_mfma_peak": round(f_d / t_d / 1e9 / PEAK_BF16_TFLOPS, 3),
+            "permute_gate_up_down_as_one_launch": round(t_1 * 1e3, 2),
+            "one_launch_frac_mfma_peak": round((f_g + f_d) / t_1 / 1e9 / PEAK_BF16_TFLOPS, 3),
+            "one_launch_wait_ran_into_its_bound": int(counters[-1].item())}
 
 
 def backward_measurement(dev, x, weights, m0):

@@ -179,22 +179,26 @@ int wx_dual_swiglu_ffn(const void* x_tiled, void* out, const int32_t* expert_off
                        int64_t inter0, int64_t inter1, const int64_t* host_rows_per_expert,
                        const int32_t* out_row_id, wx_stream_t stream);
 
-/* wx_dual_swiglu_ffn (optionally with wx_dual_down_proj_residual's closing add) as ONE launch where that pays: when
- * host_rows_per_expert is given and each of the two GEMMs is a single round of 128 x 128 tiles (at most one per CU:
- * the denoise step's few thousand action tokens), gate/up tiles and down tiles share one grid, and a down tile starts
- * as soon as the gate/up tiles of its 128 rows have finished instead of after a launch boundary.  Every other shape,
- * or a NULL workspace, runs the two launches of wx_dual_swiglu_ffn; results are bit-identical either way.
+/* wx_dual_swiglu_ffn (optionally with the permute in front and wx_dual_down_proj_residual's closing add behind) as
+ * ONE launch where that pays: when host_rows_per_expert is given and each of the two GEMMs is a single round of
+ * 128 x 128 tiles (at most one per CU: the denoise step's few thousand action tokens), gate/up tiles and down tiles
+ * share one grid, and a down tile starts as soon as the gate/up tiles of its 128 rows have finished instead of after a
+ * launch boundary.  Every other shape, or a NULL workspace, runs the launches of wx_[permute_rows_tiled +]
+ * wx_dual_swiglu_ffn; results are bit-identical either way.  The host's row counts only choose the form.
+ * x_rows: NULL, or the activations in token order, [num_rows, hidden] bf16 (out_row_id required): the permute is then
+ * part of the call and x_tiled only a work buffer -- in the one launch the gate/up tiles read the token rows through
+ * out_row_id and x_tiled is not touched; the other shapes fill it with wx_permute_rows_tiled first.
  * residual: NULL or as for wx_dual_down_proj_residual (then out_row_id is required).
  * workspace: wx_ffn_fused_workspace_bytes() bytes of device memory, 4-byte aligned, ZERO before its first use; a
  * launch leaves it zero again.  Calls that share a workspace must not overlap (one workspace per stream).
- * Inside the one launch the down tiles wait on counters in the workspace that the gate/up tiles advance; the wait is
- * bounded, and a wait that runs into its bound stores 1 into the workspace's last int (and the result is undefined).
+ * Inside the one launch tiles wait on counters in the workspace that other tiles advance; every wait is bounded
+ * (seconds), and a wait that runs into its bound stores 1 into the workspace's last int (the result is then undefined).
  * No counterpart in the reference, whose experts are separate nn.Linear launches (act.py:79-82, 142-154). */
 size_t wx_ffn_fused_workspace_bytes(void);
-int wx_dual_swiglu_ffn_fused(const void* x_tiled, void* out, const void* residual, const int32_t* expert_offsets,
-                             const void* gate0, const void* up0, const void* down0, const void* gate1,
-                             const void* up1, const void* down1, void* hmid, int64_t num_rows, int64_t hidden,
-                             int64_t inter0, int64_t inter1, const int64_t* host_rows_per_expert,
+int wx_dual_swiglu_ffn_fused(const void* x_rows, void* x_tiled, void* out, const void* residual,
+                             const int32_t* expert_offsets, const void* gate0, const void* up0, const void* down0,
+                             const void* gate1, const void* up1, const void* down1, void* hmid, int64_t num_rows,
+                             int64_t hidden, int64_t inter0, int64_t inter1, const int64_t* host_rows_per_expert,
                              const int32_t* out_row_id, void* workspace, wx_stream_t stream);
 
 /* The two launches of wx_dual_swiglu_ffn on their own, for callers that put work between them (and for
@@ -404,7 +408,8 @@ int wx_unpermute_rows_rmsnorm_bwd(const void* grad_sorted, const void* x, const 
  * partition's outputs (sorted_row_id required); the six weights packed (wx_pack_tiled); x_tiled and hmid: work
  * buffers of wx_tiled_bytes(wx_padded_sorted_rows(num_rows), hidden) bytes and wx_padded_sorted_rows(num_rows) *
  * max(inter0, inter1) bf16; norm_weight: bf16 [hidden] or NULL (no norm); add_residual != 0 returns x + block(x).
- * ffn_workspace: NULL, or the workspace of wx_dual_swiglu_ffn_fused (same rules), which then runs the two GEMMs. */
+ * ffn_workspace: NULL, or the workspace of wx_dual_swiglu_ffn_fused (same rules), which then runs the two GEMMs
+ * and, when there is no norm, the permute as well. */
 int wx_moe_block_forward(const void* x, void* out, const int32_t* row_id_map, const int32_t* sorted_row_id,
                          const int32_t* expert_offsets, const void* gate0, const void* up0, const void* down0,
                          const void* gate1, const void* up1, const void* down1, void* x_tiled, void* hmid,

@@ -81,9 +81,9 @@ def test_argument_errors_without_a_gpu():
     assert lib.wx_unpermute_rows_rmsnorm_bwd(*([None] * 3), 1e-6, *([None] * 4), 4, 8192, None, 0, None) == -2  # cols > 4096
     assert lib.wx_unpermute_rows_rmsnorm_bwd(*([None] * 3), 1e-6, *([None] * 4), 4, 2048, None, 0, None) == -1  # null pointers
     assert lib.wx_ffn_fused_workspace_bytes() >= 8
-    assert lib.wx_dual_swiglu_ffn_fused(*([None] * 11), 4, 64, 64, 64, None, None, None, None) == -1  # null pointers
-    assert lib.wx_dual_swiglu_ffn_fused(*([None] * 11), 0, 64, 64, 64, None, None, None, None) == 0   # nothing to do
-    assert lib.wx_dual_swiglu_ffn_fused(*([None] * 11), 4, 64, 48, 64, None, None, None, None) == -2  # inter % 32
+    assert lib.wx_dual_swiglu_ffn_fused(*([None] * 12), 4, 64, 64, 64, None, None, None, None) == -1  # null pointers
+    assert lib.wx_dual_swiglu_ffn_fused(*([None] * 12), 0, 64, 64, 64, None, None, None, None) == 0   # nothing to do
+    assert lib.wx_dual_swiglu_ffn_fused(*([None] * 12), 4, 64, 48, 64, None, None, None, None) == -2  # inter % 32
     assert lib.wx_moe_block_forward(*([None] * 13), -1, 64, 64, 64, None, None, 1e-6, 0, None, None) == -1
     assert lib.wx_moe_block_forward(*([None] * 13), 0, 64, 64, 64, None, None, 1e-6, 0, None, None) == 0   # nothing to do
     assert lib.wx_moe_block_forward(*([None] * 13), 4, 64, 64, 64, None, None, 1e-6, 0, None, None) == -1  # no sorted_row_id

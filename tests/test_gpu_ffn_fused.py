@@ -41,10 +41,11 @@ def _two_launches(p, xt, hm, out, res, off, inv, T, H, I0, I1, rows, stream):
                   inv.data_ptr(), stream)
 
 
-def _one_launch(p, xt, hm, out, res, off, inv, T, H, I0, I1, rows, ws, stream):
-    _lib.call("wx_dual_swiglu_ffn_fused", xt.data_ptr(), out.data_ptr(), None if res is None else res.data_ptr(),
-              off.data_ptr(), p[0], p[1], p[2], p[3], p[4], p[5], hm.data_ptr(), T, H, I0, I1, rows, inv.data_ptr(),
-              None if ws is None else ws.data_ptr(), stream)
+def _one_launch(p, xt, hm, out, res, off, inv, T, H, I0, I1, rows, ws, stream, x_rows=None):
+    """x_rows: the activations in token order; xt is then the buffer that the call permutes them into."""
+    _lib.call("wx_dual_swiglu_ffn_fused", None if x_rows is None else x_rows.data_ptr(), xt.data_ptr(), out.data_ptr(),
+              None if res is None else res.data_ptr(), off.data_ptr(), p[0], p[1], p[2], p[3], p[4], p[5], hm.data_ptr(),
+              T, H, I0, I1, rows, inv.data_ptr(), None if ws is None else ws.data_ptr(), stream)
 
 
 # one round of 128 x 128 tiles per GEMM (the shapes that run as one launch): a denoise step's 2048 action tokens, all
@@ -66,9 +67,13 @@ def test_one_launch_ffn_equals_two_launches(dev, T, m0, H, I0, I1, with_res, kno
     r = res if with_res else None
     work = _workspace(dev)
     _two_launches(p, xt, hm[0], out[0], r, off, inv, T, H, I0, I1, rows, stream)
-    for call in range(3):  # every call after the first runs on the workspace the one before it left
+    xt2 = torch.full_like(xt, 3.0)
+    for call in range(4):  # every call after the first runs on the workspace the one before it left
         out[1].fill_(9.0)
-        _one_launch(p, xt, hm[1], out[1], r, off, inv, T, H, I0, I1, rows, work, stream)
+        if call < 2:
+            _one_launch(p, xt, hm[1], out[1], r, off, inv, T, H, I0, I1, rows, work, stream)
+        else:  # ... and with the permute inside the launch (the gate/up tiles read the token rows)
+            _one_launch(p, xt2, hm[1], out[1], r, off, inv, T, H, I0, I1, rows, work, stream, x_rows=x)
         torch.cuda.synchronize()
         assert torch.equal(out[0], out[1]), f"call {call}"
         assert torch.equal(hm[0], hm[1]), f"call {call}"
@@ -89,7 +94,7 @@ def test_one_launch_ffn_with_row_counts_that_are_not_the_devices(dev, hint):
     for -- gate/up workgroups then take several tiles each, and so do down workgroups, each tile behind its own wait
     -- and the result does not change."""
     T, m0, H, I0, I1 = 4096, 2049, 1024, 64, 1024
-    _, packed, _, _, res, off, inv, xt = _case(dev, T, m0, H, I0, I1, 17)
+    _, packed, _, x, res, off, inv, xt = _case(dev, T, m0, H, I0, I1, 17)
     p = [t.data_ptr() for t in packed]
     stream = torch.cuda.current_stream().cuda_stream
     pad = native.padded_sorted_rows(T)
@@ -97,8 +102,12 @@ def test_one_launch_ffn_with_row_counts_that_are_not_the_devices(dev, hint):
     out = [torch.full((T, H), v, dtype=torch.bfloat16, device=dev) for v in (7.0, 9.0)]
     work = _workspace(dev)
     _two_launches(p, xt, hm[0], out[0], res, off, inv, T, H, I0, I1, None, stream)
+    xt2 = torch.full_like(xt, 3.0)
     for call in range(2):
-        _one_launch(p, xt, hm[1], out[1], res, off, inv, T, H, I0, I1, _lib.i64x2(hint), work, stream)
+        if call == 0:
+            _one_launch(p, xt, hm[1], out[1], res, off, inv, T, H, I0, I1, _lib.i64x2(hint), work, stream)
+        else:
+            _one_launch(p, xt2, hm[1], out[1], res, off, inv, T, H, I0, I1, _lib.i64x2(hint), work, stream, x_rows=x)
         torch.cuda.synchronize()
         assert torch.equal(out[0], out[1]) and torch.equal(hm[0], hm[1]), f"call {call}"
         assert int(work.abs().sum()) == 0
@@ -119,19 +128,22 @@ def test_one_launch_ffn_without_a_workspace_is_the_two_launches(dev):
     assert torch.equal(out[0], out[1]) and torch.equal(hm[0], hm[1])
     lib = _lib.load()
     work = _workspace(dev)
-    assert lib.wx_dual_swiglu_ffn_fused(xt.data_ptr(), out[1].data_ptr(), None, off.data_ptr(), *p, hm[1].data_ptr(), T, H,
-                                        I0, I1, rows, inv.data_ptr(), work.data_ptr() + 2, stream) == -1
+    assert lib.wx_dual_swiglu_ffn_fused(None, xt.data_ptr(), out[1].data_ptr(), None, off.data_ptr(), *p, hm[1].data_ptr(),
+                                        T, H, I0, I1, rows, inv.data_ptr(), work.data_ptr() + 2, stream) == -1
     assert b"aligned" in lib.wx_last_error_string()
-    assert lib.wx_dual_swiglu_ffn_fused(xt.data_ptr(), out[1].data_ptr(), out[0].data_ptr(), off.data_ptr(), *p,
+    assert lib.wx_dual_swiglu_ffn_fused(None, xt.data_ptr(), out[1].data_ptr(), out[0].data_ptr(), off.data_ptr(), *p,
                                         hm[1].data_ptr(), T, H, I0, I1, rows, None, work.data_ptr(), stream) == -1
     assert b"out_row_id" in lib.wx_last_error_string()  # a residual is added in token order
+    assert lib.wx_dual_swiglu_ffn_fused(out[0].data_ptr(), xt.data_ptr(), out[1].data_ptr(), None, off.data_ptr(), *p,
+                                        hm[1].data_ptr(), T, H, I0, I1, rows, None, work.data_ptr(), stream) == -1
+    assert b"out_row_id" in lib.wx_last_error_string()  # ... and rows are gathered through it
 
 
 def test_one_launch_ffn_replays_from_a_hip_graph(dev):
     """Captured once, replayed with the program's own eager launches and synchronisations in between: every replay
     equals the eager result, and the counters are zero after each."""
     T, m0, H, I0, I1 = 2048, 0, 1024, 512, 1024
-    _, packed, _, _, res, off, inv, xt = _case(dev, T, m0, H, I0, I1, 11)
+    _, packed, _, x, res, off, inv, xt = _case(dev, T, m0, H, I0, I1, 11)
     p = [t.data_ptr() for t in packed]
     pad = native.padded_sorted_rows(T)
     rows = _lib.i64x2((m0, T - m0))
@@ -144,13 +156,15 @@ def test_one_launch_ffn_replays_from_a_hip_graph(dev):
     with torch.cuda.stream(side):
         _one_launch(p, xt, hm[1], out[1], res, off, inv, T, H, I0, I1, rows, work, side.cuda_stream)
     torch.cuda.current_stream().wait_stream(side)
+    xt2 = torch.zeros_like(xt)
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):
-        _one_launch(p, xt, hm[1], out[1], res, off, inv, T, H, I0, I1, rows, work,
-                    torch.cuda.current_stream().cuda_stream)
+        _one_launch(p, xt2, hm[1], out[1], res, off, inv, T, H, I0, I1, rows, work,
+                    torch.cuda.current_stream().cuda_stream, x_rows=x)
     for replay in range(4):
         out[1].zero_()
         hm[1].zero_()
+        xt2.zero_()
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(out[0], out[1]) and torch.equal(hm[0], hm[1]), f"replay {replay}"
@@ -177,7 +191,7 @@ def test_block_forward_with_and_without_the_one_launch_ffn(dev, residual, monkey
     rows = _lib.i64x2((T - n1, n1))
     got = {}
     for flag in (True, False):
-        monkeypatch.setattr(native, "_one_launch_ffn", flag)
+        monkeypatch.setattr(native, "_one_launch_ffn", flag)  # (what native.set_one_launch_ffn sets)
         got[flag] = native.packed_block_forward(experts, x, rmap, inv, off, rows, residual=residual)
     torch.cuda.synchronize()
     assert torch.equal(got[True], got[False])

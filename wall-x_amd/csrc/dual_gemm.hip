@@ -245,19 +245,27 @@ __device__ __forceinline__ unsigned char* lds_array() {
 // The fused FFN launch: gate/up tiles (producers) and down tiles (consumers) in one grid.  A down tile of row block
 // rb reads the intermediate rows that the gate/up tiles of the same row block write, so it waits until `ready[rb]`
 // has reached the number of those tiles.  Workgroups are dispatched in index order and the producers come first, so
-// a consumer only ever waits for workgroups that are already running and never wait themselves; its wait is bounded
-// all the same (kFusedSpinLimit polls, then `*error` is set and the tile goes ahead).  The last consumer past the
-// wait of a row block clears its two counters, so a launch leaves the workspace as it found it: all zero.
+// a consumer only ever waits for workgroups that are already running and never wait themselves.  Its wait is
+// bounded all the same (kFusedWaitTicks of the 100 MHz clock; then `*error` is set and the tile goes ahead on
+// whatever is there).  The last consumer past the wait of a row block clears the row block's counters, so a launch
+// leaves the workspace as it found it: all zero.
+// The producers can read their A operand from the token rows themselves (AROWS below: `x` through `gather`), which
+// makes the permute into the K-tiled activation matrix part of the launch.
 constexpr int kFusedMaxRowBlocks = 256;   // 128-row blocks per expert
-constexpr int kFusedSpinLimit = 1 << 20;
+constexpr long long kFusedWaitTicks = 500000000ll;  // 5 s
 constexpr int kFusedCounterStride = 64;   // ints between two counters: 256 bytes, so that the polls of different row
-                                          // blocks (and the producers' increments) spread over the memory channels
+                                          // blocks (and the increments) spread over the memory channels
+constexpr int kFusedCounters = 2 * kFusedMaxRowBlocks * kFusedCounterStride;  // ints of one counter array
 struct FusedSync {
   int* ready;     // [2 * kFusedMaxRowBlocks] x stride: gate/up tiles finished, by expert and row block
-  int* passed;    // [2 * kFusedMaxRowBlocks] x stride: down tiles past their wait
+  int* passed;    // ... down tiles past their wait
   int* error;     // set to 1 when a wait ran into its bound
   int need[2];    // gate/up tiles per row block of expert e
   int consumers;  // down tiles per row block
+  // AROWS: the activations in token order, [tokens, hidden] bf16 row-major, and the partition's sorted_row_id
+  // (sorted position -> token)
+  const __bf16* x;
+  const int32_t* gather;
 };
 
 // KA / KB (generic mode only): the operand is stored with K as its slow dimension -- A as [k, m], B as [k, n] --
@@ -266,8 +274,9 @@ struct FusedSync {
 // The kernel's body is a function of its own so that one launch can run two of them side by side (the fused FFN
 // launch below: some workgroups run the gate/up form, the others the down form).  `wg` of `n_wg` is the workgroup's
 // place among those that share this body's tile list (blockIdx.x of gridDim.x in a plain launch).
-// ROLE: 0 = a plain launch; 1 / 2 = producer / consumer of a fused launch (see FusedSync).
-template <int MODE, typename TS, bool KA, bool KB, int ROLE>
+// ROLE: 0 = a plain launch; 1 / 2 = producer / consumer of a fused launch (see FusedSync).  AROWS (gate/up form of a fused launch): the A operand is read from the token rows themselves,
+// fs.x through fs.gather, instead of from a K-tiled copy of them.
+template <int MODE, typename TS, bool KA, bool KB, int ROLE, bool AROWS = false>
 __device__ __forceinline__ void dual_gemm_body(const Params& p, const int wg, const int n_wg, const FusedSync& fs) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stub; the body uses gfx950-only builtins
   constexpr int BM = TS::BM, BN = TS::BN, FM = TS::FM, FN = TS::FN;
@@ -337,7 +346,8 @@ __device__ __forceinline__ void dual_gemm_body(const Params& p, const int wg, co
   // ---- problem table (uniform) ------------------------------------------------------------------
   // (kept as two named structs, selected per tile, so everything stays in scalar registers)
   Group g0 = p.g[0], g1 = p.g[1];
-  int sorted_first[2] = {0, 0};  // kDown: sorted position of each expert's first row
+  int sorted_first[2] = {0, 0};  // tiled modes: sorted position of each expert's first row
+  int sorted_total = 0;          // ... and the number of sorted rows
   if constexpr (TILED_IN) {
     const int o0 = p.offsets[0], o1 = p.offsets[1], o2 = p.offsets[2];
     g0.m = o1 - o0;
@@ -362,9 +372,10 @@ __device__ __forceinline__ void dual_gemm_body(const Params& p, const int wg, co
         g0.c += static_cast<int64_t>(o0) * g0.ldc;
         g1.c += static_cast<int64_t>(o1) * g1.ldc;
       }
-      sorted_first[0] = o0;
-      sorted_first[1] = o1;
     }
+    sorted_first[0] = o0;
+    sorted_first[1] = o1;
+    sorted_total = o2;
   }
   constexpr int kTileN = SWIGLU ? BN / 2 : BN;  // output columns per tile
   int tiles_m[2], tiles_n[2];
@@ -515,26 +526,46 @@ __device__ __forceinline__ void dual_gemm_body(const Params& p, const int wg, co
     if constexpr (TILED_IN) {
       // this wave's row blocks of the A tile and of the B tile at K step 0; a K step later they sit one column
       // block further, i.e. (row blocks of the matrix) KiB ahead
-      const int64_t a_blk = (G.a_row0 + row0) / kBlkRows + wave * kLoadsA;
       const int64_t b_blk = col0 / kBlkRows + b_wave * kLoadsB;
-      L.a_base = G.a + (a_blk << 9);
       L.b_base = b_src + (b_blk << 9);
-      L.a_step = static_cast<int64_t>(G.lda) << 10;
       L.b_step = static_cast<int64_t>(G.ldb) << 10;
-      const int64_t a_left = (static_cast<int64_t>(G.k / kBlkCols) * G.lda - a_blk) << 10;
       const int64_t b_left = (static_cast<int64_t>(G.k / kBlkCols) * G.ldb - b_blk) << 10;
-      L.a_bytes = static_cast<uint32_t>(a_left < 0 ? 0 : (a_left > 0x7fffff00ll ? 0x7fffff00ll : a_left));
       L.b_bytes = static_cast<uint32_t>(b_left < 0 ? 0 : (b_left > 0x7fffff00ll ? 0x7fffff00ll : b_left));
-      L.a_cur = reinterpret_cast<const char*>(L.a_base);
       L.b_cur = reinterpret_cast<const char*>(L.b_base);
-      L.a_left = L.a_bytes;
       L.b_left = L.b_bytes;
-      L.a_dec = static_cast<uint32_t>(L.a_step > 0x7fffff00ll ? 0x7fffff00ll : L.a_step);
       L.b_dec = static_cast<uint32_t>(L.b_step > 0x7fffff00ll ? 0x7fffff00ll : L.b_step);
 #pragma unroll
-      for (int i = 0; i < kLoadsA; ++i) L.voff_a[i] = static_cast<uint32_t>(i * kBlkBytes + lane * 16);
-#pragma unroll
       for (int i = 0; i < kLoadsB; ++i) L.voff_b[i] = static_cast<uint32_t>(i * kBlkBytes + lane * 16);
+      if constexpr (AROWS) {
+        // A from the token rows: sorted row r of the tile is row gather[...] of the row-major activations; a load
+        // instruction fetches 64 bytes of 16 such rows (lane -> row lane / 4, and the chunk that belongs in LDS slot
+        // lane % 4), rows past the expert's last row read as zero.  The host keeps the matrix below 2 GiB.
+        const int rows_a = G.m - row0 < BM ? G.m - row0 : BM;
+        L.a_base = fs.x;
+        L.a_bytes = static_cast<uint32_t>(sorted_total) * static_cast<uint32_t>(G.k) * 2u;
+        L.a_step = 0;
+        L.a_cur = nullptr;
+        L.a_left = L.a_dec = 0;
+#pragma unroll
+        for (int i = 0; i < kLoadsA; ++i) {
+          const int r = ld_row0 + 16 * i;
+          uint32_t v = 0x80000000u;
+          if (r < rows_a)
+            v = static_cast<uint32_t>(fs.gather[sorted_first[tc.group] + row0 + r]) * static_cast<uint32_t>(G.k) * 2u + ld_chunk * 16u;
+          L.voff_a[i] = v;
+        }
+      } else {
+        const int64_t a_blk = (G.a_row0 + row0) / kBlkRows + wave * kLoadsA;
+        L.a_base = G.a + (a_blk << 9);
+        L.a_step = static_cast<int64_t>(G.lda) << 10;
+        const int64_t a_left = (static_cast<int64_t>(G.k / kBlkCols) * G.lda - a_blk) << 10;
+        L.a_bytes = static_cast<uint32_t>(a_left < 0 ? 0 : (a_left > 0x7fffff00ll ? 0x7fffff00ll : a_left));
+        L.a_cur = reinterpret_cast<const char*>(L.a_base);
+        L.a_left = L.a_bytes;
+        L.a_dec = static_cast<uint32_t>(L.a_step > 0x7fffff00ll ? 0x7fffff00ll : L.a_step);
+#pragma unroll
+        for (int i = 0; i < kLoadsA; ++i) L.voff_a[i] = static_cast<uint32_t>(i * kBlkBytes + lane * 16);
+      }
     } else {
       const int rows_a = G.m - row0 < BM ? G.m - row0 : BM;
       const int rows_b = G.n - col0 < kTileN ? G.n - col0 : kTileN;
@@ -637,14 +668,19 @@ __device__ __forceinline__ void dual_gemm_body(const Params& p, const int wg, co
     if constexpr (TILED_IN) {
       // steps past K (ring padding) and blocks past the end of the matrix read as zero through the bounds check
       const bool real = ks * BK < L.K;
-      ra = make_rsrc(L.a_cur, real ? L.a_left : 0u);
       P.rb = make_rsrc(L.b_cur, real ? L.b_left : 0u);
       // on to the next K step.  The byte counts are clamped for huge matrices; a clamped count is far above what
       // one step reads and stays as it is.
-      L.a_cur += L.a_step;
       L.b_cur += L.b_step;
-      if (L.a_left != 0x7fffff00u) L.a_left = L.a_left > L.a_dec ? L.a_left - L.a_dec : 0u;
       if (L.b_left != 0x7fffff00u) L.b_left = L.b_left > L.b_dec ? L.b_left - L.b_dec : 0u;
+      if constexpr (AROWS) {  // token rows: the base advances along K and keeps the absolute end of the readable range
+        const uint32_t adv = 2u * static_cast<uint32_t>(ks * BK);
+        ra = make_rsrc(L.a_base + ks * BK, real && L.a_bytes > adv ? L.a_bytes - adv : 0u);
+      } else {
+        ra = make_rsrc(L.a_cur, real ? L.a_left : 0u);
+        L.a_cur += L.a_step;
+        if (L.a_left != 0x7fffff00u) L.a_left = L.a_left > L.a_dec ? L.a_left - L.a_dec : 0u;
+      }
     } else {
       const int k0 = ks * BK;
       // advancing the base keeps the absolute end of the readable range, so rows past the matrix read as zero;
@@ -697,46 +733,45 @@ __device__ __forceinline__ void dual_gemm_body(const Params& p, const int wg, co
     for (int i = 0; i < kLoadsB; ++i) P.voff_b[i] = L.voff_b[i];
     issue_b(P, sb);
   };
-  // Fused launch, producer: this workgroup's tile of row block `rb` is in memory (its stores are write-through and
-  // every wavefront has waited for its own before the barrier); one lane counts the tile.
-  auto signal_consumers = [&](int rb) {
+  // Fused launch: what this workgroup wrote for row block `rb` is in memory (its stores are write-through and every
+  // wavefront has waited for its own before the barrier); one lane counts it.
+  auto count_done = [&](int* counters, int rb) {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
     __syncthreads();
     if (tid == 0)
-      __hip_atomic_fetch_add(fs.ready + rb * kFusedCounterStride, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_fetch_add(counters + rb * kFusedCounterStride, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   };
-  // Fused launch, consumer: wait (bounded) until the producers of row block `rb` have all counted themselves.
-  // No cache is invalidated afterwards: the launch began with clean caches, and no line of a row block's
-  // intermediate is read anywhere before that row block is complete (its 1 KiB blocks belong to one producer tile
-  // each), so no cache can hold an older version of it.
-  int passed_before = 0;  // consumers of the row block that were past their wait before this one
-  auto wait_for_producers = [&](int rb, int group) {
+  // Fused launch: wait (bounded) until counters[rb] has reached `need`, and take a number among the workgroups that
+  // get past this wait (`before`: how many were past it already; the answer travels while the tile is computed).
+  // No cache is invalidated afterwards: the launch began with clean caches, and no line of what the wait is for is
+  // read anywhere before it is complete (whole cache lines belong to one writer), so no cache can hold an older
+  // version of it.
+  auto wait_for_count = [&](const int* counters, int* passed, int rb, int need, int& before) {
     if (tid == 0) {
-      const int need = fs.need[group];
-      const int* flag = fs.ready + rb * kFusedCounterStride;
-      int polls = 0;
+      const int* flag = counters + rb * kFusedCounterStride;
+      const long long start = __builtin_amdgcn_s_memrealtime();
       while (__hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < need) {
-        if (++polls > kFusedSpinLimit) {
+        if (static_cast<long long>(__builtin_amdgcn_s_memrealtime()) - start > kFusedWaitTicks) {
           __hip_atomic_store(fs.error, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           break;
         }
         __builtin_amdgcn_s_sleep(2);
       }
-      // counted here, looked at when the tile is done: the answer travels while the tile is computed
-      passed_before = __hip_atomic_fetch_add(fs.passed + rb * kFusedCounterStride, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      before = __hip_atomic_fetch_add(passed + rb * kFusedCounterStride, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     barrier_no_fence();  // (no wait for the counter's answer here)
   };
-  // ... and once its tile is done: the consumer that was the last of its row block to get past the wait (the
-  // producers are done and every other consumer is past its wait as well) leaves the row block's counters at zero
-  // for the next launch
-  auto leave_row_block = [&](int rb) {
-    if (tid == 0 && passed_before == fs.consumers - 1) {
-      __hip_atomic_store(fs.ready + rb * kFusedCounterStride, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      __hip_atomic_store(fs.passed + rb * kFusedCounterStride, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  // ... and once the tile is done: the workgroup that was the last of its row block to get past the wait (everything
+  // the wait was for is done, and every other waiter is past its wait as well) leaves the two counters at zero for
+  // the next launch
+  auto clear_if_last = [&](int* counters, int* passed, int rb, int before, int waiters) {
+    if (tid == 0 && before == waiters - 1) {
+      __hip_atomic_store(counters + rb * kFusedCounterStride, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(passed + rb * kFusedCounterStride, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
   };
+  int passed_before = 0;
 
   f32x16 acc[FM][FN];
   bf16x8 fa[2][FM], fb[2][FN];  // two fragment sets: one feeds the MFMAs while the other is being read from LDS
@@ -1206,7 +1241,7 @@ __device__ __forceinline__ void dual_gemm_body(const Params& p, const int wg, co
 #pragma unroll
         for (int s = 0; s + 1 < kStages; ++s) issue_b_ahead(L, s, slot_b(s));
       }
-      wait_for_producers(S.row_block, tc.group);
+      wait_for_count(fs.ready, fs.passed, S.row_block, fs.need[tc.group], passed_before);
       if constexpr (LD) {
 #pragma unroll
         for (int s = 0; s < kStages; ++s) issue_a(L, s, slot_a(s), pend);
@@ -1290,9 +1325,9 @@ __device__ __forceinline__ void dual_gemm_body(const Params& p, const int wg, co
         }
       }
       epilogue(done);
-      if constexpr (ROLE == 1) signal_consumers(done.row_block);
+      if constexpr (ROLE == 1) count_done(fs.ready, done.row_block);
       if constexpr (ROLE == 2) {
-        leave_row_block(done.row_block);
+        clear_if_last(fs.ready, fs.passed, done.row_block, passed_before, fs.consumers);
         have = next_tile(tc);
         if (have) {  // (one tile per consumer unless the host's row counts were not the device's)
           if constexpr (LD) setup_loader(tc, L);
@@ -1321,11 +1356,13 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
 // The fused FFN launch (see FusedSync): workgroups [0, producers) run the gate/up form on `pg`, the rest the down
 // form on `pd`, both in the small tile shape.  `producers` is a multiple of 8, so a workgroup's index among its
 // form's workgroups names the same XCD as its index in the grid.
+// AROWS: the producers read the token rows (fs.x through fs.gather) in place of the K-tiled activations.
+template <bool AROWS>
 __global__ __launch_bounds__(SmallTile::kThreads, SmallTile::kWgPerCu) void ffn_fused_kernel(Params pg, Params pd,
                                                                                              FusedSync fs,
                                                                                              int producers) {
   const int wg = blockIdx.x;
-  if (wg < producers) dual_gemm_body<kGateUp, SmallTile, false, false, 1>(pg, wg, producers, fs);
+  if (wg < producers) dual_gemm_body<kGateUp, SmallTile, false, false, 1, AROWS>(pg, wg, producers, fs);
   else dual_gemm_body<kDown, SmallTile, false, false, 2>(pd, wg - producers, static_cast<int>(gridDim.x) - producers, fs);
 }
 
@@ -1657,6 +1694,7 @@ struct FfnArgs {
   const int32_t* out_row_id = nullptr;  // optional: sorted row r of the result goes to row out_row_id[r] of `out`
   void *keep_gate = nullptr, *keep_up = nullptr;  // optional: the gate / up projections, K-tiled like hmid
   const void* residual = nullptr;  // optional (with out_row_id): rows added to the result, laid out like `out`
+  const void* x_rows = nullptr;    // optional: the activations in token order; `x` is then built by the fused launch
 };
 
 int check_ffn(const char* who, const FfnArgs& a, bool need_gate_up, bool need_down) {
@@ -1751,12 +1789,15 @@ int launch_down(const FfnArgs& a, hipStream_t s) {
 }
 
 // Both launches as one (ffn_fused_kernel), for the shapes where each is a single round of small tiles with the row
-// counts known on the host -- a denoise step.  Returns 1 when the shape is not of that kind (nothing launched).
-constexpr size_t kFusedWorkspaceInts = 4 * kFusedMaxRowBlocks * kFusedCounterStride + 1;  // ready, passed, then the error flag
+// counts known on the host -- a denoise step.  With a.x_rows the gate/up tiles read the token rows themselves (the
+// permute happens in their loads; a.x is not touched).  Returns 1 when the shape is not of that kind (nothing launched).
+constexpr size_t kFusedWorkspaceInts = 2 * static_cast<size_t>(kFusedCounters) + 1;  // two counter arrays, then the error flag
 int launch_ffn_fused(const FfnArgs& a, int* ws, hipStream_t s) {
   if (a.host_rows == nullptr || ws == nullptr || a.keep_gate != nullptr) return 1;
   // (whatever the real split of the rows: the counters hold this many row blocks per expert)
   if (a.rows > static_cast<int64_t>(kFusedMaxRowBlocks) * SmallTile::BM) return 1;
+  // (token rows are addressed with 31-bit byte offsets)
+  if (a.x_rows != nullptr && (a.out_row_id == nullptr || a.rows * a.hidden * 2 >= (1ll << 31))) return 1;
   const int cus = device_cu_count();
   int64_t gate_tiles = 0, down_tiles = 0;
   int need[2] = {0, 0};
@@ -1773,14 +1814,19 @@ int launch_ffn_fused(const FfnArgs& a, int* ws, hipStream_t s) {
   pg.split = pd.split = 0;
   FusedSync fs{};
   fs.ready = ws;
-  fs.passed = ws + 2 * kFusedMaxRowBlocks * kFusedCounterStride;
-  fs.error = ws + 4 * kFusedMaxRowBlocks * kFusedCounterStride;
+  fs.passed = ws + kFusedCounters;
+  fs.error = ws + 2 * kFusedCounters;
   fs.need[0] = need[0];
   fs.need[1] = need[1];
   fs.consumers = static_cast<int>(down_cols);
+  fs.x = static_cast<const __bf16*>(a.x_rows);
+  fs.gather = a.out_row_id;
   const int producers = static_cast<int>((gate_tiles + kXcds - 1) / kXcds * kXcds);
   const int consumers = static_cast<int>((down_tiles + kXcds - 1) / kXcds * kXcds);
-  hipLaunchKernelGGL(ffn_fused_kernel, dim3(producers + consumers), dim3(SmallTile::kThreads), 0, s, pg, pd, fs, producers);
+  if (a.x_rows != nullptr)
+    hipLaunchKernelGGL(ffn_fused_kernel<true>, dim3(producers + consumers), dim3(SmallTile::kThreads), 0, s, pg, pd, fs, producers);
+  else
+    hipLaunchKernelGGL(ffn_fused_kernel<false>, dim3(producers + consumers), dim3(SmallTile::kThreads), 0, s, pg, pd, fs, producers);
   return check_launch("ffn_fused_kernel");
 }
 
@@ -1788,7 +1834,7 @@ int launch_ffn_fused(const FfnArgs& a, int* ws, hipStream_t s) {
 
 extern "C" size_t wx_ffn_fused_workspace_bytes(void) { return kFusedWorkspaceInts * sizeof(int); }
 
-extern "C" int wx_dual_swiglu_ffn_fused(const void* x_tiled, void* out, const void* residual,
+extern "C" int wx_dual_swiglu_ffn_fused(const void* x_rows, void* x_tiled, void* out, const void* residual,
                                         const int32_t* expert_offsets, const void* gate0, const void* up0,
                                         const void* down0, const void* gate1, const void* up1, const void* down1,
                                         void* hmid, int64_t num_rows, int64_t hidden, int64_t inter0, int64_t inter1,
@@ -1804,9 +1850,16 @@ extern "C" int wx_dual_swiglu_ffn_fused(const void* x_tiled, void* out, const vo
     if (reinterpret_cast<uintptr_t>(residual) & 15) return fail(WX_ERR_INVALID_ARGUMENT, "%s: residual must be 16-byte aligned", who);
     a.residual = residual;
   }
+  if (x_rows != nullptr) {
+    if (!out_row_id) return fail(WX_ERR_INVALID_ARGUMENT, "%s: x_rows needs out_row_id (the rows are gathered through it)", who);
+    if (reinterpret_cast<uintptr_t>(x_rows) & 15) return fail(WX_ERR_INVALID_ARGUMENT, "%s: x_rows must be 16-byte aligned", who);
+    a.x_rows = x_rows;
+  }
   if (reinterpret_cast<uintptr_t>(workspace) & 3) return fail(WX_ERR_INVALID_ARGUMENT, "%s: workspace must be 4-byte aligned", who);
   const int rc = launch_ffn_fused(a, static_cast<int*>(workspace), as_stream(stream));
   if (rc <= 0) return rc;
+  if (x_rows != nullptr)
+    if (int rc2 = wx_permute_rows_tiled(x_rows, x_tiled, nullptr, out_row_id, expert_offsets, num_rows, hidden, stream)) return rc2;
   if (int rc2 = launch_gate_up(a, as_stream(stream))) return rc2;
   return launch_down(a, as_stream(stream));
 }

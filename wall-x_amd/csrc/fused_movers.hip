@@ -595,6 +595,11 @@ extern "C" int wx_moe_block_forward(const void* x, void* out, const int32_t* row
   if (num_rows < 0) return fail(WX_ERR_INVALID_ARGUMENT, "%s: negative row count", who);
   if (num_rows == 0) return WX_OK;
   if (!sorted_row_id) return fail(WX_ERR_INVALID_ARGUMENT, "%s: sorted_row_id is required", who);
+  if (ffn_workspace != nullptr && norm_weight == nullptr)
+    // one launch for the permute and both GEMMs where the shape allows it, else the launches below
+    return wx_dual_swiglu_ffn_fused(x, x_tiled, out, add_residual ? x : nullptr, expert_offsets, gate0, up0, down0, gate1,
+                                    up1, down1, hmid, num_rows, hidden, inter0, inter1, host_rows_per_expert,
+                                    sorted_row_id, ffn_workspace, stream);
   if (int rc = norm_weight != nullptr
                    ? wx_rmsnorm_permute_rows_tiled(x, norm_weight, eps, x_tiled, sorted_row_id, expert_offsets, num_rows,
                                                    hidden, stream)
@@ -602,8 +607,8 @@ extern "C" int wx_moe_block_forward(const void* x, void* out, const int32_t* row
                                            stream))
     return rc;
   if (ffn_workspace != nullptr)  // one launch for both GEMMs where the shape allows it, else the two below
-    return wx_dual_swiglu_ffn_fused(x_tiled, out, add_residual ? x : nullptr, expert_offsets, gate0, up0, down0, gate1,
-                                    up1, down1, hmid, num_rows, hidden, inter0, inter1, host_rows_per_expert,
+    return wx_dual_swiglu_ffn_fused(nullptr, x_tiled, out, add_residual ? x : nullptr, expert_offsets, gate0, up0, down0,
+                                    gate1, up1, down1, hmid, num_rows, hidden, inter0, inter1, host_rows_per_expert,
                                     sorted_row_id, ffn_workspace, stream);
   if (int rc = wx_dual_swiglu_gate_up(x_tiled, hmid, expert_offsets, gate0, up0, gate1, up1, num_rows, hidden, inter0,
                                       inter1, host_rows_per_expert, stream))

@@ -41,7 +41,7 @@ PROTOTYPES = {
     "wx_permute_rows_tiled": (_i32, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _vp]),
     "wx_dual_swiglu_ffn": (_i32, [_vp] * 10 + [_i64] * 4 + [_vp, _vp, _vp]),
     "wx_ffn_fused_workspace_bytes": (_sz, []),
-    "wx_dual_swiglu_ffn_fused": (_i32, [_vp] * 11 + [_i64] * 4 + [_vp, _vp, _vp, _vp]),
+    "wx_dual_swiglu_ffn_fused": (_i32, [_vp] * 12 + [_i64] * 4 + [_vp, _vp, _vp, _vp]),
     "wx_dual_swiglu_gate_up": (_i32, [_vp] * 7 + [_i64] * 4 + [_vp, _vp]),
     "wx_dual_swiglu_gate_up_keep": (_i32, [_vp] * 9 + [_i64] * 4 + [_vp, _vp]),
     "wx_dual_down_proj": (_i32, [_vp] * 5 + [_i64] * 4 + [_vp, _vp, _vp]),

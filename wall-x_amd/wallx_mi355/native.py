@@ -804,8 +804,17 @@ class HostRows:
         return self.rows
 
 
-# The two GEMMs of a block forward as one launch where the shape allows it (wx_dual_swiglu_ffn_fused); off: always two.
+# The block forward's permute and two GEMMs as one launch where the shape allows it (wx_dual_swiglu_ffn_fused: a
+# denoise step's few thousand tokens); off: always the separate launches.  WALLX_MI355_ONE_LAUNCH_FFN=0 starts with it off.
 _one_launch_ffn = os.environ.get("WALLX_MI355_ONE_LAUNCH_FFN", "1") != "0"
+
+
+def set_one_launch_ffn(flag: bool) -> bool:
+    """Switches the one-launch form of the block forward on or off; returns the previous setting.  Results are
+    bit-identical either way."""
+    global _one_launch_ffn
+    old, _one_launch_ffn = _one_launch_ffn, bool(flag)
+    return old
 
 _ffn_scratch = {}  # (device index, stream handle, capturing) -> (tiled activations, intermediate, capture id, counters)
 
