@@ -44,8 +44,10 @@ def parse():
     ap.add_argument("--cpu-seqs", type=int, default=32, help="sequences of the batch the CPU baseline runs (32 = all)")
     ap.add_argument("--kernel-loop", default=None,
                     choices=["gate_up", "down", "down_unpermute", "permute", "permute_plain", "unpermute", "partition", "copy",
-                             "mrope", "mrope_packed", "mrope_copy", "config2_index"],
-                    help="profiling aid: run only this kernel --steps times (no JSON line); 'copy' is a plain "
+                             "layer_one_launch", "mrope", "mrope_packed", "mrope_copy", "config2_index"],
+                    help="profiling aid: run only this kernel --steps times (no JSON line); 'layer_one_launch' is "
+                         "permute, gate/up and down as the one launch a denoise step gets (three launches at config "
+                         "3, where it does not apply); 'copy' is a plain "
                          "device-to-device copy of the [T, H] activations, the known-size yardstick for HBM counters; "
                          "'mrope' / 'mrope_packed' are the M-RoPE apply at config 2 from the two tables / from the "
                          "packed table, 'mrope_copy' a device copy of q and k of the same shape, 'config2_index' the "
@@ -163,6 +165,13 @@ def main():
         _lib.call("wx_unpermute_rows", y_sorted.data_ptr(), y.data_ptr(), row_id_map.data_ptr(), None, T, 1, H,
                   _lib.WX_BF16, stream)
 
+    counters = torch.zeros(_lib.load().wx_ffn_fused_workspace_bytes() // 4, dtype=torch.int32, device=dev)
+
+    def layer_one_launch():  # permute, gate/up and down as one launch where the shape allows it (a denoise step)
+        _lib.call("wx_dual_swiglu_ffn_fused", x.data_ptr(), x_tiled.data_ptr(), y.data_ptr(), None, offsets.data_ptr(),
+                  pg0.data_ptr(), pu0.data_ptr(), pd0.data_ptr(), pg1.data_ptr(), pu1.data_ptr(), pd1.data_ptr(),
+                  hmid.data_ptr(), T, H, I0, I1, _lib.i64x2((m0, m1)), inverse.data_ptr(), counters.data_ptr(), stream)
+
     def step():  # partition -> permute -> gate/up + SwiGLU -> down with the unpermute in its stores
         partition()
         permute()
@@ -175,7 +184,7 @@ def main():
                 t.zero_()
         permute(); gate_up(); down()
         fn = {"gate_up": gate_up, "down": down, "down_unpermute": down_unpermute, "permute": permute,
-              "permute_plain": permute_plain,
+              "permute_plain": permute_plain, "layer_one_launch": layer_one_launch,
               "unpermute": unpermute, "partition": partition,
               "copy": lambda: x_sorted.copy_(x)}[args.kernel_loop]
         for _ in range(args.steps):
