@@ -194,10 +194,34 @@ __device__ __forceinline__ void tile_coords(int v, const int* tiles_m, const int
   tc.tm = first_m + (in_patch - q * rows);
   tc.tn = q;
 }
+// The share of `n` tiles that XCD `x` walks when they are dealt out as evenly as possible, the XCDs taking their
+// places in the dealing order from `first` on (the first n % 8 places get one tile more): how many, and the index of
+// the first one (every XCD's share is a contiguous range).
+__device__ __forceinline__ void xcd_share(int n, int x, int first, int& count, int& start) {
+  const int q = n / kXcds, r = n % kXcds;
+  const int pos = (x - first + kXcds) % kXcds;
+  count = q + (pos < r ? 1 : 0);
+  start = pos * q + (pos < r ? pos : r);
+}
+// Workgroup slot t (XCD t % 8, place t / 8 among that XCD's workgroups and rounds) -> tile.  Each expert's tiles
+// are dealt to the XCDs separately, expert 1's starting at the XCD where expert 0's remainder ended, so every XCD
+// walks its share of expert 0 and then its share of expert 1, at most ceil(total / 8) tiles in all.  With one list
+// cut into eight ranges instead, a short second expert would sit at the end of the last XCD's range alone: cheap
+// tiles (the action expert's down projection, a tenth of the contraction) then replace expensive ones on one XCD
+// only, and the other seven run a longer list.
 __device__ __forceinline__ bool map_tile(int t, int total, const int* tiles_m, const int* tiles_n, TileCoord& tc) {
-  const int per = (total + kXcds - 1) / kXcds;
-  const int v = (t % kXcds) * per + t / kXcds;
-  if (v >= total) return false;
+  const int all0 = tiles_m[0] * tiles_n[0];
+  const int n0 = all0 < total ? all0 : total, n1 = total - n0;  // (a first launch of a tail split stops at `total`)
+  const int x = t % kXcds, j = t / kXcds;
+  int count, start;
+  xcd_share(n0, x, 0, count, start);
+  int v = start + j;
+  if (j >= count) {
+    const int j1 = j - count;
+    xcd_share(n1, x, n0 % kXcds, count, start);
+    if (j1 >= count) return false;
+    v = n0 + start + j1;
+  }
   tile_coords(v, tiles_m, tiles_n, tc);
   return true;
 }
@@ -217,6 +241,19 @@ __host__ __device__ inline int tail_split_point(int tiles0, int tiles1, int k0, 
   const int tail1 = tail < tiles1 ? tail : tiles1, tail0 = tail - tail1;
   const int counted = (tiles1 > 0 && tiles0 > 0 && 2ll * k1 <= k0) ? tail0 : tail;
   return 2 * counted <= cus ? full : total;
+}
+
+// The tile count that decides between the two tile shapes.  The small shape pays when the large tiles would leave
+// half of the CUs idle.  Tiles of an expert whose contraction is at most half as long as the other's do not count:
+// in the small shape they ride along as a cheap second helping of the first workgroups (4096 VL rows next to a
+// handful of action rows in the down launch: 128 tiles of K = 11008 and 8 of K = 1024 are one round of small tiles
+// plus a tenth, not 136 large tiles on 256 CUs).  Evaluated identically by the host and by both launches.
+__host__ __device__ inline long long shape_deciding_tiles(long long tiles0, long long tiles1, int k0, int k1) {
+  if (tiles0 > 0 && tiles1 > 0) {
+    if (2ll * k1 <= k0) return tiles0;
+    if (2ll * k0 <= k1) return tiles1;
+  }
+  return tiles0 + tiles1;
 }
 
 // Workgroup barrier without the fences of __syncthreads().  Those fences make the compiler wait for EVERY
@@ -388,7 +425,7 @@ __device__ __forceinline__ void dual_gemm_body(const Params& p, const int wg, co
   if (p.gate != 0) {
     constexpr int kBigN = SWIGLU ? BigTile::BN / 2 : BigTile::BN;
     auto big = [](int m, int n) { return (m <= 0 || n <= 0) ? 0 : ((m + BigTile::BM - 1) / BigTile::BM) * ((n + kBigN - 1) / kBigN); };
-    const bool few = big(g0.m, g0.n) + big(g1.m, g1.n) <= p.gate_tiles;
+    const bool few = shape_deciding_tiles(big(g0.m, g0.n), big(g1.m, g1.n), g0.k, g1.k) <= p.gate_tiles;
     if (few != (p.gate == 1)) return;  // uniform: the other tile shape's launch does this problem
   }
   int total = tiles_m[0] * tiles_n[0] + tiles_m[1] * tiles_n[1];  // the host bounds this below 2^31
@@ -1454,7 +1491,8 @@ int check_dims(const char* who, int64_t m, int64_t n, int64_t k, bool k_in_rows 
 // over the chip.  If the bounds fall on both sides of that threshold the choice is made on the device: both
 // shapes are launched and the one on the wrong side returns immediately.
 // tiles_by_expert: the host's exact 256 x 256 tile counts per expert, or null when only the device knows the row
-// split.  The fused FFN launches use the tail split: a second launch with 128 x 128 tiles takes the ragged last
+// split (the bounds are then on the plain sum of the tiles; where they straddle the threshold and the device
+// chooses, it chooses by shape_deciding_tiles like the host would).  The fused FFN launches use the tail split: a second launch with 128 x 128 tiles takes the ragged last
 // round when that pays; when the host cannot tell, both launches are made and the device decides (the second
 // returns at once if there is nothing to split).
 template <int MODE, bool KA = false, bool KB = false>
@@ -1462,7 +1500,14 @@ int launch_mfma(Params p, int64_t tiles_lo, int64_t tiles_hi, hipStream_t s, con
                 const int64_t* tiles_by_expert = nullptr) {
   const int cus = device_cu_count();
   const int threshold = cus / 2;
-  const bool small = tiles_lo <= threshold, big = tiles_hi > threshold;
+  bool small = tiles_lo <= threshold, big = tiles_hi > threshold;
+  if (tiles_by_expert != nullptr) {  // the host knows the split: the count that decides is shape_deciding_tiles'
+    small = shape_deciding_tiles(tiles_by_expert[0], tiles_by_expert[1], p.g[0].k, p.g[1].k) <= threshold;
+    big = !small;
+  } else if (!small && tiles_lo <= cus && (2ll * p.g[0].k <= p.g[1].k || 2ll * p.g[1].k <= p.g[0].k)) {
+    // at most one round of large tiles, and one expert's tiles may not count: the device has to choose
+    small = true;
+  }
   p.gate_tiles = threshold;
   p.split = 0;
   p.split_cus = cus;

@@ -932,6 +932,10 @@ def packed_block_forward(experts: PackedExperts, x: torch.Tensor, row_id_map: to
                                             x_tiled.data_ptr(), hmid.data_ptr(), T, H, I0, I1, host_rows_c, norm_ptr,
                                             float(eps), int(bool(residual)),
                                             counters.data_ptr() if _one_launch_ffn else None, stream))
+    if _checked and _one_launch_ffn and cap == 0 and int(counters[-1].item()):
+        counters.zero_()
+        raise RuntimeError("packed_block_forward: a wait inside the one-launch FFN ran into its bound (the result is "
+                           "undefined); native.set_one_launch_ffn(False) runs the separate launches")
     return out
 
 
