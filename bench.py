@@ -597,6 +597,12 @@ def config4_measurement(dev, weights):
         flops = 6.0 * H * (n_vl * I0 + n_act * I1)
         out[name] = {"us": round(t * 1e3, 1), "tflops": round(flops / t / 1e9, 1),
                      "us_with_host_row_counts": round(th * 1e3, 1)}
+        # the two figures above are one call between two events on an idle GPU (launch latency included); the same
+        # calls queued back to back, 50 per event pair, as a serving loop issues them
+        tq, _ = event_ms(lambda: moe.moe_layer_forward(x, types, weights), 6, warm=1, batch=50)
+        tqh, _ = event_ms(lambda: moe.moe_layer_forward(x, types, weights, host_rows=(n_vl, n_act)), 6, warm=1, batch=50)
+        out[name]["us_per_call_50_calls_queued"] = round(tq * 1e3, 1)
+        out[name]["us_per_call_50_calls_queued_with_host_row_counts"] = round(tqh * 1e3, 1)
         # the drop-in module called the way the reference's decoder calls it: every layer gets the same token-type
         # tensor and the CPU row ranges (act.py:257-261, 1274-1283), so the partition is shared between the layers
         x3, types2 = x.view(1, T, H), types.view(1, T)
