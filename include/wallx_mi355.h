@@ -181,8 +181,8 @@ int wx_dual_swiglu_ffn(const void* x_tiled, void* out, const int32_t* expert_off
 
 /* wx_dual_swiglu_ffn (optionally with the permute in front and wx_dual_down_proj_residual's closing add behind) as
  * ONE launch where that pays: when host_rows_per_expert is given and each of the two GEMMs is a single round of
- * 128 x 128 tiles (at most one per CU: the denoise step's few thousand action tokens), gate/up tiles and down tiles
- * share one grid, and a down tile starts as soon as the gate/up tiles of its 128 rows have finished instead of after a
+ * 128 x 128 tiles (at most one per CU: the denoise step's few thousand action tokens), or, without the host's row
+ * counts, for up to two rows per CU (512 on an MI355X), gate/up tiles and down tiles share one grid, and a down tile starts as soon as the gate/up tiles of its 128 rows have finished instead of after a
  * launch boundary.  Every other shape, or a NULL workspace, runs the launches of wx_[permute_rows_tiled +]
  * wx_dual_swiglu_ffn; results are bit-identical either way.  The host's row counts only choose the form.
  * x_rows: NULL, or the activations in token order, [num_rows, hidden] bf16 (out_row_id required): the permute is then

@@ -53,7 +53,8 @@ def _one_launch(p, xt, hm, out, res, off, inv, T, H, I0, I1, rows, ws, stream, x
 @pytest.mark.parametrize("T,m0,H,I0,I1,with_res,known_rows", [
     (2048, 0, 2048, 1536, 1024, False, True), (2048, 0, 2048, 1536, 1024, True, True), (1024, 1024, 256, 512, 1024, False, True),
     (1500, 700, 512, 448, 320, True, True), (129, 1, 1024, 64, 1024, False, True), (300, 300, 96, 32, 32, True, True),
-    (2048, 0, 2048, 1536, 1024, False, False),   # rows only known on the device
+    (2048, 0, 2048, 1536, 1024, False, False),   # rows only known on the device: too many for the one launch ...
+    (512, 0, 2048, 1536, 1024, False, False), (300, 200, 512, 448, 320, True, False),   # ... and few enough for it
     (4096, 100, 2048, 1024, 1024, True, True),   # more tiles than CUs
 ])
 def test_one_launch_ffn_equals_two_launches(dev, T, m0, H, I0, I1, with_res, known_rows):

@@ -1392,7 +1392,9 @@ __global__ __launch_bounds__(TS::kThreads, TS::kWgPerCu) void dual_gemm_kernel(P
 
 // The fused FFN launch (see FusedSync): workgroups [0, producers) run the gate/up form on `pg`, the rest the down
 // form on `pd`, both in the small tile shape.  `producers` is a multiple of 8, so a workgroup's index among its
-// form's workgroups names the same XCD as its index in the grid.
+// form's workgroups names the same XCD as its index in the grid.  (A workgroup that waits is a consumer, and what
+// it waits for belongs to workgroups with lower indices, which never wait: whatever part of the grid is resident,
+// the launch makes progress.)
 // AROWS: the producers read the token rows (fs.x through fs.gather) in place of the K-tiled activations.
 template <bool AROWS>
 __global__ __launch_bounds__(SmallTile::kThreads, SmallTile::kWgPerCu) void ffn_fused_kernel(Params pg, Params pd,
@@ -1838,7 +1840,7 @@ int launch_down(const FfnArgs& a, hipStream_t s) {
 // permute happens in their loads; a.x is not touched).  Returns 1 when the shape is not of that kind (nothing launched).
 constexpr size_t kFusedWorkspaceInts = 2 * static_cast<size_t>(kFusedCounters) + 1;  // two counter arrays, then the error flag
 int launch_ffn_fused(const FfnArgs& a, int* ws, hipStream_t s) {
-  if (a.host_rows == nullptr || ws == nullptr || a.keep_gate != nullptr) return 1;
+  if (ws == nullptr || a.keep_gate != nullptr) return 1;
   // (whatever the real split of the rows: the counters hold this many row blocks per expert)
   if (a.rows > static_cast<int64_t>(kFusedMaxRowBlocks) * SmallTile::BM) return 1;
   // (token rows are addressed with 31-bit byte offsets)
@@ -1848,10 +1850,25 @@ int launch_ffn_fused(const FfnArgs& a, int* ws, hipStream_t s) {
   int need[2] = {0, 0};
   const int64_t down_cols = ceil_div(a.hidden, SmallTile::BN);
   for (int e = 0; e < 2; ++e) {
-    const int64_t row_blocks = ceil_div(a.host_rows[e], SmallTile::BM);
     need[e] = static_cast<int>(ceil_div(a.inter[e], SmallTile::BN / 2));
-    gate_tiles += row_blocks * need[e];
-    down_tiles += row_blocks * down_cols;
+    if (a.host_rows != nullptr) {
+      const int64_t row_blocks = ceil_div(a.host_rows[e], SmallTile::BM);
+      gate_tiles += row_blocks * need[e];
+      down_tiles += row_blocks * down_cols;
+    }
+  }
+  const bool rows_known = a.host_rows != nullptr;
+  if (!rows_known) {
+    // The split of the rows is only known on the device.  The launch is right for any split (workgroups take as
+    // many tiles as there are), so what the host has to settle is whether it is the faster form whatever the split.
+    // Up to two rows per CU it is: 24-27 against 29-34 us with every row on the narrow expert, 2-9 % ahead with a
+    // mix, within 4 % with every row on the wide expert (256 and 512 rows, experts 11008 / 1024).  Beyond that, rows
+    // on the wide expert cost the one workgroup of producers per CU more than they cost the separate launches' large
+    // tiles (+12 % at 1024 rows, +19 % at 2048, against -25 % / -31 % with none); with two workgroups of producers
+    // per CU the consumers land wherever a producer has left, two of them on one CU while others idle (+25 % on a
+    // half-and-half split of 1024 rows).  So larger problems take the one launch only with the host's row counts.
+    if (a.rows > 2 * cus) return 1;
+    gate_tiles = down_tiles = cus;
   }
   if (gate_tiles == 0 || gate_tiles > cus || down_tiles > cus) return 1;
   Params pg = gate_up_params(a), pd = down_params(a);
