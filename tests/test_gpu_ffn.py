@@ -757,6 +757,27 @@ def test_moe_block_backward_with_one_expert_frozen(dev, frozen_expert):
         assert got is not None and torch.equal(got, want)
 
 
+@pytest.mark.parametrize("rows0,rows1,out0,out1,n", [(4200, 300, 512, 256, 384), (6000, 0, 768, 128, 256),
+                                                     (3000, 500, 512, 256, 384)])
+def test_weight_gradients_with_the_wide_experts_contraction_in_two_halves(dev, rows0, rows1, out0, out1, n):
+    """moe._weight_grads: dW_e = a_e^T b_e.  With 4096 rows or more on expert 0 and a tile count that fills the chip
+    better that way, its contraction runs as two halves in one launch and the two bf16 results are added (one
+    rounding more than the single product); fewer rows take the plain dual launch.  Both against the fp32 product,
+    tolerance 2e-2 * rms + 1e-2 * |ref|."""
+    g = torch.Generator().manual_seed(rows0 + out0)
+    a0, a1 = torch.randn(rows0, out0, generator=g).to(torch.bfloat16), torch.randn(rows1, out1, generator=g).to(torch.bfloat16)
+    b0, b1 = torch.randn(rows0, n, generator=g).to(torch.bfloat16), torch.randn(rows1, n, generator=g).to(torch.bfloat16)
+    g0, g1 = moe._weight_grads(a0.to(dev), a1.to(dev), b0.to(dev), b1.to(dev), n, n, (True, True))
+    for got, a, b in ((g0, a0, b0), (g1, a1, b1)):
+        ref = a.float().T @ b.float()
+        assert got.shape == ref.shape
+        rms = float(ref.pow(2).mean().sqrt()) if ref.numel() else 0.0
+        bad = (got.float().cpu() - ref).abs() > 2e-2 * rms + 1e-2 * ref.abs()
+        assert not bad.any(), f"{int(bad.sum())} of {bad.numel()} outside tolerance"
+    only0, none1 = moe._weight_grads(a0.to(dev), a1.to(dev), b0.to(dev), b1.to(dev), n, n, (True, False))
+    assert none1 is None and torch.equal(only0, g0)
+
+
 def test_moe_block_under_bf16_autocast_takes_fp32_input(dev):
     """Under bf16 autocast (the reference trains that way, train_qact.py:65) the nn.Linear layers of the reference block
     take an fp32 input and answer in bf16; the drop-in does the same, forward and backward.  Outside autocast an fp32

@@ -166,6 +166,36 @@ def _dual(a0, a1, w0, w1, n0, n1, trans_a, trans_b, want=(True, True)):
     return (o0 if want[0] else None), (o1 if want[1] else None)
 
 
+_cu_counts = {}
+
+
+def _cus(device: torch.device) -> int:
+    n = _cu_counts.get(device.index)
+    if n is None:
+        n = _cu_counts[device.index] = torch.cuda.get_device_properties(device).multi_processor_count
+    return n
+
+
+def _weight_grads(a0, a1, b0, b1, n0, n1, want):
+    """The experts' weight gradients dW_e = a_e^T b_e (a_e [rows_e, out_e], b_e [rows_e, n_e]: the contraction runs over
+    the expert's tokens) as one launch, like _dual -- unless the wide expert's output is an awkward number of 256 x 256
+    tiles for the chip.  11008 x 2048 is 344 tiles: two rounds on 256 CUs for 1.34 rounds of work.  Its contraction
+    is tens of thousands of tokens long, so it is cut in two: both halves go into one launch as its two problems (688
+    tiles of half the length: three rounds of half the time), their bf16 results are added, and the narrow expert's
+    gradient (a few cheap tiles) takes a launch of its own.  The sum of two rounded halves carries one rounding more
+    than the single product; the gradient tests' tolerance covers it."""
+    if want[0] and a0.size(0) >= 4096:
+        cus = _cus(a0.device)
+        tiles = -(-a0.size(1) // 256) * -(-n0 // 256)
+        if -(-2 * tiles // cus) < 2 * -(-tiles // cus):
+            h = a0.size(0) // 2
+            first, second = _dual(a0[:h], a0[h:], b0[:h], b0[h:], n0, n0, True, False)
+            first.add_(second)
+            other = _dual(None, a1, None, b1, n0, n1, True, False, want=(False, True))[1] if want[1] else None
+            return first, other
+    return _dual(a0, a1, b0, b1, n0, n1, True, False, want=want)
+
+
 class _MoeBlockFunction(torch.autograd.Function):
     """[RMSNorm ->] permute -> both experts' SwiGLU FFN -> unpermute [+ residual] with a backward (act.py:105-162,
     and the decoder layer's lines around it, act.py:256-265, under autograd).
@@ -265,11 +295,11 @@ class _MoeBlockFunction(torch.autograd.Function):
         # weight gradients only of the experts that train: fine-tuning with the VL side frozen (the reference's
         # freeze_vlm mode trains `moe.experts.1.*` alone, qwen_vl_act_trainer.py:530-536) skips the three large ones
         if need[5] or need[8]:  # gate weights
-            grads[0], grads[3] = _dual(dg0, dg1, x0, x1, H, H, True, False, want=(need[5], need[8]))
+            grads[0], grads[3] = _weight_grads(dg0, dg1, x0, x1, H, H, (need[5], need[8]))
         if need[6] or need[9]:  # up weights
-            grads[1], grads[4] = _dual(du0, du1, x0, x1, H, H, True, False, want=(need[6], need[9]))
+            grads[1], grads[4] = _weight_grads(du0, du1, x0, x1, H, H, (need[6], need[9]))
         if need[7] or need[10]:  # down weights
-            grads[2], grads[5] = _dual(dy0, dy1, hm0, hm1, I0, I1, True, False, want=(need[7], need[10]))
+            grads[2], grads[5] = _weight_grads(dy0, dy1, hm0, hm1, I0, I1, (need[7], need[10]))
         dx = dnorm = None
         if need_x or need_norm:
             # dX = dG Wg + dU Wu: the second product accumulates onto the first in its epilogue (bf16 + bf16, rounded
