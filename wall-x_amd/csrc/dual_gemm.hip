@@ -1494,9 +1494,10 @@ int check_dims(const char* who, int64_t m, int64_t n, int64_t k, bool k_in_rows 
 // shapes are launched and the one on the wrong side returns immediately.
 // tiles_by_expert: the host's exact 256 x 256 tile counts per expert, or null when only the device knows the row
 // split (the bounds are then on the plain sum of the tiles; where they straddle the threshold and the device
-// chooses, it chooses by shape_deciding_tiles like the host would).  The fused FFN launches use the tail split: a second launch with 128 x 128 tiles takes the ragged last
-// round when that pays; when the host cannot tell, both launches are made and the device decides (the second
-// returns at once if there is nothing to split).
+// chooses, it chooses by shape_deciding_tiles like the host would).  A launch of large tiles uses the tail split: a
+// second launch with 128 x 128 tiles takes the ragged last round when that pays (the row-major op, whose sizes the
+// host knows, decides it on the host); when the host cannot tell, both launches are made and the device decides (the
+// second returns at once if there is nothing to split).
 template <int MODE, bool KA = false, bool KB = false>
 int launch_mfma(Params p, int64_t tiles_lo, int64_t tiles_hi, hipStream_t s, const char* who,
                 const int64_t* tiles_by_expert = nullptr) {
@@ -1522,7 +1523,7 @@ int launch_mfma(Params p, int64_t tiles_lo, int64_t tiles_hi, hipStream_t s, con
     p.gate = small ? 2 : 0;
     using Big = BigTileFor<MODE>;
     static_assert(Big::kWgPerCu == 1, "the split counts one large tile per CU and round");
-    bool split = MODE != kGeneric && tiles_hi > cus;
+    bool split = (MODE != kGeneric || tiles_by_expert != nullptr) && tiles_hi > cus;
     if (split && tiles_by_expert != nullptr) {
       const int64_t all = tiles_by_expert[0] + tiles_by_expert[1];
       split = all < INT32_MAX && tail_split_point(static_cast<int>(tiles_by_expert[0]), static_cast<int>(tiles_by_expert[1]),
@@ -1530,12 +1531,10 @@ int launch_mfma(Params p, int64_t tiles_lo, int64_t tiles_hi, hipStream_t s, con
     }
     p.split = split ? 1 : 0;
     hipLaunchKernelGGL((dual_gemm_kernel<MODE, Big, KA, KB>), dim3(cus), dim3(Big::kThreads), 0, s, p);
-    if constexpr (MODE != kGeneric) {
-      if (split) {
-        p.split = 2;
-        hipLaunchKernelGGL((dual_gemm_kernel<MODE, TailTile, KA, KB>), dim3(cus * TailTile::kWgPerCu),
-                           dim3(TailTile::kThreads), 0, s, p);
-      }
+    if (split) {
+      p.split = 2;
+      hipLaunchKernelGGL((dual_gemm_kernel<MODE, TailTile, KA, KB>), dim3(cus * TailTile::kWgPerCu),
+                         dim3(TailTile::kThreads), 0, s, p);
     }
   }
   return check_launch(who);
@@ -1637,10 +1636,13 @@ int dual_gemm_impl(const void* in0, const void* in1, const void* w0, const void*
     const int64_t tiles = ceil_div(mm0, BigTile::BM) * ceil_div(n0, BigTile::BN) + ceil_div(mm1, BigTile::BM) * ceil_div(n1, BigTile::BN);
     const char* who = "dual_gemm_kernel<generic>";
     gemm_path_note(WX_GEMM_PATH_MFMA);
-    if (!trans_a && trans_b) return launch_mfma<kGeneric, false, false>(p, tiles, tiles, s, who);
-    if (!trans_a && !trans_b) return launch_mfma<kGeneric, false, true>(p, tiles, tiles, s, who);
-    if (trans_a && trans_b) return launch_mfma<kGeneric, true, false>(p, tiles, tiles, s, who);
-    return launch_mfma<kGeneric, true, true>(p, tiles, tiles, s, who);
+    // (the host knows both problems' sizes: it settles the tile shape and the split of a ragged last round itself)
+    const int64_t by_expert[2] = {ceil_div(mm0, BigTile::BM) * ceil_div(n0, BigTile::BN),
+                                  ceil_div(mm1, BigTile::BM) * ceil_div(n1, BigTile::BN)};
+    if (!trans_a && trans_b) return launch_mfma<kGeneric, false, false>(p, tiles, tiles, s, who, by_expert);
+    if (!trans_a && !trans_b) return launch_mfma<kGeneric, false, true>(p, tiles, tiles, s, who, by_expert);
+    if (trans_a && trans_b) return launch_mfma<kGeneric, true, false>(p, tiles, tiles, s, who, by_expert);
+    return launch_mfma<kGeneric, true, true>(p, tiles, tiles, s, who, by_expert);
   }
   gemm_path_note(WX_GEMM_PATH_FMA);
   hipLaunchKernelGGL(dual_gemm_reference_layout_kernel, dim3(device_cu_count() * 4), dim3(256), 0, s, p, trans_a, trans_b);
