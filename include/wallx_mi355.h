@@ -182,8 +182,8 @@ int wx_dual_swiglu_ffn(const void* x_tiled, void* out, const int32_t* expert_off
 /* wx_dual_swiglu_ffn (optionally with the permute in front and wx_dual_down_proj_residual's closing add behind) as
  * ONE launch where that pays: when host_rows_per_expert is given and each of the two GEMMs is a single round of
  * 128 x 128 tiles (at most one per CU: the denoise step's few thousand action tokens), or, without the host's row
- * counts, for up to two rows per CU (512 on an MI355X), gate/up tiles and down tiles share one grid, and a down tile starts as soon as the gate/up tiles of its 128 rows have finished instead of after a
- * launch boundary.  Every other shape, or a NULL workspace, runs the launches of wx_[permute_rows_tiled +]
+ * counts, for up to two rows per CU (512 on an MI355X), gate/up tiles and down tiles share one grid, and a down tile
+ * starts as soon as the gate/up tiles of its 128 rows have finished instead of after a launch boundary.  Every other shape, or a NULL workspace, runs the launches of wx_[permute_rows_tiled +]
  * wx_dual_swiglu_ffn; results are bit-identical either way.  The host's row counts only choose the form.
  * x_rows: NULL, or the activations in token order, [num_rows, hidden] bf16 (out_row_id required): the permute is then
  * part of the call and x_tiled only a work buffer -- in the one launch the gate/up tiles read the token rows through
@@ -193,6 +193,9 @@ int wx_dual_swiglu_ffn(const void* x_tiled, void* out, const int32_t* expert_off
  * launch leaves it zero again.  Calls that share a workspace must not overlap (one workspace per stream).
  * Inside the one launch tiles wait on counters in the workspace that other tiles advance; every wait is bounded
  * (seconds), and a wait that runs into its bound stores 1 into the workspace's last int (the result is then undefined).
+ * A launch alone on the GPU, or two of them at once on two streams, cannot run into the bound (the tiles waited for
+ * always hold or get a place on the chip); a caller that keeps three or more in flight together on one GPU should
+ * read that int, or pass a NULL workspace.
  * No counterpart in the reference, whose experts are separate nn.Linear launches (act.py:79-82, 142-154). */
 size_t wx_ffn_fused_workspace_bytes(void);
 int wx_dual_swiglu_ffn_fused(const void* x_rows, void* x_tiled, void* out, const void* residual,

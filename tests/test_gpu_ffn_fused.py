@@ -196,3 +196,37 @@ def test_block_forward_with_and_without_the_one_launch_ffn(dev, residual, monkey
         got[flag] = native.packed_block_forward(experts, x, rmap, inv, off, rows, residual=residual)
     torch.cuda.synchronize()
     assert torch.equal(got[True], got[False])
+
+
+def test_one_launch_ffn_on_two_streams_at_once(dev):
+    """Two streams issue the one launch at the same time, each with a workspace of its own (what
+    native.packed_block_forward keeps per stream): workgroups of both launches share the CUs, each launch's down tiles
+    wait on its own counters, and both results are those of the separate launches.  (With two such launches resident
+    an XCD's 64 workgroup places cannot all be held by waiting down workgroups of the other launch -- one launch has
+    at most 32 of them per XCD -- so the gate/up workgroups of either always find a place.)"""
+    T, m0, H, I0, I1 = 2048, 0, 2048, 1536, 1024
+    pad = native.padded_sorted_rows(T)
+    rows = _lib.i64x2((m0, T - m0))
+    lanes = []
+    for seed in (21, 22):
+        _, packed, _, x, res, off, inv, xt = _case(dev, T, m0, H, I0, I1, seed)
+        p = [t.data_ptr() for t in packed]
+        hm = [torch.zeros(pad * max(I0, I1), dtype=torch.bfloat16, device=dev) for _ in range(2)]
+        out = [torch.empty(T, H, dtype=torch.bfloat16, device=dev) for _ in range(2)]
+        _two_launches(p, xt, hm[0], out[0], res, off, inv, T, H, I0, I1, rows, torch.cuda.current_stream().cuda_stream)
+        lanes.append(dict(packed=packed, p=p, x=x, res=res, off=off, inv=inv, xt=torch.zeros_like(xt), hm=hm, out=out,
+                          work=_workspace(dev), stream=torch.cuda.Stream()))
+    torch.cuda.synchronize()
+    for rep in range(3):
+        for ln in lanes:
+            ln["out"][1].zero_()
+            ln["hm"][1].zero_()
+        torch.cuda.synchronize()
+        for _ in range(12):  # the host issues faster than a launch runs: the two streams' launches overlap
+            for ln in lanes:
+                _one_launch(ln["p"], ln["xt"], ln["hm"][1], ln["out"][1], ln["res"], ln["off"], ln["inv"], T, H, I0, I1,
+                            rows, ln["work"], ln["stream"].cuda_stream, x_rows=ln["x"])
+        torch.cuda.synchronize()
+        for i, ln in enumerate(lanes):
+            assert torch.equal(ln["out"][0], ln["out"][1]) and torch.equal(ln["hm"][0], ln["hm"][1]), f"rep {rep} stream {i}"
+            assert int(ln["work"].abs().sum()) == 0, f"rep {rep} stream {i}: counters or the error flag left set"

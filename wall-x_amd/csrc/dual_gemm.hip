@@ -281,10 +281,13 @@ __device__ __forceinline__ unsigned char* lds_array() {
 
 // The fused FFN launch: gate/up tiles (producers) and down tiles (consumers) in one grid.  A down tile of row block
 // rb reads the intermediate rows that the gate/up tiles of the same row block write, so it waits until `ready[rb]`
-// has reached the number of those tiles.  Workgroups are dispatched in index order and the producers come first, so
-// a consumer only ever waits for workgroups that are already running and never wait themselves.  Its wait is
-// bounded all the same (kFusedWaitTicks of the 100 MHz clock; then `*error` is set and the tile goes ahead on
-// whatever is there).  The last consumer past the wait of a row block clears the row block's counters, so a launch
+// has reached the number of those tiles.  An XCD places its share of a launch's workgroups in index order and the
+// producers come first, so on every XCD the producers have their places before a consumer gets one, and producers
+// never wait: a launch alone on the chip always makes progress.  So do two of them in flight together on their own
+// workspaces (an XCD has 64 places for workgroups of this size, a launch at most 32 consumers per XCD, and a
+// launch's consumers hold no place on an XCD where its producers still wait for one: waiting workgroups cannot
+// fill an XCD).  The wait is bounded all the same (kFusedWaitTicks of the 100 MHz clock; then `*error` is set and
+// the tile goes ahead on whatever is there), which is what three or more concurrent launches would fall back on.  The last consumer past the wait of a row block clears the row block's counters, so a launch
 // leaves the workspace as it found it: all zero.
 // The producers can read their A operand from the token rows themselves (AROWS below: `x` through `gather`), which
 // makes the permute into the K-tiled activation matrix part of the launch.
