@@ -196,6 +196,9 @@ int wx_dual_swiglu_ffn(const void* x_tiled, void* out, const int32_t* expert_off
  * A launch alone on the GPU, or two of them at once on two streams, cannot run into the bound (the tiles waited for
  * always hold or get a place on the chip); a caller that keeps three or more in flight together on one GPU should
  * read that int, or pass a NULL workspace.
+ * Unless the previous one launch of the calling thread on the same workspace ran on the same six weight tensors (a
+ * loop over one layer), the one launch also requests the gate/up weights ahead of its K loops, for weights that come
+ * from HBM as every layer of a model's do.
  * No counterpart in the reference, whose experts are separate nn.Linear launches (act.py:79-82, 142-154). */
 size_t wx_ffn_fused_workspace_bytes(void);
 int wx_dual_swiglu_ffn_fused(const void* x_rows, void* x_tiled, void* out, const void* residual,

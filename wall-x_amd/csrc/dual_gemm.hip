@@ -301,6 +301,9 @@ struct FusedSync {
   int* passed;    // ... down tiles past their wait
   int* error;     // set to 1 when a wait ran into its bound
   int need[2];    // gate/up tiles per row block of expert e
+  const __bf16* warm_b[2][2];  // the producers' weights (gate, up of expert e), K-tiled; null: nothing to warm
+  int warm_ldb[2];             // their row blocks per column block
+  int warm_k;                  // their contraction length
   int consumers;  // down tiles per row block
   // AROWS: the activations in token order, [tokens, hidden] bf16 row-major, and the partition's sorted_row_id
   // (sorted position -> token)
@@ -811,6 +814,45 @@ __device__ __forceinline__ void dual_gemm_body(const Params& p, const int wg, co
       __hip_atomic_store(passed + rb * kFusedCounterStride, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
   };
+  // Fused launch, consumer, wavefronts that issue no loads: while the workgroup waits for its row block they pull
+  // a share of the PRODUCERS' weights through this XCD's L2, so that weights which come from HBM (every layer of a
+  // model has its own) are on their way before the producers' ring, four K steps deep, asks for them.  Workgroup c
+  // of the consumers sits on the XCD of producer workgroup c and takes that producer's tile: the K steps
+  // k = tm (mod kGroupM) of its gate and up column blocks (the producers of an XCD that share a column tile are the
+  // kGroupM tile rows of a patch).  The loads are LDS-direct into the still unused first A slot and are waited for
+  // before the barrier that ends the wait.  fs.warm_b is null when the host expects the weights in the caches.
+  bool warm_pending = true;
+  auto warm_producer_weights = [&]() {
+    if constexpr (ROLE == 2) {
+      const int total_g = tiles_m[0] * fs.need[0] + tiles_m[1] * fs.need[1];
+      TileCoord tg;
+      if (wg < total_g && map_tile(wg, total_g, tiles_m, fs.need, tg)) {
+        const int e = tg.group;
+        static_assert(TS::kWaves - kLoadWaves == 4, "two wavefronts per matrix, each every other K step of the share");
+        const int q = wave - kLoadWaves;  // 0 .. 3: matrix q & 1, half q >> 1 of the share
+        const __bf16* base = fs.warm_b[e][q & 1];
+        if (base != nullptr) {
+          const int ldb = fs.warm_ldb[e];
+          const int nkb = fs.warm_k / kBlkCols;
+          const int64_t bytes = (static_cast<int64_t>(nkb) * ldb) << 10;
+          if (bytes < 0x7fffff00ll) {
+            const __amdgpu_buffer_rsrc_t r = make_rsrc(base, static_cast<uint32_t>(bytes));
+            unsigned char* dummy = slot_a(0) + q * 1024;
+            constexpr int kGuBlocks = TS::BN / 2 / kBlkRows;  // row blocks of a gate/up column tile, per matrix
+            const int blk0 = tg.tn * kGuBlocks;
+            for (int ks = tg.tm % kGroupM + kGroupM * (q >> 1); ks < nkb; ks += 2 * kGroupM) {
+#pragma unroll
+              for (int i = 0; i < kGuBlocks; ++i) {
+                const uint32_t off = static_cast<uint32_t>((static_cast<int64_t>(ks) * ldb + blk0 + i) << 10) + lane * 16;
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(r, LDS_PTR(dummy), 16, off, 0, 0, 0);
+              }
+            }
+            __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));
+          }
+        }
+      }
+    }
+  };
   int passed_before = 0;
 
   f32x16 acc[FM][FN];
@@ -1280,6 +1322,12 @@ __device__ __forceinline__ void dual_gemm_body(const Params& p, const int wg, co
       if constexpr (LD) {
 #pragma unroll
         for (int s = 0; s + 1 < kStages; ++s) issue_b_ahead(L, s, slot_b(s));
+      }
+      if constexpr (!LD && ASYM) {
+        if (warm_pending) {
+          warm_pending = false;
+          warm_producer_weights();
+        }
       }
       wait_for_count(fs.ready, fs.passed, S.row_block, fs.need[tc.group], passed_before);
       if constexpr (LD) {
@@ -1843,6 +1891,29 @@ int launch_down(const FfnArgs& a, hipStream_t s) {
 // Both launches as one (ffn_fused_kernel), for the shapes where each is a single round of small tiles with the row
 // counts known on the host -- a denoise step.  With a.x_rows the gate/up tiles read the token rows themselves (the
 // permute happens in their loads; a.x is not touched).  Returns 1 when the shape is not of that kind (nothing launched).
+// Whether the one launch that last used workspace `ws` from this thread ran on the same weights (they are then
+// taken to be in the caches still, and the launch does not pull them in ahead of its K loops: in a loop over one
+// layer that would cost 0.9 us per launch, where for a model's layers, each with weights of its own, it saves 2).
+// A guess that only decides this; a few workspaces (streams) per thread are remembered.
+bool weights_of_last_launch(const void* ws, const FfnArgs& a) {
+  struct Seen { const void* ws; const void* w[6]; };
+  constexpr int kSeen = 8;
+  thread_local Seen seen[kSeen] = {};
+  thread_local int next = 0;
+  const void* w[6] = {a.gate[0], a.up[0], a.down[0], a.gate[1], a.up[1], a.down[1]};
+  for (Seen& s : seen) {
+    if (s.ws != ws) continue;
+    bool same = true;
+    for (int i = 0; i < 6; ++i) { same = same && s.w[i] == w[i]; s.w[i] = w[i]; }
+    return same;
+  }
+  Seen& s = seen[next];
+  next = (next + 1) % kSeen;
+  s.ws = ws;
+  for (int i = 0; i < 6; ++i) s.w[i] = w[i];
+  return false;
+}
+
 constexpr size_t kFusedWorkspaceInts = 2 * static_cast<size_t>(kFusedCounters) + 1;  // two counter arrays, then the error flag
 int launch_ffn_fused(const FfnArgs& a, int* ws, hipStream_t s) {
   if (ws == nullptr || a.keep_gate != nullptr) return 1;
@@ -1886,6 +1957,14 @@ int launch_ffn_fused(const FfnArgs& a, int* ws, hipStream_t s) {
   fs.need[0] = need[0];
   fs.need[1] = need[1];
   fs.consumers = static_cast<int>(down_cols);
+  if (!weights_of_last_launch(ws, a)) {
+    for (int e = 0; e < 2; ++e) {
+      fs.warm_b[e][0] = pg.g[e].b0;
+      fs.warm_b[e][1] = pg.g[e].b1;
+      fs.warm_ldb[e] = pg.g[e].ldb;
+    }
+    fs.warm_k = static_cast<int>(a.hidden);
+  }
   fs.x = static_cast<const __bf16*>(a.x_rows);
   fs.gather = a.out_row_id;
   const int producers = static_cast<int>((gate_tiles + kXcds - 1) / kXcds * kXcds);
