@@ -676,7 +676,21 @@ def config4_measurement(dev, weights):
                 stack_distinct()
             tg2, _ = event_ms(graph2.replay, 10, warm=3)
             out[name]["us_per_layer_hip_graph_replay_36_distinct_action_experts"] = round(tg2 * 1e3 / layers, 1)
-            del graph2, per_layer
+            del graph2
+            native.set_one_launch_ffn(False)
+            try:
+                side.wait_stream(torch.cuda.current_stream())
+                with torch.cuda.stream(side):
+                    stack_distinct()
+                torch.cuda.current_stream().wait_stream(side)
+                graph4 = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph4):
+                    stack_distinct()
+                tg4, _ = event_ms(graph4.replay, 10, warm=3)
+            finally:
+                native.set_one_launch_ffn(True)
+            out[name]["us_per_layer_hip_graph_replay_36_distinct_action_experts_three_launches"] = round(tg4 * 1e3 / layers, 1)
+            del graph4, per_layer
     return out
 
 
