@@ -757,6 +757,50 @@ def test_moe_block_backward_with_one_expert_frozen(dev, frozen_expert):
         assert got is not None and torch.equal(got, want)
 
 
+def test_moe_block_backward_takes_the_row_counts_from_the_partitions_read_back(dev, monkeypatch):
+    """The backward needs the per-expert row counts on the host (act.py:1274-1283 has them there).  They come from the
+    asynchronous read-back that the cached partition started; once it has landed, a forward + backward copies nothing
+    to the host, and the gradients are those of a backward that waited for expert_offsets."""
+    class Cfg:
+        experts = [{"hidden_size": 128, "intermediate_size": 320, "hidden_act": "silu"},
+                   {"hidden_size": 128, "intermediate_size": 128, "hidden_act": "silu"}]
+
+    g = torch.Generator().manual_seed(14)
+    block = moe.SparseMoeBlock(Cfg(), 2).to(torch.bfloat16)
+    with torch.no_grad():
+        for prm in block.parameters():
+            prm.copy_(_bf(prm.shape, g, 0.08))
+    block = block.to(dev)
+    x = _bf((1, 600, 128), g).to(dev)
+    types = (torch.rand(1, 600, generator=g) > 0.6).to(dev)
+    dy = _bf((1, 600, 128), g).to(dev)
+
+    def step(prepare=None):
+        for prm in block.parameters():
+            prm.grad = None
+        xd = x.clone().requires_grad_(True)
+        y = block(xd, types)
+        if prepare is not None:
+            prepare()
+        y.backward(dy)
+        return [xd.grad.clone()] + [prm.grad.clone() for prm in block.parameters()]
+
+    first = step()          # partitions; the read-back may or may not have landed when the backward starts
+    torch.cuda.synchronize()
+    copies = []
+    to_host = torch.Tensor.cpu
+
+    def counting(self, *a, **k):
+        copies.append(tuple(self.shape))
+        return to_host(self, *a, **k)
+
+    second = step(lambda: monkeypatch.setattr(torch.Tensor, "cpu", counting))
+    monkeypatch.setattr(torch.Tensor, "cpu", to_host)
+    assert copies == [], f"the backward copied {copies} to the host"
+    for a, b in zip(first, second):
+        assert torch.equal(a, b)
+
+
 @pytest.mark.parametrize("rows0,rows1,out0,out1,n", [(4200, 300, 512, 256, 384), (6000, 0, 768, 128, 256),
                                                      (3000, 500, 512, 256, 384)])
 def test_weight_gradients_with_the_wide_experts_contraction_in_two_halves(dev, rows0, rows1, out0, out1, n):

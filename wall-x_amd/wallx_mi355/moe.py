@@ -209,8 +209,8 @@ class _MoeBlockFunction(torch.autograd.Function):
     The normed, sorted rows the weight gradients contract over are recomputed (one pass, where the plain block
     permutes x), and the unpermute of dX carries the norm's backward and the residual branch's gradient (one pass,
     which also sums the norm weight's gradient).  Intermediate sizes that are not multiples of 64 recompute the two
-    projections instead.  The per-expert row counts are read back from the device once per backward (the forward
-    never synchronises)."""
+    projections instead.  The per-expert row counts come from the partition's asynchronous read-back (Routing.host_rows);
+    only a routing without one makes the backward wait for a copy of expert_offsets (the forward never synchronises)."""
 
     N_FIXED = 8  # inputs in front of the six weights
 
@@ -235,6 +235,13 @@ class _MoeBlockFunction(torch.autograd.Function):
         n0 = _MoeBlockFunction.N_FIXED
         frozen = tuple(not n for n in ctx.needs_input_grad[n0:n0 + 6])
         res_in_stores = x if (residual and sorted_row_id is not None) else None
+        # the partition's own read-back of the row counts, once it has landed (never consulted while capturing): one
+        # dispatch per GEMM in the forward, and a backward that starts without a synchronisation
+        ctx.rows_when_ready = scratch.get("rows_when_ready")
+        rows = None
+        if ctx.rows_when_ready is not None and \
+                native.capture_id(torch.cuda.current_stream(x.device).cuda_stream) == 0:
+            rows = ctx.rows_when_ready()
         saved = [x, row_id_map, expert_offsets]
         if ctx.has_norm:
             saved.append(norm_weight)
@@ -242,12 +249,13 @@ class _MoeBlockFunction(torch.autograd.Function):
             saved.append(sorted_row_id)
         if ctx.keep:
             y, gate_keep, up_keep, scratch["hmid"] = native.dual_swiglu_ffn_keep(
-                scratch["x_tiled"], T, expert_offsets, w, hmid=scratch.get("hmid"), out_row_id=sorted_row_id,
-                frozen=frozen, residual=res_in_stores)
+                scratch["x_tiled"], T, expert_offsets, w, hmid=scratch.get("hmid"), host_rows=rows,
+                out_row_id=sorted_row_id, frozen=frozen, residual=res_in_stores)
             saved += [gate_keep, up_keep]
         else:
             y = native.dual_swiglu_ffn(scratch["x_tiled"], T, expert_offsets, w, hmid=scratch.get("hmid"),
-                                       out_row_id=sorted_row_id, cache_packed=frozen, residual=res_in_stores)
+                                       host_rows=rows, out_row_id=sorted_row_id, cache_packed=frozen,
+                                       residual=res_in_stores)
         ctx.save_for_backward(*saved, *weights)
         if sorted_row_id is None:
             if residual:
@@ -268,8 +276,12 @@ class _MoeBlockFunction(torch.autograd.Function):
         n0 = _MoeBlockFunction.N_FIXED
         need = (None,) * 5 + tuple(ctx.needs_input_grad[n0:n0 + 6])  # need[5..10]: the six weights
         need_x, need_norm = ctx.needs_input_grad[0], ctx.has_norm and ctx.needs_input_grad[1]
-        o = expert_offsets.cpu().tolist()
-        m0, m1 = o[1] - o[0], o[2] - o[1]
+        rows = ctx.rows_when_ready() if ctx.rows_when_ready is not None else None
+        if rows is not None:
+            m0, m1 = int(rows[0]), int(rows[1])
+        else:  # no read-back under way (a routing made by hand or under capture), or it has not landed: wait for one
+            o = expert_offsets.cpu().tolist()
+            m0, m1 = o[1] - o[0], o[2] - o[1]
         dy = dy.contiguous().to(torch.bfloat16)
         if ctx.has_norm:  # the experts' input rows: normed, in sorted order
             xs = native.rmsnorm_permute_rows(x.detach(), norm_weight.detach(), ctx.eps, sorted_row_id)
@@ -445,7 +457,7 @@ class SparseMoeBlock(nn.Module):
         need = native.padded_sorted_rows(x.size(0)) * max(self._dims[1:])
         if self._hmid is None or self._hmid.numel() < need or self._hmid.device != x.device:
             self._hmid = torch.empty(need, dtype=torch.bfloat16, device=x.device)
-        scratch = {"x_tiled": self._x_tiled, "hmid": self._hmid}
+        scratch = {"x_tiled": self._x_tiled, "hmid": self._hmid, "rows_when_ready": routing.rows_when_ready}
         y = _MoeBlockFunction.apply(x, norm_weight, routing.row_id_map, routing.expert_offsets,
                                     routing.sorted_row_id, scratch, float(eps), bool(residual), *flat)
         self._x_tiled = scratch["x_tiled"]
